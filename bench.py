@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""Benchmark of SLAYER's temporal kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one pass of the hot path over one batch of synthetic input, forward and backward:
+
+    forward : a = psp(spikes)  (conv, 77-tap SRM kernel)   s = spike(u)   d = delayShift(s, 1)
+    backward: gd = shift(g, -1)   gs = spikeBackward(gd, u')   ga = corr(gs, SRM kernel)
+
+on the NMNIST-CNN-shaped activation tensor (12, 16, 34, 34, 300), fp32, all inputs resident in
+HBM.  The spike kernel updates its input in place, so each step works on its own pre-made copy
+of the membrane potential (made before the timed region).  Prints ONE JSON line:
+neuron-timesteps/s of the chain, the HBM roofline of the dominant kernel (HIP-event timing on
+the launch stream) and the CPU oracle timed on the host cores beside it.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+SHAPE = (12, 16, 34, 34, 300)
+HBM_PEAK_GBS = 8000.0                     # MI355X HBM3E, published
+# algorithmic bytes per neuron-timestep (fp32 tensors read + written once)
+AB = {"psp_conv": 8, "spike": 12, "shift": 8, "shift_bwd": 8, "spike_bwd": 12, "psp_corr": 8}
+KERNEL_OF = {"psp_conv": "fir_tiled_kernel<true>", "spike": "spike_stream_kernel<64>",
+             "shift": "shift_kernel<4>", "shift_bwd": "shift_kernel<4>", "spike_bwd": "spike_bwd_kernel<4>",
+             "psp_corr": "fir_tiled_kernel<false>"}
+
+
+def neuron_params():
+    return {"theta": 10.0, "tauSr": 10.0, "tauRef": 1.0, "scaleRef": 2.0, "tauRho": 1.0, "scaleRho": 1.0}
+
+
+def make_inputs(shape, device, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    spikes = (torch.rand(shape, generator=g) < 0.02).float()
+    u0 = torch.randn(shape, generator=g) * 5.0
+    g1 = torch.Generator(device="cpu").manual_seed(seed + 1)
+    grad = torch.randn(shape, generator=g1)
+    return spikes.to(device), u0.to(device), grad.to(device)
+
+
+def cpu_baseline(shape, srm, ref, params, rows_fraction=8):
+    """The CPU oracle on a bounded sample of the same workload (every rows_fraction-th batch
+    slice), all host threads."""
+    from oracle import oracle as O
+    threads = O.max_threads()
+    O.set_threads(threads)
+    rows = (shape[0] * shape[1] * shape[2] * shape[3]) // rows_fraction
+    rows -= rows % (shape[2] * shape[3])
+    sub = (1, rows // (shape[2] * shape[3]), shape[2], shape[3], shape[4])
+    rng = np.random.default_rng(0)
+    spikes = (rng.random(sub) < 0.02).astype(np.float32)
+    u0 = (rng.standard_normal(sub) * 5).astype(np.float32)
+    grad = rng.standard_normal(sub).astype(np.float32)
+    theta, tau, scale = params["theta"], params["tauRho"] * params["theta"], params["scaleRho"]
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        O.conv(spikes, srm, 1.0)
+        s, u = O.get_spikes(u0, ref, theta, 1.0)
+        O.shift(s, 1.0, 1.0)
+        gd = O.shift(grad, -1.0, 1.0)
+        gs = O.spike_bwd(gd, u, theta, tau, scale)
+        O.corr(gs, srm, 1.0)
+        times.append(time.perf_counter() - t0)
+    best = sorted(times)[len(times) // 2]
+    O.set_threads(1)
+    return {"value": spikes.size / best, "unit": "neuron-timesteps/s", "cores": threads, "kind": "port",
+            "sample": "oracle chain (conv77+spike+shift, shift+spike_bwd+corr77) on %s, median of 3, %.2f s"
+                      % (str(sub), best)}
+
+
+def flip_rate(device, srm_t, ref_t, params):
+    """Fraction of spike samples that differ between the GPU chain psp -> scale -> spike and the
+    CPU oracle chain run with separately rounded multiply and add (the only difference between
+    the two is the fp32 rounding of the filter sum upstream of the threshold)."""
+    from oracle import oracle as O
+    from slayerpytorch_amd import slayerCuda
+    rng = np.random.default_rng(0)
+    shape = (2, 16, 34, 34, 300)
+    spikes = (rng.random(shape) < 0.02).astype(np.float32)
+    gain = np.float32(14.0)          # puts about 2 % of the samples above threshold
+    a = slayerCuda.conv(torch.from_numpy(spikes).to(device), srm_t, 1.0) * float(gain)
+    s_gpu = slayerCuda.getSpikes(a.contiguous(), ref_t, params["theta"], 1.0).cpu().numpy()
+    a_cpu = O.conv(spikes, srm_t.cpu().numpy(), 1.0, fused=False) * gain
+    s_cpu, _ = O.get_spikes(a_cpu, ref_t.cpu().numpy(), params["theta"], 1.0)
+    return float((s_gpu != s_cpu).mean()), float((s_cpu != 0).mean())
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: every kernel on this path treats neuron rows independently, "
+                 "so N GPUs is N independent copies of this run; use --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+
+    from slayerpytorch_amd import slayerCuda
+    from slayerpytorch_amd.slayer import alphaKernel
+
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    params = neuron_params()
+    srm = np.array(alphaKernel(params["tauSr"], 1.0, SHAPE[-1]), dtype=np.float32)
+    ref = np.array(alphaKernel(params["tauRef"], 1.0, SHAPE[-1], mult=-params["scaleRef"] * params["theta"]),
+                   dtype=np.float32)
+    srm_t, ref_t = torch.from_numpy(srm).to(device), torch.from_numpy(ref).to(device)
+    theta, tau, scale = params["theta"], params["tauRho"] * params["theta"], params["scaleRho"]
+
+    spikes, u0, grad = make_inputs(SHAPE, device)
+    numel = spikes.numel()
+    total = args.steps + args.warmup
+    pool = [u0.clone() for _ in range(total)]          # spike() consumes one copy per step
+    names = list(AB)
+    events = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in names]
+              for _ in range(args.steps)]
+
+    def step(i, ev=None):
+        u = pool[i]
+
+        def run(k, fn):
+            if ev is not None:
+                ev[k][0].record()
+            out = fn()
+            if ev is not None:
+                ev[k][1].record()
+            return out
+
+        run(0, lambda: slayerCuda.conv(spikes, srm_t, 1.0))
+        s = run(1, lambda: slayerCuda.getSpikes(u, ref_t, theta, 1.0))
+        run(2, lambda: slayerCuda.shift(s, 1.0, 1.0))
+        gd = run(3, lambda: slayerCuda.shift(grad, 1.0, 1.0, sign=-1.0))
+        gs = run(4, lambda: slayerCuda.spikeBackward(gd, u, theta, tau, scale))
+        run(5, lambda: slayerCuda.corr(gs, srm_t, 1.0))
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(args.warmup + i, events[i])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    ms_per_step = elapsed / args.steps * 1e3
+    per_kernel_ms = {n: float(np.mean([events[i][k][0].elapsed_time(events[i][k][1]) for i in range(args.steps)]))
+                     for k, n in enumerate(names)}
+    dominant = max(per_kernel_ms, key=per_kernel_ms.get)
+    achieved = AB[dominant] * numel / (per_kernel_ms[dominant] * 1e-3) / 1e9
+    chain_gbs = sum(AB.values()) * numel / (sum(per_kernel_ms.values()) * 1e-3) / 1e9
+
+    result = {
+        "metric": "neuron-timesteps/s spike+psp+shift fwd/bwd at 1 MI355X; % HBM peak GB/s",
+        "value": numel / (elapsed / args.steps),
+        "unit": "neuron-timesteps/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "NMNIST-CNN-shaped activation tensor (12,16,34,34,300): psp conv (77 taps) + spike "
+                               "(11-tap refractory) + shift fwd, shift + spike pdf + psp corr bwd",
+                   "elements": numel, "algorithmic_bytes_per_element": sum(AB.values())},
+        "roofline": {"bound": "hbm", "kernel": KERNEL_OF[dominant], "op": dominant, "achieved": achieved,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None},
+        "chain_hbm_frac": chain_gbs / HBM_PEAK_GBS,
+        "per_kernel_ms": per_kernel_ms,
+        "per_kernel_hbm_frac": {n: AB[n] * numel / (per_kernel_ms[n] * 1e-3) / 1e9 / HBM_PEAK_GBS for n in names},
+    }
+    del pool
+    flips, rate = flip_rate(device, srm_t, ref_t, params)
+    result["spike_flip_rate"] = flips
+    result["spike_rate"] = rate
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(SHAPE, srm, ref, params)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

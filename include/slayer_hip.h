@@ -1,0 +1,174 @@
+/*
+ * slayer_hip.h - C ABI of libslayer_hip.so: SLAYER's per-neuron temporal kernels for AMD
+ * MI355X (gfx950), hand-written HIP.
+ *
+ * This is the drop-in boundary for the reference's two pybind11 extension modules,
+ * `slayerCuda` (src/cuda/slayerKernels.cu:136-145) and `slayerLoihiCuda`
+ * (src/cuda/slayerLoihiKernels.cu:48-51).  Each entry point below names the reference
+ * binding it replaces.
+ *
+ * Conventions shared by every entry point
+ *   - All tensors are dense, contiguous float32 device buffers shaped [nNeurons][T] with time
+ *     innermost ("neuron row" = T consecutive samples).  Any leading tensor shape
+ *     (N,C,H,W,...) is flattened into nNeurons by the caller.
+ *   - Pointers are device pointers valid on the CURRENT HIP device; the caller selects the
+ *     device (the reference bindings call cudaSetDevice on the tensor's device).
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only
+ *     enqueue work: no allocation, no free, no host synchronisation, no global state.
+ *   - The library never allocates device memory.  Outputs (and the one workspace, see
+ *     slayer_delay_grad_f32) are allocated by the caller.
+ *   - Return value: SLAYER_OK (0) or one of the SLAYER_E* codes; nothing has been launched
+ *     when a SLAYER_EINVAL / SLAYER_EUNSUPPORTED code is returned.  Empty tensors
+ *     (nNeurons == 0 or T == 0) are a successful no-op.
+ */
+#ifndef SLAYER_HIP_H_INCLUDED
+#define SLAYER_HIP_H_INCLUDED
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SLAYER_HIP_ABI_VERSION 1
+
+enum {
+    SLAYER_OK = 0,
+    SLAYER_EINVAL = 1,       /* null pointer, negative size, refDelay == 0, ... */
+    SLAYER_EUNSUPPORTED = 2, /* size outside what the kernels index (see each function) */
+    SLAYER_ELAUNCH = 3       /* the HIP runtime reported an error for the launch */
+};
+
+/* ABI version of the loaded library (== SLAYER_HIP_ABI_VERSION it was built with). */
+int slayer_hip_abi_version(void);
+
+/* Static, human readable text for a status code. */
+const char *slayer_status_string(int status);
+
+/* Text of the last HIP runtime error seen by this thread inside the library ("" if none). */
+const char *slayer_last_hip_error(void);
+
+/*
+ * Debug/validation knob, process wide: 0 (default) = tiled LDS kernels wherever the sizes
+ * allow; 1 = always use the generic one-thread-per-sample / one-thread-per-neuron kernels
+ * (the ones that also serve sizes the tiled kernels do not cover).  Both produce the same
+ * results.  Returns the previous value.  No counterpart in the reference.
+ */
+int slayer_force_generic_kernels(int on);
+
+/*
+ * SRM spike generation with refractory feedback.
+ * Replaces slayerCuda.getSpikes -> getSpikesCuda (src/cuda/slayerKernels.cu:14-39),
+ * kernel src/cuda/spikeKernels.h:9-38.
+ *
+ * For each neuron row, t ascending: if u[t] >= theta then s[t] = 1/Ts and
+ * u[t+j] += nu[j] for j in [0, nuSize) with t+j < T; else s[t] = 0.  `u` is updated IN
+ * PLACE (it holds the post-refractory membrane potential on return); `s` is written.
+ * Results are bit-identical to the sequential fp32 loop.  nuSize may be 0.
+ */
+int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_t nNeurons, int64_t T,
+                          int64_t nuSize, float theta, float Ts, void *stream);
+
+/*
+ * Causal temporal convolution (PSP filter, forward).
+ * Replaces slayerCuda.conv -> convCuda (src/cuda/slayerKernels.cu:41-57),
+ * kernel src/cuda/convKernels.h:10-35.
+ *
+ * out[n][t] = Ts * sum_{i=0..F-1, t-i>=0} in[n][t-i] * filt[i], accumulated in fp32 by
+ * fused multiply-add in tap order i = 0,1,...  `out` must not alias `in`.  F >= 1... F == 0
+ * yields zeros.
+ */
+int slayer_conv_f32(float *out, const float *in, const float *filt, int64_t nNeurons, int64_t T,
+                    int64_t F, float Ts, void *stream);
+
+/*
+ * Anti-causal temporal correlation (PSP filter, backward; adjoint of slayer_conv_f32).
+ * Replaces slayerCuda.corr -> corrCuda (src/cuda/slayerKernels.cu:59-75),
+ * kernel src/cuda/convKernels.h:37-62.
+ *
+ * out[n][t] = Ts * sum_{i=0..F-1, t+i<T} in[n][t+i] * filt[i].
+ */
+int slayer_corr_f32(float *out, const float *in, const float *filt, int64_t nNeurons, int64_t T,
+                    int64_t F, float Ts, void *stream);
+
+/*
+ * Time shift by one delay for all rows, delay given by value.
+ * Replaces slayerCuda.shift(Tensor, float[, Ts]) -> shiftFlCuda / shiftFl1Cuda
+ * (src/cuda/slayerKernels.cu:114-134), kernel src/cuda/shiftKernels.h:9-34.
+ *
+ * k = (int)(delay / Ts)  (fp32 quotient truncated toward zero);
+ * out[n][t] = (0 <= t-k < T) ? in[n][t-k] : 0.  `out` must not alias `in`.
+ */
+int slayer_shift_f32(float *out, const float *in, float delay, int64_t nNeurons, int64_t T,
+                     float Ts, void *stream);
+
+/*
+ * Time shift with delays read from device memory.
+ * Replaces slayerCuda.shift(Tensor, Tensor[, Ts]) -> shiftCuda / shift1Cuda
+ * (src/cuda/slayerKernels.cu:77-112), kernels src/cuda/shiftKernels.h:9-61.
+ *
+ * lutSize == 1: every row is shifted by lut[0] (read on the device: unlike the reference's
+ * `.item()` there is no host synchronisation).  Otherwise lutSize must equal nPerBatch and
+ * row (b, m) of the [nBatch][nPerBatch][T] tensor is shifted by lut[m]; one launch covers
+ * all batches.  `sign` (+1 or -1) multiplies every delay before use, so that the backward
+ * pass (shift by -delay, src/slayer.py:957,979) needs no negated copy of the table.
+ */
+int slayer_shift_lut_f32(float *out, const float *in, const float *lut, int64_t lutSize,
+                         int64_t nBatch, int64_t nPerBatch, int64_t T, float Ts, float sign,
+                         void *stream);
+
+/*
+ * Surrogate gradient of the spike function, fused into one pass.
+ * Replaces the torch expression chain of _spikeFunction.backward (src/slayer.py:857-865) and
+ * slayerLoihi._spike.backward (src/slayerLoihi.py:278-283); native precedent evalRhoKernel
+ * (src/cuda/spikeKernels.h:41-52).
+ *
+ * gradIn[i] = gradOut[i] * (scale / tau) * exp(-|u[i] - theta| / tau), tau = tauRho * theta.
+ * gradIn may alias gradOut.  tau must be non-zero.
+ */
+int slayer_spike_bwd_f32(float *gradIn, const float *gradOut, const float *u, float theta,
+                         float tau, float scale, int64_t numel, void *stream);
+
+/* Bytes of caller-provided device workspace that slayer_delay_grad_f32 needs (may be 0). */
+int64_t slayer_delay_grad_workspace_bytes(int64_t nBatch, int64_t nPerBatch, int64_t T);
+
+/*
+ * Gradient with respect to a per-neuron delay table, fused into one pass plus a small
+ * deterministic reduction.
+ * Replaces the conv + multiply + sum of _delayFunction.backward (src/slayer.py:949-955).
+ *
+ * gradDelay[m] = Ts * sum_{b,t} gradOut[b][m][t] * (out[b][m][t-1] - out[b][m][t]) / Ts,
+ * out[.][.][-1] = 0, for the [nBatch][nPerBatch][T] tensors `out` (the shifted signal) and
+ * `gradOut`.  `workspace` must hold slayer_delay_grad_workspace_bytes(...) bytes.
+ */
+int slayer_delay_grad_f32(float *gradDelay, const float *out, const float *gradOut,
+                          float *workspace, int64_t nBatch, int64_t nPerBatch, int64_t T, float Ts,
+                          void *stream);
+
+/*
+ * Loihi CUBA (current based) integer neuron.
+ * Replaces slayerLoihiCuda.getSpikes -> getSpikesCuda (src/cuda/slayerLoihiKernels.cu:12-46),
+ * kernel and launcher src/cuda/spikeLoihiKernels.h:9-96.
+ *
+ * Per neuron row, int32 state (current, voltage) starting at 0, weightScale = 1 << (6+wgtExp):
+ *   t = 0 : s = v = u = 0, the input sample is ignored;
+ *   t >= 1: current = decay(current, iDecay) + weightScale * (int)w[t]
+ *           voltage = decay(voltage, vDecay) + current
+ *           decay(x, d) = sign(x) * ((|x| * (4096 - d)) >> 12)      (32-bit wrap-around)
+ *           spike = voltage > theta and the neuron is not refractory; a spike makes the neuron
+ *           refractory until refDelay steps later; while refractory (and at the spike) the
+ *           voltage carried to the next step is 0.
+ *           s[t] = spike, u[t] = current, v[t] = spike ? vDecay : carried voltage.
+ * Outputs are exact integers stored as float32, bit-identical to the sequential loop.
+ * refDelay must be >= 1 (the reference reads an unwritten sample for 0): SLAYER_EINVAL.
+ * wgtExp must satisfy 6 + wgtExp < 32.
+ */
+int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const float *w, int64_t nNeurons,
+                                int64_t T, uint32_t wgtExp, int32_t theta, uint32_t iDecay,
+                                uint32_t vDecay, uint32_t refDelay, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* SLAYER_HIP_H_INCLUDED */

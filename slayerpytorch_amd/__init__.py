@@ -1,0 +1,12 @@
+"""slayerpytorch_amd: SLAYER's per-neuron temporal kernels for AMD MI355X (gfx950).
+
+``slayerCuda`` / ``slayerLoihiCuda`` are drop-in replacements of the reference's two extension
+modules, bound to hand-written HIP kernels through the C ABI of ``libslayer_hip.so``;
+``layer`` / ``loihi`` are the host-side layer engines that wrap them in autograd Functions.
+"""
+from . import slayerCuda, slayerLoihiCuda            # noqa: F401
+from .slayer import spikeLayer as layer               # noqa: F401
+from .slayerLoihi import spikeLayer as loihi          # noqa: F401
+from .slayerLoihi import quantize                     # noqa: F401
+
+__all__ = ["slayerCuda", "slayerLoihiCuda", "layer", "loihi", "quantize"]

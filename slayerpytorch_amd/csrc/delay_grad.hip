@@ -1,0 +1,84 @@
+// Gradient of a time shift with respect to its per-neuron delay table:
+//
+//   gradDelay[m] = Ts * sum_{b,t} gradOut[b][m][t] * d[b][m][t],
+//   d[b][m][t]   = out[b][m][t] * (-1/Ts) + out[b][m][t-1] * (1/Ts)        (out[.][.][-1] = 0)
+//
+// i.e. the 2-tap causal difference of the shifted signal, weighted by the incoming gradient and
+// reduced over batch and time.  HBM-bound (8 B per neuron-timestep: both tensors read once).
+// Pass 1: one wavefront per neuron row reduces its T products (lanes along time, coalesced) to
+// one partial sum in the caller's workspace.  Pass 2: one lane per table entry adds the
+// nBatch partials in batch order and scales by Ts.  The summation order is fixed, so results
+// are reproducible from run to run.
+#include "common.h"
+
+namespace slayer {
+
+__global__ __launch_bounds__(256) void delay_grad_rows_kernel(float *__restrict__ partial,
+                                                              const float *__restrict__ out,
+                                                              const float *__restrict__ gradOut,
+                                                              int64_t rows, int64_t T, float f0, float f1)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t wavesPerGrid = static_cast<int64_t>(gridDim.x) * (blockDim.x / kWave);
+    for (int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
+         row < rows; row += wavesPerGrid) {
+        const float *y = out + row * T;
+        const float *g = gradOut + row * T;
+        float acc = 0.0f;
+        for (int64_t t = lane; t < T; t += kWave) {
+            float d = y[t] * f0;
+            if (t > 0) d = __builtin_fmaf(y[t - 1], f1, d);
+            acc = __builtin_fmaf(g[t], d, acc);
+        }
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) acc += __shfl_down(acc, off, kWave);
+        if (lane == 0) partial[row] = acc;
+    }
+}
+
+__global__ __launch_bounds__(256) void delay_grad_batch_kernel(float *__restrict__ gradDelay,
+                                                               const float *__restrict__ partial,
+                                                               int64_t nBatch, int64_t nPerBatch, float Ts)
+{
+    const int64_t m = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (m >= nPerBatch) return;
+    float acc = 0.0f;
+    for (int64_t b = 0; b < nBatch; ++b) acc += partial[b * nPerBatch + m];
+    gradDelay[m] = acc * Ts;
+}
+
+}  // namespace slayer
+
+extern "C" int64_t slayer_delay_grad_workspace_bytes(int64_t nBatch, int64_t nPerBatch, int64_t T)
+{
+    (void)T;
+    if (nBatch <= 0 || nPerBatch <= 0) return 0;
+    return nBatch * nPerBatch * static_cast<int64_t>(sizeof(float));
+}
+
+extern "C" int slayer_delay_grad_f32(float *gradDelay, const float *out, const float *gradOut,
+                                     float *workspace, int64_t nBatch, int64_t nPerBatch, int64_t T,
+                                     float Ts, void *stream)
+{
+    using namespace slayer;
+    if (nBatch < 0 || nPerBatch < 0 || T < 0) return SLAYER_EINVAL;
+    if (nPerBatch == 0) return SLAYER_OK;
+    if (!gradDelay) return SLAYER_EINVAL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t rows = nBatch * nPerBatch;
+    const int64_t outBlocks = ceil_div(nPerBatch, 256);
+    if (outBlocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+    if (rows > 0 && T > 0) {
+        if (!out || !gradOut || !workspace) return SLAYER_EINVAL;
+        int64_t blocks = ceil_div(rows, 4);  // four wavefronts (rows) per work-group
+        if (blocks > 262144) blocks = 262144;
+        hipLaunchKernelGGL(delay_grad_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
+                           workspace, out, gradOut, rows, T, -1.0f / Ts, 1.0f / Ts);
+        int status = launch_status();
+        if (status != SLAYER_OK) return status;
+    }
+    // with no samples to reduce (nBatch == 0 or T == 0) the loop below is empty and yields zeros
+    hipLaunchKernelGGL(delay_grad_batch_kernel, dim3(static_cast<unsigned>(outBlocks)), dim3(256), 0, st,
+                       gradDelay, workspace, (rows > 0 && T > 0) ? nBatch : 0, nPerBatch, Ts);
+    return launch_status();
+}

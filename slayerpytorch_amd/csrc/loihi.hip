@@ -1,0 +1,186 @@
+// Loihi CUBA neuron: int32 current/voltage with sign-magnitude decay (>>12), integer
+// threshold, refractory delay.  Sequential in time per neuron, parallel over neurons.
+//
+// HBM-bound (16 B per neuron-timestep: read w, write spike, voltage, current).  Same streaming
+// scheme as the SRM spike kernel: a 64-lane work-group owns 64 consecutive rows and moves them
+// through LDS in 32-sample chunks, lanes along time for the 128-byte global segments, lane =
+// row for the sequential update.  The neuron state (current, voltage, refractory countdown)
+// stays in registers across chunks.  The chunk's input tile is overwritten in place by the
+// current; the voltage has its own tile; spikes travel as one 32-bit mask per lane.
+//
+// Refractory bookkeeping: the sequential formulation keeps a counter that is incremented at a
+// spike and decremented refDelay steps later by re-reading the spike it wrote then.  Because a
+// spike needs the counter to be zero, the counter only takes the values 0 and 1, and "1" lasts
+// exactly until refDelay steps after the spike.  A countdown register set to refDelay at a
+// spike and decremented once per step (before the threshold test) is therefore the same
+// automaton, without the read-back.
+#include "common.h"
+
+namespace slayer {
+
+constexpr int kLoihiChunk = 32;
+
+// sign(x) * ((|x| * (4096 - decay)) >> 12) in 32-bit wrap-around arithmetic
+__device__ __forceinline__ uint32_t loihi_decay(int x, uint32_t keep)
+{
+    const uint32_t ux = static_cast<uint32_t>(x);
+    const uint32_t mag = (x >= 0) ? ux : (0u - ux);
+    const uint32_t scaled = (mag * keep) >> 12;
+    return (x >= 0) ? scaled : (0u - scaled);
+}
+
+struct LoihiState {
+    int current;
+    int voltage;
+    uint32_t countdown;  // steps until the neuron may spike again (0 = not refractory)
+};
+
+struct LoihiParams {
+    uint32_t weightScale, keepI, keepV, refDelay, vDecay;
+    int theta;
+};
+
+// One time step (t >= 1).  Returns the spike; cOut / vOut are the reported current / voltage.
+__device__ __forceinline__ uint32_t loihi_step(LoihiState &st, const LoihiParams &p, float w,
+                                               float &cOut, float &vOut)
+{
+    const int cNew = static_cast<int>(loihi_decay(st.current, p.keepI) +
+                                      p.weightScale * static_cast<uint32_t>(trunc_sat(w)));
+    const int vNew = static_cast<int>(loihi_decay(st.voltage, p.keepV) + static_cast<uint32_t>(cNew));
+    if (st.countdown > 0) --st.countdown;
+    const bool refractory = st.countdown != 0;
+    const uint32_t spike = (vNew > p.theta && !refractory) ? 1u : 0u;
+    st.voltage = (spike || refractory) ? 0 : vNew;
+    if (spike) st.countdown = p.refDelay;
+    st.current = cNew;
+    cOut = static_cast<float>(cNew);
+    vOut = spike ? static_cast<float>(static_cast<int>(p.vDecay)) : static_cast<float>(st.voltage);
+    return spike;
+}
+
+// ---- generic kernel: one lane per neuron, straight from global memory ---------------------------
+__global__ __launch_bounds__(256) void loihi_generic_kernel(float *__restrict__ s, float *__restrict__ v,
+                                                            float *__restrict__ u,
+                                                            const float *__restrict__ w, int64_t rows,
+                                                            int64_t T, LoihiParams p)
+{
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (row >= rows) return;
+    const int64_t base = row * T;
+    LoihiState st = {0, 0, 0u};
+    s[base] = 0.0f; v[base] = 0.0f; u[base] = 0.0f;
+    for (int64_t t = 1; t < T; ++t) {
+        float c, vo;
+        const uint32_t spike = loihi_step(st, p, w[base + t], c, vo);
+        s[base + t] = static_cast<float>(spike);
+        u[base + t] = c;
+        v[base + t] = vo;
+    }
+}
+
+// ---- streaming kernel -------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void loihi_stream_kernel(float *__restrict__ s, float *__restrict__ v,
+                                                          float *__restrict__ u,
+                                                          const float *__restrict__ w, int64_t rows,
+                                                          int T, LoihiParams p)
+{
+    __shared__ float tileC[kWave * kLoihiChunk];  // input, then current
+    __shared__ float tileV[kWave * kLoihiChunk];  // voltage
+
+    const int lane = threadIdx.x;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kWave;
+    const int nChunks = (T + kLoihiChunk - 1) / kLoihiChunk;
+    const int segT = lane & 31;
+    const int segR = lane >> 5;
+
+    // rotated tile: sample k of row r at column (k + r) mod 32 -> 32 distinct banks either way
+    auto slot = [](int r, int k) { return r * kLoihiChunk + ((k + r) & (kLoihiChunk - 1)); };
+
+    LoihiState st = {0, 0, 0u};
+
+    for (int c = 0; c < nChunks; ++c) {
+        const int tBase = c * kLoihiChunk;
+        {
+            const int t = tBase + segT;
+#pragma unroll 8
+            for (int it = 0; it < 32; ++it) {
+                const int r = 2 * it + segR;
+                const int64_t row = row0 + r;
+                float x = 0.0f;
+                if (row < rows && t < T) x = w[row * static_cast<int64_t>(T) + t];
+                tileC[slot(r, segT)] = x;
+            }
+        }
+        __syncthreads();
+
+        uint32_t fired = 0;
+        const int steps = min(kLoihiChunk, T - tBase);
+        for (int k = 0; k < steps; ++k) {
+            const int i = slot(lane, k);
+            float cOut = 0.0f, vOut = 0.0f;
+            if (tBase + k > 0) {
+                const uint32_t spike = loihi_step(st, p, tileC[i], cOut, vOut);
+                fired |= spike << k;
+            }
+            tileC[i] = cOut;
+            tileV[i] = vOut;
+        }
+        __syncthreads();
+
+        {
+            const int t = tBase + segT;
+#pragma unroll 8
+            for (int it = 0; it < 32; ++it) {
+                const int r = 2 * it + segR;
+                const int64_t row = row0 + r;
+                const int i = slot(r, segT);
+                const float cv = tileC[i];
+                const float vv = tileV[i];
+                const uint32_t m = __shfl(fired, r, kWave);
+                const float sv = ((m >> segT) & 1u) ? 1.0f : 0.0f;
+                if (row < rows && t < T) {
+                    const int64_t g = row * static_cast<int64_t>(T) + t;
+                    s[g] = sv;
+                    v[g] = vv;
+                    u[g] = cv;
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+}  // namespace slayer
+
+extern "C" int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const float *w,
+                                           int64_t nNeurons, int64_t T, uint32_t wgtExp, int32_t theta,
+                                           uint32_t iDecay, uint32_t vDecay, uint32_t refDelay,
+                                           void *stream)
+{
+    using namespace slayer;
+    if (nNeurons < 0 || T < 0) return SLAYER_EINVAL;
+    if (refDelay == 0 || wgtExp > 25) return SLAYER_EINVAL;
+    if (nNeurons == 0 || T == 0) return SLAYER_OK;
+    if (!s || !v || !u || !w) return SLAYER_EINVAL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    LoihiParams p;
+    p.weightScale = 1u << (6 + wgtExp);
+    p.keepI = 4096u - iDecay;
+    p.keepV = 4096u - vDecay;
+    p.refDelay = refDelay;
+    p.vDecay = vDecay;
+    p.theta = theta;
+
+    const int64_t groups = ceil_div(nNeurons, kWave);
+    if (!generic_forced() && T < (1LL << 30) && groups < (1LL << 31)) {
+        hipLaunchKernelGGL(loihi_stream_kernel, dim3(static_cast<unsigned>(groups)), dim3(kWave), 0, st,
+                           s, v, u, w, nNeurons, static_cast<int>(T), p);
+        return launch_status();
+    }
+    const int64_t blocks = ceil_div(nNeurons, 256);
+    if (blocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+    hipLaunchKernelGGL(loihi_generic_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, s, v,
+                       u, w, nNeurons, T, p);
+    return launch_status();
+}

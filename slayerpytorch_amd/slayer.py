@@ -1,0 +1,220 @@
+"""Host side of the SRM hot path: the part of the reference's ``slayer.spikeLayer`` that feeds
+and wraps the temporal kernels, re-hosted on PyTorch-ROCm.
+
+Mirrors, with the same names, signatures and side effects:
+
+* kernel generators ``calculateSrmKernel`` / ``calculateRefKernel`` / ``_calculateAlphaKernel``
+  (src/slayer.py:98-123),
+* ``spikeLayer.psp`` / ``spike`` / ``delayShift`` / ``delay`` (src/slayer.py:130-142, 333-391),
+* autograd Functions ``_spikeFunction``, ``_pspFunction``, ``_delayLayer``, ``_delayFunction``,
+  ``_delayFunctionNoGradient`` (src/slayer.py:817-979),
+* ``dense`` (src/slayer.py:144-172, 393-437) only as plumbing for end-to-end checks: it is a
+  plain ``conv3d`` and not part of the accelerated path.
+
+Differences from the reference, all on the host: backward passes use the fused
+``slayerCuda.spikeBackward`` / ``slayerCuda.delayGrad`` kernels instead of chains of
+elementwise torch ops, and scalars saved for backward stay Python floats (no 0-dim device
+tensors, hence no device-to-host synchronisation in backward).
+"""
+import math
+
+import numpy as np
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import slayerCuda
+
+
+def alphaKernel(tau, Ts, tSample, mult=1.0, EPSILON=0.01):
+    """Samples ``mult * t/tau * exp(1 - t/tau)`` at t = 0, Ts, 2Ts, ... < tSample and stops
+    (exclusively) at the first sample past the peak whose magnitude is below ``EPSILON``
+    (src/slayer.py:114-123).  Evaluated in float64; returns a Python list."""
+    values = []
+    for t in np.arange(0, tSample, Ts):
+        v = mult * t / tau * math.exp(1 - t / tau)
+        if abs(v) < EPSILON and t > tau:
+            break
+        values.append(v)
+    return values
+
+
+class spikeLayer(nn.Module):
+    """SRM spiking layer engine: PSP filter, spike function and delays on NCHWT tensors.
+
+    ``neuronDesc`` needs ``theta, tauSr, tauRef, scaleRef, tauRho, scaleRho``; ``simulationDesc``
+    needs ``Ts, tSample`` (src/slayer.py:47-96).
+    """
+
+    def __init__(self, neuronDesc, simulationDesc, fullRefKernel=False):
+        super().__init__()
+        self.neuron = neuronDesc
+        self.simulation = simulationDesc
+        self.fullRefKernel = fullRefKernel
+        self.register_buffer("srmKernel", self.calculateSrmKernel())
+        self.register_buffer("refKernel", self.calculateRefKernel())
+
+    def calculateSrmKernel(self):
+        return torch.FloatTensor(self._calculateAlphaKernel(self.neuron["tauSr"]))
+
+    def calculateRefKernel(self):
+        mult = -self.neuron["scaleRef"] * self.neuron["theta"]
+        if self.fullRefKernel:
+            kernel = self._calculateAlphaKernel(tau=self.neuron["tauRef"], mult=mult, EPSILON=0.0001)
+        else:
+            kernel = self._calculateAlphaKernel(tau=self.neuron["tauRef"], mult=mult)
+        return torch.FloatTensor(kernel)
+
+    def _calculateAlphaKernel(self, tau, mult=1, EPSILON=0.01):
+        return alphaKernel(tau, self.simulation["Ts"], self.simulation["tSample"], mult, EPSILON)
+
+    def psp(self, spike):
+        """PSP filtering of a spike tensor (same shape out)."""
+        return _pspFunction.apply(spike, self.srmKernel, self.simulation["Ts"])
+
+    def spike(self, membranePotential):
+        """Spike function with refractory response.  A contiguous ``membranePotential`` is
+        updated in place with the refractory response, as in the reference."""
+        return _spikeFunction.apply(membranePotential, self.refKernel, self.neuron, self.simulation["Ts"])
+
+    def delayShift(self, input, delay, Ts=1):
+        """Delays ``input`` in time by ``delay`` (number, one-element tensor, or one value per
+        neuron); the gradient flows to ``input`` only."""
+        return _delayFunctionNoGradient.apply(input, delay, Ts)
+
+    def delay(self, inputSize):
+        """Learnable per-neuron (or per-channel) delay module for inputs of spatial shape
+        ``inputSize`` = C or (C, H, W)."""
+        return _delayLayer(inputSize, self.simulation["Ts"])
+
+    def dense(self, inFeatures, outFeatures, weightScale=10, preHookFx=None):
+        """Fully connected synapse applied per time step (plain conv3d, not accelerated here)."""
+        return _denseLayer(inFeatures, outFeatures, weightScale, preHookFx)
+
+
+class _denseLayer(nn.Conv3d):
+    """(outFeatures, inFeatures, 1, 1, 1) weight applied at every time step."""
+
+    def __init__(self, inFeatures, outFeatures, weightScale=1, preHookFx=None):
+        if isinstance(inFeatures, int):
+            kernel, inChannels = (1, 1, 1), inFeatures
+        elif len(inFeatures) == 2:
+            kernel, inChannels = (inFeatures[1], inFeatures[0], 1), 1
+        elif len(inFeatures) == 3:
+            kernel, inChannels = (inFeatures[1], inFeatures[0], 1), inFeatures[2]
+        else:
+            raise Exception("inFeatures should not be more than 3 dimension. It was: {}".format(inFeatures))
+        if not isinstance(outFeatures, int):
+            raise Exception("outFeatures should not be more than 1 dimesnion. It was: {}".format(outFeatures))
+        super().__init__(inChannels, outFeatures, kernel, bias=False)
+        if weightScale != 1:
+            self.weight = nn.Parameter(weightScale * self.weight)
+        self.preHookFx = preHookFx
+
+    def forward(self, input):
+        weight = self.weight if self.preHookFx is None else self.preHookFx(self.weight)
+        return F.conv3d(input, weight, self.bias, self.stride, self.padding, self.dilation, self.groups)
+
+
+class _spikeFunction(torch.autograd.Function):
+    """Forward: ``slayerCuda.getSpikes``; backward: spike-function surrogate gradient
+    ``gradOutput * scaleRho/(tauRho*theta) * exp(-|u - theta| / (tauRho*theta))``
+    (src/slayer.py:817-865)."""
+
+    @staticmethod
+    def forward(ctx, membranePotential, refractoryResponse, neuron, Ts):
+        theta = neuron["theta"]
+        # A contiguous input IS the buffer the kernel updates in place; a non-contiguous one is
+        # copied and keeps its values.  Either way the tensor saved for backward is the
+        # caller's, exactly as in the reference.
+        spikes = slayerCuda.getSpikes(membranePotential.contiguous(), refractoryResponse, theta, Ts)
+        ctx.save_for_backward(membranePotential)
+        ctx.theta = float(theta)
+        ctx.pdfTimeConstant = float(neuron["tauRho"] * neuron["theta"])
+        ctx.pdfScale = float(neuron["scaleRho"])
+        return spikes
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        (membranePotential,) = ctx.saved_tensors
+        gradInput = slayerCuda.spikeBackward(gradOutput.contiguous(), membranePotential.contiguous(),
+                                             ctx.theta, ctx.pdfTimeConstant, ctx.pdfScale)
+        return gradInput, None, None, None
+
+
+class _pspFunction(torch.autograd.Function):
+    """Forward: causal conv with the SRM kernel; backward: correlation with the same kernel;
+    the kernel itself gets no gradient (src/slayer.py:875-899)."""
+
+    @staticmethod
+    def forward(ctx, spike, filter, Ts):
+        psp = slayerCuda.conv(spike.contiguous(), filter, Ts)
+        ctx.save_for_backward(filter)
+        ctx.Ts = float(Ts)
+        return psp
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        (filter,) = ctx.saved_tensors
+        gradInput = slayerCuda.corr(gradOutput.contiguous(), filter, ctx.Ts)
+        return gradInput, None, None
+
+
+class _delayLayer(nn.Module):
+    """Learnable delay, one per neuron (C,H,W) or one per channel when the input's H and W
+    exceed the parameter's (src/slayer.py:901-928).  Initialised U[0,1)."""
+
+    def __init__(self, inputSize, Ts):
+        super().__init__()
+        if isinstance(inputSize, int):
+            shape = (inputSize, 1, 1)
+        elif len(inputSize) == 3:
+            shape = (inputSize[0], inputSize[1], inputSize[2])
+        else:
+            raise Exception("inputSize can only be 1 or 2 dimension. It was: {}".format(inputSize))
+        self.delay = nn.Parameter(torch.rand(shape), requires_grad=True)
+        self.Ts = Ts
+
+    def forward(self, input):
+        N, C, H, W, Ns = input.shape
+        if input.numel() != self.delay.numel() * Ns * N:
+            return _delayFunction.apply(input, self.delay.repeat((1, H, W)), self.Ts)
+        return _delayFunction.apply(input, self.delay, self.Ts)
+
+
+class _delayFunction(torch.autograd.Function):
+    """Shift by a per-neuron delay table with gradients for both the input (shift by the
+    negated delay) and the delays (src/slayer.py:930-957)."""
+
+    @staticmethod
+    def forward(ctx, input, delay, Ts):
+        output = slayerCuda.shift(input.contiguous(), delay.data.contiguous(), Ts)
+        ctx.save_for_backward(output, delay.data)
+        ctx.Ts = float(Ts)
+        return output
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        output, delay = ctx.saved_tensors
+        gradOutput = gradOutput.contiguous()
+        gradDelay = slayerCuda.delayGrad(output, gradOutput, ctx.Ts).reshape(gradOutput.shape[1:-1])
+        gradInput = slayerCuda.shift(gradOutput, delay.contiguous(), ctx.Ts, sign=-1.0)
+        return gradInput, gradDelay, None
+
+
+class _delayFunctionNoGradient(torch.autograd.Function):
+    """Shift by a fixed delay (number or tensor); backward shifts the gradient by the negated
+    delay (src/slayer.py:959-979)."""
+
+    @staticmethod
+    def forward(ctx, input, delay, Ts=1):
+        if isinstance(delay, torch.Tensor):
+            delay = delay.detach().to(device=input.device, dtype=input.dtype).contiguous()
+        output = slayerCuda.shift(input.contiguous(), delay, Ts)
+        ctx.delay = delay
+        ctx.Ts = float(Ts)
+        return output
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        return slayerCuda.shift(gradOutput.contiguous(), ctx.delay, ctx.Ts, sign=-1.0), None, None

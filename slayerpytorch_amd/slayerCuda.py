@@ -1,0 +1,219 @@
+"""``slayerCuda`` for MI355X: same callables as the reference's pybind11 extension
+(src/cuda/slayerKernels.cu:136-145), implemented over the C ABI of ``libslayer_hip.so``.
+
+===================================  ==========================================================
+callable                             reference binding it replaces
+===================================  ==========================================================
+``getSpikes(u, nu, theta, Ts)``      ``getSpikesCuda``  src/cuda/slayerKernels.cu:14-39
+``conv(input, filter, Ts)``          ``convCuda``       src/cuda/slayerKernels.cu:41-57
+``corr(input, filter, Ts)``          ``corrCuda``       src/cuda/slayerKernels.cu:59-75
+``shift(input, lut[, Ts])``          ``shiftCuda`` / ``shift1Cuda``     :77-112
+``shift(input, delay[, Ts])``        ``shiftFlCuda`` / ``shiftFl1Cuda`` :114-134
+===================================  ==========================================================
+
+Argument checks mirror the reference's ``CHECK_INPUT`` / ``CHECK_DEVICE`` assertions and are
+made before anything is launched, so they can be exercised without a GPU.  Scalars may be
+Python numbers or 0-dim tensors, as with pybind11's float conversion.  Outputs are allocated
+with ``torch.empty_like``; kernels are enqueued on PyTorch's current stream of the tensor's
+device and never synchronise with the host.
+
+``spikeBackward``, ``delayGrad`` and the ``sign`` argument of ``shift`` have no counterpart in
+the reference extension: they are the fused forms of the elementwise chains in
+``_spikeFunction.backward`` / ``_delayFunction.backward`` (src/slayer.py:857-865, 944-957).
+"""
+import numbers
+
+import torch
+
+from . import _lib
+
+__all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "delayGrad"]
+
+
+def _check_input(x, name):
+    if not isinstance(x, torch.Tensor):
+        raise TypeError("%s must be a torch.Tensor, got %s" % (name, type(x).__name__))
+    if not x.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)
+    if not x.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)
+    if x.dtype != torch.float32:
+        raise RuntimeError("expected scalar type Float but found %s for %s" % (x.dtype, name))
+
+
+def _check_device(x, y, xname, yname):
+    if x.device.index != y.device.index:
+        raise RuntimeError("%s and %s must be in same CUDA device" % (xname, yname))
+
+
+def _scalar(x, name):
+    if isinstance(x, torch.Tensor):
+        if x.numel() != 1:
+            raise TypeError("%s must be a number or a one-element tensor" % name)
+        return float(x)
+    if isinstance(x, numbers.Real):
+        return float(x)
+    try:
+        return float(x)   # numpy scalars and other objects with __float__
+    except Exception:
+        raise TypeError("%s must be a number, got %s" % (name, type(x).__name__))
+
+
+def _ptr(x):
+    return x.data_ptr() if x.numel() else None
+
+
+def _rows(x):
+    T = x.shape[-1] if x.dim() else 1
+    return (x.numel() // T if T else 0), T
+
+
+class _on_device_of:
+    """Makes the tensor's device current (like the reference's cudaSetDevice) and yields the
+    raw handle of PyTorch's current stream there."""
+
+    def __init__(self, x):
+        self.guard = torch.cuda.device(x.device)
+
+    def __enter__(self):
+        self.guard.__enter__()
+        return torch.cuda.current_stream().cuda_stream
+
+    def __exit__(self, *exc):
+        return self.guard.__exit__(*exc)
+
+
+def getSpikes(d_u, d_nu, theta, Ts):
+    """Spikes of the membrane potential ``d_u`` (N,C,H,W,T); ``d_u`` is updated IN PLACE with
+    the refractory response ``d_nu`` of every spike.  Returns the spike tensor (``1/Ts`` at
+    spikes)."""
+    _check_input(d_u, "d_u")
+    _check_input(d_nu, "d_nu")
+    _check_device(d_u, d_nu, "d_u", "d_nu")
+    if d_u.dim() < 4:
+        raise IndexError("Dimension out of range (getSpikes expects a 5 dimensional N,C,H,W,T tensor, "
+                         "got %d dimensions)" % d_u.dim())
+    if d_u.dim() != 5:
+        raise RuntimeError("getSpikes expects a 5 dimensional (N,C,H,W,T) tensor, got %d dimensions"
+                           % d_u.dim())
+    theta = _scalar(theta, "theta")
+    Ts = _scalar(Ts, "Ts")
+    lib = _lib.load()
+    d_s = torch.empty_like(d_u)
+    n, T = _rows(d_u)
+    nuSize = d_nu.shape[-1] if d_nu.dim() else 1
+    with _on_device_of(d_u) as stream:
+        _lib.check(lib.slayer_get_spikes_f32(_ptr(d_s), _ptr(d_u), _ptr(d_nu), n, T, nuSize, theta, Ts,
+                                             stream), "slayer_get_spikes_f32")
+    return d_s
+
+
+def _fir(entry, name, input, filter, Ts):
+    _check_input(input, "input")
+    _check_input(filter, "filter")
+    _check_device(input, filter, "input", "filter")
+    Ts = _scalar(Ts, "Ts")
+    lib = _lib.load()
+    output = torch.empty_like(input)
+    n, T = _rows(input)
+    with _on_device_of(input) as stream:
+        _lib.check(getattr(lib, entry)(_ptr(output), _ptr(input), _ptr(filter), n, T, filter.numel(), Ts,
+                                       stream), entry)
+    return output
+
+
+def conv(input, filter, Ts):
+    """Causal convolution in time (last axis) of every neuron row with ``filter``, times ``Ts``."""
+    return _fir("slayer_conv_f32", "conv", input, filter, Ts)
+
+
+def corr(input, filter, Ts):
+    """Anti-causal correlation in time (adjoint of :func:`conv`), times ``Ts``."""
+    return _fir("slayer_corr_f32", "corr", input, filter, Ts)
+
+
+def shift(input, shiftLUT, Ts=1.0, sign=1.0):
+    """Shifts every neuron row in time by ``int(delay / Ts)`` samples (zero fill).
+
+    ``shiftLUT`` is a number (one delay for all rows), a one-element tensor (same, read on the
+    device) or a tensor with one delay per neuron of a batch item (``numel == C*H*W``).
+    ``sign`` (+1/-1, extension) multiplies the delays, for the backward shift.
+    """
+    _check_input(input, "input")
+    sign = float(sign)
+    if isinstance(shiftLUT, torch.Tensor):
+        _check_input(shiftLUT, "shiftLUT")
+        _check_device(input, shiftLUT, "input", "shiftLUT")
+        Ts = _scalar(Ts, "Ts")
+        n, T = _rows(input)
+        if shiftLUT.numel() == 1:
+            nBatch, nPerBatch = 1, n
+        else:
+            nBatch = input.shape[0]
+            nPerBatch = (n // nBatch) if nBatch else 0
+            if shiftLUT.numel() != nPerBatch:
+                raise RuntimeError("shift and number of neurons must be same")
+        lib = _lib.load()
+        output = torch.empty_like(input)
+        with _on_device_of(input) as stream:
+            _lib.check(lib.slayer_shift_lut_f32(_ptr(output), _ptr(input), _ptr(shiftLUT),
+                                                shiftLUT.numel(), nBatch, nPerBatch, T, Ts, sign, stream),
+                       "slayer_shift_lut_f32")
+        return output
+    delay = _scalar(shiftLUT, "shiftLUT")
+    Ts = _scalar(Ts, "Ts")
+    lib = _lib.load()
+    output = torch.empty_like(input)
+    n, T = _rows(input)
+    with _on_device_of(input) as stream:
+        _lib.check(lib.slayer_shift_f32(_ptr(output), _ptr(input), delay * sign, n, T, Ts, stream),
+                   "slayer_shift_f32")
+    return output
+
+
+def spikeBackward(gradOutput, membranePotential, theta, tau, scale):
+    """``gradOutput * scale/tau * exp(-|membranePotential - theta| / tau)`` in one pass
+    (``tau`` is the scaled time constant ``tauRho * theta``)."""
+    _check_input(gradOutput, "gradOutput")
+    _check_input(membranePotential, "membranePotential")
+    _check_device(gradOutput, membranePotential, "gradOutput", "membranePotential")
+    if gradOutput.shape != membranePotential.shape:
+        raise RuntimeError("gradOutput and membranePotential must have the same shape")
+    theta, tau, scale = _scalar(theta, "theta"), _scalar(tau, "tau"), _scalar(scale, "scale")
+    lib = _lib.load()
+    gradInput = torch.empty_like(gradOutput)
+    with _on_device_of(gradOutput) as stream:
+        _lib.check(lib.slayer_spike_bwd_f32(_ptr(gradInput), _ptr(gradOutput), _ptr(membranePotential),
+                                            theta, tau, scale, gradOutput.numel(), stream),
+                   "slayer_spike_bwd_f32")
+    return gradInput
+
+
+def delayGrad(output, gradOutput, Ts):
+    """Gradient of ``shift`` with respect to its per-neuron delays: ``Ts * sum over batch and
+    time of gradOutput * (output[t-1] - output[t]) / Ts``; shape ``output.shape[1:-1]``."""
+    _check_input(output, "output")
+    _check_input(gradOutput, "gradOutput")
+    _check_device(output, gradOutput, "output", "gradOutput")
+    if output.shape != gradOutput.shape:
+        raise RuntimeError("output and gradOutput must have the same shape")
+    if output.dim() < 2:
+        raise RuntimeError("delayGrad expects at least (batch, time) dimensions")
+    Ts = _scalar(Ts, "Ts")
+    lib = _lib.load()
+    n, T = _rows(output)
+    nBatch = output.shape[0]
+    nPerBatch = (n // nBatch) if nBatch else 0
+    shape = tuple(output.shape[1:-1])
+    if nBatch == 0:
+        nPerBatch = 1
+        for d in shape:
+            nPerBatch *= d
+    gradDelay = torch.empty(shape, dtype=output.dtype, device=output.device)
+    nbytes = lib.slayer_delay_grad_workspace_bytes(nBatch, nPerBatch, T)
+    workspace = torch.empty((max(nbytes, 4) // 4,), dtype=torch.float32, device=output.device)
+    with _on_device_of(output) as stream:
+        _lib.check(lib.slayer_delay_grad_f32(_ptr(gradDelay), _ptr(output), _ptr(gradOutput),
+                                             workspace.data_ptr(), nBatch, nPerBatch, T, Ts, stream),
+                   "slayer_delay_grad_f32")
+    return gradDelay

@@ -1,0 +1,114 @@
+"""Host side of the Loihi hot path: the part of the reference's ``slayerLoihi.spikeLayer``
+that feeds and wraps the Loihi neuron kernel, re-hosted on PyTorch-ROCm.
+
+Mirrors: threshold ``theta = vThMant * 2**6`` (src/slayerLoihi.py:47-56), the integer PSP and
+refractory kernel generators (:58-89), ``spikeLoihi`` / ``spikeLoihiFull`` (:91-122), the
+autograd Function ``_spike`` (:243-283) and the quantised ``dense`` default (:124-139,
+src/quantizeParams.py).
+"""
+import numpy as np
+import torch
+
+from . import slayer, slayerCuda, slayerLoihiCuda
+
+
+class quantizeWeights(torch.autograd.Function):
+    """``round(w / step) * step`` with a straight-through gradient (src/quantizeParams.py:3-31)."""
+
+    @staticmethod
+    def forward(ctx, weights, step=1):
+        return torch.round(weights / step) * step
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        return gradOutput, None
+
+
+def quantize(weights, step=1):
+    return quantizeWeights.apply(weights, step)
+
+
+def loihiPspKernel(iDecay, vDecay, wgtExp=0):
+    """Voltage response of the CUBA neuron to one input spike of weight 1, as a float list:
+    integer recurrence started at ``1 << (7 + wgtExp)`` (a weight of 2), run until the voltage
+    reaches zero (the final 0 is kept) and halved (src/slayerLoihi.py:66-79)."""
+    u = [1 << (6 + wgtExp + 1)]
+    v = [u[-1]]
+    while v[-1] > 0:
+        uNext = (u[-1] * ((1 << 12) - iDecay)) >> 12
+        vNext = ((v[-1] * ((1 << 12) - vDecay)) >> 12) + uNext
+        u.append(uNext)
+        v.append(vNext)
+    return [float(x) / 2 for x in v]
+
+
+def loihiRefKernel(theta, vDecay, refDelay, SCALE=1000):
+    """Absolute refractory block (``refDelay`` samples of ``-SCALE*theta``, first one 0) followed
+    by ``-2 *`` the decaying threshold sequence (src/slayerLoihi.py:81-89)."""
+    absolute = np.ones(refDelay) * (-SCALE * theta)
+    absolute[0] = 0
+    relative = [theta]
+    while relative[-1] > 0:
+        relative.append((relative[-1] * ((1 << 12) - vDecay)) >> 12)
+    return np.concatenate((absolute, -2 * np.array(relative))).astype("float32")
+
+
+class spikeLayer(slayer.spikeLayer):
+    """Loihi flavour of :class:`slayer.spikeLayer`.  ``neuronDesc`` needs ``vThMant, vDecay,
+    iDecay, refDelay, wgtExp, tauRho, scaleRho``; ``theta`` is derived and ``scaleRho`` is
+    divided by the PSP kernel's maximum, both written back into ``neuronDesc`` as the
+    reference does."""
+
+    def __init__(self, neuronDesc, simulationDesc):
+        if neuronDesc["type"] == "LOIHI":
+            neuronDesc["theta"] = neuronDesc["vThMant"] * 2 ** 6
+        super().__init__(neuronDesc, simulationDesc)
+        self.maxPspKernel = torch.max(self.srmKernel).cpu().data.item()
+        neuronDesc["scaleRho"] /= self.maxPspKernel
+
+    def calculateSrmKernel(self):
+        return torch.tensor(loihiPspKernel(self.neuron["iDecay"], self.neuron["vDecay"], self.neuron["wgtExp"]))
+
+    def calculateRefKernel(self, SCALE=1000):
+        return torch.tensor(loihiRefKernel(self.neuron["theta"], self.neuron["vDecay"],
+                                           self.neuron["refDelay"], SCALE))
+
+    def spikeLoihi(self, weightedSpikes):
+        """Loihi neuron dynamics on weighted (unfiltered) input spikes -> output spikes, with the
+        SLAYER surrogate gradient attached."""
+        return _spike.apply(weightedSpikes, self.srmKernel, self.neuron, self.simulation["Ts"])
+
+    def spikeLoihiFull(self, weightedSpikes):
+        """Same dynamics without autograd; returns ``(spike, voltage, current)``."""
+        return _spike.loihi(weightedSpikes, self.neuron, self.simulation["Ts"])
+
+    def dense(self, inFeatures, outFeatures, weightScale=100, preHookFx=lambda x: quantize(x, step=2)):
+        return super().dense(inFeatures, outFeatures, weightScale, preHookFx)
+
+
+class _spike(torch.autograd.Function):
+    @staticmethod
+    def loihi(weightedSpikes, neuron, Ts):
+        if weightedSpikes.dtype == torch.int32:
+            Ts = 1
+        spike, voltage, current = slayerLoihiCuda.getSpikes(
+            (weightedSpikes * Ts).contiguous(), neuron["wgtExp"], neuron["theta"], neuron["iDecay"],
+            neuron["vDecay"], neuron["refDelay"])
+        return spike / Ts, voltage, current
+
+    @staticmethod
+    def forward(ctx, weightedSpikes, srmKernel, neuron, Ts):
+        spike, voltage, current = _spike.loihi(weightedSpikes, neuron, Ts)
+        ctx.save_for_backward(voltage, srmKernel.clone().detach())
+        ctx.theta = float(neuron["theta"])
+        ctx.pdfTimeConstant = float(neuron["tauRho"] * neuron["theta"])
+        ctx.pdfScale = float(neuron["scaleRho"])
+        ctx.Ts = float(Ts)
+        return spike
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        voltage, srmKernel = ctx.saved_tensors
+        weighted = slayerCuda.spikeBackward(gradOutput.contiguous(), voltage, ctx.theta,
+                                            ctx.pdfTimeConstant, ctx.pdfScale)
+        return slayerCuda.corr(weighted, srmKernel, ctx.Ts), None, None, None

@@ -1,0 +1,262 @@
+"""Parity of the HIP kernels with the CPU oracle on the same seeded inputs.  Every call goes
+through the Python modules ``slayerCuda`` / ``slayerLoihiCuda``, i.e. ctypes -> C ABI of
+libslayer_hip.so.  Integer/threshold work (spike, Loihi, shift) must be bit-exact; fp32 filters
+must stay within 1e-5 relative (they are in fact bit-exact against the fused-multiply-add
+oracle, which is asserted too).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from slayerpytorch_amd import _lib, slayerCuda, slayerLoihiCuda
+from slayerpytorch_amd.slayer import alphaKernel
+
+from _util import rel_err
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-5       # psp / corr / spike pdf / delay gradient: max |gpu - oracle| <= REL_TOL * max |oracle|
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+@pytest.fixture(params=[0, 1], ids=["tiled", "generic"])
+def impl(request):
+    lib = _lib.load()
+    old = lib.slayer_force_generic_kernels(request.param)
+    yield request.param
+    lib.slayer_force_generic_kernels(old)
+
+
+# ------------------------------------------------------------------------------------------ shift
+@pytest.mark.parametrize("shape", [(5, 10, 20, 30, 100), (3, 7, 1, 1, 33), (2, 3, 2, 2, 1), (1, 1, 1, 1, 5000),
+                                   (4, 130, 1, 1, 350)])
+def test_shift_per_neuron_exact(shape):
+    rng = np.random.default_rng(9)
+    Ts = 0.1
+    x = rng.standard_normal(shape).astype(np.float32)
+    d = (rng.random(shape[1:4]) * 2 - 1).astype(np.float32) * shape[-1] * Ts / 4
+    d.reshape(-1)[0] = 0.0
+    got = host(slayerCuda.shift(dev(x), dev(d), Ts))
+    assert np.array_equal(bits(got), bits(O.shift(x, d, Ts)))
+    # negated table (backward direction)
+    got = host(slayerCuda.shift(dev(x), dev(d), Ts, sign=-1.0))
+    assert np.array_equal(bits(got), bits(O.shift(x, -d, Ts)))
+
+
+@pytest.mark.parametrize("delay,Ts", [(4, 1.0), (-3, 1.0), (0, 1.0), (-0.25, 0.1), (0.3, 0.1), (1000.0, 1.0),
+                                      (-1e12, 1.0), (2.5, 0.5)])
+@pytest.mark.parametrize("T", [300, 350, 33])
+def test_shift_scalar_exact(delay, Ts, T):
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((3, 5, 2, 2, T)).astype(np.float32)
+    want = O.shift(x, delay, Ts)
+    assert np.array_equal(bits(host(slayerCuda.shift(dev(x), delay, Ts))), bits(want))
+    # one-element tensor: read on the device, same result
+    assert np.array_equal(bits(host(slayerCuda.shift(dev(x), dev(np.array([delay], np.float32)), Ts))), bits(want))
+    if Ts == 1.0:
+        assert np.array_equal(bits(host(slayerCuda.shift(dev(x), delay))), bits(want))      # Ts defaults to 1
+
+
+def test_shift_unaligned_storage_offset():
+    rng = np.random.default_rng(11)
+    base = dev(rng.standard_normal(2 * 3 * 64 + 1).astype(np.float32))
+    x = base[1:].reshape(2, 3, 1, 1, 64)                       # 4-byte aligned only
+    got = host(slayerCuda.shift(x, 5.0, 1.0))
+    assert np.array_equal(got, O.shift(host(x), 5.0, 1.0))
+
+
+# ------------------------------------------------------------------------------------------ conv / corr
+FIR_CASES = [
+    # (rows shape, T, F)
+    ((2, 16, 5, 5), 300, 77), ((1, 1, 1, 3), 350, 77), ((3, 70), 64, 8), ((2, 33), 2000, 8),
+    ((5, 7), 100, 1), ((5, 7), 100, 2), ((5, 7), 100, 3), ((5, 7), 100, 4), ((5, 7), 100, 5),
+    ((4, 9), 37, 11), ((4, 9), 40, 12), ((4, 9), 41, 13), ((3, 3), 500, 110), ((3, 3), 500, 160),
+    ((2, 5), 30, 77), ((2, 2), 1, 5), ((1, 40), 700, 330), ((1, 3), 50, 500),
+]
+
+
+@pytest.mark.parametrize("rows,T,Fl", FIR_CASES)
+@pytest.mark.parametrize("op", ["conv", "corr"])
+def test_fir_matches_oracle(impl, rows, T, Fl, op):
+    rng = np.random.default_rng(T * 1000 + Fl)
+    x = rng.standard_normal(rows + (T,)).astype(np.float32)
+    f = rng.standard_normal(Fl).astype(np.float32)
+    Ts = 0.7
+    got = host(getattr(slayerCuda, op)(dev(x), dev(f), Ts))
+    want = getattr(O, op)(x, f, Ts, fused=True)
+    assert rel_err(got, want) <= REL_TOL
+    assert rel_err(got, getattr(O, op)(x, f, Ts, fused=False)) <= REL_TOL
+    assert np.array_equal(bits(got), bits(want)), "not bit-identical to the fused-multiply-add chain"
+
+
+def test_fir_sparse_spike_input_and_alpha_kernel(impl):
+    rng = np.random.default_rng(5)
+    x = (rng.random((4, 2, 34, 34, 300)) < 0.02).astype(np.float32)
+    f = np.array(alphaKernel(10.0, 1.0, 300), dtype=np.float32)
+    got = host(slayerCuda.conv(dev(x), dev(f), 1.0))
+    assert np.array_equal(bits(got), bits(O.conv(x, f, 1.0)))
+
+
+def test_fir_is_left_padded_conv3d(impl):
+    # the identity the reference's test_slayer011 asserts: psp == pspLayer, ||diff|| / numel < 1e-6
+    rng = np.random.default_rng(6)
+    x = dev((rng.random((2, 4, 8, 8, 200)) < 0.1).astype(np.float32))
+    f = dev(np.array(alphaKernel(10.0, 1.0, 200), dtype=np.float32))
+    padded = torch.nn.functional.pad(x.reshape(2, 1, 1, -1, 200), (f.numel() - 1, 0))
+    want = torch.nn.functional.conv3d(padded, torch.flip(f, [0]).reshape(1, 1, 1, 1, -1)).reshape(x.shape)
+    got = slayerCuda.conv(x, f, 1.0)
+    assert (torch.norm(got - want) / got.numel()).item() < 1e-6
+
+
+def test_fir_adjoint_identity(impl):
+    rng = np.random.default_rng(7)
+    x, y = dev(rng.standard_normal((6, 50, 300)).astype(np.float32)), dev(rng.standard_normal((6, 50, 300)).astype(np.float32))
+    f = dev(np.array(alphaKernel(10.0, 1.0, 300), dtype=np.float32))
+    lhs = (slayerCuda.conv(x, f, 1.0).double() * y.double()).sum().item()
+    rhs = (x.double() * slayerCuda.corr(y, f, 1.0).double()).sum().item()
+    assert abs(lhs - rhs) <= 1e-5 * abs(lhs)
+
+
+# ------------------------------------------------------------------------------------------ spike
+SPIKE_CASES = [
+    # (shape, nuSize)
+    ((2, 16, 6, 6, 300), 11), ((1, 3, 1, 1, 350), 11), ((2, 130, 1, 1, 64), 11), ((1, 1, 1, 1, 2000), 8),
+    ((3, 5, 2, 2, 95), 1), ((3, 5, 2, 2, 96), 0), ((2, 9, 3, 1, 97), 33), ((2, 9, 3, 1, 130), 34),
+    ((2, 9, 3, 1, 200), 97), ((1, 70, 1, 1, 500), 110), ((1, 20, 1, 1, 501), 160), ((2, 2, 2, 2, 1), 11),
+    ((1, 4, 1, 1, 7), 11),
+]
+
+
+@pytest.mark.parametrize("shape,nuSize", SPIKE_CASES)
+def test_spikes_bit_exact(impl, shape, nuSize):
+    rng = np.random.default_rng(shape[-1] + nuSize)
+    u = (rng.standard_normal(shape) * 6).astype(np.float32)
+    nu = (-rng.random(nuSize) * 12).astype(np.float32)
+    if nuSize > 2:
+        nu[0] = 0.0
+    theta, Ts = 10.0, 0.5
+    want_s, want_u = O.get_spikes(u, nu, theta, Ts)
+    ud = dev(u)
+    s = slayerCuda.getSpikes(ud, dev(nu), theta, Ts)
+    assert np.array_equal(bits(host(s)), bits(want_s))
+    assert np.array_equal(bits(host(ud)), bits(want_u)), "membrane potential must be updated in place, bit-exact"
+    assert want_s.sum() > 0 or shape[-1] < 8
+
+
+def test_spikes_dense_firing_and_positive_feedback(impl):
+    # every sample above threshold, and a refractory kernel that pushes u up (runaway firing)
+    rng = np.random.default_rng(3)
+    u = (np.abs(rng.standard_normal((2, 8, 3, 3, 150))) * 5 + 10).astype(np.float32)
+    for nu in (np.array([0, -1, -0.5, 3, 2], np.float32), np.array([1.0], np.float32)):
+        want_s, want_u = O.get_spikes(u, nu, 10.0, 1.0)
+        ud = dev(u)
+        s = slayerCuda.getSpikes(ud, dev(nu), 10.0, 1.0)
+        assert np.array_equal(bits(host(s)), bits(want_s)) and np.array_equal(bits(host(ud)), bits(want_u))
+
+
+def test_spikes_special_cases(impl):
+    rng = np.random.default_rng(4)
+    u = (rng.standard_normal((1, 4, 2, 2, 90)) * 6).astype(np.float32)
+    nu = np.array(alphaKernel(1.0, 1.0, 300, mult=-20), dtype=np.float32)
+    ud = dev(u)
+    s = slayerCuda.getSpikes(ud, dev(nu), float("inf"), 1.0)
+    assert not host(s).any() and np.array_equal(host(ud), u)
+    one = np.zeros((1, 1, 1, 1, 40), np.float32)
+    one[..., 7] = 10.0
+    od = dev(one)
+    s = host(slayerCuda.getSpikes(od, dev(nu), 10.0, 0.25))
+    assert s[..., 7] == 4.0 and s.sum() == 4.0
+    want = one.copy()
+    want[..., 7:7 + len(nu)] += nu
+    assert np.array_equal(host(od), want)
+
+
+# ------------------------------------------------------------------------------------------ spike backward
+@pytest.mark.parametrize("n", [1, 7, 4096, 12 * 16 * 34 * 34 * 3 + 1, 1 << 20])
+def test_spike_bwd(n):
+    rng = np.random.default_rng(n)
+    u = (rng.standard_normal(n) * 8).astype(np.float32)
+    g = rng.standard_normal(n).astype(np.float32)
+    for theta, tau, scale in [(10.0, 10.0, 1.0), (10.0, 1.0, 1.0), (5120.0, 5120.0, 1 / 195.0)]:
+        got = host(slayerCuda.spikeBackward(dev(g), dev(u), theta, tau, scale))
+        want = O.spike_bwd(g, u, theta, tau, scale)
+        np.testing.assert_allclose(got, want, rtol=REL_TOL, atol=1e-30)
+        ref64 = g.astype(np.float64) * scale / tau * np.exp(-np.abs(u.astype(np.float64) - theta) / tau)
+        assert rel_err(got, ref64) <= REL_TOL
+
+
+# ------------------------------------------------------------------------------------------ delay gradient
+@pytest.mark.parametrize("shape,Ts", [((4, 6, 1, 1, 80), 0.1), ((64, 20, 1, 1, 2000), 1.0), ((3, 2, 5, 7, 33), 0.5),
+                                      ((1, 1, 1, 1, 1), 1.0)])
+def test_delay_grad(shape, Ts):
+    rng = np.random.default_rng(shape[-1])
+    y = rng.standard_normal(shape).astype(np.float32)
+    g = rng.standard_normal(shape).astype(np.float32)
+    got = host(slayerCuda.delayGrad(dev(y), dev(g), Ts))
+    want = O.delay_grad(y, g, Ts)
+    assert got.shape == shape[1:-1]
+    assert rel_err(got, want) <= REL_TOL
+    # the three-pass formulation of the reference: conv with [-1, 1]/Ts (Ts argument 1), multiply, sum
+    diff = slayerCuda.conv(dev(y), dev(np.array([-1, 1], np.float32)) / Ts, 1)
+    ref = torch.sum(dev(g).double() * diff.double(), [0, -1]) * Ts
+    assert rel_err(got, host(ref)) <= REL_TOL
+
+
+# ------------------------------------------------------------------------------------------ Loihi
+def loihi_input(rng, shape, p=0.05):
+    return (2 * rng.integers(-128, 128, size=shape) * (rng.random(shape) < p)).astype(np.float32)
+
+
+@pytest.mark.parametrize("shape", [(2, 16, 8, 8, 300), (1, 3, 1, 1, 350), (2, 130, 1, 1, 64), (64, 200), (5, 1),
+                                   (1, 1, 1, 1, 2000), (70, 33)])
+@pytest.mark.parametrize("refDelay", [1, 2, 17])
+def test_loihi_bit_exact(impl, shape, refDelay):
+    rng = np.random.default_rng(sum(shape) + refDelay)
+    w = loihi_input(rng, shape, p=0.3)
+    want = O.loihi_get_spikes(w, 0, 80 * 64, 1024, 128, refDelay)
+    got = slayerLoihiCuda.getSpikes(dev(w), 0, 80 * 64, 1024, 128, refDelay)
+    for a, b, name in zip(got, want, ("spike", "voltage", "current")):
+        assert np.array_equal(bits(host(a)), bits(b)), name
+    assert want[0].sum() > 0 or shape[-1] < 8
+
+
+@pytest.mark.parametrize("params", [(1, 10 * 64, 2048, 256, 3), (0, 64, 0, 0, 1), (2, 5000, 4095, 4095, 2),
+                                    (0, 1, 4096, 4096, 1), (3, 300000, 100, 10, 500)])
+def test_loihi_parameters_wraparound_and_truncation(impl, params):
+    rng = np.random.default_rng(8)
+    w = (rng.standard_normal((3, 40, 150)) * 40).astype(np.float32)           # non-integers: (int) truncates toward zero
+    w[0, 0, 5] = np.nan
+    w[0, 1, 5] = 1e20
+    w[0, 2, 5] = -1e20
+    want = O.loihi_get_spikes(w, *params)
+    got = slayerLoihiCuda.getSpikes(dev(w), *params)
+    for a, b, name in zip(got, want, ("spike", "voltage", "current")):
+        assert np.array_equal(bits(host(a)), bits(b)), name
+
+
+# ------------------------------------------------------------------------------------------ empty tensors
+def test_empty_tensors():
+    e = torch.empty((0, 3, 1, 1, 10), device="cuda")
+    f = dev(np.ones(3, np.float32))
+    assert slayerCuda.conv(e, f, 1.0).shape == e.shape
+    assert slayerCuda.corr(e, f, 1.0).shape == e.shape
+    assert slayerCuda.shift(e, 2.0).shape == e.shape
+    assert slayerCuda.getSpikes(e, f, 1.0, 1.0).shape == e.shape
+    assert [t.shape for t in slayerLoihiCuda.getSpikes(e, 0, 64, 0, 0, 1)] == [e.shape] * 3
+    z = torch.empty((2, 3, 1, 1, 0), device="cuda")
+    assert slayerCuda.conv(z, f, 1.0).shape == z.shape
+    assert slayerCuda.getSpikes(z, f, 1.0, 1.0).shape == z.shape
+    assert host(slayerCuda.delayGrad(z, z, 1.0)).tolist() == [[[0.0]]] * 3
+    torch.cuda.synchronize()
