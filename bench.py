@@ -48,7 +48,7 @@ def make_inputs(shape, device, seed=0):
     return spikes.to(device), u0.to(device), grad.to(device)
 
 
-def cpu_baseline(shape, srm, ref, params, rows_fraction=8):
+def cpu_baseline(shape, srm, ref, params, rows_fraction=1):
     """The CPU oracle on a bounded sample of the same workload (every rows_fraction-th batch
     slice), all host threads."""
     from oracle import oracle as O

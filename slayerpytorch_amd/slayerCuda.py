@@ -201,14 +201,12 @@ def delayGrad(output, gradOutput, Ts):
         raise RuntimeError("delayGrad expects at least (batch, time) dimensions")
     Ts = _scalar(Ts, "Ts")
     lib = _lib.load()
-    n, T = _rows(output)
+    T = output.shape[-1]
     nBatch = output.shape[0]
-    nPerBatch = (n // nBatch) if nBatch else 0
     shape = tuple(output.shape[1:-1])
-    if nBatch == 0:
-        nPerBatch = 1
-        for d in shape:
-            nPerBatch *= d
+    nPerBatch = 1
+    for d in shape:
+        nPerBatch *= d
     gradDelay = torch.empty(shape, dtype=output.dtype, device=output.device)
     nbytes = lib.slayer_delay_grad_workspace_bytes(nBatch, nPerBatch, T)
     workspace = torch.empty((max(nbytes, 4) // 4,), dtype=torch.float32, device=output.device)
