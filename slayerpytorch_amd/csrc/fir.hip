@@ -8,23 +8,22 @@
 // zeros, which leaves the chain's value unchanged.
 //
 // Tiled kernel.  The convolution is the correlation on a reversed time axis, so both share one
-// core: Y[m] = sum_i X[m+i] * filt[i].  A work-group of 256 lanes owns 32 neuron rows and one
-// time tile; it stages the rows' samples (plus the F-1 sample halo) into LDS as X[32][LD]
-// (reversed for the convolution).  Lane l works on row (l & 31); each half-wave is one "slot"
-// that takes 8-output chunks of the tile.  A lane keeps a 12-sample register window of X and
-// slides it 4 samples per 4 taps with one 16-byte LDS read, so one LDS read feeds 32 FMAs;
-// LD = 4 (mod 32) makes those reads bank-conflict free across the 32 rows of a slot.  Filter
-// taps are wave-uniform and come through scalar loads.  An FIR with F = 77 taps needs 154
-// flop per 8 bytes moved, which is at the FP32 ridge of the machine: the kernel is built to
-// be FMA-issue bound, not LDS or HBM bound.
+// core: Y[m] = sum_i X[m+i] * filt[i].  A work-group of 256 lanes owns R consecutive neuron
+// rows and one time tile; it stages the rows' samples (plus the F-1 sample halo, zero padded)
+// into LDS as X[R][LD] with 16-byte loads (reversed in time for the convolution).  The tile is
+// then cut into chunks of 8 consecutive outputs of one row; lanes take chunks in row-major
+// order, so neighbouring lanes produce neighbouring outputs and the results leave as 16-byte
+// stores.  A lane keeps a 12-sample register window of X and slides it 4 samples per 4 taps
+// with one 16-byte LDS read, i.e. one LDS read feeds 32 FMAs.  Filter taps are wave-uniform
+// and come through scalar loads.  An FIR with F = 77 taps needs 154 flop per 8 bytes moved,
+// which is at the FP32 ridge of the machine: the kernel is meant to be FMA-issue bound.
 #include "common.h"
 
 namespace slayer {
 
-constexpr int kFirRows = 32;    // rows per work-group
-constexpr int kFirSlots = 8;    // half-waves per work-group
-constexpr int kFirU = 8;        // outputs per lane per chunk
-constexpr int kFirMaxLD = 388;  // LDS row pitch limit: 32*388*4 B = 48.5 KiB, three groups per CU
+constexpr int kFirU = 8;              // outputs per lane per chunk
+constexpr int kFirMaxLdsFloats = 12288;  // 48 KiB of LDS per work-group at most
+constexpr int kFirMaxPitch = 512;     // longest LDS row (samples) the tiled kernel stages
 
 // ---- generic kernel: one lane per output sample (any F, any T) ---------------------------------
 template <bool CAUSAL>
@@ -64,52 +63,89 @@ __device__ __forceinline__ void fma_quad(float (&acc)[kFirU], const float4 &a, c
     }
 }
 
-template <bool CAUSAL>
+// i / d for 0 <= i < 2^24 with a precomputed float reciprocal (estimate plus one correction)
+__device__ __forceinline__ void divmod_small(int i, int d, float inv, int &q, int &r)
+{
+    q = static_cast<int>(static_cast<float>(i) * inv);
+    r = i - q * d;
+    if (r < 0) { --q; r += d; }
+    else if (r >= d) { ++q; r -= d; }
+}
+
+// VEC: rows are whole 16-byte vectors (T % 4 == 0, pointers 16-byte aligned)
+template <bool CAUSAL, bool VEC>
 __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
                                                         const float *__restrict__ in,
                                                         const float *__restrict__ filt,
-                                                        int64_t rows, int T, int F, int TT, int LD,
+                                                        int64_t rows, int T, int F, int TT, int LD, int R,
                                                         float Ts)
 {
     extern __shared__ __align__(16) float X[];
 
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kFirRows;
-    const int t0 = blockIdx.y * TT;                 // first output time of the tile
-    const int tt = min(TT, T - t0);                 // outputs in this tile
+    const int tid = threadIdx.x;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
+    const int nRows = static_cast<int>(min(static_cast<int64_t>(R), rows - row0));
+    const int t0 = blockIdx.y * TT;                   // first output time of the tile
+    const int tt = min(TT, T - t0);                   // outputs in this tile
     const int ttp = (tt + kFirU - 1) & ~(kFirU - 1);  // rounded up to whole chunks
-    const int tHi = t0 + ttp - 1;                   // time stored at X[.][0] when reversed
-    const int used = ttp + F + 4;                   // samples of a row the core may read
+    const int tHi = t0 + ttp - 1;                     // time stored at X[.][0] when reversed
 
-    // stage: X[r][j] = in[row0+r][time(j)], zero outside the row; time(j) = t0+j (corr) or tHi-j (conv)
-    for (int r = wave; r < kFirRows; r += 4) {
-        const int64_t row = row0 + r;
-        const float *src = in + row * static_cast<int64_t>(T);
-        float *dst = X + r * LD;
-        for (int j = lane; j < used; j += kWave) {
-            const int time = CAUSAL ? (tHi - j) : (t0 + j);
-            float v = 0.0f;
-            if (row < rows && time >= 0 && time < T) v = src[time];
-            dst[j] = v;
+    // ---- stage: X[r][j] = in[row0+r][time(j)], zero outside the row;
+    //      time(j) = t0 + j (correlation) or tHi - j (convolution)
+    {
+        const int LD4 = LD >> 2;
+        const float invLD4 = 1.0f / static_cast<float>(LD4);
+        const int quads = nRows * LD4;
+        for (int q = tid; q < quads; q += 256) {
+            int r, j4;
+            divmod_small(q, LD4, invLD4, r, j4);
+            const float *src = in + (row0 + r) * static_cast<int64_t>(T);
+            const int j = j4 << 2;
+            float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (CAUSAL) {
+                const int tl = tHi - j - 3;            // lowest time of the quad; X order is descending
+                if (VEC) {
+                    if (tl >= 0 && tl + 3 < T) {
+                        const float4 g = *reinterpret_cast<const float4 *>(src + tl);
+                        v = make_float4(g.w, g.z, g.y, g.x);
+                    }
+                } else {
+                    if (tl + 3 >= 0 && tl + 3 < T) v.x = src[tl + 3];
+                    if (tl + 2 >= 0 && tl + 2 < T) v.y = src[tl + 2];
+                    if (tl + 1 >= 0 && tl + 1 < T) v.z = src[tl + 1];
+                    if (tl >= 0 && tl < T) v.w = src[tl];
+                }
+            } else {
+                const int tl = t0 + j;
+                if (VEC) {
+                    if (tl + 3 < T) v = *reinterpret_cast<const float4 *>(src + tl);
+                } else {
+                    if (tl < T) v.x = src[tl];
+                    if (tl + 1 < T) v.y = src[tl + 1];
+                    if (tl + 2 < T) v.z = src[tl + 2];
+                    if (tl + 3 < T) v.w = src[tl + 3];
+                }
+            }
+            *reinterpret_cast<float4 *>(X + r * LD + j) = v;
         }
     }
     __syncthreads();
 
-    const int r = lane & 31;
-    const int slot = wave * 2 + (lane >> 5);
-    const int64_t row = row0 + r;
-    const float *xr = X + r * LD;
+    // ---- compute: work item = (row, chunk of 8 outputs), row-major over lanes
     const int nChunks = ttp / kFirU;
+    const float invChunks = 1.0f / static_cast<float>(nChunks);
+    const int items = nRows * nChunks;
     const int F4 = F & ~3;
 
-    for (int c = slot; c < nChunks; c += kFirSlots) {
+    for (int w = tid; w < items; w += 256) {
+        int r, c;
+        divmod_small(w, nChunks, invChunks, r, c);
         const int m0 = c * kFirU;
         float acc[kFirU];
 #pragma unroll
         for (int j = 0; j < kFirU; ++j) acc[j] = 0.0f;
 
-        const float4 *xq = reinterpret_cast<const float4 *>(xr + m0);
+        const float4 *xq = reinterpret_cast<const float4 *>(X + r * LD + m0);
         float4 qa = xq[0], qb = xq[1], qc = xq[2];
         int i = 0, q = 3;
         // three 4-tap blocks per trip so that the window rotates through registers without moves
@@ -137,25 +173,71 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
             const float f0 = filt[i];
             const float f1 = (i + 1 < F) ? filt[i + 1] : 0.0f;
             const float f2 = (i + 2 < F) ? filt[i + 2] : 0.0f;
-            const float w[12] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w, qc.x, qc.y, qc.z, qc.w};
+            const float wv[12] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w, qc.x, qc.y, qc.z, qc.w};
 #pragma unroll
             for (int j = 0; j < kFirU; ++j) {
-                acc[j] = __builtin_fmaf(w[j], f0, acc[j]);
-                if (i + 1 < F) acc[j] = __builtin_fmaf(w[j + 1], f1, acc[j]);
-                if (i + 2 < F) acc[j] = __builtin_fmaf(w[j + 2], f2, acc[j]);
+                acc[j] = __builtin_fmaf(wv[j], f0, acc[j]);
+                if (i + 1 < F) acc[j] = __builtin_fmaf(wv[j + 1], f1, acc[j]);
+                if (i + 2 < F) acc[j] = __builtin_fmaf(wv[j + 2], f2, acc[j]);
             }
         }
 
-        if (row < rows) {
-            float *dst = out + row * static_cast<int64_t>(T);
+        // ---- store the 8 outputs: times t0+m0 .. +7 (correlation) or tHi-m0-7 .. tHi-m0 (convolution)
+        float *dst = out + (row0 + r) * static_cast<int64_t>(T);
+        float y[kFirU];
 #pragma unroll
-            for (int j = 0; j < kFirU; ++j) {
-                const int m = m0 + j;
-                const int time = CAUSAL ? (tHi - m) : (t0 + m);
-                if (time >= t0 && time < t0 + tt) dst[time] = acc[j] * Ts;
-            }
+        for (int j = 0; j < kFirU; ++j) y[j] = (CAUSAL ? acc[kFirU - 1 - j] : acc[j]) * Ts;
+        const int tl = CAUSAL ? (tHi - m0 - (kFirU - 1)) : (t0 + m0);   // lowest time of the chunk
+        if (VEC) {
+            // tl is a multiple of 4 and so is the tile's end, so each half is all in or all out
+            if (tl >= t0 && tl + 3 < t0 + tt)
+                *reinterpret_cast<float4 *>(dst + tl) = make_float4(y[0], y[1], y[2], y[3]);
+            if (tl + 4 >= t0 && tl + 7 < t0 + tt)
+                *reinterpret_cast<float4 *>(dst + tl + 4) = make_float4(y[4], y[5], y[6], y[7]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < kFirU; ++j)
+                if (tl + j >= t0 && tl + j < t0 + tt) dst[tl + j] = y[j];
         }
     }
+}
+
+struct FirPlan {
+    int TT, LD, R, nTiles;
+};
+
+// Chooses the time tile, the LDS row pitch and the rows per work-group.
+static bool plan_fir(int64_t rows, int64_t T, int64_t F, FirPlan &p)
+{
+    // a row of X holds ttp + F + 4 samples (chunk-rounded tile, halo, window over-read)
+    const int64_t ttMax = (kFirMaxPitch - 4 - F) & ~static_cast<int64_t>(kFirU - 1);
+    if (F < 1 || ttMax < 64) return false;
+    const int64_t nTiles = ceil_div(T, ttMax);
+    if (nTiles > 65535) return false;
+    int64_t TT = ceil_div(ceil_div(T, nTiles), kFirU) * kFirU;
+    if (nTiles == 1) TT = T;
+    const int64_t ttp = ceil_div(TT, kFirU) * kFirU;
+    const int64_t LD = (ttp + F + 4 + 3) & ~static_cast<int64_t>(3);
+    const int64_t nChunks = ttp / kFirU;
+    // rows per group: fill the 256 lanes evenly with (row, chunk) items, stay within the LDS
+    // budget, and prefer small tiles (more groups per CU overlap staging with compute)
+    const int64_t rMax = kFirMaxLdsFloats / LD;
+    if (rMax < 1) return false;
+    int64_t best = 1;
+    double bestScore = -1.0;
+    for (int64_t r = 1; r <= rMax && r <= 64; ++r) {
+        const int64_t items = r * nChunks;
+        const double eff = static_cast<double>(items) / static_cast<double>(ceil_div(items, 256) * 256);
+        // at least ~3 passes of work per staging, mild preference for less LDS
+        const double score = eff - (items < 512 ? 0.25 : 0.0) - 0.02 * static_cast<double>(r * LD) / kFirMaxLdsFloats;
+        if (score > bestScore) { bestScore = score; best = r; }
+    }
+    if (best > rows) best = rows;
+    p.TT = static_cast<int>(TT);
+    p.LD = static_cast<int>(LD);
+    p.R = static_cast<int>(best);
+    p.nTiles = static_cast<int>(nTiles);
+    return true;
 }
 
 template <bool CAUSAL>
@@ -167,23 +249,19 @@ static int launch_fir(float *out, const float *in, const float *filt, int64_t ro
     if (!out || !in || (F > 0 && !filt)) return SLAYER_EINVAL;
     if (T >= (1LL << 30)) return SLAYER_EUNSUPPORTED;
 
-    // largest tile (multiple of the chunk) whose row pitch fits the LDS budget
-    const int64_t ttMax = (kFirMaxLD - 4 - F) & ~static_cast<int64_t>(kFirU - 1);
-    const bool tiled = !generic_forced() && F >= 1 && ttMax >= 64 && rows < (1LL << 31) * kFirRows;
-    if (tiled) {
-        const int64_t nTiles = ceil_div(T, ttMax);
-        int64_t TT = ceil_div(ceil_div(T, nTiles), kFirU) * kFirU;
-        if (nTiles == 1) TT = T;
-        const int64_t ttp = ceil_div(TT, kFirU) * kFirU;
-        int64_t LD = ttp + F + 4;
-        LD = ((LD - 4 + 31) / 32) * 32 + 4;  // 4 (mod 32): conflict-free 16-byte reads per slot
-        const int64_t rowTiles = ceil_div(rows, kFirRows);
-        if (nTiles <= 65535 && LD <= kFirMaxLD) {
-            dim3 grid(static_cast<unsigned>(rowTiles), static_cast<unsigned>(nTiles)), block(256);
-            const size_t lds = static_cast<size_t>(kFirRows) * LD * sizeof(float);
-            hipLaunchKernelGGL(fir_tiled_kernel<CAUSAL>, grid, block, lds, stream, out, in, filt, rows,
-                               static_cast<int>(T), static_cast<int>(F), static_cast<int>(TT),
-                               static_cast<int>(LD), Ts);
+    FirPlan p;
+    if (!generic_forced() && plan_fir(rows, T, F, p)) {
+        const int64_t rowTiles = ceil_div(rows, p.R);
+        if (rowTiles < (1LL << 31)) {
+            dim3 grid(static_cast<unsigned>(rowTiles), static_cast<unsigned>(p.nTiles)), block(256);
+            const size_t lds = static_cast<size_t>(p.R) * p.LD * sizeof(float);
+            const bool vec = (T % 4 == 0) && aligned16(out) && aligned16(in);
+            if (vec)
+                hipLaunchKernelGGL((fir_tiled_kernel<CAUSAL, true>), grid, block, lds, stream, out, in, filt,
+                                   rows, static_cast<int>(T), static_cast<int>(F), p.TT, p.LD, p.R, Ts);
+            else
+                hipLaunchKernelGGL((fir_tiled_kernel<CAUSAL, false>), grid, block, lds, stream, out, in, filt,
+                                   rows, static_cast<int>(T), static_cast<int>(F), p.TT, p.LD, p.R, Ts);
             return launch_status();
         }
     }

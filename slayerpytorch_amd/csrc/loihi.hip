@@ -84,8 +84,9 @@ __global__ __launch_bounds__(64) void loihi_stream_kernel(float *__restrict__ s,
                                                           const float *__restrict__ w, int64_t rows,
                                                           int T, LoihiParams p)
 {
-    __shared__ float tileC[kWave * kLoihiChunk];  // input, then current
-    __shared__ float tileV[kWave * kLoihiChunk];  // voltage
+    constexpr int P = kLoihiChunk + 1;  // padded pitch: column k of row r sits in bank (r + k) mod 32
+    __shared__ float tileC[kWave * P];  // input, then current
+    __shared__ float tileV[kWave * P];  // voltage
 
     const int lane = threadIdx.x;
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kWave;
@@ -93,8 +94,7 @@ __global__ __launch_bounds__(64) void loihi_stream_kernel(float *__restrict__ s,
     const int segT = lane & 31;
     const int segR = lane >> 5;
 
-    // rotated tile: sample k of row r at column (k + r) mod 32 -> 32 distinct banks either way
-    auto slot = [](int r, int k) { return r * kLoihiChunk + ((k + r) & (kLoihiChunk - 1)); };
+    auto slot = [](int r, int k) { return r * P + k; };
 
     LoihiState st = {0, 0, 0u};
 

@@ -18,6 +18,11 @@
 // The ring is rotated by the row number (sample t of row r lives at column (t + r) mod L), so
 // both access patterns - a fixed column over 32 rows and 32 consecutive columns of one row -
 // hit 32 different LDS banks.
+//
+// Short refractory kernels (nuSize <= 24, the normal case) use a faster variant of the same
+// scheme: the samples the refractory kernel can still reach live in a per-lane register
+// window instead of the ring, so the in-place additions are register adds and LDS only
+// transposes the chunk on its way in and out.
 #include "common.h"
 
 namespace slayer {
@@ -130,6 +135,99 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
     }
 }
 
+// ---- register-window kernel (nuSize <= NU) -----------------------------------------------------------
+// NU: window length, a compile-time bound on nuSize.  Lane = row keeps v[0 .. 32+NU-2], the
+// membrane potential of 32 + NU - 1 consecutive time steps.  Each trip loads the next 32
+// samples of every row (transposed through LDS), walks 32 time steps - a spike adds nu[0..NU)
+// onto v[k .. k+NU) - and retires the 32 oldest samples.  The walk therefore lags the loads by
+// NU - 1 steps.  Taps beyond nuSize are -0.0f, whose addition changes no value; positions
+// before the first and after the last sample hold NaN, which never reaches the threshold.
+template <int NU>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) void spike_window_kernel(float *__restrict__ s, float *u,
+                                                          const float *__restrict__ nu,
+                                                          int64_t rows, int T, int nuSize,
+                                                          float theta, float Ts)
+{
+    constexpr int C = kSpikeChunk;
+    constexpr int LAG = NU - 1;
+    constexpr int P = C + 1;  // padded pitch: column k of row r sits in bank (r + k) mod 32
+    __shared__ float tile[kWave * P];
+
+    const int lane = threadIdx.x;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kWave;
+    const float amplitude = 1.0f / Ts;
+    const float quiet = __builtin_nanf("");
+    const int segT = lane & 31;
+    const int segR = lane >> 5;
+    auto slot = [](int r, int k) { return r * P + k; };
+
+    float tap[NU];
+#pragma unroll
+    for (int j = 0; j < NU; ++j) tap[j] = (j < nuSize) ? nu[j] : -0.0f;
+
+    float v[C + LAG];
+#pragma unroll
+    for (int k = 0; k < LAG; ++k) v[k] = quiet;
+
+    const int trips = (T + LAG + C - 1) / C;
+    for (int it = 0; it < trips; ++it) {
+        const int tLoad = it * C;       // first time step loaded in this trip
+        const int tWalk = tLoad - LAG;  // first time step walked (and retired) in this trip
+
+        // load: lanes along time, two 128-byte row segments per instruction
+        {
+            const int t = tLoad + segT;
+#pragma unroll 8
+            for (int i = 0; i < 32; ++i) {
+                const int r = 2 * i + segR;
+                const int64_t row = row0 + r;
+                float x = quiet;
+                if (row < rows && t < T) x = u[row * static_cast<int64_t>(T) + t];
+                tile[slot(r, segT)] = x;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < C; ++k) v[LAG + k] = tile[slot(lane, k)];
+        __syncthreads();
+
+        // walk 32 time steps
+        uint32_t fired = 0;
+#pragma unroll
+        for (int k = 0; k < C; ++k) {
+            if (v[k] >= theta) {
+                fired |= 1u << k;
+#pragma unroll
+                for (int j = 0; j < NU; ++j) v[k + j] += tap[j];
+            }
+        }
+
+        // retire: the 32 oldest samples are final
+#pragma unroll
+        for (int k = 0; k < C; ++k) tile[slot(lane, k)] = v[k];
+        __syncthreads();
+        {
+            const int t = tWalk + segT;
+#pragma unroll 8
+            for (int i = 0; i < 32; ++i) {
+                const int r = 2 * i + segR;
+                const int64_t row = row0 + r;
+                const float uv = tile[slot(r, segT)];
+                const uint32_t m = __shfl(fired, r, kWave);
+                const float sv = ((m >> segT) & 1u) ? amplitude : 0.0f;
+                if (row < rows && t >= 0 && t < T) {
+                    const int64_t g = row * static_cast<int64_t>(T) + t;
+                    u[g] = uv;
+                    s[g] = sv;
+                }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < LAG; ++k) v[k] = v[C + k];
+    }
+}
+
 // ---- surrogate gradient ------------------------------------------------------------------------------
 template <int VEC>
 __global__ __launch_bounds__(256) void spike_bwd_kernel(float *gradIn, const float *gradOut,
@@ -167,6 +265,21 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
 
     const int64_t groups = ceil_div(nNeurons, kWave);
     const bool stream_ok = !generic_forced() && T < (1LL << 30) && groups < (1LL << 31);
+#define SLAYER_SPIKE_WINDOW(NU)                                                                          \
+    do {                                                                                                \
+        hipLaunchKernelGGL(spike_window_kernel<NU>, dim3(static_cast<unsigned>(groups)), dim3(kWave), 0,  \
+                           st, s, u, nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize), theta,  \
+                           Ts);                                                                         \
+        return launch_status();                                                                         \
+    } while (0)
+    if (stream_ok && nuSize <= 24) {
+        if (nuSize <= 4) SLAYER_SPIKE_WINDOW(4);
+        if (nuSize <= 8) SLAYER_SPIKE_WINDOW(8);
+        if (nuSize <= 12) SLAYER_SPIKE_WINDOW(12);
+        if (nuSize <= 16) SLAYER_SPIKE_WINDOW(16);
+        SLAYER_SPIKE_WINDOW(24);
+    }
+#undef SLAYER_SPIKE_WINDOW
     if (stream_ok && nuSize <= 33) {
         hipLaunchKernelGGL(spike_stream_kernel<64>, dim3(static_cast<unsigned>(groups)), dim3(kWave), 0,
                            st, s, u, nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize), theta,
