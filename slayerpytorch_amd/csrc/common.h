@@ -37,6 +37,47 @@ __device__ __forceinline__ int trunc_sat(float x)
 // Number of whole sampling steps in a delay: fp32 quotient truncated toward zero.
 __device__ __forceinline__ int delay_steps(float delay, float Ts) { return trunc_sat(delay / Ts); }
 
+// ---- buffer addressing -------------------------------------------------------------------------
+// address = base (128-bit descriptor in scalar registers) + per-lane byte offset (one vector
+// register) + wave-uniform byte offset (scalar register).  Lets a wave touch many rows of a tile
+// without a 64-bit address register per access.  Both offsets are 32 bit: kernels that use it
+// keep tiles below 2 GiB (rows of at most kBufferMaxT samples).
+typedef __amdgpu_buffer_rsrc_t BufferRsrc;
+constexpr int64_t kBufferMaxT = 1 << 22;
+
+__device__ __forceinline__ BufferRsrc make_buffer(const void *base)
+{
+    // raw buffer, no stride/swizzle, 32-bit data format; range = the whole 32-bit offset space
+    // (validity of every access is established by the caller's own predicates)
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x7fffffff, 0x00020000);
+}
+
+__device__ __forceinline__ float buffer_load(BufferRsrc b, int laneBytes, int uniformBytes)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(b, laneBytes, uniformBytes, 0));
+}
+
+typedef float float4_ext __attribute__((ext_vector_type(4)));
+typedef unsigned int uint4_ext __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float4 buffer_load4(BufferRsrc b, int laneBytes, int uniformBytes)
+{
+    const uint4_ext x = __builtin_amdgcn_raw_buffer_load_b128(b, laneBytes, uniformBytes, 0);
+    const float4_ext f = __builtin_bit_cast(float4_ext, x);
+    return make_float4(f.x, f.y, f.z, f.w);
+}
+
+__device__ __forceinline__ void buffer_store4(BufferRsrc b, int laneBytes, int uniformBytes, float4 v)
+{
+    const float4_ext f = {v.x, v.y, v.z, v.w};
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4_ext, f), b, laneBytes, uniformBytes, 0);
+}
+
+__device__ __forceinline__ void buffer_store(BufferRsrc b, int laneBytes, int uniformBytes, float x)
+{
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, x), b, laneBytes, uniformBytes, 0);
+}
+
 }  // namespace slayer
 
 #endif

@@ -72,6 +72,19 @@ __device__ __forceinline__ void divmod_small(int i, int d, float inv, int &q, in
     else if (r >= d) { ++q; r -= d; }
 }
 
+// (row, column) = divmod(index, width) advanced incrementally: the work index grows by 256 per
+// trip, so the pair moves by (256 / width, 256 % width) with one carry.
+struct RowCol {
+    int r, c;
+    __device__ __forceinline__ void init(int index, int width, float inv) { divmod_small(index, width, inv, r, c); }
+    __device__ __forceinline__ void advance(int dr, int dc, int width)
+    {
+        r += dr;
+        c += dc;
+        if (c >= width) { c -= width; ++r; }
+    }
+};
+
 // VEC: rows are whole 16-byte vectors (T % 4 == 0, pointers 16-byte aligned)
 template <bool CAUSAL, bool VEC>
 __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
@@ -89,11 +102,48 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
     const int tt = min(TT, T - t0);                   // outputs in this tile
     const int ttp = (tt + kFirU - 1) & ~(kFirU - 1);  // rounded up to whole chunks
     const int tHi = t0 + ttp - 1;                     // time stored at X[.][0] when reversed
+    const int LD4 = LD >> 2;
+
+    // The tile's rows as 32-bit offsets from its first row (a tile spans far less than 2 GiB).
+    const BufferRsrc bufIn = make_buffer(in + row0 * static_cast<int64_t>(T));
+    const BufferRsrc bufOut = make_buffer(out + row0 * static_cast<int64_t>(T));
 
     // ---- stage: X[r][j] = in[row0+r][time(j)], zero outside the row;
     //      time(j) = t0 + j (correlation) or tHi - j (convolution)
-    {
-        const int LD4 = LD >> 2;
+    if (VEC) {
+        // samples of the row that the tile needs: times [tA, tB), whole 16-byte vectors
+        const int tA = CAUSAL ? max(0, tHi + 1 - LD) : t0;
+        const int tB = CAUSAL ? min(T, tHi + 1) : min(T, t0 + LD);
+        const int nq = (tB - tA) >> 2;               // source vectors per row
+        const int jA = CAUSAL ? (tHi + 1 - tB) : 0;  // X columns [jA, jA + 4 nq) receive them
+        {
+            RowCol rc;
+            rc.init(tid, nq, 1.0f / static_cast<float>(nq));
+            const int dr = 256 / nq, dc = 256 % nq;
+            const int total = nRows * nq;
+            for (int g = tid; g < total; g += 256, rc.advance(dr, dc, nq)) {
+                const float4 v = buffer_load4(bufIn, (rc.r * T + tA + (rc.c << 2)) * 4, 0);
+                if (CAUSAL)  // descending time: the vector lands mirrored
+                    *reinterpret_cast<float4 *>(X + rc.r * LD + (jA + ((nq - 1 - rc.c) << 2))) =
+                        make_float4(v.w, v.z, v.y, v.x);
+                else
+                    *reinterpret_cast<float4 *>(X + rc.r * LD + (rc.c << 2)) = v;
+            }
+        }
+        // zero padding: columns [0, jA) and [jA + 4 nq, LD)
+        const int zq = LD4 - nq;
+        if (zq > 0) {
+            RowCol rc;
+            rc.init(tid, zq, 1.0f / static_cast<float>(zq));
+            const int dr = 256 / zq, dc = 256 % zq;
+            const int total = nRows * zq;
+            const int head = jA >> 2;
+            for (int g = tid; g < total; g += 256, rc.advance(dr, dc, zq)) {
+                const int j4 = (rc.c < head) ? rc.c : (rc.c + nq);
+                *reinterpret_cast<float4 *>(X + rc.r * LD + (j4 << 2)) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            }
+        }
+    } else {
         const float invLD4 = 1.0f / static_cast<float>(LD4);
         const int quads = nRows * LD4;
         for (int q = tid; q < quads; q += 256) {
@@ -103,28 +153,17 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
             const int j = j4 << 2;
             float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if (CAUSAL) {
-                const int tl = tHi - j - 3;            // lowest time of the quad; X order is descending
-                if (VEC) {
-                    if (tl >= 0 && tl + 3 < T) {
-                        const float4 g = *reinterpret_cast<const float4 *>(src + tl);
-                        v = make_float4(g.w, g.z, g.y, g.x);
-                    }
-                } else {
-                    if (tl + 3 >= 0 && tl + 3 < T) v.x = src[tl + 3];
-                    if (tl + 2 >= 0 && tl + 2 < T) v.y = src[tl + 2];
-                    if (tl + 1 >= 0 && tl + 1 < T) v.z = src[tl + 1];
-                    if (tl >= 0 && tl < T) v.w = src[tl];
-                }
+                const int tl = tHi - j - 3;  // lowest time of the quad; X order is descending
+                if (tl + 3 >= 0 && tl + 3 < T) v.x = src[tl + 3];
+                if (tl + 2 >= 0 && tl + 2 < T) v.y = src[tl + 2];
+                if (tl + 1 >= 0 && tl + 1 < T) v.z = src[tl + 1];
+                if (tl >= 0 && tl < T) v.w = src[tl];
             } else {
                 const int tl = t0 + j;
-                if (VEC) {
-                    if (tl + 3 < T) v = *reinterpret_cast<const float4 *>(src + tl);
-                } else {
-                    if (tl < T) v.x = src[tl];
-                    if (tl + 1 < T) v.y = src[tl + 1];
-                    if (tl + 2 < T) v.z = src[tl + 2];
-                    if (tl + 3 < T) v.w = src[tl + 3];
-                }
+                if (tl < T) v.x = src[tl];
+                if (tl + 1 < T) v.y = src[tl + 1];
+                if (tl + 2 < T) v.z = src[tl + 2];
+                if (tl + 3 < T) v.w = src[tl + 3];
             }
             *reinterpret_cast<float4 *>(X + r * LD + j) = v;
         }
@@ -133,14 +172,15 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
 
     // ---- compute: work item = (row, chunk of 8 outputs), row-major over lanes
     const int nChunks = ttp / kFirU;
-    const float invChunks = 1.0f / static_cast<float>(nChunks);
     const int items = nRows * nChunks;
     const int F4 = F & ~3;
+    RowCol item;
+    item.init(tid, nChunks, 1.0f / static_cast<float>(nChunks));
+    const int itemDr = 256 / nChunks, itemDc = 256 % nChunks;
 
-    for (int w = tid; w < items; w += 256) {
-        int r, c;
-        divmod_small(w, nChunks, invChunks, r, c);
-        const int m0 = c * kFirU;
+    for (int w = tid; w < items; w += 256, item.advance(itemDr, itemDc, nChunks)) {
+        const int r = item.r;
+        const int m0 = item.c * kFirU;
         float acc[kFirU];
 #pragma unroll
         for (int j = 0; j < kFirU; ++j) acc[j] = 0.0f;
@@ -183,18 +223,18 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
         }
 
         // ---- store the 8 outputs: times t0+m0 .. +7 (correlation) or tHi-m0-7 .. tHi-m0 (convolution)
-        float *dst = out + (row0 + r) * static_cast<int64_t>(T);
         float y[kFirU];
 #pragma unroll
         for (int j = 0; j < kFirU; ++j) y[j] = (CAUSAL ? acc[kFirU - 1 - j] : acc[j]) * Ts;
-        const int tl = CAUSAL ? (tHi - m0 - (kFirU - 1)) : (t0 + m0);   // lowest time of the chunk
+        const int tl = CAUSAL ? (tHi - m0 - (kFirU - 1)) : (t0 + m0);  // lowest time of the chunk
         if (VEC) {
             // tl is a multiple of 4 and so is the tile's end, so each half is all in or all out
-            if (tl >= t0 && tl + 3 < t0 + tt)
-                *reinterpret_cast<float4 *>(dst + tl) = make_float4(y[0], y[1], y[2], y[3]);
+            const int off = (r * T + tl) * 4;
+            if (tl >= t0 && tl + 3 < t0 + tt) buffer_store4(bufOut, off, 0, make_float4(y[0], y[1], y[2], y[3]));
             if (tl + 4 >= t0 && tl + 7 < t0 + tt)
-                *reinterpret_cast<float4 *>(dst + tl + 4) = make_float4(y[4], y[5], y[6], y[7]);
+                buffer_store4(bufOut, off + 16, 0, make_float4(y[4], y[5], y[6], y[7]));
         } else {
+            float *dst = out + (row0 + r) * static_cast<int64_t>(T);
 #pragma unroll
             for (int j = 0; j < kFirU; ++j)
                 if (tl + j >= t0 && tl + j < t0 + tt) dst[tl + j] = y[j];
@@ -211,7 +251,7 @@ static bool plan_fir(int64_t rows, int64_t T, int64_t F, FirPlan &p)
 {
     // a row of X holds ttp + F + 4 samples (chunk-rounded tile, halo, window over-read)
     const int64_t ttMax = (kFirMaxPitch - 4 - F) & ~static_cast<int64_t>(kFirU - 1);
-    if (F < 1 || ttMax < 64) return false;
+    if (F < 1 || ttMax < 64 || T > kBufferMaxT) return false;
     const int64_t nTiles = ceil_div(T, ttMax);
     if (nTiles > 65535) return false;
     int64_t TT = ceil_div(ceil_div(T, nTiles), kFirU) * kFirU;

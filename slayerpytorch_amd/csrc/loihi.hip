@@ -79,70 +79,92 @@ __global__ __launch_bounds__(256) void loihi_generic_kernel(float *__restrict__ 
 }
 
 // ---- streaming kernel -------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void loihi_stream_kernel(float *__restrict__ s, float *__restrict__ v,
-                                                          float *__restrict__ u,
-                                                          const float *__restrict__ w, int64_t rows,
-                                                          int T, LoihiParams p)
+// Global traffic uses buffer addressing (per-lane offset + wave-uniform offset per row pair); the
+// 32 loads of a chunk are issued one chunk ahead and stay in flight during the sequential update.
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 8))) void loihi_stream_kernel(
+    float *__restrict__ s, float *__restrict__ v, float *__restrict__ u, const float *__restrict__ w,
+    int64_t rows, int T, LoihiParams p)
 {
-    constexpr int P = kLoihiChunk + 1;  // padded pitch: column k of row r sits in bank (r + k) mod 32
+    constexpr int C = kLoihiChunk;
+    constexpr int P = C + 1;  // padded pitch: column k of row r sits in bank (r + k) mod 32
     __shared__ float tileC[kWave * P];  // input, then current
     __shared__ float tileV[kWave * P];  // voltage
 
     const int lane = threadIdx.x;
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kWave;
-    const int nChunks = (T + kLoihiChunk - 1) / kLoihiChunk;
+    const bool fullTile = row0 + kWave <= rows;
+    const int nChunks = (T + C - 1) / C;
     const int segT = lane & 31;
     const int segR = lane >> 5;
-
     auto slot = [](int r, int k) { return r * P + k; };
+
+    const int64_t tileBase = row0 * static_cast<int64_t>(T);
+    const BufferRsrc bufW = make_buffer(w + tileBase);
+    const BufferRsrc bufS = make_buffer(s + tileBase);
+    const BufferRsrc bufV = make_buffer(v + tileBase);
+    const BufferRsrc bufU = make_buffer(u + tileBase);
+    const int laneOff = (segR * T + segT) * 4;
+    const int pairStride = 2 * T * 4;
+
+    float pre[C];
+    auto issue_loads = [&](int tBase) {
+        const int off = laneOff + tBase * 4;
+        if (fullTile && tBase + C <= T) {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) pre[i] = buffer_load(bufW, off, i * pairStride);
+        } else {
+            const bool tOk = tBase + segT < T;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                pre[i] = 0.0f;
+                if (tOk && row0 + 2 * i + segR < rows) pre[i] = buffer_load(bufW, off, i * pairStride);
+            }
+        }
+    };
 
     LoihiState st = {0, 0, 0u};
 
+    issue_loads(0);
     for (int c = 0; c < nChunks; ++c) {
-        const int tBase = c * kLoihiChunk;
-        {
-            const int t = tBase + segT;
-#pragma unroll 8
-            for (int it = 0; it < 32; ++it) {
-                const int r = 2 * it + segR;
-                const int64_t row = row0 + r;
-                float x = 0.0f;
-                if (row < rows && t < T) x = w[row * static_cast<int64_t>(T) + t];
-                tileC[slot(r, segT)] = x;
-            }
-        }
+        const int tBase = c * C;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) tileC[slot(2 * i + segR, segT)] = pre[i];
         __syncthreads();
+        issue_loads(tBase + C);  // past the end of the rows this loads nothing
 
+        // sequential update: lane = row
         uint32_t fired = 0;
-        const int steps = min(kLoihiChunk, T - tBase);
-        for (int k = 0; k < steps; ++k) {
+        const int first = (c == 0) ? 1 : 0;  // t = 0 is forced to zero
+        if (c == 0) {
+            tileC[slot(lane, 0)] = 0.0f;
+            tileV[slot(lane, 0)] = 0.0f;
+        }
+#pragma unroll 8
+        for (int k = first; k < C; ++k) {
             const int i = slot(lane, k);
-            float cOut = 0.0f, vOut = 0.0f;
-            if (tBase + k > 0) {
-                const uint32_t spike = loihi_step(st, p, tileC[i], cOut, vOut);
-                fired |= spike << k;
-            }
+            float cOut, vOut;
+            const uint32_t spike = loihi_step(st, p, tileC[i], cOut, vOut);
+            fired |= spike << k;
             tileC[i] = cOut;
             tileV[i] = vOut;
         }
         __syncthreads();
 
         {
-            const int t = tBase + segT;
+            const int off = laneOff + tBase * 4;
+            const bool fast = fullTile && tBase + C <= T;
+            const bool tOk = tBase + segT < T;
 #pragma unroll 8
-            for (int it = 0; it < 32; ++it) {
-                const int r = 2 * it + segR;
-                const int64_t row = row0 + r;
-                const int i = slot(r, segT);
-                const float cv = tileC[i];
-                const float vv = tileV[i];
+            for (int i = 0; i < 32; ++i) {
+                const int r = 2 * i + segR;
+                const float cv = tileC[slot(r, segT)];
+                const float vv = tileV[slot(r, segT)];
                 const uint32_t m = __shfl(fired, r, kWave);
                 const float sv = ((m >> segT) & 1u) ? 1.0f : 0.0f;
-                if (row < rows && t < T) {
-                    const int64_t g = row * static_cast<int64_t>(T) + t;
-                    s[g] = sv;
-                    v[g] = vv;
-                    u[g] = cv;
+                if (fast || (tOk && row0 + r < rows)) {
+                    buffer_store(bufS, off, i * pairStride, sv);
+                    buffer_store(bufV, off, i * pairStride, vv);
+                    buffer_store(bufU, off, i * pairStride, cv);
                 }
             }
         }
@@ -173,7 +195,7 @@ extern "C" int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const f
     p.theta = theta;
 
     const int64_t groups = ceil_div(nNeurons, kWave);
-    if (!generic_forced() && T < (1LL << 30) && groups < (1LL << 31)) {
+    if (!generic_forced() && T <= kBufferMaxT && groups < (1LL << 31)) {
         hipLaunchKernelGGL(loihi_stream_kernel, dim3(static_cast<unsigned>(groups)), dim3(kWave), 0, st,
                            s, v, u, w, nNeurons, static_cast<int>(T), p);
         return launch_status();

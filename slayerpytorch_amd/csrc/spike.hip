@@ -142,11 +142,15 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
 // onto v[k .. k+NU) - and retires the 32 oldest samples.  The walk therefore lags the loads by
 // NU - 1 steps.  Taps beyond nuSize are -0.0f, whose addition changes no value; positions
 // before the first and after the last sample hold NaN, which never reaches the threshold.
+//
+// Global traffic uses buffer addressing: one per-lane byte offset (row parity and time within
+// the segment) plus a wave-uniform scalar offset per row pair, so the 32 loads of a trip need
+// no per-load address registers, are all issued together one trip ahead of their use, and stay
+// in flight while the current trip is walked.
 template <int NU>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) void spike_window_kernel(float *__restrict__ s, float *u,
-                                                          const float *__restrict__ nu,
-                                                          int64_t rows, int T, int nuSize,
-                                                          float theta, float Ts)
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) void spike_window_kernel(
+    float *__restrict__ s, float *u, const float *__restrict__ nu, int64_t rows, int T, int nuSize,
+    float theta, float Ts)
 {
     constexpr int C = kSpikeChunk;
     constexpr int LAG = NU - 1;
@@ -155,11 +159,17 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) void
 
     const int lane = threadIdx.x;
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kWave;
+    const bool fullTile = row0 + kWave <= rows;
     const float amplitude = 1.0f / Ts;
     const float quiet = __builtin_nanf("");
     const int segT = lane & 31;
     const int segR = lane >> 5;
     auto slot = [](int r, int k) { return r * P + k; };
+
+    const BufferRsrc bufU = make_buffer(u + row0 * static_cast<int64_t>(T));
+    const BufferRsrc bufS = make_buffer(s + row0 * static_cast<int64_t>(T));
+    const int laneOff = (segR * T + segT) * 4;  // byte offset of (row parity, time in segment)
+    const int pairStride = 2 * T * 4;           // bytes between row pairs
 
     float tap[NU];
 #pragma unroll
@@ -169,27 +179,35 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) void
 #pragma unroll
     for (int k = 0; k < LAG; ++k) v[k] = quiet;
 
-    const int trips = (T + LAG + C - 1) / C;
-    for (int it = 0; it < trips; ++it) {
-        const int tLoad = it * C;       // first time step loaded in this trip
-        const int tWalk = tLoad - LAG;  // first time step walked (and retired) in this trip
-
-        // load: lanes along time, two 128-byte row segments per instruction
-        {
-            const int t = tLoad + segT;
-#pragma unroll 8
+    float pre[C];
+    auto issue_loads = [&](int tLoad) {
+        const int off = laneOff + tLoad * 4;
+        if (fullTile && tLoad + C <= T) {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) pre[i] = buffer_load(bufU, off, i * pairStride);
+        } else {
+            const bool tOk = tLoad + segT < T;
+#pragma unroll
             for (int i = 0; i < 32; ++i) {
-                const int r = 2 * i + segR;
-                const int64_t row = row0 + r;
-                float x = quiet;
-                if (row < rows && t < T) x = u[row * static_cast<int64_t>(T) + t];
-                tile[slot(r, segT)] = x;
+                pre[i] = quiet;
+                if (tOk && row0 + 2 * i + segR < rows) pre[i] = buffer_load(bufU, off, i * pairStride);
             }
         }
+    };
+
+    const int trips = (T + LAG + C - 1) / C;
+    issue_loads(0);
+    for (int it = 0; it < trips; ++it) {
+        const int tWalk = it * C - LAG;  // first time step walked (and retired) in this trip
+
+        // transpose the loaded chunk through LDS: lane = row gets its next 32 samples
+#pragma unroll
+        for (int i = 0; i < 32; ++i) tile[slot(2 * i + segR, segT)] = pre[i];
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < C; ++k) v[LAG + k] = tile[slot(lane, k)];
         __syncthreads();
+        issue_loads((it + 1) * C);  // past the end of the rows this loads nothing
 
         // walk 32 time steps
         uint32_t fired = 0;
@@ -207,18 +225,28 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) void
         for (int k = 0; k < C; ++k) tile[slot(lane, k)] = v[k];
         __syncthreads();
         {
-            const int t = tWalk + segT;
+            const int off = laneOff + tWalk * 4;
+            if (fullTile && tWalk >= 0 && tWalk + C <= T) {
 #pragma unroll 8
-            for (int i = 0; i < 32; ++i) {
-                const int r = 2 * i + segR;
-                const int64_t row = row0 + r;
-                const float uv = tile[slot(r, segT)];
-                const uint32_t m = __shfl(fired, r, kWave);
-                const float sv = ((m >> segT) & 1u) ? amplitude : 0.0f;
-                if (row < rows && t >= 0 && t < T) {
-                    const int64_t g = row * static_cast<int64_t>(T) + t;
-                    u[g] = uv;
-                    s[g] = sv;
+                for (int i = 0; i < 32; ++i) {
+                    const int r = 2 * i + segR;
+                    const float uv = tile[slot(r, segT)];
+                    const uint32_t m = __shfl(fired, r, kWave);
+                    buffer_store(bufU, off, i * pairStride, uv);
+                    buffer_store(bufS, off, i * pairStride, ((m >> segT) & 1u) ? amplitude : 0.0f);
+                }
+            } else {
+                const int t = tWalk + segT;
+                const bool tOk = t >= 0 && t < T;
+#pragma unroll 8
+                for (int i = 0; i < 32; ++i) {
+                    const int r = 2 * i + segR;
+                    const float uv = tile[slot(r, segT)];
+                    const uint32_t m = __shfl(fired, r, kWave);
+                    if (tOk && row0 + r < rows) {
+                        buffer_store(bufU, off, i * pairStride, uv);
+                        buffer_store(bufS, off, i * pairStride, ((m >> segT) & 1u) ? amplitude : 0.0f);
+                    }
                 }
             }
         }
@@ -265,6 +293,7 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
 
     const int64_t groups = ceil_div(nNeurons, kWave);
     const bool stream_ok = !generic_forced() && T < (1LL << 30) && groups < (1LL << 31);
+    const bool window_ok = stream_ok && T <= kBufferMaxT;
 #define SLAYER_SPIKE_WINDOW(NU)                                                                          \
     do {                                                                                                \
         hipLaunchKernelGGL(spike_window_kernel<NU>, dim3(static_cast<unsigned>(groups)), dim3(kWave), 0,  \
@@ -272,7 +301,7 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
                            Ts);                                                                         \
         return launch_status();                                                                         \
     } while (0)
-    if (stream_ok && nuSize <= 24) {
+    if (window_ok && nuSize <= 24) {
         if (nuSize <= 4) SLAYER_SPIKE_WINDOW(4);
         if (nuSize <= 8) SLAYER_SPIKE_WINDOW(8);
         if (nuSize <= 12) SLAYER_SPIKE_WINDOW(12);
