@@ -18,6 +18,15 @@ int note_hip_error(hipError_t err)
     return SLAYER_ELAUNCH;
 }
 
+int compute_units()
+{
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
+        return 256;
+    return cus;
+}
+
 bool generic_forced() { return g_force_generic.load(std::memory_order_relaxed) != 0; }
 
 }  // namespace slayer

@@ -17,6 +17,9 @@ int note_hip_error(hipError_t err);
 // Status of the launch that was just enqueued on this thread.
 inline int launch_status() { return note_hip_error(hipGetLastError()); }
 
+// Compute units of the current device (256 on MI355X); persistent kernels size their grid by it.
+int compute_units();
+
 // True when slayer_force_generic_kernels(1) is in effect.
 bool generic_forced();
 
@@ -36,6 +39,28 @@ __device__ __forceinline__ int trunc_sat(float x)
 
 // Number of whole sampling steps in a delay: fp32 quotient truncated toward zero.
 __device__ __forceinline__ int delay_steps(float delay, float Ts) { return trunc_sat(delay / Ts); }
+
+// i / d for 0 <= i < 2^24 with a precomputed float reciprocal (estimate plus one correction)
+__device__ __forceinline__ void divmod_small(int i, int d, float inv, int &q, int &r)
+{
+    q = static_cast<int>(static_cast<float>(i) * inv);
+    r = i - q * d;
+    if (r < 0) { --q; r += d; }
+    else if (r >= d) { ++q; r -= d; }
+}
+
+// (row, column) = divmod(index, width) advanced incrementally: the work index grows by 256 per
+// trip, so the pair moves by (256 / width, 256 % width) with one carry.
+struct RowCol {
+    int r, c;
+    __device__ __forceinline__ void init(int index, int width, float inv) { divmod_small(index, width, inv, r, c); }
+    __device__ __forceinline__ void advance(int dr, int dc, int width)
+    {
+        r += dr;
+        c += dc;
+        if (c >= width) { c -= width; ++r; }
+    }
+};
 
 // ---- buffer addressing -------------------------------------------------------------------------
 // address = base (128-bit descriptor in scalar registers) + per-lane byte offset (one vector

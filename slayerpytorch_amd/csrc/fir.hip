@@ -63,28 +63,6 @@ __device__ __forceinline__ void fma_quad(float (&acc)[kFirU], const float4 &a, c
     }
 }
 
-// i / d for 0 <= i < 2^24 with a precomputed float reciprocal (estimate plus one correction)
-__device__ __forceinline__ void divmod_small(int i, int d, float inv, int &q, int &r)
-{
-    q = static_cast<int>(static_cast<float>(i) * inv);
-    r = i - q * d;
-    if (r < 0) { --q; r += d; }
-    else if (r >= d) { ++q; r -= d; }
-}
-
-// (row, column) = divmod(index, width) advanced incrementally: the work index grows by 256 per
-// trip, so the pair moves by (256 / width, 256 % width) with one carry.
-struct RowCol {
-    int r, c;
-    __device__ __forceinline__ void init(int index, int width, float inv) { divmod_small(index, width, inv, r, c); }
-    __device__ __forceinline__ void advance(int dr, int dc, int width)
-    {
-        r += dr;
-        c += dc;
-        if (c >= width) { c -= width; ++r; }
-    }
-};
-
 // VEC: rows are whole 16-byte vectors (T % 4 == 0, pointers 16-byte aligned)
 template <bool CAUSAL, bool VEC>
 __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,

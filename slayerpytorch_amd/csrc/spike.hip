@@ -19,10 +19,9 @@
 // both access patterns - a fixed column over 32 rows and 32 consecutive columns of one row -
 // hit 32 different LDS banks.
 //
-// Short refractory kernels (nuSize <= 24, the normal case) use a faster variant of the same
-// scheme: the samples the refractory kernel can still reach live in a per-lane register
-// window instead of the ring, so the in-place additions are register adds and LDS only
-// transposes the chunk on its way in and out.
+// Short refractory kernels (nuSize <= 24, the normal case) take the row-tile kernel further
+// down instead: fewer rows per wavefront, long contiguous runs per row, and a per-lane register
+// window in place of the ring.
 #include "common.h"
 
 namespace slayer {
@@ -135,124 +134,179 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
     }
 }
 
-// ---- register-window kernel (nuSize <= NU) -----------------------------------------------------------
-// NU: window length, a compile-time bound on nuSize.  Lane = row keeps v[0 .. 32+NU-2], the
-// membrane potential of 32 + NU - 1 consecutive time steps.  Each trip loads the next 32
-// samples of every row (transposed through LDS), walks 32 time steps - a spike adds nu[0..NU)
-// onto v[k .. k+NU) - and retires the 32 oldest samples.  The walk therefore lags the loads by
-// NU - 1 steps.  Taps beyond nuSize are -0.0f, whose addition changes no value; positions
-// before the first and after the last sample hold NaN, which never reaches the threshold.
-//
-// Global traffic uses buffer addressing: one per-lane byte offset (row parity and time within
-// the segment) plus a wave-uniform scalar offset per row pair, so the 32 loads of a trip need
-// no per-load address registers, are all issued together one trip ahead of their use, and stay
-// in flight while the current trip is walked.
-template <int NU>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) void spike_window_kernel(
-    float *__restrict__ s, float *u, const float *__restrict__ nu, int64_t rows, int T, int nuSize,
-    float theta, float Ts)
+// ---- row-tile kernel (nuSize <= NU) --------------------------------------------------------------------
+// The fast path.  A wavefront owns kTileRows consecutive rows and moves them through LDS in
+// pieces of Tc samples per row (the whole row when it is short enough), so that global memory
+// is read and written as long contiguous runs with 16-byte accesses per lane - the access
+// pattern of a plain copy.  Lanes 0..kTileRows-1 then walk their row in LDS order:
+// 32 samples at a time are pulled into a register window v[0 .. 32+LAG), a spike adds
+// nu[0..NU) onto v[k .. k+NU) (the same fp32 additions, in the same order, as the sequential
+// loop), and the 32 oldest samples go back to LDS together with a 32-bit spike mask.  The last
+// LAG samples of a piece are not final until the next piece arrives; they wait in v[0..LAG).
+// Taps beyond nuSize are -0.0f, whose addition changes no value; slots before the first and
+// after the last sample hold NaN, which never reaches the threshold.
+// Leaving most lanes idle during the walk is deliberate: the kernel is bound by HBM traffic,
+// not by the vector ALU, and short tiles keep many wavefronts (and bytes) in flight per CU.
+constexpr int kTileRows = 16;
+constexpr int kTileMaxPiece = 352;  // longest piece (samples per row) a tile stages at once
+
+template <int NU, bool VEC>
+__global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, float *u,
+                                                        const float *__restrict__ nu, int64_t rows,
+                                                        int T, int nuSize, int Tc, int P, int MP,
+                                                        int64_t tiles, float theta, float Ts)
 {
-    constexpr int C = kSpikeChunk;
-    constexpr int LAG = NU - 1;
-    constexpr int P = C + 1;  // padded pitch: column k of row r sits in bank (r + k) mod 32
-    __shared__ float tile[kWave * P];
+    constexpr int LAG = (NU + 2) & ~3;  // look-ahead of the walk, rounded to whole 16-byte vectors
+    constexpr int G = 32;               // samples per walk group = bits of a spike mask
+    constexpr int V = VEC ? 4 : 1;      // samples per global access
+    constexpr int NB = kTileRows * kTileMaxPiece / V / kWave;  // accesses per lane per piece, at most
+    extern __shared__ __align__(16) float lds[];
+    float *tile = lds;                                                    // [kTileRows][P], P = 4 (mod 32)
+    uint32_t *masks = reinterpret_cast<uint32_t *>(lds + kTileRows * P);  // [kTileRows][MP]
 
     const int lane = threadIdx.x;
-    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kWave;
-    const bool fullTile = row0 + kWave <= rows;
     const float amplitude = 1.0f / Ts;
     const float quiet = __builtin_nanf("");
-    const int segT = lane & 31;
-    const int segR = lane >> 5;
-    auto slot = [](int r, int k) { return r * P + k; };
-
-    const BufferRsrc bufU = make_buffer(u + row0 * static_cast<int64_t>(T));
-    const BufferRsrc bufS = make_buffer(s + row0 * static_cast<int64_t>(T));
-    const int laneOff = (segR * T + segT) * 4;  // byte offset of (row parity, time in segment)
-    const int pairStride = 2 * T * 4;           // bytes between row pairs
 
     float tap[NU];
 #pragma unroll
     for (int j = 0; j < NU; ++j) tap[j] = (j < nuSize) ? nu[j] : -0.0f;
 
-    float v[C + LAG];
-#pragma unroll
-    for (int k = 0; k < LAG; ++k) v[k] = quiet;
+    float v[G + LAG];
 
-    float pre[C];
-    auto issue_loads = [&](int tLoad) {
-        const int off = laneOff + tLoad * 4;
-        if (fullTile && tLoad + C <= T) {
+    // A "step" is one piece of one tile.  The global loads of a step are issued one step ahead
+    // into x[] and stay in flight while the previous step is walked and retired.
+    float x[NB * V];
+    auto rows_of = [&](int64_t t) { return static_cast<int>(min(static_cast<int64_t>(kTileRows), rows - t * kTileRows)); };
+    auto issue = [&](int64_t t, int tL) {
+        const BufferRsrc bufU = make_buffer(u + t * kTileRows * static_cast<int64_t>(T));
+        const int n = min(Tc, T - tL);
+        const int perRow = n / V;
+        const int total = rows_of(t) * perRow;
+        RowCol rc;
+        rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
+        const int dr = kWave / perRow, dc = kWave % perRow;
 #pragma unroll
-            for (int i = 0; i < 32; ++i) pre[i] = buffer_load(bufU, off, i * pairStride);
-        } else {
-            const bool tOk = tLoad + segT < T;
-#pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                pre[i] = quiet;
-                if (tOk && row0 + 2 * i + segR < rows) pre[i] = buffer_load(bufU, off, i * pairStride);
+        for (int b = 0; b < NB; ++b) {
+            if (lane + b * kWave < total) {
+                const int off = (rc.r * T + tL + rc.c * V) * 4;
+                if (VEC) {
+                    const float4 q = buffer_load4(bufU, off, 0);
+                    x[4 * b] = q.x; x[4 * b + 1] = q.y; x[4 * b + 2] = q.z; x[4 * b + 3] = q.w;
+                } else {
+                    x[b] = buffer_load(bufU, off, 0);
+                }
             }
+            rc.advance(dr, dc, perRow);
+        }
+    };
+    auto commit = [&](int64_t t, int tL) {  // tile[r][LAG + c] = u[row][tL + c]
+        const int n = min(Tc, T - tL);
+        const int perRow = n / V;
+        const int total = rows_of(t) * perRow;
+        RowCol rc;
+        rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
+        const int dr = kWave / perRow, dc = kWave % perRow;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            if (lane + b * kWave < total) {
+                float *dst = tile + rc.r * P + LAG + rc.c * V;
+                if (VEC) *reinterpret_cast<float4 *>(dst) = make_float4(x[4 * b], x[4 * b + 1], x[4 * b + 2], x[4 * b + 3]);
+                else *dst = x[b];
+            }
+            rc.advance(dr, dc, perRow);
         }
     };
 
-    const int trips = (T + LAG + C - 1) / C;
-    issue_loads(0);
-    for (int it = 0; it < trips; ++it) {
-        const int tWalk = it * C - LAG;  // first time step walked (and retired) in this trip
+    int64_t t = blockIdx.x;
+    int tL = 0;
+    if (t < tiles) issue(t, tL);
+    while (t < tiles) {
+        const int nRows = rows_of(t);
+        const int n = min(Tc, T - tL);  // new samples per row in this piece
+        const bool last = tL + n == T;
+        const int tW = tL - LAG;        // time of tile column 0 (columns [0, LAG) are carried over)
 
-        // transpose the loaded chunk through LDS: lane = row gets its next 32 samples
-#pragma unroll
-        for (int i = 0; i < 32; ++i) tile[slot(2 * i + segR, segT)] = pre[i];
+        commit(t, tL);
         __syncthreads();
-#pragma unroll
-        for (int k = 0; k < C; ++k) v[LAG + k] = tile[slot(lane, k)];
-        __syncthreads();
-        issue_loads((it + 1) * C);  // past the end of the rows this loads nothing
-
-        // walk 32 time steps
-        uint32_t fired = 0;
-#pragma unroll
-        for (int k = 0; k < C; ++k) {
-            if (v[k] >= theta) {
-                fired |= 1u << k;
-#pragma unroll
-                for (int j = 0; j < NU; ++j) v[k + j] += tap[j];
-            }
+        {   // next step: next piece of this tile, or first piece of this group's next tile
+            const int64_t tn = last ? t + gridDim.x : t;
+            const int tLn = last ? 0 : tL + Tc;
+            if (tn < tiles) issue(tn, tLn);
         }
 
-        // retire: the 32 oldest samples are final
+        // ---- walk: lane = row.  Columns [0, W) become final in this step.
+        const int W = last ? n + LAG : n;
+        if (lane < kTileRows) {
+            float *mine = tile + lane * P;
+            if (tL == 0) {
 #pragma unroll
-        for (int k = 0; k < C; ++k) tile[slot(lane, k)] = v[k];
-        __syncthreads();
-        {
-            const int off = laneOff + tWalk * 4;
-            if (fullTile && tWalk >= 0 && tWalk + C <= T) {
-#pragma unroll 8
-                for (int i = 0; i < 32; ++i) {
-                    const int r = 2 * i + segR;
-                    const float uv = tile[slot(r, segT)];
-                    const uint32_t m = __shfl(fired, r, kWave);
-                    buffer_store(bufU, off, i * pairStride, uv);
-                    buffer_store(bufS, off, i * pairStride, ((m >> segT) & 1u) ? amplitude : 0.0f);
+                for (int k = 0; k < LAG; ++k) v[k] = quiet;
+            }
+            const int groups = (W + G - 1) / G;
+            for (int g = 0; g < groups; ++g) {
+                const int c0 = g * G;
+                if (c0 + G <= n) {
+#pragma unroll
+                    for (int k = 0; k < G; k += 4) {
+                        const float4 q = *reinterpret_cast<const float4 *>(mine + LAG + c0 + k);
+                        v[LAG + k] = q.x; v[LAG + k + 1] = q.y; v[LAG + k + 2] = q.z; v[LAG + k + 3] = q.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < G; ++k) v[LAG + k] = (c0 + k < n) ? mine[LAG + c0 + k] : quiet;
                 }
-            } else {
-                const int t = tWalk + segT;
-                const bool tOk = t >= 0 && t < T;
-#pragma unroll 8
-                for (int i = 0; i < 32; ++i) {
-                    const int r = 2 * i + segR;
-                    const float uv = tile[slot(r, segT)];
-                    const uint32_t m = __shfl(fired, r, kWave);
-                    if (tOk && row0 + r < rows) {
-                        buffer_store(bufU, off, i * pairStride, uv);
-                        buffer_store(bufS, off, i * pairStride, ((m >> segT) & 1u) ? amplitude : 0.0f);
+                uint32_t fired = 0;
+#pragma unroll
+                for (int k = 0; k < G; ++k) {
+                    if (v[k] >= theta) {
+                        fired |= 1u << k;
+#pragma unroll
+                        for (int j = 0; j < NU; ++j) v[k + j] += tap[j];
                     }
                 }
+#pragma unroll
+                for (int k = 0; k < G; k += 4)
+                    *reinterpret_cast<float4 *>(mine + c0 + k) = make_float4(v[k], v[k + 1], v[k + 2], v[k + 3]);
+                masks[lane * MP + g] = fired;
+#pragma unroll
+                for (int k = 0; k < LAG; ++k) v[k] = v[G + k];
             }
         }
         __syncthreads();
-#pragma unroll
-        for (int k = 0; k < LAG; ++k) v[k] = v[C + k];
+
+        // ---- retire: columns [first, W) leave as u' and s, times tW + column
+        {
+            const BufferRsrc bufU = make_buffer(u + t * kTileRows * static_cast<int64_t>(T));
+            const BufferRsrc bufS = make_buffer(s + t * kTileRows * static_cast<int64_t>(T));
+            const int first = (tL == 0) ? LAG : 0;  // before the first sample there is nothing to store
+            const int perRow = (W - first) / V;
+            const int total = nRows * perRow;
+            RowCol rc;
+            rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
+            const int dr = kWave / perRow, dc = kWave % perRow;
+#pragma unroll 4
+            for (int g0 = lane; g0 < total; g0 += kWave) {
+                const int col = first + rc.c * V;
+                const int off = (rc.r * T + tW + col) * 4;
+                const float *src = tile + rc.r * P + col;
+                const uint32_t m = masks[rc.r * MP + (col >> 5)] >> (col & 31);
+                if (VEC) {
+                    buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(src));
+                    buffer_store4(bufS, off, 0,
+                                  make_float4((m & 1u) ? amplitude : 0.0f, (m & 2u) ? amplitude : 0.0f,
+                                              (m & 4u) ? amplitude : 0.0f, (m & 8u) ? amplitude : 0.0f));
+                } else {
+                    buffer_store(bufU, off, 0, src[0]);
+                    buffer_store(bufS, off, 0, (m & 1u) ? amplitude : 0.0f);
+                }
+                rc.advance(dr, dc, perRow);
+            }
+        }
+        __syncthreads();
+
+        if (last) { t += gridDim.x; tL = 0; }
+        else tL += Tc;
     }
 }
 
@@ -294,21 +348,38 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
     const int64_t groups = ceil_div(nNeurons, kWave);
     const bool stream_ok = !generic_forced() && T < (1LL << 30) && groups < (1LL << 31);
     const bool window_ok = stream_ok && T <= kBufferMaxT;
-#define SLAYER_SPIKE_WINDOW(NU)                                                                          \
+#define SLAYER_SPIKE_TILE(NU)                                                                             \
     do {                                                                                                \
-        hipLaunchKernelGGL(spike_window_kernel<NU>, dim3(static_cast<unsigned>(groups)), dim3(kWave), 0,  \
-                           st, s, u, nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize), theta,  \
-                           Ts);                                                                         \
+        constexpr int lag = (NU + 2) & ~3;                                                              \
+        const int cols = (lag + Tc + 31) & ~31; /* the walk goes in groups of 32 columns */             \
+        const int P = cols + 4; /* 4 (mod 32): rows are 16-byte aligned and start in different banks */ \
+        const int MP = cols / 32 + 1;                                                                   \
+        const size_t lds = (static_cast<size_t>(kTileRows) * P + kTileRows * MP) * sizeof(float);       \
+        const int64_t resident = static_cast<int64_t>(cus) * (160 * 1024 / static_cast<int64_t>(lds));  \
+        const unsigned grid = static_cast<unsigned>(tiles < resident ? tiles : resident);               \
+        if (vec)                                                                                        \
+            hipLaunchKernelGGL((spike_tile_kernel<NU, true>), dim3(grid), dim3(kWave), lds, st, s, u,   \
+                               nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize), Tc, P, MP,  \
+                               tiles, theta, Ts);                                                       \
+        else                                                                                            \
+            hipLaunchKernelGGL((spike_tile_kernel<NU, false>), dim3(grid), dim3(kWave), lds, st, s, u,  \
+                               nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize), Tc, P, MP,  \
+                               tiles, theta, Ts);                                                       \
         return launch_status();                                                                         \
     } while (0)
+    const int64_t tiles = ceil_div(nNeurons, kTileRows);
     if (window_ok && nuSize <= 24) {
-        if (nuSize <= 4) SLAYER_SPIKE_WINDOW(4);
-        if (nuSize <= 8) SLAYER_SPIKE_WINDOW(8);
-        if (nuSize <= 12) SLAYER_SPIKE_WINDOW(12);
-        if (nuSize <= 16) SLAYER_SPIKE_WINDOW(16);
-        SLAYER_SPIKE_WINDOW(24);
+        // short rows travel whole; long rows in pieces of 256 samples (1 KiB per row)
+        const int Tc = (T <= kTileMaxPiece) ? static_cast<int>(T) : 256;
+        const bool vec = (T % 4 == 0) && aligned16(s) && aligned16(u);
+        const int cus = compute_units();
+        if (nuSize <= 4) SLAYER_SPIKE_TILE(4);
+        if (nuSize <= 8) SLAYER_SPIKE_TILE(8);
+        if (nuSize <= 12) SLAYER_SPIKE_TILE(12);
+        if (nuSize <= 16) SLAYER_SPIKE_TILE(16);
+        SLAYER_SPIKE_TILE(24);
     }
-#undef SLAYER_SPIKE_WINDOW
+#undef SLAYER_SPIKE_TILE
     if (stream_ok && nuSize <= 33) {
         hipLaunchKernelGGL(spike_stream_kernel<64>, dim3(static_cast<unsigned>(groups)), dim3(kWave), 0,
                            st, s, u, nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize), theta,
