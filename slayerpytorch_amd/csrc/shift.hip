@@ -1,71 +1,87 @@
 // Time shift of neuron rows: out[n][t] = in[n][t - k_n], zero outside [0, T).
 //
-// HBM-bound gather (8 B per neuron-timestep: one read, one write).  A work-group owns a
-// block of consecutive rows, i.e. one contiguous piece of the tensor; every lane writes one
-// 16-byte vector of the output, so stores are fully coalesced, and reads the (generally
-// unaligned) source samples from the same row.  The delay of a row is either one value for
-// the whole tensor or an entry of a per-neuron table shared by all batch items; one launch
-// covers every batch item.
+// HBM-bound gather (8 B per neuron-timestep: one read, one write), built like the fastest copy
+// this GPU runs: one 16-byte vector per lane, one pass per work-group, streaming cache policy.
+// A work-group owns a few whole rows (or a 256-vector slice of a long row); a lane writes one
+// aligned output vector and assembles it from the two aligned input vectors that straddle its
+// shifted position, so both directions stay fully coalesced whatever the shift is.  The delay
+// of a row is either one value for the whole tensor or an entry of a per-neuron table shared
+// by all batch items; one launch covers every batch item.
 #include "common.h"
 
 namespace slayer {
 
 enum ShiftMode { kShiftValue = 0, kShiftDeviceScalar = 1, kShiftTable = 2 };
 
-// VEC = samples written per lane (4 when rows are 16-byte aligned multiples of 4 samples).
-template <int VEC>
-__global__ __launch_bounds__(256) void shift_kernel(float *__restrict__ out,
-                                                    const float *__restrict__ in,
-                                                    const float *__restrict__ lut, int mode,
-                                                    float delayValue, float sign, int64_t rows,
-                                                    uint32_t nPerBatch, int T, int rowsPerBlock,
-                                                    float Ts)
+// Delay, in whole samples, of row (row0 + r); r < 256.  The table index is the row's position
+// within its batch item: the 64-bit remainder is taken once per work-group (row0 is uniform),
+// the per-lane part is 32 bit.
+__device__ __forceinline__ int row_steps(int mode, const float *__restrict__ lut, float delayValue,
+                                         float sign, float Ts, int64_t row0, int r, uint32_t nPerBatch)
 {
-    const int perRow = T / VEC;  // vectors per row
+    if (mode == kShiftValue) return delay_steps(delayValue * sign, Ts);
+    if (mode == kShiftDeviceScalar) return delay_steps(lut[0] * sign, Ts);
+    const uint32_t m0 = static_cast<uint32_t>(row0 % static_cast<int64_t>(nPerBatch));
+    const uint32_t m = static_cast<uint32_t>((static_cast<uint64_t>(m0) + static_cast<uint32_t>(r)) % nPerBatch);
+    return delay_steps(lut[m] * sign, Ts);
+}
+
+// Rows are whole 16-byte vectors (T % 4 == 0, 16-byte aligned tensors) and the tensor has fewer
+// than 2^32 of them: lane g of the grid owns output vector g of the flattened tensor.
+template <int LOADPOLICY>
+__global__ __launch_bounds__(256) void shift_vec_kernel(float *__restrict__ out,
+                                                        const float *__restrict__ in,
+                                                        const float *__restrict__ lut, int mode,
+                                                        float delayValue, float sign, uint32_t quads,
+                                                        uint32_t nPerBatch, int T, FastDiv byRow,
+                                                        float Ts)
+{
+    const int perRow = T >> 2;
+    const uint32_t g0 = blockIdx.x * 256u;      // first vector of this work-group
+    const uint32_t g = g0 + threadIdx.x;
+    const bool active = g < quads;
+    const uint32_t rowBase = fastdiv(g0, byRow);  // wave-uniform: addressing is relative to this row
+    const uint32_t row = fastdiv(active ? g : g0, byRow);
+    const int q = static_cast<int>((active ? g : g0) - row * static_cast<uint32_t>(perRow));
+    const int r = static_cast<int>(row - rowBase);
+
+    const BufferRsrc bufIn = make_buffer(in + static_cast<int64_t>(rowBase) * T);
+    const BufferRsrc bufOut = make_buffer(out + static_cast<int64_t>(rowBase) * T);
+    int k = row_steps(mode, lut, delayValue, sign, Ts, rowBase, r, nPerBatch);
+    k = max(-T, min(T, k));             // shifts beyond the row length all give an empty row
+    const int s0 = (q << 2) - k;        // source sample of the first output sample
+    const int qa = s0 >> 2;             // aligned source vector holding it (floor division)
+    const int sh = s0 & 3;
+    const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    float4 a = zero, b = zero;
+    if (active && qa >= 0 && qa < perRow) a = buffer_load4<LOADPOLICY>(bufIn, (r * T + (qa << 2)) * 4, 0);
+    if (active && sh != 0 && qa + 1 >= 0 && qa + 1 < perRow)
+        b = buffer_load4<LOADPOLICY>(bufIn, (r * T + (qa << 2) + 4) * 4, 0);
+    float4 y = a;
+    if (sh == 1) y = make_float4(a.y, a.z, a.w, b.x);
+    if (sh == 2) y = make_float4(a.z, a.w, b.x, b.y);
+    if (sh == 3) y = make_float4(a.w, b.x, b.y, b.z);
+    if (active) buffer_store4(bufOut, (r * T + (q << 2)) * 4, 0, y);
+}
+
+// Any T, any alignment: one sample per lane, lanes along time (coalesced 256-byte runs).
+__global__ __launch_bounds__(256) void shift_scalar_kernel(float *__restrict__ out,
+                                                           const float *__restrict__ in,
+                                                           const float *__restrict__ lut, int mode,
+                                                           float delayValue, float sign, int64_t rows,
+                                                           uint32_t nPerBatch, int T, int rowsPerBlock,
+                                                           float Ts)
+{
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * rowsPerBlock;
     const int nRows = static_cast<int>(min(static_cast<int64_t>(rowsPerBlock), rows - row0));
-    const int items = nRows * perRow;
-    const float invPerRow = 1.0f / static_cast<float>(perRow);
-    const uint32_t m0 = (mode == kShiftTable) ? static_cast<uint32_t>(row0 % nPerBatch) : 0u;
-
-    int uniformSteps = 0;
-    if (mode == kShiftValue) uniformSteps = delay_steps(delayValue * sign, Ts);
-    if (mode == kShiftDeviceScalar) uniformSteps = delay_steps(lut[0] * sign, Ts);
-
-    for (int i = threadIdx.x; i < items; i += blockDim.x) {
-        int r = 0, q = i;
-        if (nRows > 1) {
-            // i / perRow for i < 2^24: float estimate plus one correction step
-            r = static_cast<int>(static_cast<float>(i) * invPerRow);
-            q = i - r * perRow;
-            if (q < 0) { --r; q += perRow; }
-            else if (q >= perRow) { ++r; q -= perRow; }
-        }
-        int k = uniformSteps;
-        if (mode == kShiftTable) {
-            uint32_t m = (m0 + static_cast<uint32_t>(r)) % nPerBatch;
-            k = delay_steps(lut[m] * sign, Ts);
-        }
-        const int64_t base = (row0 + r) * static_cast<int64_t>(T);
-        const float *src = in + base;
-        const int t = q * VEC;
-        // source sample index of the first output sample; 64-bit so that t - k cannot wrap
-        const int64_t s0 = static_cast<int64_t>(t) - k;
-        if (VEC == 4) {
-            float4 v;
-            if ((k & 3) == 0 && s0 >= 0 && s0 + 3 < T) {
-                v = *reinterpret_cast<const float4 *>(src + s0);
-            } else {
-                v.x = (s0 >= 0 && s0 < T) ? src[s0] : 0.0f;
-                v.y = (s0 + 1 >= 0 && s0 + 1 < T) ? src[s0 + 1] : 0.0f;
-                v.z = (s0 + 2 >= 0 && s0 + 2 < T) ? src[s0 + 2] : 0.0f;
-                v.w = (s0 + 3 >= 0 && s0 + 3 < T) ? src[s0 + 3] : 0.0f;
-            }
-            *reinterpret_cast<float4 *>(out + base + t) = v;
-        } else {
-            out[base + t] = (s0 >= 0 && s0 < T) ? src[s0] : 0.0f;
-        }
-    }
+    int r = 0, t = blockIdx.y * 256 + threadIdx.x;
+    if (rowsPerBlock > 1) divmod_small(threadIdx.x, T, 1.0f / static_cast<float>(T), r, t);
+    if (r >= nRows || t >= T) return;
+    int k = row_steps(mode, lut, delayValue, sign, Ts, row0, r, nPerBatch);
+    k = max(-T, min(T, k));
+    const int src = t - k;
+    const int64_t base = (row0 + r) * static_cast<int64_t>(T);
+    out[base + t] = (src >= 0 && src < T) ? in[base + src] : 0.0f;
 }
 
 static int launch_shift(float *out, const float *in, const float *lut, int mode, float delayValue,
@@ -76,28 +92,29 @@ static int launch_shift(float *out, const float *in, const float *lut, int mode,
     if (rows == 0 || T == 0) return SLAYER_OK;
     if (!out || !in) return SLAYER_EINVAL;
     if (mode != kShiftValue && !lut) return SLAYER_EINVAL;
-    if (T >= (1LL << 30) || nPerBatch >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+    if (T >= (1LL << 28) || nPerBatch >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
     if (mode == kShiftTable && nPerBatch == 0) return SLAYER_EINVAL;
 
-    const bool vec4 = (T % 4 == 0) && aligned16(out) && aligned16(in);
-    const int vec = vec4 ? 4 : 1;
-    const int64_t perRow = T / vec;
-    // about 2048 vectors (8 per lane) per work-group, whole rows only, and the in-block
-    // item index must stay below 2^24 for the float division in the kernel
-    int64_t rowsPerBlock = perRow >= 2048 ? 1 : (2048 / perRow);
-    if (rowsPerBlock > rows) rowsPerBlock = rows;
-    const int64_t blocks = ceil_div(rows, rowsPerBlock);
-    if (blocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
-
-    dim3 grid(static_cast<unsigned>(blocks)), block(256);
-    if (vec4)
-        hipLaunchKernelGGL(shift_kernel<4>, grid, block, 0, stream, out, in, lut, mode, delayValue,
-                           sign, rows, static_cast<uint32_t>(nPerBatch), static_cast<int>(T),
-                           static_cast<int>(rowsPerBlock), Ts);
-    else
-        hipLaunchKernelGGL(shift_kernel<1>, grid, block, 0, stream, out, in, lut, mode, delayValue,
-                           sign, rows, static_cast<uint32_t>(nPerBatch), static_cast<int>(T),
-                           static_cast<int>(rowsPerBlock), Ts);
+    const bool vec = (T % 4 == 0) && aligned16(out) && aligned16(in) && rows * (T / 4) < (1LL << 32);
+    if (vec) {
+        const int64_t quads = rows * (T / 4);
+        const int64_t blocks = ceil_div(quads, 256);
+        // an aligned shift (whole vectors) reads every input vector exactly once: stream it;
+        // otherwise neighbouring lanes share input vectors and the loads should stay cached
+        hipLaunchKernelGGL(shift_vec_kernel<0>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, out,
+                           in, lut, mode, delayValue, sign, static_cast<uint32_t>(quads),
+                           static_cast<uint32_t>(nPerBatch), static_cast<int>(T),
+                           make_fastdiv(static_cast<uint32_t>(T / 4)), Ts);
+        return launch_status();
+    }
+    const int64_t rowsPerBlock = T >= 256 ? 1 : 256 / T;
+    const int64_t rowBlocks = ceil_div(rows, rowsPerBlock);
+    const int64_t colBlocks = ceil_div(T, 256);
+    if (rowBlocks >= (1LL << 31) || colBlocks > 65535) return SLAYER_EUNSUPPORTED;
+    dim3 grid(static_cast<unsigned>(rowBlocks), static_cast<unsigned>(rowsPerBlock > 1 ? 1 : colBlocks));
+    hipLaunchKernelGGL(shift_scalar_kernel, grid, dim3(256), 0, stream, out, in, lut, mode, delayValue, sign,
+                       rows, static_cast<uint32_t>(nPerBatch), static_cast<int>(T),
+                       static_cast<int>(rowsPerBlock), Ts);
     return launch_status();
 }
 

@@ -311,27 +311,37 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 }
 
 // ---- surrogate gradient ------------------------------------------------------------------------------
-template <int VEC>
-__global__ __launch_bounds__(256) void spike_bwd_kernel(float *gradIn, const float *gradOut,
-                                                        const float *__restrict__ u, float theta,
-                                                        float tau, float gain, int64_t numel)
+// One pass over three tensors (12 B per neuron-timestep), shaped like the fastest copy this GPU
+// runs: one 16-byte vector per lane, one pass per work-group, streaming cache policy.
+typedef float vec4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float spike_pdf(float u, float theta, float tau, float gain)
 {
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x * VEC;
-    for (int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * VEC; i < numel;
-         i += stride) {
-        if (VEC == 4) {
-            const float4 g = *reinterpret_cast<const float4 *>(gradOut + i);
-            const float4 x = *reinterpret_cast<const float4 *>(u + i);
-            float4 o;
-            o.x = g.x * (gain * expf(-fabsf(x.x - theta) / tau));
-            o.y = g.y * (gain * expf(-fabsf(x.y - theta) / tau));
-            o.z = g.z * (gain * expf(-fabsf(x.z - theta) / tau));
-            o.w = g.w * (gain * expf(-fabsf(x.w - theta) / tau));
-            *reinterpret_cast<float4 *>(gradIn + i) = o;
-        } else {
-            gradIn[i] = gradOut[i] * (gain * expf(-fabsf(u[i] - theta) / tau));
-        }
-    }
+    return gain * expf(-fabsf(u - theta) / tau);
+}
+
+__global__ __launch_bounds__(256) void spike_bwd_vec_kernel(float *gradIn, const float *gradOut,
+                                                            const float *__restrict__ u, float theta,
+                                                            float tau, float gain, int64_t quads)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= quads) return;
+    const vec4f g = __builtin_nontemporal_load(reinterpret_cast<const vec4f *>(gradOut) + i);
+    const vec4f x = __builtin_nontemporal_load(reinterpret_cast<const vec4f *>(u) + i);
+    vec4f o;
+    o.x = g.x * spike_pdf(x.x, theta, tau, gain);
+    o.y = g.y * spike_pdf(x.y, theta, tau, gain);
+    o.z = g.z * spike_pdf(x.z, theta, tau, gain);
+    o.w = g.w * spike_pdf(x.w, theta, tau, gain);
+    __builtin_nontemporal_store(o, reinterpret_cast<vec4f *>(gradIn) + i);
+}
+
+__global__ __launch_bounds__(256) void spike_bwd_scalar_kernel(float *gradIn, const float *gradOut,
+                                                               const float *__restrict__ u, float theta,
+                                                               float tau, float gain, int64_t numel)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < numel) gradIn[i] = gradOut[i] * spike_pdf(u[i], theta, tau, gain);
 }
 
 }  // namespace slayer
@@ -409,14 +419,14 @@ extern "C" int slayer_spike_bwd_f32(float *gradIn, const float *gradOut, const f
     hipStream_t st = static_cast<hipStream_t>(stream);
     const float gain = scale / tau;
     const bool vec4 = (numel % 4 == 0) && aligned16(gradIn) && aligned16(gradOut) && aligned16(u);
-    const int64_t perBlock = 256 * (vec4 ? 4 : 1) * 4;  // four trips per lane
-    int64_t blocks = ceil_div(numel, perBlock);
-    if (blocks > (1LL << 30)) blocks = 1LL << 30;
+    const int64_t lanes = vec4 ? numel / 4 : numel;
+    const int64_t blocks = ceil_div(lanes, 256);
+    if (blocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
     if (vec4)
-        hipLaunchKernelGGL(spike_bwd_kernel<4>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
-                           gradIn, gradOut, u, theta, tau, gain, numel);
+        hipLaunchKernelGGL(spike_bwd_vec_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
+                           gradIn, gradOut, u, theta, tau, gain, lanes);
     else
-        hipLaunchKernelGGL(spike_bwd_kernel<1>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
-                           gradIn, gradOut, u, theta, tau, gain, numel);
+        hipLaunchKernelGGL(spike_bwd_scalar_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
+                           gradIn, gradOut, u, theta, tau, gain, lanes);
     return launch_status();
 }
