@@ -30,9 +30,9 @@ SHAPE = (12, 16, 34, 34, 300)
 HBM_PEAK_GBS = 8000.0                     # MI355X HBM3E, published
 # algorithmic bytes per neuron-timestep (fp32 tensors read + written once)
 AB = {"psp_conv": 8, "spike": 12, "shift": 8, "shift_bwd": 8, "spike_bwd": 12, "psp_corr": 8}
-KERNEL_OF = {"psp_conv": "fir_tiled_kernel<true>", "spike": "spike_stream_kernel<64>",
-             "shift": "shift_kernel<4>", "shift_bwd": "shift_kernel<4>", "spike_bwd": "spike_bwd_kernel<4>",
-             "psp_corr": "fir_tiled_kernel<false>"}
+KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, true>", "spike": "slayer::spike_tile_kernel<12, true>",
+             "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
+             "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_tiled_kernel<false, true>"}
 
 
 def neuron_params():
@@ -88,7 +88,7 @@ def flip_rate(device, srm_t, ref_t, params):
     rng = np.random.default_rng(0)
     shape = (2, 16, 34, 34, 300)
     spikes = (rng.random(shape) < 0.02).astype(np.float32)
-    gain = np.float32(14.0)          # puts about 2 % of the samples above threshold
+    gain = np.float32(9.0)           # puts about 2 % of the samples above threshold
     a = slayerCuda.conv(torch.from_numpy(spikes).to(device), srm_t, 1.0) * float(gain)
     s_gpu = slayerCuda.getSpikes(a.contiguous(), ref_t, params["theta"], 1.0).cpu().numpy()
     a_cpu = O.conv(spikes, srm_t.cpu().numpy(), 1.0, fused=False) * gain

@@ -53,6 +53,8 @@ def _scalar(x, name):
         return float(x)
     if isinstance(x, numbers.Real):
         return float(x)
+    if isinstance(x, (str, bytes)):
+        raise TypeError("%s must be a number, got %s" % (name, type(x).__name__))
     try:
         return float(x)   # numpy scalars and other objects with __float__
     except Exception:

@@ -1,0 +1,426 @@
+"""The host-side layer engines on the GPU: autograd Functions, side effects, the reference's
+golden vectors through the HIP path, analogues of the reference's own tests for this path
+(test_slayer002/003/009/010/011, test_slayerLoihi001/002) and size-independent properties at
+the benchmark's full tensor sizes.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import slayerpytorch_amd as snn
+from oracle import oracle as O
+from slayerpytorch_amd import slayerCuda, slayerLoihiCuda
+from slayerpytorch_amd.slayer import alphaKernel
+
+from _util import golden, raster_from_aer, rel_err
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+REL_TOL = 1e-5
+
+
+def neuron(**kw):
+    d = {"theta": 10.0, "tauSr": 10.0, "tauRef": 1.0, "scaleRef": 2.0, "tauRho": 1.0, "scaleRho": 1.0}
+    d.update(kw)
+    return d
+
+
+def loihi_neuron(**kw):
+    d = {"type": "LOIHI", "vThMant": 80, "vDecay": 128, "iDecay": 1024, "refDelay": 1, "wgtExp": 0,
+         "tauRho": 1, "scaleRho": 1}
+    d.update(kw)
+    return d
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+# ------------------------------------------------------------------------------------------ psp
+def test_psp_forward_backward_matches_oracle():
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 300}).to(DEV)
+    rng = np.random.default_rng(0)
+    x = (rng.random((3, 4, 5, 5, 300)) < 0.05).astype(np.float32)
+    g = rng.standard_normal(x.shape).astype(np.float32)
+    xt = dev(x).requires_grad_(True)
+    y = layer.psp(xt)
+    y.backward(dev(g))
+    srm = host(layer.srmKernel)
+    assert np.array_equal(host(y), O.conv(x, srm, 1.0))
+    assert np.array_equal(host(xt.grad), O.corr(g, srm, 1.0))
+    assert layer.srmKernel.grad is None
+
+
+def test_psp_equals_padded_conv3d_layer():
+    # reference test_slayer011: psp == pspLayer (left-padded conv3d with the flipped kernel), ||d|| / numel < 1e-6
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 300}).to(DEV)
+    x = (torch.rand((2, 2, 34, 34, 300), device=DEV) < 0.02).float()
+    k = layer.srmKernel
+    padded = F.pad(x.reshape(2, 1, 1, -1, 300), (k.numel() - 1, 0))
+    want = F.conv3d(padded, torch.flip(k, [0]).reshape(1, 1, 1, 1, -1)).reshape(x.shape) * 1.0
+    got = layer.psp(x)
+    assert (torch.norm(got - want) / got.numel()).item() < 1e-6
+
+
+def test_psp_accepts_non_contiguous_input_and_tensor_Ts():
+    layer = snn.layer(neuron(), {"Ts": 0.5, "tSample": 100}).to(DEV)
+    x = torch.randn((2, 3, 4, 100, 5), device=DEV).permute(0, 1, 2, 4, 3)       # time last, not contiguous
+    assert not x.is_contiguous()
+    want = O.conv(host(x.contiguous()), host(layer.srmKernel), 0.5)
+    assert np.array_equal(host(layer.psp(x)), want)
+    # the extension accepts a 0-dim tensor wherever the reference passed one for Ts
+    got = slayerCuda.conv(x.contiguous(), layer.srmKernel, torch.tensor(0.5, device=DEV))
+    assert np.array_equal(host(got), want)
+
+
+# ------------------------------------------------------------------------------------------ spike
+def test_spike_forward_side_effect_and_backward():
+    nd = neuron(tauRho=0.7, scaleRho=1.3)
+    layer = snn.layer(nd, {"Ts": 1.0, "tSample": 300}).to(DEV)
+    rng = np.random.default_rng(1)
+    u = (rng.standard_normal((2, 8, 6, 6, 300)) * 5).astype(np.float32)
+    g = rng.standard_normal(u.shape).astype(np.float32)
+    ref = host(layer.refKernel)
+    want_s, want_u = O.get_spikes(u, ref, 10.0, 1.0)
+
+    ut = dev(u)
+    src = ut.clone().requires_grad_(True)
+    pre = src * 1.0                                   # contiguous non-leaf: spike() updates it in place
+    s = layer.spike(pre)
+    assert np.array_equal(host(s), want_s)
+    assert np.array_equal(host(pre), want_u), "membrane potential must reflect the refractory response"
+    s.backward(dev(g))
+    # the gradient uses the post-refractory potential that was saved
+    want_g = O.spike_bwd(g, want_u, 10.0, 0.7 * 10.0, 1.3)
+    np.testing.assert_allclose(host(src.grad), want_g, rtol=REL_TOL, atol=1e-30)
+
+
+def test_spike_non_contiguous_input_is_left_untouched():
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 64}).to(DEV)
+    rng = np.random.default_rng(2)
+    u = (rng.standard_normal((2, 3, 4, 64, 5)) * 6).astype(np.float32)
+    ut = dev(u).permute(0, 1, 2, 4, 3)
+    before = host(ut).copy()
+    s = layer.spike(ut)
+    want_s, _ = O.get_spikes(before, host(layer.refKernel), 10.0, 1.0)
+    assert np.array_equal(host(s), want_s)
+    assert np.array_equal(host(ut), before)          # the kernel worked on a contiguous copy
+
+
+def test_get_spikes_requires_five_dimensions():
+    f = torch.ones(3, device=DEV)
+    with pytest.raises(IndexError):
+        slayerCuda.getSpikes(torch.zeros((4, 10), device=DEV), f, 1.0, 1.0)
+    with pytest.raises(RuntimeError):
+        slayerCuda.getSpikes(torch.zeros((1, 2, 3, 10), device=DEV), f, 1.0, 1.0)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        slayerCuda.conv(torch.zeros((4, 10, 3), device=DEV).permute(0, 2, 1), f, 1.0)
+    with pytest.raises(RuntimeError, match="Float"):
+        slayerCuda.conv(torch.zeros((4, 10), device=DEV, dtype=torch.float64), f, 1.0)
+    with pytest.raises(RuntimeError, match="shift and number of neurons must be same"):
+        slayerCuda.shift(torch.zeros((2, 3, 1, 1, 10), device=DEV), torch.zeros(5, device=DEV), 1.0)
+
+
+# ------------------------------------------------------------------------------------------ delay
+def check_shift(x, y, k):
+    if k > 0:
+        return torch.equal(x[:-k], y[k:]) and not y[:k].any()
+    if k == 0:
+        return torch.equal(x, y)
+    return torch.equal(x[-k:], y[:k]) and not y[k:].any()
+
+
+def test_shift_per_neuron_like_reference_test009():
+    Ts = 0.1
+    layer = snn.layer(neuron(), {"Ts": Ts, "tSample": 50}).to(DEV)
+    N, C, H, W, D = 5, 10, 20, 30, 500
+    delay = layer.delay((C, H, W)).to(DEV)
+    x = torch.randn((N, C, H, W, D), device=DEV)
+    delay.delay.data = torch.rand(delay.delay.shape, device=DEV) * 2 - 1
+    y = slayerCuda.shift(x, delay.delay.data, Ts)
+    d = host(delay.delay.data)
+    xs, ys = x.cpu(), y.cpu()
+    rng = np.random.default_rng(0)
+    for _ in range(400):                              # a random sample of neurons; all rows are checked below
+        n, c, h, w = rng.integers(N), rng.integers(C), rng.integers(H), rng.integers(W)
+        k = int(np.float32(d[c, h, w]) / np.float32(Ts))
+        assert check_shift(xs[n, c, h, w], ys[n, c, h, w], k)
+    assert np.array_equal(host(y), O.shift(host(x), d, Ts))
+    y4 = layer.delayShift(x, 4)
+    assert torch.equal(y4[..., 4:], x[..., :-4]) and not y4[..., :4].any()
+
+
+def test_delay_shift_backward_shifts_the_other_way():
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 100}).to(DEV)
+    x = torch.randn((2, 3, 4, 4, 100), device=DEV, requires_grad=True)
+    g = torch.randn_like(x)
+    for delay in (3, 3.0, torch.tensor(3.0), torch.tensor([3.0], device=DEV)):
+        x.grad = None
+        layer.delayShift(x, delay).backward(g)
+        assert np.array_equal(host(x.grad), O.shift(host(g), -3, 1.0))
+    d = torch.rand((3, 4, 4), device=DEV) * 20 - 5
+    x.grad = None
+    layer.delayShift(x, d).backward(g)
+    assert np.array_equal(host(x.grad), O.shift(host(g), -host(d), 1.0))
+
+
+def test_delay_layer_gradients_like_reference_test010():
+    """Autograd delay gradient == -sum(e * d(psp)/dt) * Ts, in both operator orders."""
+    Ts, Ns, N, Nin, Nout = 0.1, 500, 5, 25, 1
+    nd = neuron(tauSr=1.0)
+    layer = snn.layer(nd, {"Ts": Ts, "tSample": 50}).to(DEV)
+    torch.manual_seed(0)
+    fc1 = layer.dense(Nin, Nout).to(DEV)
+    delay = layer.delay((Nin, 1, 1)).to(DEV)
+    spikeIn = ((torch.rand((N, Nin, 1, 1, Ns), device=DEV) > 0.8).float() / Ts)
+    spikeDes = ((torch.rand((N, Nout, 1, 1, Ns), device=DEV) > 0.8).float() / Ts)
+
+    def loss_of(spikeOut):
+        err = layer.psp(spikeOut - spikeDes)
+        return 0.5 * torch.sum(err ** 2) * Ts
+
+    grads = []
+
+    class Probe(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):
+            return x.view_as(x)
+
+        @staticmethod
+        def backward(ctx, g):
+            grads.append(g)
+            return g
+
+    pspDelayed = delay(layer.psp(spikeIn))
+    uOut = fc1(Probe.apply(pspDelayed))
+    loss_of(layer.spike(uOut)).backward()
+    errorRec = grads[0]
+    diffFilter = torch.tensor([1, -1], dtype=torch.float, device=DEV) / Ts
+    dpsp_dt = slayerCuda.conv(pspDelayed.detach().contiguous(), diffFilter, 1)
+    manual = -torch.sum(errorRec * dpsp_dt, [0, -1], keepdim=True).reshape((Nin, 1, 1)) * Ts
+    assert torch.norm(manual - delay.delay.grad).item() < 1e-4
+    assert torch.norm(manual).item() > 1e-3
+
+    # delay before psp gives the same gradient (both are time-invariant linear maps)
+    delay.delay.grad = None
+    loss_of(layer.spike(fc1(layer.psp(delay(spikeIn))))).backward()
+    assert torch.norm(manual - delay.delay.grad).item() < 1e-4
+
+
+def test_delay_layer_per_channel_broadcast_and_oracle_gradient():
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 64}).to(DEV)
+    delay = layer.delay(3).to(DEV)                       # one delay per channel, input has H, W > 1
+    delay.delay.data = torch.tensor([0.0, 2.0, 5.0], device=DEV).reshape(3, 1, 1)
+    x = torch.randn((2, 3, 4, 5, 64), device=DEV, requires_grad=True)
+    g = torch.randn_like(x)
+    y = delay(x)
+    y.backward(g)
+    lut = np.repeat(np.array([0.0, 2.0, 5.0], np.float32), 20).reshape(3, 4, 5)
+    assert np.array_equal(host(y), O.shift(host(x), lut, 1.0))
+    assert np.array_equal(host(x.grad), O.shift(host(g), -lut, 1.0))
+    per_neuron = O.delay_grad(host(y), host(g), 1.0)    # (3, 4, 5): summed over the repeat by autograd
+    assert rel_err(host(delay.delay.grad).reshape(3), per_neuron.reshape(3, -1).sum(1)) < 1e-4
+
+
+# ------------------------------------------------------------------------------------------ golden chains
+def test_golden_250_25_1_spike_chain_like_reference_test002():
+    snn_d = golden("snn_250_25_1.npz")
+    Ts, Ns = 0.1, 500
+    nd = neuron(tauSr=1.0)
+    layer = snn.layer(nd, {"Ts": Ts, "tSample": 50}, fullRefKernel=True).to(DEV)
+    assert layer.srmKernel.numel() == 77 and layer.refKernel.numel() == 160
+    fc1, fc2 = layer.dense(250, 25).to(DEV), layer.dense(25, 1).to(DEV)
+    fc1.weight.data = dev(snn_d["w1learned"]).reshape(25, 250, 1, 1, 1)
+    fc2.weight.data = dev(snn_d["w2learned"]).reshape(1, 25, 1, 1, 1)
+    x = dev(raster_from_aer(snn_d["spikeIn"], 250, Ns, Ts, 1 / Ts)).reshape(1, 250, 1, 1, Ns)
+    uHid = fc1(layer.psp(x))
+    pre = host(uHid).copy()
+    sHid = layer.spike(uHid)
+    want = raster_from_aer(snn_d["spikeHid"], 25, Ns, Ts, 1 / Ts)
+    assert np.array_equal(host(sHid).reshape(25, Ns), want)
+    sOut = layer.spike(layer.psp(fc2(sHid)))
+    assert np.array_equal(np.nonzero(host(sOut).reshape(-1))[0], np.array([203, 355, 447]))
+    # spike function triples recorded for hidden neuron 0: u before, u after, spikes
+    d = snn_d["spikeFuncHid"][:-1]
+    assert np.abs(pre.reshape(25, Ns)[0] - d[:, 0]).max() < 2e-3
+    assert np.abs(host(uHid).reshape(25, Ns)[0] - d[:, 1]).max() < 2e-3
+    assert np.array_equal(host(sHid).reshape(25, Ns)[0], d[:, 2])
+
+
+def test_golden_gradients_like_reference_test003():
+    snn_d = golden("snn_250_25_1.npz")
+    Ts, Ns = 0.1, 500
+    nd = neuron(tauSr=1.0, tauRho=0.1)
+    layer = snn.layer(nd, {"Ts": Ts, "tSample": 50}, fullRefKernel=True).to(DEV)
+    fc1, fc2 = layer.dense(250, 25).to(DEV), layer.dense(25, 1).to(DEV)
+    fc1.weight = torch.nn.Parameter(dev(snn_d["w1Initial"]).reshape(25, 250, 1, 1, 1))
+    fc2.weight = torch.nn.Parameter(dev(snn_d["w2Initial"]).reshape(1, 25, 1, 1, 1))
+    x = dev(raster_from_aer(snn_d["spikeIn"], 250, Ns, Ts, 1 / Ts)).reshape(1, 250, 1, 1, Ns)
+    des = dev(raster_from_aer(snn_d["spikeOut"], 1, Ns, Ts, 1 / Ts)).reshape(1, 1, 1, 1, Ns)
+    s1 = layer.spike(layer.psp(fc1(x)))
+    s2 = layer.spike(layer.psp(fc2(s1)))
+    err = layer.psp(s2 - des)
+    loss = 0.5 * torch.sum(err ** 2) * Ts
+    loss.backward()
+    g2 = host(fc2.weight.grad).reshape(1, 25)
+    g1 = host(fc1.weight.grad).reshape(25, 250)
+    assert np.linalg.norm(snn_d["gradW2Initial"] - g2) / g2.size < 1e-4
+    assert np.linalg.norm(snn_d["gradW1Initial"] - g1) / g1.size < 1e-4
+
+
+# ------------------------------------------------------------------------------------------ Loihi
+def test_loihi_chip_recordings_like_reference_loihi_test001():
+    snn_d, chip = golden("snn_250_25_1.npz"), golden("loihi_chip.npz")
+    Ts, Ns = 0.1, 500
+    layer = snn.loihi(loihi_neuron(), {"Ts": Ts, "tSample": 50}).to(DEV)
+    fc1, fc2 = layer.dense(250, 25).to(DEV), layer.dense(25, 1).to(DEV)
+    W1 = np.round(snn_d["w1learned"].astype(np.float64) * 4 / 2) * 2
+    W2 = np.round(snn_d["w2learned"].astype(np.float64) * 4 / 2) * 2
+    fc1.weight.data = dev(W1.astype(np.float32)).reshape(25, 250, 1, 1, 1)
+    fc2.weight.data = dev(W2.astype(np.float32)).reshape(1, 25, 1, 1, 1)
+    x = dev(raster_from_aer(snn_d["spikeIn"], 250, Ns, Ts, 1 / Ts, offset=49)).reshape(1, 250, 1, 1, Ns)
+    sH, vH, _ = layer.spikeLoihiFull(fc1(x))
+    sH = layer.delayShift(sH, 1)
+    sO, vO, _ = layer.spikeLoihiFull(fc2(sH))
+    sO = layer.delayShift(sO, 1)
+    want = raster_from_aer(chip["hiddenSpikes"], 25, Ns, Ts, 1 / Ts, time_first=False)
+    assert torch.norm(sH.reshape(25, Ns).cpu() - torch.from_numpy(want)).item() < 1e-3
+    assert np.array_equal(np.nonzero(host(sO).reshape(-1))[0], np.array([57, 60]))
+    assert torch.norm(vH[0, 24, 0, 0, :-1].cpu() - torch.from_numpy(chip["hiddenVoltage24"]).float()).item() < 1e-3
+    assert torch.norm(vO[..., :-1].cpu().reshape(-1) - torch.from_numpy(chip["outputVoltage"]).float()).item() < 1e-3
+
+
+@pytest.mark.parametrize("refDelay", [2, 9, 17])
+def test_loihi_random_network_like_reference_loihi_test002(refDelay):
+    rng = np.random.default_rng(refDelay)
+    numSrc, numDst, T = 128, 64, 200
+    layer = snn.loihi(loihi_neuron(refDelay=refDelay, scaleRho=768), {"Ts": 1, "tSample": T}).to(DEV)
+    weight = np.round((rng.random((numDst, numSrc)) - 0.5) * 10) * 2
+    w = weight.dot(rng.random((numSrc, T)) > 0.8).astype(np.float32)
+    spike, voltage, current = layer.spikeLoihiFull(dev(w))                  # 2-D input, as in the reference test
+    want = O.loihi_get_spikes(w, 0, 80 * 64, 1024, 128, refDelay)
+    assert np.array_equal(host(spike), want[0]) and np.array_equal(host(voltage), want[1])
+    assert np.array_equal(host(current), want[2])
+
+
+def test_loihi_autograd_backward():
+    Ts = 1.0
+    nd = loihi_neuron(scaleRho=2.0)
+    layer = snn.loihi(nd, {"Ts": Ts, "tSample": 300}).to(DEV)
+    rng = np.random.default_rng(3)
+    w = (2 * rng.integers(-64, 64, size=(2, 6, 5, 5, 300)) * (rng.random((2, 6, 5, 5, 300)) < 0.3)).astype(np.float32)
+    g = rng.standard_normal(w.shape).astype(np.float32)
+    wt = dev(w).requires_grad_(True)
+    s = layer.spikeLoihi(wt)
+    s.backward(dev(g))
+    ws, wv, _ = O.loihi_get_spikes(w, 0, 5120, 1024, 128, 1)
+    assert np.array_equal(host(s), ws) and ws.sum() > 0
+    psp = host(layer.srmKernel)
+    want = O.corr(O.spike_bwd(g, wv, 5120.0, 5120.0, nd["scaleRho"]), psp, Ts)
+    assert rel_err(host(wt.grad), want) < REL_TOL
+    assert len(psp) == 110 and nd["scaleRho"] == pytest.approx(2.0 / 195.0)
+
+
+def test_loihi_Ts_scaling_of_input_and_output():
+    layer = snn.loihi(loihi_neuron(), {"Ts": 0.1, "tSample": 20}).to(DEV)
+    rng = np.random.default_rng(4)
+    w = (20 * rng.integers(-30, 60, size=(1, 9, 1, 1, 200))).astype(np.float32)      # spikes of amplitude 1/Ts times weights
+    s, v, u = layer.spikeLoihiFull(dev(w))
+    ws, wv, wu = O.loihi_get_spikes((w * np.float32(0.1)).astype(np.float32), 0, 5120, 1024, 128, 1)
+    assert np.array_equal(host(s), ws / np.float32(0.1)) and np.array_equal(host(v), wv)
+    with pytest.raises(ValueError):
+        slayerLoihiCuda.getSpikes(dev(w), 0, 5120, 1024, 128, 0)
+
+
+# ------------------------------------------------------------------------------------------ full sizes
+FULL = (12, 16, 34, 34, 300)          # largest activation tensor of the NMNIST-CNN-shaped config
+
+
+def test_full_size_spike_sampled_rows_and_checksum():
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 300}).to(DEV)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    u = torch.randn(FULL, generator=g) * 5.0
+    ud = u.to(DEV)
+    s = slayerCuda.getSpikes(ud, layer.refKernel, 10.0, 1.0)
+    rows = np.random.default_rng(0).choice(12 * 16 * 34 * 34, 4096, replace=False)
+    un = u.reshape(-1, 300).numpy()[rows].reshape(1, 4096, 1, 1, 300)
+    want_s, want_u = O.get_spikes(un, host(layer.refKernel), 10.0, 1.0)
+    idx = torch.from_numpy(rows).to(DEV)
+    assert np.array_equal(host(s.reshape(-1, 300)[idx]), want_s.reshape(4096, 300))
+    assert np.array_equal(host(ud.reshape(-1, 300)[idx]), want_u.reshape(4096, 300))
+    # size-independent properties: spikes are 0 or 1/Ts and sit on supra-threshold samples (nu[0] = 0);
+    # the refractory update is linear in the spikes: u_after = u_before + conv(spikes, nu) up to rounding
+    assert torch.all((s == 0) | (s == 1.0))
+    assert torch.all(ud[s > 0] >= 10.0)
+    assert 0.005 < (s > 0).float().mean().item() < 0.05
+    rebuilt = u.to(DEV) + slayerCuda.conv(s, layer.refKernel, 1.0)
+    assert (rebuilt - ud).abs().max().item() < 1e-4
+
+
+def test_full_size_psp_linearity_adjoint_and_sampled_rows():
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 300}).to(DEV)
+    k = layer.srmKernel
+    g = torch.Generator(device="cpu").manual_seed(1)
+    x = (torch.rand(FULL, generator=g) < 0.02).float().to(DEV)
+    y = torch.randn(FULL, generator=g).to(DEV)
+    cx = slayerCuda.conv(x, k, 1.0)
+    cy = slayerCuda.corr(y, k, 1.0)
+    lhs = (cx.double() * y.double()).sum().item()
+    rhs = (x.double() * cy.double()).sum().item()
+    assert abs(lhs - rhs) <= 1e-6 * abs(lhs)                                   # <conv x, y> = <x, corr y>
+    both = slayerCuda.conv(2.0 * x + y, k, 1.0)
+    assert rel_err(host(both[0, 0]), host(2.0 * cx[0, 0] + slayerCuda.conv(y, k, 1.0)[0, 0])) < REL_TOL
+    rows = np.random.default_rng(1).choice(12 * 16 * 34 * 34, 2048, replace=False)
+    idx = torch.from_numpy(rows).to(DEV)
+    assert np.array_equal(host(cx.reshape(-1, 300)[idx]), O.conv(host(x.reshape(-1, 300)[idx]), host(k), 1.0))
+    assert np.array_equal(host(cy.reshape(-1, 300)[idx]), O.corr(host(y.reshape(-1, 300)[idx]), host(k), 1.0))
+
+
+def test_full_size_shift_roundtrip():
+    g = torch.Generator(device="cpu").manual_seed(2)
+    x = torch.randn(FULL, generator=g).to(DEV)
+    y = slayerCuda.shift(x, 1.0, 1.0)
+    assert torch.equal(y[..., 1:], x[..., :-1]) and not y[..., 0].any()
+    back = slayerCuda.shift(y, 1.0, 1.0, sign=-1.0)
+    assert torch.equal(back[..., :-1], x[..., :-1]) and not back[..., -1].any()
+
+
+def test_full_size_loihi_sampled_rows():
+    shape = (8, 16, 32, 32, 300)      # largest tensor of the Loihi DVS-gesture-shaped config
+    g = torch.Generator(device="cpu").manual_seed(3)
+    w = (2 * torch.randint(-128, 128, shape, generator=g) * (torch.rand(shape, generator=g) < 0.05)).float()
+    s, v, u = slayerLoihiCuda.getSpikes(w.to(DEV), 0, 5120, 1024, 128, 1)
+    rows = np.random.default_rng(3).choice(8 * 16 * 32 * 32, 4096, replace=False)
+    want = O.loihi_get_spikes(w.reshape(-1, 300).numpy()[rows], 0, 5120, 1024, 128, 1)
+    idx = torch.from_numpy(rows).to(DEV)
+    for got, exp in zip((s, v, u), want):
+        assert np.array_equal(host(got.reshape(-1, 300)[idx]), exp)
+    assert want[0].sum() > 0
+    # invariants of the neuron: first sample is zero, spikes are 0/1, reported voltage at a spike is vDecay
+    assert not s[..., 0].any() and not v[..., 0].any() and not u[..., 0].any()
+    assert torch.all((s == 0) | (s == 1)) and torch.all(v[s > 0] == 128)
+
+
+def test_delay_stress_config_shapes():
+    # long-sequence delay config: (64, 256, 1, 1, 2000) with delays U[0, 62], tauSr = 1 (8 taps)
+    layer = snn.layer(neuron(tauSr=1.0), {"Ts": 1.0, "tSample": 2000}).to(DEV)
+    assert layer.srmKernel.numel() == 8
+    g = torch.Generator(device="cpu").manual_seed(4)
+    x = (torch.rand((64, 256, 1, 1, 2000), generator=g) < 0.005).float().to(DEV).requires_grad_(True)
+    delay = layer.delay(256).to(DEV)
+    delay.delay.data = (torch.rand((256, 1, 1), generator=g) * 62).to(DEV)
+    y = delay(layer.psp(x))
+    grad = torch.randn(y.shape, generator=g).to(DEV)
+    y.backward(grad)
+    a = O.conv(host(x), host(layer.srmKernel), 1.0)
+    want_y = O.shift(a, host(delay.delay.data), 1.0)
+    assert np.array_equal(host(y), want_y)
+    assert rel_err(host(delay.delay.grad), O.delay_grad(want_y, host(grad), 1.0)) < REL_TOL
+    want_gx = O.corr(O.shift(host(grad), -host(delay.delay.data), 1.0), host(layer.srmKernel), 1.0)
+    assert np.array_equal(host(x.grad), want_gx)

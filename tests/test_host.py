@@ -1,0 +1,135 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every symbol the
+header declares, and the Python modules reject bad arguments before anything is launched, with
+the error behaviour of the reference bindings (src/cuda/slayerKernels.cu:7-10, 35, 102;
+src/cuda/slayerLoihiKernels.cu:12-19)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from slayerpytorch_amd import _lib, slayerCuda, slayerLoihiCuda
+import slayerpytorch_amd as snn
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "slayer_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(slayer_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_symbols()
+    assert len(names) >= 13 and "slayer_conv_f32" in names and "slayer_loihi_get_spikes_f32" in names
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in names:
+        assert hasattr(lib, name), "libslayer_hip.so does not export %s" % name
+    assert sorted(_lib.SIGNATURES) == names, "python binding table and header disagree"
+
+
+def test_abi_version_and_status_strings():
+    lib = _lib.load()
+    assert lib.slayer_hip_abi_version() == _lib.ABI_VERSION == 1
+    assert lib.slayer_status_string(0) == b"ok"
+    assert lib.slayer_status_string(1) == b"invalid argument"
+    assert lib.slayer_status_string(77) == b"unknown status"
+    with pytest.raises(_lib.SlayerHipError, match="invalid argument"):
+        _lib.check(1, "slayer_conv_f32")
+
+
+def test_argument_validation_in_the_c_abi_without_launch():
+    lib = _lib.load()
+    # empty tensors are a successful no-op, whatever the pointers
+    assert lib.slayer_conv_f32(None, None, None, 0, 10, 3, 1.0, None) == 0
+    assert lib.slayer_get_spikes_f32(None, None, None, 5, 0, 3, 1.0, 1.0, None) == 0
+    # null pointers with work to do, negative sizes, refDelay 0, bad sign
+    assert lib.slayer_conv_f32(None, None, None, 4, 10, 3, 1.0, None) == 1
+    assert lib.slayer_corr_f32(None, None, None, -1, 10, 3, 1.0, None) == 1
+    assert lib.slayer_shift_f32(None, None, 1.0, 4, 10, 1.0, None) == 1
+    assert lib.slayer_shift_lut_f32(None, None, None, 3, 2, 4, 10, 1.0, 1.0, None) == 1     # lutSize != nPerBatch
+    assert lib.slayer_shift_lut_f32(None, None, None, 4, 0, 4, 10, 1.0, 0.5, None) == 1     # sign must be +-1
+    assert lib.slayer_loihi_get_spikes_f32(None, None, None, None, 0, 0, 0, 64, 0, 0, 0, None) == 1   # refDelay 0
+    assert lib.slayer_loihi_get_spikes_f32(None, None, None, None, 0, 0, 26, 64, 0, 0, 1, None) == 1  # 1 << 32
+    assert lib.slayer_spike_bwd_f32(None, None, None, 1.0, 0.0, 1.0, 4, None) == 1
+    assert lib.slayer_delay_grad_workspace_bytes(64, 256, 2000) == 64 * 256 * 4
+    assert lib.slayer_delay_grad_workspace_bytes(0, 256, 2000) == 0
+
+
+def test_cpu_tensors_are_rejected_like_the_reference():
+    x = torch.zeros(1, 2, 1, 1, 10)
+    f = torch.ones(3)
+    for call in (lambda: slayerCuda.conv(x, f, 1.0), lambda: slayerCuda.corr(x, f, 1.0),
+                 lambda: slayerCuda.shift(x, f, 1.0), lambda: slayerCuda.shift(x, 1.0),
+                 lambda: slayerCuda.getSpikes(x, f, 1.0, 1.0),
+                 lambda: slayerLoihiCuda.getSpikes(x, 0, 64, 0, 0, 1)):
+        with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+            call()
+
+
+def test_non_tensor_and_bad_scalar_arguments():
+    f = torch.ones(3)
+    with pytest.raises(TypeError):
+        slayerCuda.conv([1.0, 2.0], f, 1.0)
+    with pytest.raises(TypeError):
+        slayerLoihiCuda.getSpikes(None, 0, 64, 0, 0, 1)
+
+
+def test_loihi_integer_arguments_follow_unsigned_conversion():
+    from slayerpytorch_amd.slayerLoihiCuda import _unsigned
+    assert _unsigned(5, "x") == 5 and _unsigned(torch.tensor(7), "x") == 7
+    import numpy as np
+    assert _unsigned(np.int64(3), "x") == 3
+    for bad in (-1, 1.5, "3", 1 << 32, torch.tensor(1.0)):
+        with pytest.raises(TypeError):
+            _unsigned(bad, "x")
+
+
+def test_scalar_conversion_accepts_numbers_and_one_element_tensors():
+    from slayerpytorch_amd.slayerCuda import _scalar
+    import numpy as np
+    assert _scalar(2, "Ts") == 2.0 and _scalar(torch.tensor(0.5), "Ts") == 0.5
+    assert _scalar(np.float32(0.25), "Ts") == 0.25
+    with pytest.raises(TypeError):
+        _scalar(torch.ones(2), "Ts")
+    with pytest.raises(TypeError):
+        _scalar("1.0", "Ts")
+
+
+def test_layer_objects_build_without_gpu():
+    neuron = {"theta": 10, "tauSr": 10.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
+    layer = snn.layer(neuron, {"Ts": 1.0, "tSample": 300})
+    assert layer.srmKernel.numel() == 77 and layer.refKernel.numel() == 11
+    assert set(layer.state_dict()) == {"srmKernel", "refKernel"}        # buffers travel with the state dict
+    assert layer.refKernel[1].item() == pytest.approx(-20.0)
+    delay = layer.delay((4, 3, 2))
+    assert delay.delay.shape == (4, 3, 2) and delay.delay.requires_grad
+    assert layer.delay(5).delay.shape == (5, 1, 1)
+    fc = layer.dense(12, 7)
+    assert fc.weight.shape == (7, 12, 1, 1, 1)
+    assert layer.dense((3, 4, 2), 5).weight.shape == (5, 2, 4, 3, 1)
+    ld = {"type": "LOIHI", "vThMant": 80, "vDecay": 128, "iDecay": 1024, "refDelay": 1, "wgtExp": 0,
+          "tauRho": 1, "scaleRho": 1}
+    loihi = snn.loihi(ld, {"Ts": 1, "tSample": 300})
+    assert ld["theta"] == 5120 and loihi.maxPspKernel == 195.0 and ld["scaleRho"] == pytest.approx(1 / 195.0)
+    w = loihi.dense(8, 4)
+    q = w.preHookFx(w.weight)
+    assert torch.all(q == torch.round(q / 2) * 2)                        # weights quantised in steps of 2
+
+
+def test_dropin_modules_re_export_the_extension_api():
+    import importlib
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "slayerpytorch_amd", "dropin"))
+    try:
+        sc = importlib.import_module("slayerCuda")
+        slc = importlib.import_module("slayerLoihiCuda")
+    finally:
+        sys.path.pop(0)
+        sys.modules.pop("slayerCuda", None)
+        sys.modules.pop("slayerLoihiCuda", None)
+    for name in ("getSpikes", "conv", "corr", "shift"):
+        assert getattr(sc, name) is getattr(slayerCuda, name)
+    assert slc.getSpikes is slayerLoihiCuda.getSpikes
