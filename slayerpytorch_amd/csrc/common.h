@@ -62,6 +62,19 @@ struct RowCol {
     }
 };
 
+// Synchronisation inside a work-group that is a single wavefront.  LDS executes the accesses of
+// one wavefront in program order, so data written by one lane is visible to the other lanes of
+// the same wavefront in any later instruction; all that is needed is to keep the compiler from
+// moving LDS accesses across this point.  Unlike __syncthreads() it does not wait for the
+// wavefront's outstanding global loads and stores, which is the point: prefetches and stores
+// stay in flight across it.
+__device__ __forceinline__ void wave_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // Division of a 32-bit unsigned number by a constant chosen on the host (Granlund-Montgomery):
 // q = (t + ((n - t) >> s1)) >> s2 with t = mulhi(n, m).  Exact for every n and every d >= 1.
 struct FastDiv {
@@ -122,15 +135,17 @@ __device__ __forceinline__ float4 buffer_load4(BufferRsrc b, int laneBytes, int 
     return make_float4(f.x, f.y, f.z, f.w);
 }
 
+template <int POLICY = kStream>
 __device__ __forceinline__ void buffer_store4(BufferRsrc b, int laneBytes, int uniformBytes, float4 v)
 {
     const float4_ext f = {v.x, v.y, v.z, v.w};
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4_ext, f), b, laneBytes, uniformBytes, kStream);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4_ext, f), b, laneBytes, uniformBytes, POLICY);
 }
 
+template <int POLICY = kStream>
 __device__ __forceinline__ void buffer_store(BufferRsrc b, int laneBytes, int uniformBytes, float x)
 {
-    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, x), b, laneBytes, uniformBytes, kStream);
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, x), b, laneBytes, uniformBytes, POLICY);
 }
 
 }  // namespace slayer

@@ -1,12 +1,14 @@
 // Loihi CUBA neuron: int32 current/voltage with sign-magnitude decay (>>12), integer
 // threshold, refractory delay.  Sequential in time per neuron, parallel over neurons.
 //
-// HBM-bound (16 B per neuron-timestep: read w, write spike, voltage, current).  Same streaming
-// scheme as the SRM spike kernel: a 64-lane work-group owns 64 consecutive rows and moves them
-// through LDS in 32-sample chunks, lanes along time for the 128-byte global segments, lane =
-// row for the sequential update.  The neuron state (current, voltage, refractory countdown)
-// stays in registers across chunks.  The chunk's input tile is overwritten in place by the
-// current; the voltage has its own tile; spikes travel as one 32-bit mask per lane.
+// HBM-bound (16 B per neuron-timestep: read w, write spike, voltage, current).  Same row-tile
+// scheme as the SRM spike kernel: a 64-lane work-group owns 16 consecutive rows and moves them
+// through LDS in pieces of up to 128 samples per row, so global memory is read and written as
+// contiguous runs with 16-byte accesses; lanes 0..15 then update their row sequentially, 32
+// samples at a time from registers.  The neuron state (current, voltage, refractory countdown)
+// stays in registers across pieces.  The piece's input tile is overwritten in place by the
+// current; the voltage has its own tile; spikes travel as 32-bit masks.  Work-groups are
+// persistent and issue the loads of the next piece before updating the current one.
 //
 // Refractory bookkeeping: the sequential formulation keeps a counter that is incremented at a
 // spike and decremented refDelay steps later by re-reading the spike it wrote then.  Because a
@@ -16,46 +18,62 @@
 // automaton, without the read-back.
 #include "common.h"
 
+#ifndef LOIHI_ROWS
+#define LOIHI_ROWS 64
+#define LOIHI_LPP 1
+#endif
+#define LOIHI_PIECE 64
+
 namespace slayer {
 
-constexpr int kLoihiChunk = 32;
 
-// sign(x) * ((|x| * (4096 - decay)) >> 12) in 32-bit wrap-around arithmetic
+// The update below is written without branches: one time step is about 30 vector instructions.
+
+// float -> int32 the way the hardware converts: toward zero, saturating, NaN -> 0
+// (v_cvt_i32_f32; a C cast would be undefined for the out-of-range inputs).
+__device__ __forceinline__ int cvt_trunc_sat(float x)
+{
+    int r;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
+
+// sign(x) * ((|x| * keep) >> 12) in 32-bit wrap-around arithmetic, keep = 4096 - decay
 __device__ __forceinline__ uint32_t loihi_decay(int x, uint32_t keep)
 {
-    const uint32_t ux = static_cast<uint32_t>(x);
-    const uint32_t mag = (x >= 0) ? ux : (0u - ux);
+    const uint32_t sgn = static_cast<uint32_t>(x >> 31);           // 0 or 0xFFFFFFFF
+    const uint32_t mag = (static_cast<uint32_t>(x) ^ sgn) - sgn;    // |x| (2^31 stays 2^31)
     const uint32_t scaled = (mag * keep) >> 12;
-    return (x >= 0) ? scaled : (0u - scaled);
+    return (scaled ^ sgn) - sgn;                                    // negated again when x < 0
 }
 
 struct LoihiState {
     int current;
     int voltage;
-    uint32_t countdown;  // steps until the neuron may spike again (0 = not refractory)
+    int countdown;  // steps until the neuron may spike again (0 = not refractory)
 };
 
 struct LoihiParams {
-    uint32_t weightScale, keepI, keepV, refDelay, vDecay;
-    int theta;
+    uint32_t weightShift, keepI, keepV, vDecay;
+    int refDelay, theta;
 };
 
-// One time step (t >= 1).  Returns the spike; cOut / vOut are the reported current / voltage.
+// One time step (t >= 1).  Returns the spike (0/1); cOut / vOut are the reported current / voltage.
 __device__ __forceinline__ uint32_t loihi_step(LoihiState &st, const LoihiParams &p, float w,
                                                float &cOut, float &vOut)
 {
-    const int cNew = static_cast<int>(loihi_decay(st.current, p.keepI) +
-                                      p.weightScale * static_cast<uint32_t>(trunc_sat(w)));
+    const uint32_t wi = static_cast<uint32_t>(cvt_trunc_sat(w));
+    const int cNew = static_cast<int>(loihi_decay(st.current, p.keepI) + (wi << p.weightShift));
     const int vNew = static_cast<int>(loihi_decay(st.voltage, p.keepV) + static_cast<uint32_t>(cNew));
-    if (st.countdown > 0) --st.countdown;
-    const bool refractory = st.countdown != 0;
-    const uint32_t spike = (vNew > p.theta && !refractory) ? 1u : 0u;
-    st.voltage = (spike || refractory) ? 0 : vNew;
-    if (spike) st.countdown = p.refDelay;
+    const int cd = max(st.countdown - 1, 0);
+    const bool quiet = cd == 0;                       // not refractory at this step
+    const bool spike = quiet & (vNew > p.theta);
+    st.voltage = (quiet & !spike) ? vNew : 0;
+    st.countdown = spike ? p.refDelay : cd;
     st.current = cNew;
     cOut = static_cast<float>(cNew);
     vOut = spike ? static_cast<float>(static_cast<int>(p.vDecay)) : static_cast<float>(st.voltage);
-    return spike;
+    return spike ? 1u : 0u;
 }
 
 // ---- generic kernel: one lane per neuron, straight from global memory ---------------------------
@@ -67,7 +85,7 @@ __global__ __launch_bounds__(256) void loihi_generic_kernel(float *__restrict__ 
     const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (row >= rows) return;
     const int64_t base = row * T;
-    LoihiState st = {0, 0, 0u};
+    LoihiState st = {0, 0, 0};
     s[base] = 0.0f; v[base] = 0.0f; u[base] = 0.0f;
     for (int64_t t = 1; t < T; ++t) {
         float c, vo;
@@ -78,97 +96,294 @@ __global__ __launch_bounds__(256) void loihi_generic_kernel(float *__restrict__ 
     }
 }
 
-// ---- streaming kernel -------------------------------------------------------------------------------
-// Global traffic uses buffer addressing (per-lane offset + wave-uniform offset per row pair); the
-// 32 loads of a chunk are issued one chunk ahead and stay in flight during the sequential update.
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 8))) void loihi_stream_kernel(
-    float *__restrict__ s, float *__restrict__ v, float *__restrict__ u, const float *__restrict__ w,
-    int64_t rows, int T, LoihiParams p)
+// ---- row-tile kernel ---------------------------------------------------------------------------------
+// R rows per tile (= lanes that update), PIECE = samples per row and piece at most.
+template <bool VEC, int R, int PIECE>
+__global__ __launch_bounds__(64) void loihi_tile_kernel(float *__restrict__ s, float *__restrict__ v,
+                                                        float *__restrict__ u, const float *__restrict__ w,
+                                                        int64_t rows, int T, int Tc, int P, int MP,
+                                                        int64_t tiles, LoihiParams p)
 {
-    constexpr int C = kLoihiChunk;
-    constexpr int P = C + 1;  // padded pitch: column k of row r sits in bank (r + k) mod 32
-    __shared__ float tileC[kWave * P];  // input, then current
-    __shared__ float tileV[kWave * P];  // voltage
+    constexpr int G = 32;           // samples per update group = bits of a spike mask
+    constexpr int V = VEC ? 4 : 1;  // samples per global access
+    constexpr int NB = R * PIECE / V / kWave;  // accesses per lane per piece, at most
+    extern __shared__ __align__(16) float lds[];
+    float *tileC = lds;                    // [R][P]: input, then current;  P = 4 (mod 32)
+    float *tileV = lds + R * P;   // [R][P]: voltage
+    uint32_t *masks = reinterpret_cast<uint32_t *>(lds + 2 * R * P);  // [R][MP]
 
     const int lane = threadIdx.x;
-    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kWave;
-    const bool fullTile = row0 + kWave <= rows;
-    const int nChunks = (T + C - 1) / C;
-    const int segT = lane & 31;
-    const int segR = lane >> 5;
-    auto slot = [](int r, int k) { return r * P + k; };
+    LoihiState st = {0, 0, 0};
 
-    const int64_t tileBase = row0 * static_cast<int64_t>(T);
-    const BufferRsrc bufW = make_buffer(w + tileBase);
-    const BufferRsrc bufS = make_buffer(s + tileBase);
-    const BufferRsrc bufV = make_buffer(v + tileBase);
-    const BufferRsrc bufU = make_buffer(u + tileBase);
-    const int laneOff = (segR * T + segT) * 4;
-    const int pairStride = 2 * T * 4;
-
-    float pre[C];
-    auto issue_loads = [&](int tBase) {
-        const int off = laneOff + tBase * 4;
-        if (fullTile && tBase + C <= T) {
+    float x[NB * V];
+    auto rows_of = [&](int64_t t) { return static_cast<int>(min(static_cast<int64_t>(R), rows - t * R)); };
+    auto issue = [&](int64_t t, int tL) {
+        const BufferRsrc bufW = make_buffer(w + t * R * static_cast<int64_t>(T));
+        const int perRow = min(Tc, T - tL) / V;
+        const int total = rows_of(t) * perRow;
+        RowCol rc;
+        rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
+        const int dr = kWave / perRow, dc = kWave % perRow;
 #pragma unroll
-            for (int i = 0; i < 32; ++i) pre[i] = buffer_load(bufW, off, i * pairStride);
-        } else {
-            const bool tOk = tBase + segT < T;
-#pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                pre[i] = 0.0f;
-                if (tOk && row0 + 2 * i + segR < rows) pre[i] = buffer_load(bufW, off, i * pairStride);
+        for (int b = 0; b < NB; ++b) {
+            if (lane + b * kWave < total) {
+                const int off = (rc.r * T + tL + rc.c * V) * 4;
+                if (VEC) {
+                    const float4 q = buffer_load4(bufW, off, 0);
+                    x[4 * b] = q.x; x[4 * b + 1] = q.y; x[4 * b + 2] = q.z; x[4 * b + 3] = q.w;
+                } else {
+                    x[b] = buffer_load(bufW, off, 0);
+                }
             }
+            rc.advance(dr, dc, perRow);
+        }
+    };
+    auto commit = [&](int64_t t, int tL) {
+        const int perRow = min(Tc, T - tL) / V;
+        const int total = rows_of(t) * perRow;
+        RowCol rc;
+        rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
+        const int dr = kWave / perRow, dc = kWave % perRow;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            if (lane + b * kWave < total) {
+                float *dst = tileC + rc.r * P + rc.c * V;
+                if (VEC) *reinterpret_cast<float4 *>(dst) = make_float4(x[4 * b], x[4 * b + 1], x[4 * b + 2], x[4 * b + 3]);
+                else *dst = x[b];
+            }
+            rc.advance(dr, dc, perRow);
         }
     };
 
-    LoihiState st = {0, 0, 0u};
+    int64_t t = blockIdx.x;
+    int tL = 0;
+    if (t < tiles) issue(t, tL);
+    while (t < tiles) {
+        const int nRows = rows_of(t);
+        const int n = min(Tc, T - tL);
+        const bool last = tL + n == T;
 
-    issue_loads(0);
-    for (int c = 0; c < nChunks; ++c) {
-        const int tBase = c * C;
-#pragma unroll
-        for (int i = 0; i < 32; ++i) tileC[slot(2 * i + segR, segT)] = pre[i];
-        __syncthreads();
-        issue_loads(tBase + C);  // past the end of the rows this loads nothing
-
-        // sequential update: lane = row
-        uint32_t fired = 0;
-        const int first = (c == 0) ? 1 : 0;  // t = 0 is forced to zero
-        if (c == 0) {
-            tileC[slot(lane, 0)] = 0.0f;
-            tileV[slot(lane, 0)] = 0.0f;
-        }
-#pragma unroll 8
-        for (int k = first; k < C; ++k) {
-            const int i = slot(lane, k);
-            float cOut, vOut;
-            const uint32_t spike = loihi_step(st, p, tileC[i], cOut, vOut);
-            fired |= spike << k;
-            tileC[i] = cOut;
-            tileV[i] = vOut;
-        }
-        __syncthreads();
-
+        commit(t, tL);
+        wave_sync();
         {
-            const int off = laneOff + tBase * 4;
-            const bool fast = fullTile && tBase + C <= T;
-            const bool tOk = tBase + segT < T;
-#pragma unroll 8
-            for (int i = 0; i < 32; ++i) {
-                const int r = 2 * i + segR;
-                const float cv = tileC[slot(r, segT)];
-                const float vv = tileV[slot(r, segT)];
-                const uint32_t m = __shfl(fired, r, kWave);
-                const float sv = ((m >> segT) & 1u) ? 1.0f : 0.0f;
-                if (fast || (tOk && row0 + r < rows)) {
-                    buffer_store(bufS, off, i * pairStride, sv);
-                    buffer_store(bufV, off, i * pairStride, vv);
-                    buffer_store(bufU, off, i * pairStride, cv);
+            const int64_t tn = last ? t + gridDim.x : t;
+            const int tLn = last ? 0 : tL + Tc;
+            if (tn < tiles) issue(tn, tLn);
+        }
+
+        // ---- sequential update: lane = row
+        if (lane < R) {
+            if (tL == 0) st = {0, 0, 0};
+            float *mineC = tileC + lane * P;
+            float *mineV = tileV + lane * P;
+            const int groups = (n + G - 1) / G;
+            for (int g = 0; g < groups; ++g) {
+                const int c0 = g * G;
+                float in[G], cur[G], vol[G];
+#pragma unroll
+                for (int k = 0; k < G; k += 4) {
+                    const float4 q = *reinterpret_cast<const float4 *>(mineC + c0 + k);
+                    in[k] = q.x; in[k + 1] = q.y; in[k + 2] = q.z; in[k + 3] = q.w;
+                }
+                uint32_t fired = 0;
+#pragma unroll
+                for (int k = 0; k < G; ++k) {
+                    if (tL + c0 + k == 0) {  // t = 0 is forced to zero and leaves the state untouched
+                        cur[k] = 0.0f;
+                        vol[k] = 0.0f;
+                    } else {
+                        fired |= loihi_step(st, p, in[k], cur[k], vol[k]) << k;
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < G; k += 4) {
+                    *reinterpret_cast<float4 *>(mineC + c0 + k) = make_float4(cur[k], cur[k + 1], cur[k + 2], cur[k + 3]);
+                    *reinterpret_cast<float4 *>(mineV + c0 + k) = make_float4(vol[k], vol[k + 1], vol[k + 2], vol[k + 3]);
+                }
+                masks[lane * MP + g] = fired;
+            }
+        }
+        wave_sync();
+
+        // ---- retire
+        {
+            const int64_t base = t * R * static_cast<int64_t>(T);
+            const BufferRsrc bufS = make_buffer(s + base);
+            const BufferRsrc bufV = make_buffer(v + base);
+            const BufferRsrc bufU = make_buffer(u + base);
+            const int perRow = n / V;
+            const int total = nRows * perRow;
+            RowCol rc;
+            rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
+            const int dr = kWave / perRow, dc = kWave % perRow;
+#pragma unroll 4
+            for (int g0 = lane; g0 < total; g0 += kWave) {
+                const int col = rc.c * V;
+                const int off = (rc.r * T + tL + col) * 4;
+                const uint32_t m = masks[rc.r * MP + (col >> 5)] >> (col & 31);
+                if (VEC) {
+                    buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + rc.r * P + col));
+                    buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + rc.r * P + col));
+                    buffer_store4(bufS, off, 0,
+                                  make_float4((m & 1u) ? 1.0f : 0.0f, (m & 2u) ? 1.0f : 0.0f,
+                                              (m & 4u) ? 1.0f : 0.0f, (m & 8u) ? 1.0f : 0.0f));
+                } else {
+                    buffer_store(bufU, off, 0, tileC[rc.r * P + col]);
+                    buffer_store(bufV, off, 0, tileV[rc.r * P + col]);
+                    buffer_store(bufS, off, 0, (m & 1u) ? 1.0f : 0.0f);
+                }
+                rc.advance(dr, dc, perRow);
+            }
+        }
+        wave_sync();
+
+        if (last) { t += gridDim.x; tL = 0; }
+        else tL += Tc;
+    }
+}
+
+// ---- line-aligned row-tile kernel ---------------------------------------------------------------------
+// Same scheme, for rows that are whole 16-byte vectors, with one refinement that matters a lot on
+// HBM: every piece of every row is a whole number of 128-byte memory lines.  Row r does not cut
+// its samples at multiples of the piece length but at the 128-byte boundaries of its own
+// storage: with o_r = (address of the row's first sample mod 128) / 4, piece j of row r holds the
+// samples [32 LPP j - o_r, 32 LPP (j+1) - o_r).  Lanes are independent in the sequential update,
+// so it does not matter that they are at slightly different times.  All four tensors are then
+// read and written as full, aligned lines (except at the two ends of a row); pieces that start
+// or end in the middle of a line make the memory system write that line twice, partially, which
+// measured about three times slower for the three output tensors.
+// R rows per tile (= lanes that update), LPP = 128-byte lines per row and piece.
+template <int R, int LPP>
+__global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, float *__restrict__ v,
+                                                         float *__restrict__ u, const float *__restrict__ w,
+                                                         int64_t rows, int T, int64_t tiles, LoihiParams p)
+{
+    constexpr int G = 32;              // samples per line = samples per update group = bits of a mask
+    constexpr int TC = G * LPP;        // samples per row and piece
+    constexpr int QP = TC / 4;         // 16-byte vectors per row and piece
+    constexpr int RPI = kWave / QP;    // rows covered by one wave-wide access
+    constexpr int NB = R / RPI;        // accesses per lane per piece
+    constexpr int P = TC + 4;          // LDS pitch = 4 (mod 32): 16-byte aligned rows in different banks
+    __shared__ __align__(16) float tileC[R * P];  // input, then current
+    __shared__ __align__(16) float tileV[R * P];  // voltage
+    __shared__ uint32_t masks[R * LPP];
+
+    const int lane = threadIdx.x;
+    const int subRow = lane / QP;         // row within an access
+    const int col = (lane % QP) * 4;      // first column of this lane's vector
+    const int pieces = (T + G - 1 + TC - 1) / TC;  // enough for the most skewed row
+
+    LoihiState st = {0, 0, 0};
+    float4 x[NB];
+
+    auto rows_of = [&](int64_t t) { return static_cast<int>(min(static_cast<int64_t>(R), rows - t * R)); };
+    // samples by which row r of tile t starts after a 128-byte boundary
+    auto skew_base = [&](int64_t t) {
+        return static_cast<int>((reinterpret_cast<uintptr_t>(w + t * R * static_cast<int64_t>(T)) >> 2) & 31);
+    };
+    auto issue = [&](int64_t t, int j) {
+        const BufferRsrc bufW = make_buffer(w + t * R * static_cast<int64_t>(T));
+        const int nRows = rows_of(t);
+        const int o0 = skew_base(t);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const int r = b * RPI + subRow;
+            const int time = TC * j - ((o0 + r * T) & 31) + col;
+            x[b] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (r < nRows && time >= 0 && time < T) x[b] = buffer_load4(bufW, (r * T + time) * 4, 0);
+        }
+    };
+
+    int64_t t = blockIdx.x;
+    int j = 0;
+    if (t < tiles) issue(t, j);
+    while (t < tiles) {
+        const int nRows = rows_of(t);
+        const int o0 = skew_base(t);
+        const bool last = j + 1 == pieces;
+
+#pragma unroll
+        for (int b = 0; b < NB; ++b) *reinterpret_cast<float4 *>(tileC + (b * RPI + subRow) * P + col) = x[b];
+        wave_sync();
+        {
+            const int64_t tn = last ? t + gridDim.x : t;
+            if (tn < tiles) issue(tn, last ? 0 : j + 1);
+        }
+
+        // ---- sequential update: lane = row; this lane's column c is its sample TC*j - o + c
+        if (R == kWave || lane < R) {
+            if (j == 0) st = {0, 0, 0};
+            float *mineC = tileC + lane * P;
+            float *mineV = tileV + lane * P;
+            const int tRow = TC * j - ((o0 + lane * T) & 31);
+            // pieces that lie inside every row need no per-sample checks
+            const bool inside = j >= 1 && TC * (j + 1) <= T;
+#pragma unroll
+            for (int g = 0; g < LPP; ++g) {
+                const int c0 = g * G;
+                float in[G], cur[G], vol[G];
+#pragma unroll
+                for (int k = 0; k < G; k += 4) {
+                    const float4 q = *reinterpret_cast<const float4 *>(mineC + c0 + k);
+                    in[k] = q.x; in[k + 1] = q.y; in[k + 2] = q.z; in[k + 3] = q.w;
+                }
+                uint32_t fired = 0;
+                if (inside) {
+#pragma unroll
+                    for (int k = 0; k < G; ++k) fired |= loihi_step(st, p, in[k], cur[k], vol[k]) << k;
+                } else {
+#pragma unroll
+                    for (int k = 0; k < G; ++k) {
+                        // sample 0 is forced to zero and leaves the state untouched; samples outside
+                        // the row do not exist
+                        const int time = tRow + c0 + k;
+                        const bool ok = time >= 1 && time < T;
+                        LoihiState next = st;
+                        float c, vo;
+                        const uint32_t spike = loihi_step(next, p, in[k], c, vo);
+                        st.current = ok ? next.current : st.current;
+                        st.voltage = ok ? next.voltage : st.voltage;
+                        st.countdown = ok ? next.countdown : st.countdown;
+                        cur[k] = ok ? c : 0.0f;
+                        vol[k] = ok ? vo : 0.0f;
+                        fired |= (ok ? spike : 0u) << k;
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < G; k += 4) {
+                    *reinterpret_cast<float4 *>(mineC + c0 + k) = make_float4(cur[k], cur[k + 1], cur[k + 2], cur[k + 3]);
+                    *reinterpret_cast<float4 *>(mineV + c0 + k) = make_float4(vol[k], vol[k + 1], vol[k + 2], vol[k + 3]);
+                }
+                masks[lane * LPP + g] = fired;
+            }
+        }
+        wave_sync();
+
+        // ---- retire: whole lines of current, voltage and spikes
+        {
+            const int64_t base = t * R * static_cast<int64_t>(T);
+            const BufferRsrc bufS = make_buffer(s + base);
+            const BufferRsrc bufV = make_buffer(v + base);
+            const BufferRsrc bufU = make_buffer(u + base);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const int r = b * RPI + subRow;
+                const int time = TC * j - ((o0 + r * T) & 31) + col;
+                if (r < nRows && time >= 0 && time < T) {
+                    const int off = (r * T + time) * 4;
+                    const uint32_t m = masks[r * LPP + (col >> 5)] >> (col & 31);
+                    buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + r * P + col));
+                    buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + r * P + col));
+                    buffer_store4(bufS, off, 0,
+                                  make_float4((m & 1u) ? 1.0f : 0.0f, (m & 2u) ? 1.0f : 0.0f,
+                                              (m & 4u) ? 1.0f : 0.0f, (m & 8u) ? 1.0f : 0.0f));
                 }
             }
         }
-        __syncthreads();
+        wave_sync();
+
+        if (last) { t += gridDim.x; j = 0; }
+        else ++j;
     }
 }
 
@@ -181,23 +396,50 @@ extern "C" int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const f
 {
     using namespace slayer;
     if (nNeurons < 0 || T < 0) return SLAYER_EINVAL;
-    if (refDelay == 0 || wgtExp > 25) return SLAYER_EINVAL;
+    if (refDelay == 0 || wgtExp > 25 || refDelay > 0x7fffffffu) return SLAYER_EINVAL;
     if (nNeurons == 0 || T == 0) return SLAYER_OK;
     if (!s || !v || !u || !w) return SLAYER_EINVAL;
     hipStream_t st = static_cast<hipStream_t>(stream);
 
     LoihiParams p;
-    p.weightScale = 1u << (6 + wgtExp);
+    p.weightShift = 6 + wgtExp;  // weight scale 1 << (6 + wgtExp)
     p.keepI = 4096u - iDecay;
     p.keepV = 4096u - vDecay;
-    p.refDelay = refDelay;
+    p.refDelay = static_cast<int>(refDelay);
     p.vDecay = vDecay;
     p.theta = theta;
 
-    const int64_t groups = ceil_div(nNeurons, kWave);
-    if (!generic_forced() && T <= kBufferMaxT && groups < (1LL << 31)) {
-        hipLaunchKernelGGL(loihi_stream_kernel, dim3(static_cast<unsigned>(groups)), dim3(kWave), 0, st,
-                           s, v, u, w, nNeurons, static_cast<int>(T), p);
+    if (!generic_forced() && T <= kBufferMaxT) {
+        constexpr int kRows = 32, kPiece = LOIHI_PIECE;
+        const int64_t tiles = ceil_div(nNeurons, kRows);
+        // rows shorter than a piece travel whole; the update goes in groups of 32 columns
+        const int Tc = T < kPiece ? static_cast<int>(T) : kPiece;
+        const int cols = (Tc + 31) & ~31;
+        const int P = cols + 4;  // 4 (mod 32): rows are 16-byte aligned and start in different banks
+        const int MP = cols / 32 + 1;
+        const size_t lds = (static_cast<size_t>(2 * kRows) * P + kRows * MP) * sizeof(float);
+        const int64_t resident = static_cast<int64_t>(compute_units()) * (160 * 1024 / static_cast<int64_t>(lds));
+        const unsigned grid = static_cast<unsigned>(tiles < resident ? tiles : resident);
+        const bool vec = (T % 4 == 0) && aligned16(s) && aligned16(v) && aligned16(u) && aligned16(w);
+        const uintptr_t phase = reinterpret_cast<uintptr_t>(w) & 127;
+        const bool samePhase = (reinterpret_cast<uintptr_t>(s) & 127) == phase &&
+                               (reinterpret_cast<uintptr_t>(v) & 127) == phase &&
+                               (reinterpret_cast<uintptr_t>(u) & 127) == phase;
+        if (vec && samePhase) {
+            constexpr int kR = LOIHI_ROWS, kLpp = LOIHI_LPP;
+            const int64_t lineTiles = ceil_div(nNeurons, kR);
+            const int64_t ldsBytes = (2LL * kR * (32 * kLpp + 4) + kR * kLpp) * 4;
+            const int64_t fit = static_cast<int64_t>(compute_units()) * (160 * 1024 / ldsBytes);
+            hipLaunchKernelGGL((loihi_lines_kernel<kR, kLpp>), dim3(static_cast<unsigned>(lineTiles < fit ? lineTiles : fit)),
+                               dim3(kWave), 0, st, s, v, u, w, nNeurons, static_cast<int>(T), lineTiles, p);
+            return launch_status();
+        }
+        if (vec)
+            hipLaunchKernelGGL((loihi_tile_kernel<true, kRows, kPiece>), dim3(grid), dim3(kWave), lds, st, s, v, u,
+                               w, nNeurons, static_cast<int>(T), Tc, P, MP, tiles, p);
+        else
+            hipLaunchKernelGGL((loihi_tile_kernel<false, kRows, kPiece>), dim3(grid), dim3(kWave), lds, st, s, v,
+                               u, w, nNeurons, static_cast<int>(T), Tc, P, MP, tiles, p);
         return launch_status();
     }
     const int64_t blocks = ceil_div(nNeurons, 256);

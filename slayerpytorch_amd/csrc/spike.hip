@@ -88,7 +88,7 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
 
     for (int c = 0; c < nChunks; ++c) {
         if (c + ahead < nChunks) load_chunk(c + ahead);
-        __syncthreads();
+        wave_sync();
 
         // process: lane = row
         uint32_t fired = 0;
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
                 for (; j < last; ++j) ring[slot(lane, t + j)] += nu[j];
             }
         }
-        __syncthreads();
+        wave_sync();
 
         // store: finished chunk c leaves the ring
         {
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
                 }
             }
         }
-        __syncthreads();
+        wave_sync();
     }
 }
 
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         const int tW = tL - LAG;        // time of tile column 0 (columns [0, LAG) are carried over)
 
         commit(t, tL);
-        __syncthreads();
+        wave_sync();
         {   // next step: next piece of this tile, or first piece of this group's next tile
             const int64_t tn = last ? t + gridDim.x : t;
             const int tLn = last ? 0 : tL + Tc;
@@ -273,7 +273,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                 for (int k = 0; k < LAG; ++k) v[k] = v[G + k];
             }
         }
-        __syncthreads();
+        wave_sync();
 
         // ---- retire: columns [first, W) leave as u' and s, times tW + column
         {
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                 rc.advance(dr, dc, perRow);
             }
         }
-        __syncthreads();
+        wave_sync();
 
         if (last) { t += gridDim.x; tL = 0; }
         else tL += Tc;
