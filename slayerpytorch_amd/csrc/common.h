@@ -127,6 +127,14 @@ __device__ __forceinline__ float buffer_load(BufferRsrc b, int laneBytes, int un
 typedef float float4_ext __attribute__((ext_vector_type(4)));
 typedef unsigned int uint4_ext __attribute__((ext_vector_type(4)));
 
+// Offset that lies outside every buffer made by make_buffer(): a load from it returns zeros and a
+// store to it is dropped by the hardware's range check.  Masking accesses this way instead of
+// branching around them keeps the number of memory instructions between two points fixed, so
+// the compiler can wait for "all but the last N" (s_waitcnt vmcnt(N)) instead of for everything.
+constexpr int kOutOfRange = static_cast<int>(0x80000000u);
+
+__device__ __forceinline__ int masked_offset(bool valid, int bytes) { return valid ? bytes : kOutOfRange; }
+
 template <int POLICY = kStream>
 __device__ __forceinline__ float4 buffer_load4(BufferRsrc b, int laneBytes, int uniformBytes)
 {

@@ -21,7 +21,6 @@
 
 namespace slayer {
 
-constexpr int kFirU = 8;              // outputs per lane per chunk
 constexpr int kFirMaxLdsFloats = 12288;  // 48 KiB of LDS per work-group at most
 constexpr int kFirMaxPitch = 512;     // longest LDS row (samples) the tiled kernel stages
 
@@ -49,13 +48,31 @@ __global__ __launch_bounds__(256) void fir_generic_kernel(float *__restrict__ ou
 }
 
 // ---- tiled kernel ---------------------------------------------------------------------------------
-__device__ __forceinline__ void fma_quad(float (&acc)[kFirU], const float4 &a, const float4 &b,
-                                         const float4 &c, float f0, float f1, float f2, float f3)
+// A lane produces U consecutive outputs from a register window of U + 4 samples held as
+// NQ = U/4 + 1 16-byte vectors q[].  ROT says which vector currently holds the oldest samples:
+// window sample e is component e % 4 of q[(ROT + e / 4) % NQ].  After a 4-tap block the oldest
+// vector is replaced by the next one from LDS and ROT advances, so the window slides without any
+// register moves once the loops are unrolled.
+template <int U, int ROT>
+__device__ __forceinline__ void window_of(float (&w)[U + 4], const float4 (&q)[U / 4 + 1])
 {
-    // window w[0..11] = (a, b, c); output j, tap s uses w[j + s]
-    const float w[12] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w, c.x, c.y, c.z, c.w};
+    constexpr int NQ = U / 4 + 1;
 #pragma unroll
-    for (int j = 0; j < kFirU; ++j) {
+    for (int v = 0; v < NQ; ++v) {
+        const float4 &x = q[(ROT + v) % NQ];
+        w[4 * v] = x.x; w[4 * v + 1] = x.y; w[4 * v + 2] = x.z; w[4 * v + 3] = x.w;
+    }
+}
+
+// taps f0..f3 are filter taps i..i+3; output j, tap s uses window sample j + s
+template <int U, int ROT>
+__device__ __forceinline__ void fma_block(float (&acc)[U], const float4 (&q)[U / 4 + 1], float f0, float f1,
+                                          float f2, float f3)
+{
+    float w[U + 4];
+    window_of<U, ROT>(w, q);
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
         acc[j] = __builtin_fmaf(w[j + 0], f0, acc[j]);
         acc[j] = __builtin_fmaf(w[j + 1], f1, acc[j]);
         acc[j] = __builtin_fmaf(w[j + 2], f2, acc[j]);
@@ -63,8 +80,128 @@ __device__ __forceinline__ void fma_quad(float (&acc)[kFirU], const float4 &a, c
     }
 }
 
+// the last 1..3 taps of a filter whose length is not a multiple of 4
+template <int U, int ROT>
+__device__ __forceinline__ void fma_rest(float (&acc)[U], const float4 (&q)[U / 4 + 1], const float *__restrict__ f,
+                                         int n)
+{
+    float w[U + 4];
+    window_of<U, ROT>(w, q);
+    const float f0 = f[0];
+    const float f1 = n > 1 ? f[1] : 0.0f;
+    const float f2 = n > 2 ? f[2] : 0.0f;
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+        acc[j] = __builtin_fmaf(w[j], f0, acc[j]);
+        if (n > 1) acc[j] = __builtin_fmaf(w[j + 1], f1, acc[j]);
+        if (n > 2) acc[j] = __builtin_fmaf(w[j + 2], f2, acc[j]);
+    }
+}
+
+// blocks B, B+1, .., NQ-1 of one trip of the main loop (NQ blocks = 4 NQ taps per trip)
+template <int U, int B>
+struct TripBlocks {
+    static __device__ __forceinline__ void run(float (&acc)[U], float4 (&q)[U / 4 + 1], const float4 *xq, int qi,
+                                               const float *__restrict__ f)
+    {
+        if constexpr (B < U / 4 + 1) {
+            fma_block<U, B>(acc, q, f[4 * B], f[4 * B + 1], f[4 * B + 2], f[4 * B + 3]);
+            q[B] = xq[qi + B];
+            TripBlocks<U, B + 1>::run(acc, q, xq, qi, f);
+        }
+    }
+};
+
+// up to NQ-1 further whole blocks after the main loop, then the rest; B = blocks done so far
+template <int U, int B>
+struct TailBlocks {
+    static __device__ __forceinline__ void run(float (&acc)[U], float4 (&q)[U / 4 + 1], const float4 *xq, int qi,
+                                               const float *__restrict__ f, int left)
+    {
+        if constexpr (B < U / 4 + 1) {
+            if (left >= 4) {
+                fma_block<U, B>(acc, q, f[0], f[1], f[2], f[3]);
+                q[B] = xq[qi];
+                TailBlocks<U, B + 1>::run(acc, q, xq, qi + 1, f + 4, left - 4);
+            } else if (left > 0) {
+                fma_rest<U, B>(acc, q, f, left);
+            }
+        }
+    }
+};
+
+// true when any of the four samples is not (plus or minus) zero
+__device__ __forceinline__ bool any_nonzero(const float4 &v)
+{
+    const uint32_t bits = __builtin_bit_cast(uint32_t, v.x) | __builtin_bit_cast(uint32_t, v.y) |
+                          __builtin_bit_cast(uint32_t, v.z) | __builtin_bit_cast(uint32_t, v.w);
+    return (bits << 1) != 0;
+}
+
+// ---- event-driven path for sparse input (spike trains) -------------------------------------------
+// When few samples of a tile are non-zero, walking the taps wastes almost all of its multiply-adds
+// on zeros.  Here a wavefront takes one row at a time, finds the row's non-zero samples ("events")
+// with ballots, and for each block of 64 outputs adds the events that can reach it, in ascending
+// order of their column: for output m the terms X[j] * filt[j - m] arrive in ascending j, i.e. in
+// ascending tap order, which is exactly the dense chain with its zero terms left out - and adding
+// a zero term never changes a finite sum - so both paths give the same bits.  All control flow is
+// wave-uniform (the event list lives in scalar registers).
+constexpr int kSparseBlocks = 7;   // 64-column blocks of an LDS row the sparse path handles (LD <= 448)
+constexpr int kSparseMaxTaps = 129;  // an event reaches at most three 64-output blocks
+
+template <bool CAUSAL>
+__device__ __forceinline__ void fir_sparse_tile(const BufferRsrc &bufOut, const float *X, const float *fL,
+                                                int nRows, int LD, int ttp, int t0, int tt, int tHi, int T,
+                                                int F, float Ts)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int nPass = (ttp + kWave - 1) / kWave;  // blocks of 64 outputs; lane's output in block k is 64 k + lane
+    for (int r = wave; r < nRows; r += 4) {
+        const float *xr = X + r * LD;
+        float acc[kSparseBlocks];
+#pragma unroll
+        for (int k = 0; k < kSparseBlocks; ++k) acc[k] = 0.0f;
+        // events in ascending column order, 64 columns at a time
+#pragma unroll
+        for (int b = 0; b < kSparseBlocks; ++b) {
+            if (b * kWave >= LD) break;
+            float v = 0.0f;
+            if (b * kWave + lane < LD) v = xr[b * kWave + lane];
+            uint64_t mask = __ballot(v != 0.0f);
+            while (mask) {
+                const int pos = __builtin_ctzll(mask);
+                mask &= mask - 1;
+                const float xv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), pos));
+                // column j = 64 b + pos is tap i = j - m of output m; it reaches the output blocks
+                // b-2, b-1 and b (F <= 129), each with its own tap; the taps are fetched together
+                float tap[3];
+                bool hit[3];
+#pragma unroll
+                for (int d = 0; d < 3; ++d) {
+                    const int i = kWave * d + pos - lane;  // tap for the output block b - d
+                    hit[d] = b - d >= 0 && b - d < nPass && static_cast<unsigned>(i) < static_cast<unsigned>(F);
+                    tap[d] = hit[d] ? fL[i] : 0.0f;
+                }
+#pragma unroll
+                for (int d = 0; d < 3; ++d)
+                    if (b - d >= 0 && hit[d]) acc[b - d] = __builtin_fmaf(xv, tap[d], acc[b - d]);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kSparseBlocks; ++k) {
+            if (k >= nPass) break;
+            const int m = k * kWave + lane;
+            const int time = CAUSAL ? (tHi - m) : (t0 + m);
+            // the blocks of 64 outputs of a row complete each other's memory lines: keep them cached
+            buffer_store<0>(bufOut, masked_offset(m < ttp && time >= t0 && time < t0 + tt, (r * T + time) * 4), 0,
+                            acc[k] * Ts);
+        }
+    }
+}
+
 // VEC: rows are whole 16-byte vectors (T % 4 == 0, pointers 16-byte aligned)
-template <bool CAUSAL, bool VEC>
+template <bool CAUSAL, bool VEC, int U>
 __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
                                                         const float *__restrict__ in,
                                                         const float *__restrict__ filt,
@@ -72,13 +209,16 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
                                                         float Ts)
 {
     extern __shared__ __align__(16) float X[];
+    float *fL = X + R * LD;                                        // filter copy for the sparse path
+    uint32_t *nzCount = reinterpret_cast<uint32_t *>(fL + F);      // non-zero input vectors, per wavefront
+    uint32_t nonZero = 0;                                          // wave-uniform
 
     const int tid = threadIdx.x;
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
     const int nRows = static_cast<int>(min(static_cast<int64_t>(R), rows - row0));
     const int t0 = blockIdx.y * TT;                   // first output time of the tile
     const int tt = min(TT, T - t0);                   // outputs in this tile
-    const int ttp = (tt + kFirU - 1) & ~(kFirU - 1);  // rounded up to whole chunks
+    const int ttp = (tt + U - 1) & ~(U - 1);  // rounded up to whole chunks
     const int tHi = t0 + ttp - 1;                     // time stored at X[.][0] when reversed
     const int LD4 = LD >> 2;
 
@@ -101,6 +241,7 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
             const int total = nRows * nq;
             for (int g = tid; g < total; g += 256, rc.advance(dr, dc, nq)) {
                 const float4 v = buffer_load4(bufIn, (rc.r * T + tA + (rc.c << 2)) * 4, 0);
+                nonZero += __builtin_popcountll(__ballot(any_nonzero(v)));
                 if (CAUSAL)  // descending time: the vector lands mirrored
                     *reinterpret_cast<float4 *>(X + rc.r * LD + (jA + ((nq - 1 - rc.c) << 2))) =
                         make_float4(v.w, v.z, v.y, v.x);
@@ -144,12 +285,25 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
                 if (tl + 3 < T) v.w = src[tl + 3];
             }
             *reinterpret_cast<float4 *>(X + r * LD + j) = v;
+            nonZero += __builtin_popcountll(__ballot(any_nonzero(v)));
         }
     }
+    for (int i = tid; i < F; i += 256) fL[i] = filt[i];
+    if ((tid & (kWave - 1)) == 0) nzCount[tid / kWave] = nonZero;
     __syncthreads();
 
+    // ---- sparse input: event-driven path
+    {
+        const uint32_t nz = nzCount[0] + nzCount[1] + nzCount[2] + nzCount[3];
+        const uint32_t vectors = static_cast<uint32_t>(nRows) * static_cast<uint32_t>(LD >> 2);
+        if (F <= kSparseMaxTaps && LD <= kSparseBlocks * kWave && nz * 8u <= vectors) {
+            fir_sparse_tile<CAUSAL>(bufOut, X, fL, nRows, LD, ttp, t0, tt, tHi, T, F, Ts);
+            return;
+        }
+    }
+
     // ---- compute: work item = (row, chunk of 8 outputs), row-major over lanes
-    const int nChunks = ttp / kFirU;
+    const int nChunks = ttp / U;
     const int items = nRows * nChunks;
     const int F4 = F & ~3;
     RowCol item;
@@ -158,104 +312,97 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
 
     for (int w = tid; w < items; w += 256, item.advance(itemDr, itemDc, nChunks)) {
         const int r = item.r;
-        const int m0 = item.c * kFirU;
-        float acc[kFirU];
+        const int m0 = item.c * U;
+        float acc[U];
 #pragma unroll
-        for (int j = 0; j < kFirU; ++j) acc[j] = 0.0f;
+        for (int j = 0; j < U; ++j) acc[j] = 0.0f;
 
+        constexpr int NQ = U / 4 + 1;
         const float4 *xq = reinterpret_cast<const float4 *>(X + r * LD + m0);
-        float4 qa = xq[0], qb = xq[1], qc = xq[2];
-        int i = 0, q = 3;
-        // three 4-tap blocks per trip so that the window rotates through registers without moves
-        for (; i + 12 <= F4; i += 12, q += 3) {
-            fma_quad(acc, qa, qb, qc, filt[i], filt[i + 1], filt[i + 2], filt[i + 3]);
-            qa = xq[q];
-            fma_quad(acc, qb, qc, qa, filt[i + 4], filt[i + 5], filt[i + 6], filt[i + 7]);
-            qb = xq[q + 1];
-            fma_quad(acc, qc, qa, qb, filt[i + 8], filt[i + 9], filt[i + 10], filt[i + 11]);
-            qc = xq[q + 2];
-        }
-        if (i + 4 <= F4) {
-            fma_quad(acc, qa, qb, qc, filt[i], filt[i + 1], filt[i + 2], filt[i + 3]);
-            const float4 n = xq[q];
-            qa = qb; qb = qc; qc = n;
-            i += 4; ++q;
-        }
-        if (i + 4 <= F4) {
-            fma_quad(acc, qa, qb, qc, filt[i], filt[i + 1], filt[i + 2], filt[i + 3]);
-            const float4 n = xq[q];
-            qa = qb; qb = qc; qc = n;
-            i += 4; ++q;
-        }
-        if (i < F) {  // 1..3 remaining taps
-            const float f0 = filt[i];
-            const float f1 = (i + 1 < F) ? filt[i + 1] : 0.0f;
-            const float f2 = (i + 2 < F) ? filt[i + 2] : 0.0f;
-            const float wv[12] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w, qc.x, qc.y, qc.z, qc.w};
+        float4 q[NQ];
 #pragma unroll
-            for (int j = 0; j < kFirU; ++j) {
-                acc[j] = __builtin_fmaf(wv[j], f0, acc[j]);
-                if (i + 1 < F) acc[j] = __builtin_fmaf(wv[j + 1], f1, acc[j]);
-                if (i + 2 < F) acc[j] = __builtin_fmaf(wv[j + 2], f2, acc[j]);
-            }
-        }
+        for (int v = 0; v < NQ; ++v) q[v] = xq[v];
+        int i = 0, qi = NQ;
+        for (; i + 4 * NQ <= F4; i += 4 * NQ, qi += NQ) TripBlocks<U, 0>::run(acc, q, xq, qi, filt + i);
+        TailBlocks<U, 0>::run(acc, q, xq, qi, filt + i, F - i);
 
-        // ---- store the 8 outputs: times t0+m0 .. +7 (correlation) or tHi-m0-7 .. tHi-m0 (convolution)
-        float y[kFirU];
+        // ---- store the U outputs: times t0+m0 .. (correlation) or tHi-m0-(U-1) .. tHi-m0 (convolution)
+        float y[U];
 #pragma unroll
-        for (int j = 0; j < kFirU; ++j) y[j] = (CAUSAL ? acc[kFirU - 1 - j] : acc[j]) * Ts;
-        const int tl = CAUSAL ? (tHi - m0 - (kFirU - 1)) : (t0 + m0);  // lowest time of the chunk
+        for (int j = 0; j < U; ++j) y[j] = (CAUSAL ? acc[U - 1 - j] : acc[j]) * Ts;
+        const int tl = CAUSAL ? (tHi - m0 - (U - 1)) : (t0 + m0);  // lowest time of the chunk
         if (VEC) {
-            // tl is a multiple of 4 and so is the tile's end, so each half is all in or all out
+            // tl is a multiple of 4 and so is the tile's end, so each vector is all in or all out.
+            // The vectors of one lane complete each other's memory lines: keep them cached.
             const int off = (r * T + tl) * 4;
-            if (tl >= t0 && tl + 3 < t0 + tt) buffer_store4(bufOut, off, 0, make_float4(y[0], y[1], y[2], y[3]));
-            if (tl + 4 >= t0 && tl + 7 < t0 + tt)
-                buffer_store4(bufOut, off + 16, 0, make_float4(y[4], y[5], y[6], y[7]));
+#pragma unroll
+            for (int v = 0; v < U / 4; ++v)
+                if (tl + 4 * v >= t0 && tl + 4 * v + 3 < t0 + tt)
+                    buffer_store4<0>(bufOut, off + 16 * v, 0, make_float4(y[4 * v], y[4 * v + 1], y[4 * v + 2], y[4 * v + 3]));
         } else {
             float *dst = out + (row0 + r) * static_cast<int64_t>(T);
 #pragma unroll
-            for (int j = 0; j < kFirU; ++j)
+            for (int j = 0; j < U; ++j)
                 if (tl + j >= t0 && tl + j < t0 + tt) dst[tl + j] = y[j];
         }
     }
 }
 
 struct FirPlan {
-    int TT, LD, R, nTiles;
+    int U, TT, LD, R, nTiles;
 };
 
-// Chooses the time tile, the LDS row pitch and the rows per work-group.
-static bool plan_fir(int64_t rows, int64_t T, int64_t F, FirPlan &p)
+// Chooses outputs per lane, the time tile, the LDS row pitch and the rows per work-group.
+static bool plan_fir(int64_t rows, int64_t T, int64_t F, FirPlan &best)
 {
-    // a row of X holds ttp + F + 4 samples (chunk-rounded tile, halo, window over-read)
-    const int64_t ttMax = (kFirMaxPitch - 4 - F) & ~static_cast<int64_t>(kFirU - 1);
-    if (F < 1 || ttMax < 64 || T > kBufferMaxT) return false;
-    const int64_t nTiles = ceil_div(T, ttMax);
-    if (nTiles > 65535) return false;
-    int64_t TT = ceil_div(ceil_div(T, nTiles), kFirU) * kFirU;
-    if (nTiles == 1) TT = T;
-    const int64_t ttp = ceil_div(TT, kFirU) * kFirU;
-    const int64_t LD = (ttp + F + 4 + 3) & ~static_cast<int64_t>(3);
-    const int64_t nChunks = ttp / kFirU;
-    // rows per group: fill the 256 lanes evenly with (row, chunk) items, stay within the LDS
-    // budget, and prefer small tiles (more groups per CU overlap staging with compute)
-    const int64_t rMax = kFirMaxLdsFloats / LD;
-    if (rMax < 1) return false;
-    int64_t best = 1;
+    if (F < 1 || T > kBufferMaxT) return false;
     double bestScore = -1.0;
-    for (int64_t r = 1; r <= rMax && r <= 64; ++r) {
-        const int64_t items = r * nChunks;
-        const double eff = static_cast<double>(items) / static_cast<double>(ceil_div(items, 256) * 256);
-        // at least ~3 passes of work per staging, mild preference for less LDS
-        const double score = eff - (items < 512 ? 0.25 : 0.0) - 0.02 * static_cast<double>(r * LD) / kFirMaxLdsFloats;
-        if (score > bestScore) { bestScore = score; best = r; }
+    for (int U = 16; U >= 8; U -= 8) {
+        // a row of X holds ttp + F + 4 samples (chunk-rounded tile, halo, window over-read)
+        const int64_t ttMax = (kFirMaxPitch - 4 - F) & ~static_cast<int64_t>(U - 1);
+        if (ttMax < 64) continue;
+        const int64_t nTiles = ceil_div(T, ttMax);
+        if (nTiles > 65535) continue;
+        int64_t TT = ceil_div(ceil_div(T, nTiles), U) * U;
+        if (nTiles == 1) TT = T;
+        const int64_t ttp = ceil_div(TT, U) * U;
+        const int64_t LD = (ttp + F + 4 + 3) & ~static_cast<int64_t>(3);
+        const int64_t nChunks = ttp / U;
+        const int64_t rMax = kFirMaxLdsFloats / LD;
+        if (rMax < 1) continue;
+        // per-item work: F taps on U outputs plus a fixed prologue/epilogue; rows per group: fill
+        // the 256 lanes evenly with (row, chunk) items and prefer small tiles (more groups per CU
+        // overlap staging with compute)
+        const double perOutput = (static_cast<double>(F) + 60.0 / U) * static_cast<double>(ttp) /
+                                 static_cast<double>(TT < T ? TT : T);
+        for (int64_t r = 1; r <= rMax && r <= 64; ++r) {
+            const int64_t items = r * nChunks;
+            const double eff = static_cast<double>(items) / static_cast<double>(ceil_div(items, 256) * 256);
+            const double score = eff / perOutput - (items < 256 ? 0.25 / F : 0.0) -
+                                 0.06 / F * static_cast<double>(r * LD) / kFirMaxLdsFloats;
+            if (score > bestScore) {
+                bestScore = score;
+                best.U = U;
+                best.TT = static_cast<int>(TT);
+                best.LD = static_cast<int>(LD);
+                best.R = static_cast<int>(r);
+                best.nTiles = static_cast<int>(nTiles);
+            }
+        }
     }
-    if (best > rows) best = rows;
-    p.TT = static_cast<int>(TT);
-    p.LD = static_cast<int>(LD);
-    p.R = static_cast<int>(best);
-    p.nTiles = static_cast<int>(nTiles);
+    if (bestScore < 0.0) return false;
+    if (best.R > rows) best.R = static_cast<int>(rows);
     return true;
+}
+
+template <bool CAUSAL, bool VEC, int U>
+static void launch_tiled(const FirPlan &p, float *out, const float *in, const float *filt, int64_t rows, int64_t T,
+                         int64_t F, float Ts, hipStream_t stream)
+{
+    dim3 grid(static_cast<unsigned>(ceil_div(rows, p.R)), static_cast<unsigned>(p.nTiles)), block(256);
+    const size_t lds = (static_cast<size_t>(p.R) * p.LD + static_cast<size_t>(F) + 4) * sizeof(float);
+    hipLaunchKernelGGL((fir_tiled_kernel<CAUSAL, VEC, U>), grid, block, lds, stream, out, in, filt, rows,
+                       static_cast<int>(T), static_cast<int>(F), p.TT, p.LD, p.R, Ts);
 }
 
 template <bool CAUSAL>
@@ -268,20 +415,13 @@ static int launch_fir(float *out, const float *in, const float *filt, int64_t ro
     if (T >= (1LL << 30)) return SLAYER_EUNSUPPORTED;
 
     FirPlan p;
-    if (!generic_forced() && plan_fir(rows, T, F, p)) {
-        const int64_t rowTiles = ceil_div(rows, p.R);
-        if (rowTiles < (1LL << 31)) {
-            dim3 grid(static_cast<unsigned>(rowTiles), static_cast<unsigned>(p.nTiles)), block(256);
-            const size_t lds = static_cast<size_t>(p.R) * p.LD * sizeof(float);
-            const bool vec = (T % 4 == 0) && aligned16(out) && aligned16(in);
-            if (vec)
-                hipLaunchKernelGGL((fir_tiled_kernel<CAUSAL, true>), grid, block, lds, stream, out, in, filt,
-                                   rows, static_cast<int>(T), static_cast<int>(F), p.TT, p.LD, p.R, Ts);
-            else
-                hipLaunchKernelGGL((fir_tiled_kernel<CAUSAL, false>), grid, block, lds, stream, out, in, filt,
-                                   rows, static_cast<int>(T), static_cast<int>(F), p.TT, p.LD, p.R, Ts);
-            return launch_status();
-        }
+    if (!generic_forced() && plan_fir(rows, T, F, p) && ceil_div(rows, p.R) < (1LL << 31)) {
+        const bool vec = (T % 4 == 0) && aligned16(out) && aligned16(in);
+        if (vec && p.U == 16) launch_tiled<CAUSAL, true, 16>(p, out, in, filt, rows, T, F, Ts, stream);
+        else if (vec) launch_tiled<CAUSAL, true, 8>(p, out, in, filt, rows, T, F, Ts, stream);
+        else if (p.U == 16) launch_tiled<CAUSAL, false, 16>(p, out, in, filt, rows, T, F, Ts, stream);
+        else launch_tiled<CAUSAL, false, 8>(p, out, in, filt, rows, T, F, Ts, stream);
+        return launch_status();
     }
     const int64_t tBlocks = ceil_div(T, 256);
     if (tBlocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;

@@ -289,14 +289,24 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
         for (int b = 0; b < NB; ++b) {
             const int r = b * RPI + subRow;
             const int time = TC * j - ((o0 + r * T) & 31) + col;
-            x[b] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            if (r < nRows && time >= 0 && time < T) x[b] = buffer_load4(bufW, (r * T + time) * 4, 0);
+            x[b] = buffer_load4(bufW, masked_offset(r < nRows && time >= 0 && time < T, (r * T + time) * 4), 0);
         }
     };
 
     int64_t t = blockIdx.x;
     int j = 0;
-    if (t < tiles) issue(t, j);
+    if (t >= tiles) return;
+    issue(t, j);
+    {
+        // The loop below keeps one piece of loads and one piece of stores in flight and waits only
+        // for the loads ("all but the 3*NB most recent memory instructions").  Entering it with the
+        // same number of stores behind the first loads - dropped by the range check - lets the
+        // compiler use that count on every trip instead of waiting for everything.
+        const BufferRsrc none = make_buffer(w);
+#pragma unroll
+        for (int b = 0; b < 3 * NB; ++b)  // distinct (all out-of-range) addresses, so none is folded away
+            buffer_store4(none, kOutOfRange + 16 * b, 0, make_float4(static_cast<float>(b), 0.0f, 0.0f, 0.0f));
+    }
     while (t < tiles) {
         const int nRows = rows_of(t);
         const int o0 = skew_base(t);
@@ -369,15 +379,13 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
             for (int b = 0; b < NB; ++b) {
                 const int r = b * RPI + subRow;
                 const int time = TC * j - ((o0 + r * T) & 31) + col;
-                if (r < nRows && time >= 0 && time < T) {
-                    const int off = (r * T + time) * 4;
-                    const uint32_t m = masks[r * LPP + (col >> 5)] >> (col & 31);
-                    buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + r * P + col));
-                    buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + r * P + col));
-                    buffer_store4(bufS, off, 0,
-                                  make_float4((m & 1u) ? 1.0f : 0.0f, (m & 2u) ? 1.0f : 0.0f,
-                                              (m & 4u) ? 1.0f : 0.0f, (m & 8u) ? 1.0f : 0.0f));
-                }
+                const int off = masked_offset(r < nRows && time >= 0 && time < T, (r * T + time) * 4);
+                const uint32_t m = masks[r * LPP + (col >> 5)] >> (col & 31);
+                buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + r * P + col));
+                buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + r * P + col));
+                buffer_store4(bufS, off, 0,
+                              make_float4((m & 1u) ? 1.0f : 0.0f, (m & 2u) ? 1.0f : 0.0f,
+                                          (m & 4u) ? 1.0f : 0.0f, (m & 8u) ? 1.0f : 0.0f));
             }
         }
         wave_sync();
