@@ -162,12 +162,14 @@ __device__ __forceinline__ void fir_sparse_tile(const BufferRsrc &bufOut, const 
         float acc[kSparseBlocks];
 #pragma unroll
         for (int k = 0; k < kSparseBlocks; ++k) acc[k] = 0.0f;
+        float xb[kSparseBlocks];  // the row, 64 columns per register
+#pragma unroll
+        for (int b = 0; b < kSparseBlocks; ++b) xb[b] = (b * kWave + lane < LD) ? xr[b * kWave + lane] : 0.0f;
         // events in ascending column order, 64 columns at a time
 #pragma unroll
         for (int b = 0; b < kSparseBlocks; ++b) {
             if (b * kWave >= LD) break;
-            float v = 0.0f;
-            if (b * kWave + lane < LD) v = xr[b * kWave + lane];
+            const float v = xb[b];
             uint64_t mask = __ballot(v != 0.0f);
             while (mask) {
                 const int pos = __builtin_ctzll(mask);
@@ -379,7 +381,7 @@ static bool plan_fir(int64_t rows, int64_t T, int64_t F, FirPlan &best)
             const int64_t items = r * nChunks;
             const double eff = static_cast<double>(items) / static_cast<double>(ceil_div(items, 256) * 256);
             const double score = eff / perOutput - (items < 256 ? 0.25 / F : 0.0) -
-                                 0.06 / F * static_cast<double>(r * LD) / kFirMaxLdsFloats;
+                                 0.25 / F * static_cast<double>(r * LD) / kFirMaxLdsFloats;
             if (score > bestScore) {
                 bestScore = score;
                 best.U = U;
