@@ -96,6 +96,64 @@ def flip_rate(device, srm_t, ref_t, params):
     return float((s_gpu != s_cpu).mean()), float((s_cpu != 0).mean())
 
 
+def other_rows(device):
+    """Quick per-op measurements of the scope rows that are not part of the headline chain, each on
+    the largest tensor its BASELINE config gives it (median of 7 event-timed launches)."""
+    from slayerpytorch_amd import slayerCuda, slayerLoihiCuda
+    from slayerpytorch_amd.slayer import alphaKernel
+    from slayerpytorch_amd.slayerLoihi import loihiPspKernel
+
+    def timed(fn, setup=None):
+        ts = []
+        for i in range(10):
+            if setup:
+                setup()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            if i >= 3:
+                ts.append(a.elapsed_time(b) * 1e-3)
+        return float(np.median(ts))
+
+    def row(name, ab, numel, seconds, shape):
+        return {"op": name, "shape": list(shape), "us": seconds * 1e6, "neuron_timesteps_per_s": numel / seconds,
+                "hbm_frac": ab * numel / seconds / 1e9 / HBM_PEAK_GBS}
+
+    out = []
+    g = torch.Generator(device="cpu").manual_seed(2)
+    # delay stress config: (64, 256, 1, 1, 2000), delays U[0, 62], 8-tap SRM kernel
+    shape = (64, 256, 1, 1, 2000)
+    x = (torch.rand(shape, generator=g) < 0.005).float().to(device)
+    grad = torch.randn(shape, generator=g).to(device)
+    lut = (torch.rand((256, 1, 1), generator=g) * 62).to(device)
+    srm8 = torch.tensor(alphaKernel(1.0, 1.0, 2000), dtype=torch.float32, device=device)
+    ref = torch.tensor(alphaKernel(1.0, 1.0, 2000, mult=-20.0), dtype=torch.float32, device=device)
+    u0 = (torch.randn(shape, generator=g) * 5).to(device)
+    ub = u0.clone()
+    n = x.numel()
+    y = slayerCuda.shift(x, lut, 1.0)
+    out.append(row("shift_per_neuron_table", 8, n, timed(lambda: slayerCuda.shift(x, lut, 1.0)), shape))
+    out.append(row("delay_gradient", 8, n, timed(lambda: slayerCuda.delayGrad(y, grad, 1.0)), shape))
+    out.append(row("psp_conv_8tap", 8, n, timed(lambda: slayerCuda.conv(x, srm8, 1.0)), shape))
+    out.append(row("psp_corr_8tap", 8, n, timed(lambda: slayerCuda.corr(grad, srm8, 1.0)), shape))
+    out.append(row("spike_T2000", 12, n, timed(lambda: slayerCuda.getSpikes(ub, ref, 10.0, 1.0), lambda: ub.copy_(u0)), shape))
+    del x, grad, u0, ub, y
+    # Loihi config: largest tensor (8, 16, 32, 32, 300)
+    shape = (8, 16, 32, 32, 300)
+    w = (2 * torch.randint(-128, 128, shape, generator=g) * (torch.rand(shape, generator=g) < 0.05)).float().to(device)
+    gl = torch.randn(shape, generator=g).to(device)
+    psp = torch.tensor(loihiPspKernel(1024, 128, 0), dtype=torch.float32, device=device)
+    n = w.numel()
+    s, v, u = slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1)
+    out.append(row("loihi_forward", 16, n, timed(lambda: slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1)), shape))
+    out.append(row("loihi_backward_pdf_plus_corr110", 20, n,
+                   timed(lambda: slayerCuda.corr(slayerCuda.spikeBackward(gl, v, 5120.0, 5120.0, 1 / 195.0), psp, 1.0)),
+                   shape))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -182,6 +240,7 @@ def main():
     flips, rate = flip_rate(device, srm_t, ref_t, params)
     result["spike_flip_rate"] = flips
     result["spike_rate"] = rate
+    result["other_rows"] = other_rows(device)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(SHAPE, srm, ref, params)
     print(json.dumps(result))

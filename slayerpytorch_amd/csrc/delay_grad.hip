@@ -13,11 +13,15 @@
 
 namespace slayer {
 
+// VEC: rows are whole 16-byte vectors (T % 4 == 0, 16-byte aligned tensors): a lane takes four
+// consecutive samples per trip and gets the sample before them from the lane to its left.
+template <bool VEC>
 __global__ __launch_bounds__(256) void delay_grad_rows_kernel(float *__restrict__ partial,
                                                               const float *__restrict__ out,
                                                               const float *__restrict__ gradOut,
                                                               int64_t rows, int64_t T, float f0, float f1)
 {
+    typedef float vec4f __attribute__((ext_vector_type(4)));
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t wavesPerGrid = static_cast<int64_t>(gridDim.x) * (blockDim.x / kWave);
     for (int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
@@ -25,10 +29,34 @@ __global__ __launch_bounds__(256) void delay_grad_rows_kernel(float *__restrict_
         const float *y = out + row * T;
         const float *g = gradOut + row * T;
         float acc = 0.0f;
-        for (int64_t t = lane; t < T; t += kWave) {
-            float d = y[t] * f0;
-            if (t > 0) d = __builtin_fmaf(y[t - 1], f1, d);
-            acc = __builtin_fmaf(g[t], d, acc);
+        if (VEC) {
+            const int64_t quads = T >> 2;
+            for (int64_t q0 = 0; q0 < quads; q0 += kWave) {
+                const int64_t q = q0 + lane;
+                vec4f yv = {0.0f, 0.0f, 0.0f, 0.0f}, gv = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (q < quads) {
+                    yv = __builtin_nontemporal_load(reinterpret_cast<const vec4f *>(y) + q);
+                    gv = __builtin_nontemporal_load(reinterpret_cast<const vec4f *>(g) + q);
+                }
+                float before = __shfl_up(yv.w, 1, kWave);   // y[4q - 1] from the lane to the left
+                if (lane == 0) before = (q0 > 0) ? y[4 * q0 - 1] : 0.0f;
+                const bool first = q == 0;                  // y[-1] does not exist: one-tap difference
+                float d0 = yv.x * f0;
+                if (!first) d0 = __builtin_fmaf(before, f1, d0);
+                const float d1 = __builtin_fmaf(yv.x, f1, yv.y * f0);
+                const float d2 = __builtin_fmaf(yv.y, f1, yv.z * f0);
+                const float d3 = __builtin_fmaf(yv.z, f1, yv.w * f0);
+                acc = __builtin_fmaf(gv.x, d0, acc);
+                acc = __builtin_fmaf(gv.y, d1, acc);
+                acc = __builtin_fmaf(gv.z, d2, acc);
+                acc = __builtin_fmaf(gv.w, d3, acc);
+            }
+        } else {
+            for (int64_t t = lane; t < T; t += kWave) {
+                float d = y[t] * f0;
+                if (t > 0) d = __builtin_fmaf(y[t - 1], f1, d);
+                acc = __builtin_fmaf(g[t], d, acc);
+            }
         }
 #pragma unroll
         for (int off = kWave / 2; off > 0; off >>= 1) acc += __shfl_down(acc, off, kWave);
@@ -72,8 +100,12 @@ extern "C" int slayer_delay_grad_f32(float *gradDelay, const float *out, const f
         if (!out || !gradOut || !workspace) return SLAYER_EINVAL;
         int64_t blocks = ceil_div(rows, 4);  // four wavefronts (rows) per work-group
         if (blocks > 262144) blocks = 262144;
-        hipLaunchKernelGGL(delay_grad_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
-                           workspace, out, gradOut, rows, T, -1.0f / Ts, 1.0f / Ts);
+        if ((T % 4 == 0) && aligned16(out) && aligned16(gradOut))
+            hipLaunchKernelGGL(delay_grad_rows_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
+                               workspace, out, gradOut, rows, T, -1.0f / Ts, 1.0f / Ts);
+        else
+            hipLaunchKernelGGL(delay_grad_rows_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
+                               workspace, out, gradOut, rows, T, -1.0f / Ts, 1.0f / Ts);
         int status = launch_status();
         if (status != SLAYER_OK) return status;
     }
