@@ -30,9 +30,9 @@ SHAPE = (12, 16, 34, 34, 300)
 HBM_PEAK_GBS = 8000.0                     # MI355X HBM3E, published
 # algorithmic bytes per neuron-timestep (fp32 tensors read + written once)
 AB = {"psp_conv": 8, "spike": 12, "shift": 8, "shift_bwd": 8, "spike_bwd": 12, "psp_corr": 8}
-KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, true, 16>", "spike": "slayer::spike_tile_kernel<12, true>",
+KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, ...> (conv)", "spike": "slayer::spike_tile_kernel<12, true>",
              "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
-             "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_tiled_kernel<false, true, 16>"}
+             "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_tiled_kernel<false, ...> (corr)"}
 
 
 def neuron_params():

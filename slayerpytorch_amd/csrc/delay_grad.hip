@@ -64,6 +64,8 @@ __global__ __launch_bounds__(256) void delay_grad_rows_kernel(float *__restrict_
     }
 }
 
+// Pass 2, few batch items: one lane per table entry adds the nBatch partials in batch order
+// (neighbouring lanes read neighbouring entries).
 __global__ __launch_bounds__(256) void delay_grad_batch_kernel(float *__restrict__ gradDelay,
                                                                const float *__restrict__ partial,
                                                                int64_t nBatch, int64_t nPerBatch, float Ts)
@@ -73,6 +75,22 @@ __global__ __launch_bounds__(256) void delay_grad_batch_kernel(float *__restrict
     float acc = 0.0f;
     for (int64_t b = 0; b < nBatch; ++b) acc += partial[b * nPerBatch + m];
     gradDelay[m] = acc * Ts;
+}
+
+// Pass 2, many batch items: one wavefront per table entry; lane l adds the partials of batch
+// items l, l+64, .. in order, then the 64 lane sums are combined in a fixed tree.
+__global__ __launch_bounds__(256) void delay_grad_batch_wave_kernel(float *__restrict__ gradDelay,
+                                                                    const float *__restrict__ partial,
+                                                                    int64_t nBatch, int64_t nPerBatch, float Ts)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t m = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
+    if (m >= nPerBatch) return;
+    float acc = 0.0f;
+    for (int64_t b = lane; b < nBatch; b += kWave) acc += partial[b * nPerBatch + m];
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) acc += __shfl_down(acc, off, kWave);
+    if (lane == 0) gradDelay[m] = acc * Ts;
 }
 
 }  // namespace slayer
@@ -110,7 +128,13 @@ extern "C" int slayer_delay_grad_f32(float *gradDelay, const float *out, const f
         if (status != SLAYER_OK) return status;
     }
     // with no samples to reduce (nBatch == 0 or T == 0) the loop below is empty and yields zeros
-    hipLaunchKernelGGL(delay_grad_batch_kernel, dim3(static_cast<unsigned>(outBlocks)), dim3(256), 0, st,
-                       gradDelay, workspace, (rows > 0 && T > 0) ? nBatch : 0, nPerBatch, Ts);
+    const int64_t batches = (rows > 0 && T > 0) ? nBatch : 0;
+    const int64_t waveBlocks = ceil_div(nPerBatch, 4);
+    if (batches >= 32 && waveBlocks < (1LL << 31))
+        hipLaunchKernelGGL(delay_grad_batch_wave_kernel, dim3(static_cast<unsigned>(waveBlocks)), dim3(256), 0, st,
+                           gradDelay, workspace, batches, nPerBatch, Ts);
+    else
+        hipLaunchKernelGGL(delay_grad_batch_kernel, dim3(static_cast<unsigned>(outBlocks)), dim3(256), 0, st,
+                           gradDelay, workspace, batches, nPerBatch, Ts);
     return launch_status();
 }
