@@ -252,8 +252,14 @@ __global__ __launch_bounds__(64) void loihi_tile_kernel(float *__restrict__ s, f
 // read and written as full, aligned lines (except at the two ends of a row); pieces that start
 // or end in the middle of a line make the memory system write that line twice, partially, which
 // measured about three times slower for the three output tensors.
+//
+// MERGE (needs LPP = 1 and rows of at least 64 samples): the memory line in which row r ends is
+// also the line in which row r+1 begins.  Stored by both rows it would be written twice,
+// partially, ten pieces apart.  Instead row r+1 keeps the results of its first line in
+// registers and hands them over when row r reaches that line, so that it goes out once, whole.
+// Only the first and the last row of a tile still write a partial line.
 // R rows per tile (= lanes that update), LPP = 128-byte lines per row and piece.
-template <int R, int LPP>
+template <int R, int LPP, bool MERGE>
 __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, float *__restrict__ v,
                                                          float *__restrict__ u, const float *__restrict__ w,
                                                          int64_t rows, int T, int64_t tiles, LoihiParams p)
@@ -273,8 +279,11 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
     const int col = (lane % QP) * 4;      // first column of this lane's vector
     const int pieces = (T + G - 1 + TC - 1) / TC;  // enough for the most skewed row
 
+    static_assert(!MERGE || (LPP == 1 && R == kWave), "line merging is written for one line per piece");
     LoihiState st = {0, 0, 0};
     float4 x[NB];
+    float headC[MERGE ? G : 1], headV[MERGE ? G : 1];  // results of this row's first line (MERGE)
+    uint32_t headFired = 0;
 
     auto rows_of = [&](int64_t t) { return static_cast<int>(min(static_cast<int64_t>(R), rows - t * R)); };
     // samples by which row r of tile t starts after a 128-byte boundary
@@ -365,6 +374,29 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
                     *reinterpret_cast<float4 *>(mineV + c0 + k) = make_float4(vol[k], vol[k + 1], vol[k + 2], vol[k + 3]);
                 }
                 masks[lane * LPP + g] = fired;
+                if (MERGE && j == 0) {
+#pragma unroll
+                    for (int k = 0; k < G; ++k) { headC[k] = cur[k]; headV[k] = vol[k]; }
+                    headFired = fired;
+                }
+            }
+            if (MERGE && j > 0) {
+                // hand this row's first line over to the row above when that row reaches it
+                const int skew = (o0 + lane * T) & 31;             // samples of that line owned by the row above
+                const int skewAbove = (o0 + (lane - 1) * T) & 31;
+                const int lastAbove = (T - 1 + skewAbove) >> 5;    // piece in which the row above ends
+                if (lane > 0 && lane < nRows && skew > 0 && j == lastAbove) {
+                    float *aboveC = tileC + (lane - 1) * P;
+                    float *aboveV = tileV + (lane - 1) * P;
+#pragma unroll
+                    for (int k = 0; k < G; k += 4) {
+                        if (k >= skew) {
+                            *reinterpret_cast<float4 *>(aboveC + k) = make_float4(headC[k], headC[k + 1], headC[k + 2], headC[k + 3]);
+                            *reinterpret_cast<float4 *>(aboveV + k) = make_float4(headV[k], headV[k + 1], headV[k + 2], headV[k + 3]);
+                        }
+                    }
+                    masks[lane - 1] |= headFired;
+                }
             }
         }
         wave_sync();
@@ -378,8 +410,16 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const int r = b * RPI + subRow;
-                const int time = TC * j - ((o0 + r * T) & 31) + col;
-                const int off = masked_offset(r < nRows && time >= 0 && time < T, (r * T + time) * 4);
+                const int skew = (o0 + r * T) & 31;
+                const int time = TC * j - skew + col;
+                bool ok = r < nRows && time >= 0 && time < T;
+                if (MERGE) {
+                    // a row's first line, when shared, goes out with the last line of the row above ..
+                    if (j == 0 && r > 0 && skew > 0) ok = false;
+                    // .. whose last line therefore extends into the row below
+                    if (r + 1 < nRows && time >= T && j == ((T - 1 + skew) >> 5)) ok = true;
+                }
+                const int off = masked_offset(ok, (r * T + time) * 4);
                 const uint32_t m = masks[r * LPP + (col >> 5)] >> (col & 31);
                 buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + r * P + col));
                 buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + r * P + col));
@@ -438,8 +478,13 @@ extern "C" int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const f
             const int64_t lineTiles = ceil_div(nNeurons, kR);
             const int64_t ldsBytes = (2LL * kR * (32 * kLpp + 4) + kR * kLpp) * 4;
             const int64_t fit = static_cast<int64_t>(compute_units()) * (160 * 1024 / ldsBytes);
-            hipLaunchKernelGGL((loihi_lines_kernel<kR, kLpp>), dim3(static_cast<unsigned>(lineTiles < fit ? lineTiles : fit)),
-                               dim3(kWave), 0, st, s, v, u, w, nNeurons, static_cast<int>(T), lineTiles, p);
+            const dim3 grid(static_cast<unsigned>(lineTiles < fit ? lineTiles : fit));
+            if (kLpp == 1 && kR == kWave && T >= 64)
+                hipLaunchKernelGGL((loihi_lines_kernel<kR, kLpp, kLpp == 1 && kR == kWave>), grid, dim3(kWave), 0, st, s, v,
+                                   u, w, nNeurons, static_cast<int>(T), lineTiles, p);
+            else
+                hipLaunchKernelGGL((loihi_lines_kernel<kR, kLpp, false>), grid, dim3(kWave), 0, st, s, v, u, w, nNeurons,
+                                   static_cast<int>(T), lineTiles, p);
             return launch_status();
         }
         if (vec)

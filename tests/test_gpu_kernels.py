@@ -109,6 +109,31 @@ def test_fir_sparse_spike_input_and_alpha_kernel(impl):
     assert np.array_equal(bits(got), bits(O.conv(x, f, 1.0)))
 
 
+@pytest.mark.parametrize("T,Fl", [(300, 77), (64, 8), (300, 129), (300, 130), (350, 77), (2000, 8), (436, 9), (440, 9),
+                                  (96, 1), (128, 128)])
+@pytest.mark.parametrize("op", ["conv", "corr"])
+def test_fir_sparse_input_edges(impl, T, Fl, op):
+    # almost-all-zero rows take the event-driven path (up to 129 taps, LDS rows up to 448 samples):
+    # events at both ends of a row, in neighbouring samples, negative zeros, an infinite sample
+    rng = np.random.default_rng(T + Fl)
+    x = np.zeros((3, 41, T), np.float32)
+    x[:, :, 0] = 1.0
+    x[:, :, T - 1] = -2.0
+    x[0, :, T // 2: T // 2 + 3] = 0.5
+    x[1, :, 1] = -0.0
+    x[2, 5, T // 3] = np.inf
+    idx = rng.integers(0, T, size=(3, 41, 2))
+    np.put_along_axis(x, idx, rng.standard_normal((3, 41, 2)).astype(np.float32), axis=2)
+    f = (rng.random(Fl) + 0.5).astype(np.float32)
+    got = host(getattr(slayerCuda, op)(dev(x), dev(f), 0.5))
+    want = getattr(O, op)(x, f, 0.5, fused=True)
+    assert np.array_equal(bits(got), bits(want))
+    # the same rows with a dense row block mixed in (the choice of path is per tile)
+    x[1] = rng.standard_normal((41, T)).astype(np.float32)
+    got = host(getattr(slayerCuda, op)(dev(x), dev(f), 0.5))
+    assert np.array_equal(bits(got), bits(getattr(O, op)(x, f, 0.5, fused=True)))
+
+
 def test_fir_is_left_padded_conv3d(impl):
     # the identity the reference's test_slayer011 asserts: psp == pspLayer, ||diff|| / numel < 1e-6
     rng = np.random.default_rng(6)
@@ -244,6 +269,30 @@ def test_loihi_parameters_wraparound_and_truncation(impl, params):
     got = slayerLoihiCuda.getSpikes(dev(w), *params)
     for a, b, name in zip(got, want, ("spike", "voltage", "current")):
         assert np.array_equal(bits(host(a)), bits(b)), name
+
+
+@pytest.mark.parametrize("T", [64, 68, 72, 100, 124, 128, 132, 196, 300, 332])
+@pytest.mark.parametrize("rows", [(1, 1), (3, 67), (2, 64), (5, 13)])
+def test_loihi_rows_sharing_memory_lines(impl, T, rows):
+    # rows that are whole 16-byte vectors but start and end inside 128-byte memory lines: the line
+    # shared by two neighbouring rows is written once, from the results of both
+    rng = np.random.default_rng(T)
+    w = loihi_input(rng, rows + (T,), p=0.3)
+    want = O.loihi_get_spikes(w, 0, 20 * 64, 1024, 128, 2)
+    got = slayerLoihiCuda.getSpikes(dev(w), 0, 20 * 64, 1024, 128, 2)
+    for a, b, name in zip(got, want, ("spike", "voltage", "current")):
+        assert np.array_equal(bits(host(a)), bits(b)), name
+    assert want[0].sum() > 0
+
+
+def test_loihi_unaligned_tensors_take_the_general_kernel():
+    rng = np.random.default_rng(77)
+    w = loihi_input(rng, (2 * 40 * 96 + 1,), p=0.3)
+    wt = dev(w)[1:].reshape(2, 40, 96)                       # 4-byte aligned storage only
+    want = O.loihi_get_spikes(w[1:].reshape(2, 40, 96), 0, 20 * 64, 1024, 128, 1)
+    got = slayerLoihiCuda.getSpikes(wt, 0, 20 * 64, 1024, 128, 1)
+    for a, b in zip(got, want):
+        assert np.array_equal(host(a), b)
 
 
 # ------------------------------------------------------------------------------------------ empty tensors
