@@ -135,10 +135,10 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
 }
 
 // ---- row-tile kernel (nuSize <= NU) --------------------------------------------------------------------
-// The fast path.  A wavefront owns kTileRows consecutive rows and moves them through LDS in
+// The fast path.  A wavefront owns R consecutive rows and moves them through LDS in
 // pieces of Tc samples per row (the whole row when it is short enough), so that global memory
 // is read and written as long contiguous runs with 16-byte accesses per lane - the access
-// pattern of a plain copy.  Lanes 0..kTileRows-1 then walk their row in LDS order:
+// pattern of a plain copy.  Lanes 0..R-1 then walk their row in LDS order:
 // 32 samples at a time are pulled into a register window v[0 .. 32+LAG), a spike adds
 // nu[0..NU) onto v[k .. k+NU) (the same fp32 additions, in the same order, as the sequential
 // loop), and the 32 oldest samples go back to LDS together with a 32-bit spike mask.  The last
@@ -147,22 +147,25 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
 // after the last sample hold NaN, which never reaches the threshold.
 // Leaving most lanes idle during the walk is deliberate: the kernel is bound by HBM traffic,
 // not by the vector ALU, and short tiles keep many wavefronts (and bytes) in flight per CU.
-constexpr int kTileRows = 16;
 constexpr int kTileMaxPiece = 352;  // longest piece (samples per row) a tile stages at once
 
-template <int NU, bool VEC>
+// LAG: look-ahead of the walk in samples (>= NU - 1, whole 16-byte vectors).  The samples that
+// leave a piece are the ones LAG before its end, so with several pieces per row LAG = 32 keeps
+// every run of stores on 128-byte boundaries of the row (partial lines are expensive to write).
+// R: rows per tile (16, or 8 when the tensor has too few rows to fill the GPU with 16-row tiles).
+template <int NU, bool VEC, int LAG, int R>
 __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, float *u,
                                                         const float *__restrict__ nu, int64_t rows,
                                                         int T, int nuSize, int Tc, int P, int MP,
                                                         int64_t tiles, float theta, float Ts)
 {
-    constexpr int LAG = (NU + 2) & ~3;  // look-ahead of the walk, rounded to whole 16-byte vectors
+    static_assert(LAG >= NU - 1 && LAG % 4 == 0, "the window must cover the refractory kernel");
     constexpr int G = 32;               // samples per walk group = bits of a spike mask
     constexpr int V = VEC ? 4 : 1;      // samples per global access
-    constexpr int NB = kTileRows * kTileMaxPiece / V / kWave;  // accesses per lane per piece, at most
+    constexpr int NB = R * kTileMaxPiece / V / kWave;  // accesses per lane per piece, at most
     extern __shared__ __align__(16) float lds[];
-    float *tile = lds;                                                    // [kTileRows][P], P = 4 (mod 32)
-    uint32_t *masks = reinterpret_cast<uint32_t *>(lds + kTileRows * P);  // [kTileRows][MP]
+    float *tile = lds;                                                    // [R][P], P = 4 (mod 32)
+    uint32_t *masks = reinterpret_cast<uint32_t *>(lds + R * P);  // [R][MP]
 
     const int lane = threadIdx.x;
     const float amplitude = 1.0f / Ts;
@@ -177,9 +180,9 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     // A "step" is one piece of one tile.  The global loads of a step are issued one step ahead
     // into x[] and stay in flight while the previous step is walked and retired.
     float x[NB * V];
-    auto rows_of = [&](int64_t t) { return static_cast<int>(min(static_cast<int64_t>(kTileRows), rows - t * kTileRows)); };
+    auto rows_of = [&](int64_t t) { return static_cast<int>(min(static_cast<int64_t>(R), rows - t * R)); };
     auto issue = [&](int64_t t, int tL) {
-        const BufferRsrc bufU = make_buffer(u + t * kTileRows * static_cast<int64_t>(T));
+        const BufferRsrc bufU = make_buffer(u + t * R * static_cast<int64_t>(T));
         const int n = min(Tc, T - tL);
         const int perRow = n / V;
         const int total = rows_of(t) * perRow;
@@ -237,7 +240,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 
         // ---- walk: lane = row.  Columns [0, W) become final in this step.
         const int W = last ? n + LAG : n;
-        if (lane < kTileRows) {
+        if (lane < R) {
             float *mine = tile + lane * P;
             if (tL == 0) {
 #pragma unroll
@@ -277,8 +280,8 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 
         // ---- retire: columns [first, W) leave as u' and s, times tW + column
         {
-            const BufferRsrc bufU = make_buffer(u + t * kTileRows * static_cast<int64_t>(T));
-            const BufferRsrc bufS = make_buffer(s + t * kTileRows * static_cast<int64_t>(T));
+            const BufferRsrc bufU = make_buffer(u + t * R * static_cast<int64_t>(T));
+            const BufferRsrc bufS = make_buffer(s + t * R * static_cast<int64_t>(T));
             const int first = (tL == 0) ? LAG : 0;  // before the first sample there is nothing to store
             const int perRow = (W - first) / V;
             const int total = nRows * perRow;
@@ -358,26 +361,38 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
     const int64_t groups = ceil_div(nNeurons, kWave);
     const bool stream_ok = !generic_forced() && T < (1LL << 30) && groups < (1LL << 31);
     const bool window_ok = stream_ok && T <= kBufferMaxT;
-#define SLAYER_SPIKE_TILE(NU)                                                                             \
+#define SLAYER_SPIKE_TILE_LAUNCH(NU, LAGV, RV)                                                           \
     do {                                                                                                \
-        constexpr int lag = (NU + 2) & ~3;                                                              \
-        const int cols = (lag + Tc + 31) & ~31; /* the walk goes in groups of 32 columns */             \
-        const int P = cols + 4; /* 4 (mod 32): rows are 16-byte aligned and start in different banks */ \
-        const int MP = cols / 32 + 1;                                                                   \
-        const size_t lds = (static_cast<size_t>(kTileRows) * P + kTileRows * MP) * sizeof(float);       \
-        const int64_t resident = static_cast<int64_t>(cus) * (160 * 1024 / static_cast<int64_t>(lds));  \
-        const unsigned grid = static_cast<unsigned>(tiles < resident ? tiles : resident);               \
         if (vec)                                                                                        \
-            hipLaunchKernelGGL((spike_tile_kernel<NU, true>), dim3(grid), dim3(kWave), lds, st, s, u,   \
-                               nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize), Tc, P, MP,  \
-                               tiles, theta, Ts);                                                       \
+            hipLaunchKernelGGL((spike_tile_kernel<NU, true, LAGV, RV>), dim3(grid), dim3(kWave), lds,   \
+                               st, s, u, nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize),   \
+                               Tc, P, MP, tiles, theta, Ts);                                            \
         else                                                                                            \
-            hipLaunchKernelGGL((spike_tile_kernel<NU, false>), dim3(grid), dim3(kWave), lds, st, s, u,  \
-                               nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize), Tc, P, MP,  \
-                               tiles, theta, Ts);                                                       \
+            hipLaunchKernelGGL((spike_tile_kernel<NU, false, LAGV, RV>), dim3(grid), dim3(kWave), lds,  \
+                               st, s, u, nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize),   \
+                               Tc, P, MP, tiles, theta, Ts);                                            \
         return launch_status();                                                                         \
     } while (0)
-    const int64_t tiles = ceil_div(nNeurons, kTileRows);
+#define SLAYER_SPIKE_TILE_LAG(NU, LAGV)                                                                  \
+    do {                                                                                                \
+        const int cols = (LAGV + Tc + 31) & ~31; /* the walk goes in groups of 32 columns */            \
+        const int P = cols + 4; /* 4 (mod 32): rows are 16-byte aligned and start in different banks */ \
+        const int MP = cols / 32 + 1;                                                                   \
+        /* 16 rows per tile unless that leaves wavefront slots of the GPU empty */                      \
+        const int64_t slots16 = static_cast<int64_t>(cus) * (160 * 1024 / ((16LL * P + 16 * MP) * 4));  \
+        const int rowsPerTile = ceil_div(nNeurons, 16) >= slots16 ? 16 : 8;                             \
+        const size_t lds = (static_cast<size_t>(rowsPerTile) * P + rowsPerTile * MP) * sizeof(float);   \
+        const int64_t tiles = ceil_div(nNeurons, rowsPerTile);                                          \
+        const int64_t resident = static_cast<int64_t>(cus) * (160 * 1024 / static_cast<int64_t>(lds));  \
+        const unsigned grid = static_cast<unsigned>(tiles < resident ? tiles : resident);               \
+        if (rowsPerTile == 16) SLAYER_SPIKE_TILE_LAUNCH(NU, LAGV, 16);                                  \
+        SLAYER_SPIKE_TILE_LAUNCH(NU, LAGV, 8);                                                          \
+    } while (0)
+#define SLAYER_SPIKE_TILE(NU)                                                                            \
+    do {                                                                                                \
+        if (T <= kTileMaxPiece) SLAYER_SPIKE_TILE_LAG(NU, ((NU + 2) & ~3));                             \
+        SLAYER_SPIKE_TILE_LAG(NU, 32);                                                                  \
+    } while (0)
     if (window_ok && nuSize <= 24) {
         // short rows travel whole; long rows in pieces of 256 samples (1 KiB per row)
         const int Tc = (T <= kTileMaxPiece) ? static_cast<int>(T) : 256;
@@ -390,6 +405,8 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
         SLAYER_SPIKE_TILE(24);
     }
 #undef SLAYER_SPIKE_TILE
+#undef SLAYER_SPIKE_TILE_LAG
+#undef SLAYER_SPIKE_TILE_LAUNCH
     if (stream_ok && nuSize <= 33) {
         hipLaunchKernelGGL(spike_stream_kernel<64>, dim3(static_cast<unsigned>(groups)), dim3(kWave), 0,
                            st, s, u, nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize), theta,
