@@ -378,24 +378,29 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
         const int cols = (LAGV + Tc + 31) & ~31; /* the walk goes in groups of 32 columns */            \
         const int P = cols + 4; /* 4 (mod 32): rows are 16-byte aligned and start in different banks */ \
         const int MP = cols / 32 + 1;                                                                   \
-        /* 16 rows per tile unless that leaves wavefront slots of the GPU empty */                      \
+        /* Rows that travel whole: 8-row tiles, one work-group per tile - many short-lived groups per   \
+           CU overlap the memory phases of some with the walks of others better than a loop does.       \
+           Rows in pieces: the group loops over the pieces; 16 rows per tile unless that would leave    \
+           wavefront slots of the GPU empty. */                                                         \
         const int64_t slots16 = static_cast<int64_t>(cus) * (160 * 1024 / ((16LL * P + 16 * MP) * 4));  \
-        const int rowsPerTile = ceil_div(nNeurons, 16) >= slots16 ? 16 : 8;                             \
+        const int rowsPerTile = (!whole && ceil_div(nNeurons, 16) >= slots16) ? 16 : 8;                 \
         const size_t lds = (static_cast<size_t>(rowsPerTile) * P + rowsPerTile * MP) * sizeof(float);   \
         const int64_t tiles = ceil_div(nNeurons, rowsPerTile);                                          \
         const int64_t resident = static_cast<int64_t>(cus) * (160 * 1024 / static_cast<int64_t>(lds));  \
-        const unsigned grid = static_cast<unsigned>(tiles < resident ? tiles : resident);               \
+        if (tiles >= (1LL << 31)) return SLAYER_EUNSUPPORTED;                                           \
+        const unsigned grid = static_cast<unsigned>((whole || tiles < resident) ? tiles : resident);    \
         if (rowsPerTile == 16) SLAYER_SPIKE_TILE_LAUNCH(NU, LAGV, 16);                                  \
         SLAYER_SPIKE_TILE_LAUNCH(NU, LAGV, 8);                                                          \
     } while (0)
 #define SLAYER_SPIKE_TILE(NU)                                                                            \
     do {                                                                                                \
-        if (T <= kTileMaxPiece) SLAYER_SPIKE_TILE_LAG(NU, ((NU + 2) & ~3));                             \
+        if (whole) SLAYER_SPIKE_TILE_LAG(NU, ((NU + 2) & ~3));                                          \
         SLAYER_SPIKE_TILE_LAG(NU, 32);                                                                  \
     } while (0)
     if (window_ok && nuSize <= 24) {
         // short rows travel whole; long rows in pieces of 256 samples (1 KiB per row)
-        const int Tc = (T <= kTileMaxPiece) ? static_cast<int>(T) : 256;
+        const bool whole = T <= kTileMaxPiece;
+        const int Tc = whole ? static_cast<int>(T) : 256;
         const bool vec = (T % 4 == 0) && aligned16(s) && aligned16(u);
         const int cus = compute_units();
         if (nuSize <= 4) SLAYER_SPIKE_TILE(4);
