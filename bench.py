@@ -11,8 +11,9 @@ One step = one pass of the hot path over one batch of synthetic input, forward a
 on the NMNIST-CNN-shaped activation tensor (12, 16, 34, 34, 300), fp32, all inputs resident in
 HBM.  The spike kernel updates its input in place, so each step works on its own pre-made copy
 of the membrane potential (made before the timed region).  Prints ONE JSON line:
-neuron-timesteps/s of the chain, the HBM roofline of the dominant kernel (HIP-event timing on
-the launch stream) and the CPU oracle timed on the host cores beside it.
+neuron-timesteps/s of the chain, the HBM roofline of the dominant kernel (HIP events around its
+launches inside the timed region, on the launch stream) and the CPU oracle timed on the host
+cores beside it.
 """
 import argparse
 import json
@@ -30,7 +31,12 @@ SHAPE = (12, 16, 34, 34, 300)
 HBM_PEAK_GBS = 8000.0                     # MI355X HBM3E, published
 # algorithmic bytes per neuron-timestep (fp32 tensors read + written once)
 AB = {"psp_conv": 8, "spike": 12, "shift": 8, "shift_bwd": 8, "spike_bwd": 12, "psp_corr": 8}
-KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, ...> (conv)", "spike": "slayer::spike_tile_kernel<12, true>",
+# HBM bytes per launch on SHAPE measured with the FETCH_SIZE and WRITE_SIZE hardware counters
+# (rocprofv3 --pmc, one counter per run, scaled by the reading of a plain copy of known size);
+# the figures and the commands are in profiles/hbm_traffic_counters.txt
+TRAFFIC_BYTES = {"psp_conv": 536.9e6, "spike": 798.8e6, "shift": 540.8e6, "shift_bwd": 540.8e6, "spike_bwd": 798.7e6,
+                 "psp_corr": 542.4e6}
+KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, ...> (conv)", "spike": "slayer::spike_tile_kernel<12, true, 12, 8>",
              "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
              "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_tiled_kernel<false, ...> (corr)"}
 
@@ -63,7 +69,8 @@ def cpu_baseline(shape, srm, ref, params, rows_fraction=1):
     grad = rng.standard_normal(sub).astype(np.float32)
     theta, tau, scale = params["theta"], params["tauRho"] * params["theta"], params["scaleRho"]
     times = []
-    for _ in range(3):
+    began = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - began < 10.0 and len(times) < 200):   # about 10 s of CPU work
         t0 = time.perf_counter()
         O.conv(spikes, srm, 1.0)
         s, u = O.get_spikes(u0, ref, theta, 1.0)
@@ -75,8 +82,8 @@ def cpu_baseline(shape, srm, ref, params, rows_fraction=1):
     best = sorted(times)[len(times) // 2]
     O.set_threads(1)
     return {"value": spikes.size / best, "unit": "neuron-timesteps/s", "cores": threads, "kind": "port",
-            "sample": "oracle chain (conv77+spike+shift, shift+spike_bwd+corr77) on %s, median of 3, %.2f s"
-                      % (str(sub), best)}
+            "sample": "oracle chain (conv77+spike+shift, shift+spike_bwd+corr77) on %s, median of %d passes, %.2f s each"
+                      % (str(sub), len(times), best)}
 
 
 def flip_rate(device, srm_t, ref_t, params):
@@ -160,6 +167,12 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--chain-only", action="store_true",
+                    help="only the headline chain (for profiler runs): no per-kernel pass, flip rate, "
+                         "other rows or CPU baseline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one plain copy of known size (a zero-delay shift of half the tensor: "
+                         "%d bytes read, as many written) to scale hardware counters by" % (4 * 6 * 16 * 34 * 34 * 300))
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every kernel on this path treats neuron rows independently, "
@@ -181,20 +194,21 @@ def main():
 
     spikes, u0, grad = make_inputs(SHAPE, device)
     numel = spikes.numel()
-    total = args.steps + args.warmup
-    pool = [u0.clone() for _ in range(total)]          # spike() consumes one copy per step
     names = list(AB)
-    events = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in names]
-              for _ in range(args.steps)]
+    probe = 0 if args.chain_only else max(args.steps, 1)   # untimed steps with an event pair around every launch
+    pool = [u0.clone() for _ in range(args.warmup + probe + args.steps)]   # spike() consumes one copy per step
 
-    def step(i, ev=None):
-        u = pool[i]
+    def event_pair():
+        return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
+    def step(u, ev=None):
+        """ev: {op index: (start, stop)} - the launches to bracket with HIP events (torch records
+        them on the current stream, which is the stream the kernels are launched on)."""
         def run(k, fn):
-            if ev is not None:
+            if ev is not None and k in ev:
                 ev[k][0].record()
             out = fn()
-            if ev is not None:
+            if ev is not None and k in ev:
                 ev[k][1].record()
             return out
 
@@ -206,20 +220,37 @@ def main():
         run(5, lambda: slayerCuda.corr(gs, srm_t, 1.0))
 
     for i in range(args.warmup):
-        step(i)
+        step(pool[i])
+    if args.copy_calibration:
+        slayerCuda.shift(grad[:6], 0.0, 1.0)
+    torch.cuda.synchronize()
+
+    # Per-kernel pass (untimed): every launch bracketed.  The event records themselves cost a few
+    # microseconds per launch, so the timed region below brackets the dominant kernel only.
+    per_kernel_ms = None
+    dominant = "psp_corr"
+    if probe:
+        evs = [{k: event_pair() for k in range(len(names))} for _ in range(probe)]
+        for i in range(probe):
+            step(pool[args.warmup + i], evs[i])
+        torch.cuda.synchronize()
+        per_kernel_ms = {n: float(np.mean([evs[i][k][0].elapsed_time(evs[i][k][1]) for i in range(probe)]))
+                         for k, n in enumerate(names)}
+        dominant = max(per_kernel_ms, key=per_kernel_ms.get)
+    kd = names.index(dominant)
+
+    evs = [{kd: event_pair()} for _ in range(args.steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(args.warmup + i, events[i])
+        step(pool[args.warmup + probe + i], evs[i])
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
     ms_per_step = elapsed / args.steps * 1e3
-    per_kernel_ms = {n: float(np.mean([events[i][k][0].elapsed_time(events[i][k][1]) for i in range(args.steps)]))
-                     for k, n in enumerate(names)}
-    dominant = max(per_kernel_ms, key=per_kernel_ms.get)
-    achieved = AB[dominant] * numel / (per_kernel_ms[dominant] * 1e-3) / 1e9
-    chain_gbs = sum(AB.values()) * numel / (sum(per_kernel_ms.values()) * 1e-3) / 1e9
+    dominant_ms = float(np.mean([evs[i][kd][0].elapsed_time(evs[i][kd][1]) for i in range(args.steps)]))
+    achieved = AB[dominant] * numel / (dominant_ms * 1e-3) / 1e9
+    chain_gbs = sum(AB.values()) * numel / (elapsed / args.steps) / 1e9
 
     result = {
         "metric": "neuron-timesteps/s spike+psp+shift fwd/bwd at 1 MI355X; % HBM peak GB/s",
@@ -231,18 +262,25 @@ def main():
                                "(11-tap refractory) + shift fwd, shift + spike pdf + psp corr bwd",
                    "elements": numel, "algorithmic_bytes_per_element": sum(AB.values())},
         "roofline": {"bound": "hbm", "kernel": KERNEL_OF[dominant], "op": dominant, "achieved": achieved,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None},
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "launch_ms": dominant_ms,
+                     "traffic": TRAFFIC_BYTES.get(dominant)},
+        # the whole step (six launches and the gaps between them) against the HBM peak
         "chain_hbm_frac": chain_gbs / HBM_PEAK_GBS,
-        "per_kernel_ms": per_kernel_ms,
-        "per_kernel_hbm_frac": {n: AB[n] * numel / (per_kernel_ms[n] * 1e-3) / 1e9 / HBM_PEAK_GBS for n in names},
     }
+    if per_kernel_ms is not None:
+        result["per_kernel_ms"] = per_kernel_ms
+        result["per_kernel_hbm_frac"] = {n: AB[n] * numel / (per_kernel_ms[n] * 1e-3) / 1e9 / HBM_PEAK_GBS
+                                         for n in names}
+        result["per_kernel_pass"] = "%d untimed steps before the timed region, an event pair around every launch" % probe
     del pool
-    flips, rate = flip_rate(device, srm_t, ref_t, params)
-    result["spike_flip_rate"] = flips
-    result["spike_rate"] = rate
-    result["other_rows"] = other_rows(device)
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(SHAPE, srm, ref, params)
+    if not args.chain_only:
+        flips, rate = flip_rate(device, srm_t, ref_t, params)
+        result["spike_flip_rate"] = flips
+        result["spike_rate"] = rate
+        result["other_rows"] = other_rows(device)
+        if not args.no_cpu_baseline:
+            result["cpu_baseline"] = cpu_baseline(SHAPE, srm, ref, params)
     print(json.dumps(result))
 
 
