@@ -19,7 +19,7 @@
 #include "common.h"
 
 #ifndef LOIHI_ROWS
-#define LOIHI_ROWS 64
+#define LOIHI_ROWS 32
 #define LOIHI_LPP 1
 #endif
 #define LOIHI_PIECE 64
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
     const int col = (lane % QP) * 4;      // first column of this lane's vector
     const int pieces = (T + G - 1 + TC - 1) / TC;  // enough for the most skewed row
 
-    static_assert(!MERGE || (LPP == 1 && R == kWave), "line merging is written for one line per piece");
+    static_assert(!MERGE || (LPP == 1 && R <= kWave), "line merging is written for one line per piece");
     LoihiState st = {0, 0, 0};
     float4 x[NB];
     float headC[MERGE ? G : 1], headV[MERGE ? G : 1];  // results of this row's first line (MERGE)
@@ -479,8 +479,8 @@ extern "C" int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const f
             const int64_t ldsBytes = (2LL * kR * (32 * kLpp + 4) + kR * kLpp) * 4;
             const int64_t fit = static_cast<int64_t>(compute_units()) * (160 * 1024 / ldsBytes);
             const dim3 grid(static_cast<unsigned>(lineTiles < fit ? lineTiles : fit));
-            if (kLpp == 1 && kR == kWave && T >= 64)
-                hipLaunchKernelGGL((loihi_lines_kernel<kR, kLpp, kLpp == 1 && kR == kWave>), grid, dim3(kWave), 0, st, s, v,
+            if (kLpp == 1 && T >= 64)
+                hipLaunchKernelGGL((loihi_lines_kernel<kR, kLpp, kLpp == 1>), grid, dim3(kWave), 0, st, s, v,
                                    u, w, nNeurons, static_cast<int>(T), lineTiles, p);
             else
                 hipLaunchKernelGGL((loihi_lines_kernel<kR, kLpp, false>), grid, dim3(kWave), 0, st, s, v, u, w, nNeurons,
