@@ -7,16 +7,20 @@
 // then one multiply by Ts, exactly like the sequential loop; samples outside [0,T) enter as
 // zeros, which leaves the chain's value unchanged.
 //
-// Tiled kernel.  The convolution is the correlation on a reversed time axis, so both share one
-// core: Y[m] = sum_i X[m+i] * filt[i].  A work-group of 256 lanes owns R consecutive neuron
-// rows and one time tile; it stages the rows' samples (plus the F-1 sample halo, zero padded)
-// into LDS as X[R][LD] with 16-byte loads (reversed in time for the convolution).  The tile is
-// then cut into chunks of 8 consecutive outputs of one row; lanes take chunks in row-major
-// order, so neighbouring lanes produce neighbouring outputs and the results leave as 16-byte
-// stores.  A lane keeps a 12-sample register window of X and slides it 4 samples per 4 taps
-// with one 16-byte LDS read, i.e. one LDS read feeds 32 FMAs.  Filter taps are wave-uniform
-// and come through scalar loads.  An FIR with F = 77 taps needs 154 flop per 8 bytes moved,
-// which is at the FP32 ridge of the machine: the kernel is meant to be FMA-issue bound.
+// Three kernels share that definition:
+//  * direct: rows of whole 16-byte vectors and filters of at most 33 taps (81 for the
+//    correlation): everything in registers, addressing of a plain copy;
+//  * tiled: the convolution is the correlation on a reversed time axis, so both share one core
+//    Y[m] = sum_i X[m+i] * filt[i].  A work-group of 256 lanes owns R consecutive neuron rows
+//    and one time tile; it stages the rows' samples (plus the F-1 sample halo, zero padded) into
+//    LDS as X[R][LD] with 16-byte loads (reversed in time for the convolution).  Dense tiles are
+//    cut into chunks of U (8 or 16) consecutive outputs of one row; lanes take chunks in row-major
+//    order, keep a (U+4)-sample register window of X and slide it 4 samples per 4 taps with one
+//    16-byte LDS read, i.e. one LDS read feeds 4 U FMAs; filter taps are wave-uniform and come
+//    through scalar loads.  Tiles whose input is almost all zeros (spike trains) take an
+//    event-driven path instead.  An FIR with F = 77 taps needs 154 flop per 8 bytes moved, which
+//    is at the FP32 ridge of the machine: on dense input the kernel is FMA-issue bound;
+//  * generic: one lane per output, any shape.
 #include "common.h"
 
 namespace slayer {
@@ -45,6 +49,84 @@ __global__ __launch_bounds__(256) void fir_generic_kernel(float *__restrict__ ou
         }
         out[row * T + t] = acc * Ts;
     }
+}
+
+// ---- direct kernel: rows of whole 16-byte vectors, everything in registers -----------------------------
+// Lane g of the grid owns a chunk of U consecutive outputs of one row (U/4 aligned 16-byte
+// vectors), reads the NV aligned input vectors that hold its U + F - 1 samples straight from
+// global memory (neighbouring lanes share them through the caches), runs the U tap chains in
+// registers and streams its results out.  No LDS, no barriers; the addressing is that of a plain
+// copy.  NV >= (F - 1 + U) / 4.
+template <bool CAUSAL, int NV, int U>
+__global__ __launch_bounds__(256) void fir_direct_kernel(float *__restrict__ out, const float *__restrict__ in,
+                                                         const float *__restrict__ filt, uint32_t chunks, int T,
+                                                         int F, FastDiv byRow, float Ts)
+{
+    constexpr int UV = U / 4;
+    const int perRow = T >> 2;                    // vectors per row
+    const int chunksPerRow = (perRow + UV - 1) / UV;
+    const uint32_t g0 = blockIdx.x * 256u;
+    const uint32_t g = g0 + threadIdx.x;
+    const bool active = g < chunks;
+    const uint32_t rowBase = fastdiv(g0, byRow);  // wave-uniform: addressing is relative to this row
+    const uint32_t row = fastdiv(active ? g : g0, byRow);
+    const int c = static_cast<int>((active ? g : g0) - row * static_cast<uint32_t>(chunksPerRow));
+    const int r = static_cast<int>(row - rowBase);
+    const BufferRsrc bufIn = make_buffer(in + static_cast<int64_t>(rowBase) * T);
+    const BufferRsrc bufOut = make_buffer(out + static_cast<int64_t>(rowBase) * T);
+
+    // window w[k] = sample 4 * first + k of the row, zero outside the row
+    const int first = CAUSAL ? UV * c + UV - NV : UV * c;
+    float w[4 * NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int qv = first + v;
+        const float4 x = buffer_load4<0>(bufIn, masked_offset(active && qv >= 0 && qv < perRow, (r * T + (qv << 2)) * 4), 0);
+        w[4 * v] = x.x; w[4 * v + 1] = x.y; w[4 * v + 2] = x.z; w[4 * v + 3] = x.w;
+    }
+    // all loads are issued before the first tap: keep them from sinking into the tap blocks
+#pragma unroll
+    for (int k = 0; k < 4 * NV; ++k) asm volatile("" : "+v"(w[k]));
+
+    float acc[U];
+#pragma unroll
+    for (int e = 0; e < U; ++e) acc[e] = 0.0f;
+    constexpr int FMAX = 4 * NV - U + 1;          // longest filter this window serves
+    constexpr int B = 8;                          // taps per block
+#pragma unroll
+    for (int ib = 0; ib < FMAX; ib += B) {
+        if (ib + B <= F) {
+            float f[B];
+#pragma unroll
+            for (int k = 0; k < B; ++k) f[k] = filt[ib + k];
+#pragma unroll
+            for (int k = 0; k < B; ++k) {
+                const int i = ib + k;
+                if (i < FMAX) {
+#pragma unroll
+                    for (int e = 0; e < U; ++e)
+                        acc[e] = __builtin_fmaf(CAUSAL ? w[4 * NV - U + e - i] : w[e + i], f[k], acc[e]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < B; ++k) {
+                const int i = ib + k;
+                if (i < FMAX && i < F) {
+                    const float fi = filt[i];
+#pragma unroll
+                    for (int e = 0; e < U; ++e)
+                        acc[e] = __builtin_fmaf(CAUSAL ? w[4 * NV - U + e - i] : w[e + i], fi, acc[e]);
+                }
+            }
+        }
+    }
+    // with several vectors per lane one store instruction leaves gaps that the lane's next store
+    // fills: those go through the cache, which merges them into whole memory lines
+#pragma unroll
+    for (int v = 0; v < UV; ++v)
+        buffer_store4<(UV > 1 ? 0 : kStream)>(bufOut, masked_offset(active && UV * c + v < perRow, (r * T + ((UV * c + v) << 2)) * 4), 0,
+                      make_float4(acc[4 * v] * Ts, acc[4 * v + 1] * Ts, acc[4 * v + 2] * Ts, acc[4 * v + 3] * Ts));
 }
 
 // ---- tiled kernel ---------------------------------------------------------------------------------
@@ -416,9 +498,35 @@ static int launch_fir(float *out, const float *in, const float *filt, int64_t ro
     if (!out || !in || (F > 0 && !filt)) return SLAYER_EINVAL;
     if (T >= (1LL << 30)) return SLAYER_EUNSUPPORTED;
 
+    const bool vec = (T % 4 == 0) && aligned16(out) && aligned16(in);
+    // Register-only kernel: always for short filters (the op is then a stream); up to 81 taps for
+    // the correlation, whose input - a gradient - is dense, where it measures 6-9 % faster than
+    // the tiled kernel.  The convolution keeps the tiled kernel for longer filters because of its
+    // event-driven path for spike trains.
+    const int64_t directMax = CAUSAL ? 33 : 81;
+    if (!generic_forced() && vec && F >= 1 && F <= directMax && T < (1LL << 28) && rows * (T / 4) < (1LL << 32)) {
+        const int U = F <= 17 ? 4 : 8;
+        const int64_t chunksPerRow = ceil_div(T / 4, U / 4);
+        const int64_t chunks = rows * chunksPerRow;
+        const dim3 grid(static_cast<unsigned>(ceil_div(chunks, 256)));
+        const FastDiv byRow = make_fastdiv(static_cast<uint32_t>(chunksPerRow));
+#define SLAYER_FIR_DIRECT(NV, UU)                                                                                  \
+    hipLaunchKernelGGL((fir_direct_kernel<CAUSAL, NV, UU>), grid, dim3(256), 0, stream, out, in, filt,             \
+                       static_cast<uint32_t>(chunks), static_cast<int>(T), static_cast<int>(F), byRow, Ts)
+        if (F <= 5) SLAYER_FIR_DIRECT(2, 4);
+        else if (F <= 9) SLAYER_FIR_DIRECT(3, 4);
+        else if (F <= 13) SLAYER_FIR_DIRECT(4, 4);
+        else if (F <= 17) SLAYER_FIR_DIRECT(5, 4);
+        else if (F <= 25) SLAYER_FIR_DIRECT(8, 8);
+        else if (F <= 33) SLAYER_FIR_DIRECT(10, 8);
+        else if (F <= 49) SLAYER_FIR_DIRECT(14, 8);
+        else if (F <= 65) SLAYER_FIR_DIRECT(18, 8);
+        else SLAYER_FIR_DIRECT(22, 8);
+#undef SLAYER_FIR_DIRECT
+        return launch_status();
+    }
     FirPlan p;
     if (!generic_forced() && plan_fir(rows, T, F, p) && ceil_div(rows, p.R) < (1LL << 31)) {
-        const bool vec = (T % 4 == 0) && aligned16(out) && aligned16(in);
         if (vec && p.U == 16) launch_tiled<CAUSAL, true, 16>(p, out, in, filt, rows, T, F, Ts, stream);
         else if (vec) launch_tiled<CAUSAL, true, 8>(p, out, in, filt, rows, T, F, Ts, stream);
         else if (p.U == 16) launch_tiled<CAUSAL, false, 16>(p, out, in, filt, rows, T, F, Ts, stream);

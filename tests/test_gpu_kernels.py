@@ -101,6 +101,23 @@ def test_fir_matches_oracle(impl, rows, T, Fl, op):
     assert np.array_equal(bits(got), bits(want)), "not bit-identical to the fused-multiply-add chain"
 
 
+@pytest.mark.parametrize("Fl", [1, 5, 6, 9, 10, 13, 14, 17, 18, 25, 26, 33, 34, 49, 50, 65, 66, 77, 81, 82])
+@pytest.mark.parametrize("T", [4, 12, 44, 300])
+def test_fir_filter_lengths_around_kernel_choices(Fl, T):
+    # the register-only kernel serves filters up to 33 taps (convolution) / 81 taps (correlation)
+    # in windows of 2..22 vectors; rows whose vector count is odd end in a half-filled chunk;
+    # an infinite sample must reach exactly the outputs within Fl taps of it
+    rng = np.random.default_rng(Fl * 1000 + T)
+    x = rng.standard_normal((3, 37, T)).astype(np.float32)
+    x[1, 3, T // 2] = np.inf
+    f = rng.standard_normal(Fl).astype(np.float32)
+    for op in ("conv", "corr"):
+        got = host(getattr(slayerCuda, op)(dev(x), dev(f), 0.5))
+        want = getattr(O, op)(x, f, 0.5, fused=True)
+        assert np.array_equal(np.isnan(got), np.isnan(want)), (op, Fl, T)
+        assert np.array_equal(np.where(np.isnan(got), 0, bits(got)), np.where(np.isnan(want), 0, bits(want))), (op, Fl, T)
+
+
 def test_fir_sparse_spike_input_and_alpha_kernel(impl):
     rng = np.random.default_rng(5)
     x = (rng.random((4, 2, 34, 34, 300)) < 0.02).astype(np.float32)
