@@ -29,6 +29,8 @@ sys.path.insert(0, ROOT)
 
 SHAPE = (12, 16, 34, 34, 300)
 HBM_PEAK_GBS = 8000.0                     # MI355X HBM3E, published
+FP32_PEAK_TFLOPS = 157.3                  # MI355X FP32 vector, published (with packed FP32; this build issues scalar FMAs: 78.6)
+SRM_TAPS = 77
 # algorithmic bytes per neuron-timestep (fp32 tensors read + written once)
 AB = {"psp_conv": 8, "spike": 12, "shift": 8, "shift_bwd": 8, "spike_bwd": 12, "psp_corr": 8}
 # HBM bytes per launch on SHAPE measured with the FETCH_SIZE and WRITE_SIZE hardware counters
@@ -84,6 +86,30 @@ def cpu_baseline(shape, srm, ref, params, rows_fraction=1):
     return {"value": spikes.size / best, "unit": "neuron-timesteps/s", "cores": threads, "kind": "port",
             "sample": "oracle chain (conv77+spike+shift, shift+spike_bwd+corr77) on %s, median of %d passes, %.2f s each"
                       % (str(sub), len(times), best)}
+
+
+def copy_ceiling(x):
+    """What plain copies of the benchmark tensor reach on this box (read + written bytes per second):
+    the runtime's device-to-device copy and this library's zero-delay shift (one 16-byte vector
+    per lane, streaming policy)."""
+    from slayerpytorch_amd import slayerCuda
+    y = torch.empty_like(x)
+
+    def timed(fn):
+        ts = []
+        for i in range(10):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            if i >= 3:
+                ts.append(a.elapsed_time(b) * 1e-3)
+        return float(np.median(ts))
+
+    nbytes = 2 * x.numel() * 4
+    return {"unit": "GB/s", "device_to_device_copy": nbytes / timed(lambda: y.copy_(x)) / 1e9,
+            "zero_delay_shift_kernel": nbytes / timed(lambda: slayerCuda.shift(x, 0.0, 1.0)) / 1e9}
 
 
 def flip_rate(device, srm_t, ref_t, params):
@@ -268,6 +294,9 @@ def main():
         # the whole step (six launches and the gaps between them) against the HBM peak
         "chain_hbm_frac": chain_gbs / HBM_PEAK_GBS,
     }
+    # the 77-tap filters sit at the FP32 ridge: also as a fraction of the FP32 vector peak
+    result["roofline"]["fp32_frac_if_fir"] = (2.0 * SRM_TAPS * numel / (dominant_ms * 1e-3) / 1e12 / FP32_PEAK_TFLOPS
+                                              if dominant in ("psp_conv", "psp_corr") else None)
     if per_kernel_ms is not None:
         result["per_kernel_ms"] = per_kernel_ms
         result["per_kernel_hbm_frac"] = {n: AB[n] * numel / (per_kernel_ms[n] * 1e-3) / 1e9 / HBM_PEAK_GBS
@@ -275,6 +304,7 @@ def main():
         result["per_kernel_pass"] = "%d untimed steps before the timed region, an event pair around every launch" % probe
     del pool
     if not args.chain_only:
+        result["measured_copy_ceiling"] = copy_ceiling(grad)
         flips, rate = flip_rate(device, srm_t, ref_t, params)
         result["spike_flip_rate"] = flips
         result["spike_rate"] = rate
