@@ -182,7 +182,7 @@ def other_rows(device):
     s, v, u = slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1)
     out.append(row("loihi_forward", 16, n, timed(lambda: slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1)), shape))
     out.append(row("loihi_backward_pdf_plus_corr110", 20, n,
-                   timed(lambda: slayerCuda.corr(slayerCuda.spikeBackward(gl, v, 5120.0, 5120.0, 1 / 195.0), psp, 1.0)),
+                   timed(lambda: slayerCuda.spikeBackwardCorr(gl, v, psp, 5120.0, 5120.0, 1 / 195.0, 1.0)),
                    shape))
     return out
 

@@ -129,6 +129,20 @@ int slayer_shift_lut_f32(float *out, const float *in, const float *lut, int64_t 
 int slayer_spike_bwd_f32(float *gradIn, const float *gradOut, const float *u, float theta,
                          float tau, float scale, int64_t numel, void *stream);
 
+/*
+ * Backward pass of the Loihi neuron in one kernel: surrogate gradient, then correlation with
+ * the PSP kernel.  Replaces the body of slayerLoihi._spike.backward (src/slayerLoihi.py:278-283:
+ * the spikePdf expression chain followed by slayerCuda.corr, src/cuda/slayerKernels.cu:59-75).
+ *
+ * gradIn[n][t] = Ts * sum_{i<F} [t+i < T] w[n][t+i] * filt[i],
+ * w[n][t]      = gradOut[n][t] * (scale / tau) * exp(-|u[n][t] - theta| / tau).
+ * Same values as slayer_spike_bwd_f32 followed by slayer_corr_f32, without the intermediate
+ * tensor.  gradIn must not alias the inputs.  tau must be non-zero.
+ */
+int slayer_spike_bwd_corr_f32(float *gradIn, const float *gradOut, const float *u,
+                              const float *filt, int64_t nNeurons, int64_t T, int64_t F,
+                              float theta, float tau, float scale, float Ts, void *stream);
+
 /* Bytes of caller-provided device workspace that slayer_delay_grad_f32 needs (may be 0). */
 int64_t slayer_delay_grad_workspace_bytes(int64_t nBatch, int64_t nPerBatch, int64_t T);
 

@@ -62,6 +62,13 @@ struct RowCol {
     }
 };
 
+// Surrogate gradient of the spike function at membrane potential u: gain * exp(-|u - theta| / tau)
+// with gain = scale / tau.
+__device__ __forceinline__ float spike_pdf(float u, float theta, float tau, float gain)
+{
+    return gain * expf(-fabsf(u - theta) / tau);
+}
+
 // Synchronisation inside a work-group that is a single wavefront.  LDS executes the accesses of
 // one wavefront in program order, so data written by one lane is visible to the other lanes of
 // the same wavefront in any later instruction; all that is needed is to keep the compiler from

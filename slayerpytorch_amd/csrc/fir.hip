@@ -28,24 +28,35 @@ namespace slayer {
 constexpr int kFirMaxLdsFloats = 12288;  // 48 KiB of LDS per work-group at most
 constexpr int kFirMaxPitch = 512;     // longest LDS row (samples) the tiled kernel stages
 
+// Optional gate on the input: the filter then runs over in[n][t] * gain * exp(-|u[n][t] - theta| / tau),
+// i.e. the spike function's surrogate gradient applied on the way in (u == nullptr: no gate).
+struct FirGate {
+    const float *u;
+    float theta, tau, gain;
+};
+
 // ---- generic kernel: one lane per output sample (any F, any T) ---------------------------------
-template <bool CAUSAL>
+template <bool CAUSAL, bool GATED>
 __global__ __launch_bounds__(256) void fir_generic_kernel(float *__restrict__ out,
                                                           const float *__restrict__ in,
                                                           const float *__restrict__ filt,
-                                                          int64_t rows, int64_t T, int64_t F, float Ts)
+                                                          int64_t rows, int64_t T, int64_t F, float Ts, FirGate gate)
 {
     const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (t >= T) return;
     for (int64_t row = blockIdx.y; row < rows; row += gridDim.y) {
         const float *x = in + row * T;
+        const float *gu = GATED ? gate.u + row * T : nullptr;
+        auto sample = [&](int64_t k) {
+            return GATED ? x[k] * spike_pdf(gu[k], gate.theta, gate.tau, gate.gain) : x[k];
+        };
         float acc = 0.0f;
         if (CAUSAL) {
             const int64_t taps = (t + 1 < F) ? (t + 1) : F;
-            for (int64_t i = 0; i < taps; ++i) acc = __builtin_fmaf(x[t - i], filt[i], acc);
+            for (int64_t i = 0; i < taps; ++i) acc = __builtin_fmaf(sample(t - i), filt[i], acc);
         } else {
             const int64_t taps = (T - t < F) ? (T - t) : F;
-            for (int64_t i = 0; i < taps; ++i) acc = __builtin_fmaf(x[t + i], filt[i], acc);
+            for (int64_t i = 0; i < taps; ++i) acc = __builtin_fmaf(sample(t + i), filt[i], acc);
         }
         out[row * T + t] = acc * Ts;
     }
@@ -285,12 +296,13 @@ __device__ __forceinline__ void fir_sparse_tile(const BufferRsrc &bufOut, const 
 }
 
 // VEC: rows are whole 16-byte vectors (T % 4 == 0, pointers 16-byte aligned)
-template <bool CAUSAL, bool VEC, int U>
+// GATED: the staged samples are in * pdf(gate.u), computed once per staged sample
+template <bool CAUSAL, bool VEC, int U, bool GATED>
 __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
                                                         const float *__restrict__ in,
                                                         const float *__restrict__ filt,
                                                         int64_t rows, int T, int F, int TT, int LD, int R,
-                                                        float Ts)
+                                                        float Ts, FirGate gate)
 {
     extern __shared__ __align__(16) float X[];
     float *fL = X + R * LD;                                        // filter copy for the sparse path
@@ -309,6 +321,8 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
     // The tile's rows as 32-bit offsets from its first row (a tile spans far less than 2 GiB).
     const BufferRsrc bufIn = make_buffer(in + row0 * static_cast<int64_t>(T));
     const BufferRsrc bufOut = make_buffer(out + row0 * static_cast<int64_t>(T));
+    const BufferRsrc bufGate = make_buffer((GATED ? gate.u : in) + row0 * static_cast<int64_t>(T));
+    auto gated = [&](float x, float u) { return x * spike_pdf(u, gate.theta, gate.tau, gate.gain); };
 
     // ---- stage: X[r][j] = in[row0+r][time(j)], zero outside the row;
     //      time(j) = t0 + j (correlation) or tHi - j (convolution)
@@ -324,7 +338,11 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
             const int dr = 256 / nq, dc = 256 % nq;
             const int total = nRows * nq;
             for (int g = tid; g < total; g += 256, rc.advance(dr, dc, nq)) {
-                const float4 v = buffer_load4(bufIn, (rc.r * T + tA + (rc.c << 2)) * 4, 0);
+                float4 v = buffer_load4(bufIn, (rc.r * T + tA + (rc.c << 2)) * 4, 0);
+                if (GATED) {
+                    const float4 g = buffer_load4(bufGate, (rc.r * T + tA + (rc.c << 2)) * 4, 0);
+                    v = make_float4(gated(v.x, g.x), gated(v.y, g.y), gated(v.z, g.z), gated(v.w, g.w));
+                }
                 nonZero += __builtin_popcountll(__ballot(any_nonzero(v)));
                 if (CAUSAL)  // descending time: the vector lands mirrored
                     *reinterpret_cast<float4 *>(X + rc.r * LD + (jA + ((nq - 1 - rc.c) << 2))) =
@@ -353,20 +371,22 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
             int r, j4;
             divmod_small(q, LD4, invLD4, r, j4);
             const float *src = in + (row0 + r) * static_cast<int64_t>(T);
+            const float *gsrc = (GATED ? gate.u : in) + (row0 + r) * static_cast<int64_t>(T);
+            auto at = [&](int t) { return GATED ? gated(src[t], gsrc[t]) : src[t]; };
             const int j = j4 << 2;
             float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if (CAUSAL) {
                 const int tl = tHi - j - 3;  // lowest time of the quad; X order is descending
-                if (tl + 3 >= 0 && tl + 3 < T) v.x = src[tl + 3];
-                if (tl + 2 >= 0 && tl + 2 < T) v.y = src[tl + 2];
-                if (tl + 1 >= 0 && tl + 1 < T) v.z = src[tl + 1];
-                if (tl >= 0 && tl < T) v.w = src[tl];
+                if (tl + 3 >= 0 && tl + 3 < T) v.x = at(tl + 3);
+                if (tl + 2 >= 0 && tl + 2 < T) v.y = at(tl + 2);
+                if (tl + 1 >= 0 && tl + 1 < T) v.z = at(tl + 1);
+                if (tl >= 0 && tl < T) v.w = at(tl);
             } else {
                 const int tl = t0 + j;
-                if (tl < T) v.x = src[tl];
-                if (tl + 1 < T) v.y = src[tl + 1];
-                if (tl + 2 < T) v.z = src[tl + 2];
-                if (tl + 3 < T) v.w = src[tl + 3];
+                if (tl < T) v.x = at(tl);
+                if (tl + 1 < T) v.y = at(tl + 1);
+                if (tl + 2 < T) v.z = at(tl + 2);
+                if (tl + 3 < T) v.w = at(tl + 3);
             }
             *reinterpret_cast<float4 *>(X + r * LD + j) = v;
             nonZero += __builtin_popcountll(__ballot(any_nonzero(v)));
@@ -479,32 +499,33 @@ static bool plan_fir(int64_t rows, int64_t T, int64_t F, FirPlan &best)
     return true;
 }
 
-template <bool CAUSAL, bool VEC, int U>
+template <bool CAUSAL, bool VEC, int U, bool GATED>
 static void launch_tiled(const FirPlan &p, float *out, const float *in, const float *filt, int64_t rows, int64_t T,
-                         int64_t F, float Ts, hipStream_t stream)
+                         int64_t F, float Ts, const FirGate &gate, hipStream_t stream)
 {
     dim3 grid(static_cast<unsigned>(ceil_div(rows, p.R)), static_cast<unsigned>(p.nTiles)), block(256);
     const size_t lds = (static_cast<size_t>(p.R) * p.LD + static_cast<size_t>(F) + 4) * sizeof(float);
-    hipLaunchKernelGGL((fir_tiled_kernel<CAUSAL, VEC, U>), grid, block, lds, stream, out, in, filt, rows,
-                       static_cast<int>(T), static_cast<int>(F), p.TT, p.LD, p.R, Ts);
+    hipLaunchKernelGGL((fir_tiled_kernel<CAUSAL, VEC, U, GATED>), grid, block, lds, stream, out, in, filt, rows,
+                       static_cast<int>(T), static_cast<int>(F), p.TT, p.LD, p.R, Ts, gate);
 }
 
-template <bool CAUSAL>
+template <bool CAUSAL, bool GATED>
 static int launch_fir(float *out, const float *in, const float *filt, int64_t rows, int64_t T,
-                      int64_t F, float Ts, hipStream_t stream)
+                      int64_t F, float Ts, const FirGate &gate, hipStream_t stream)
 {
     if (rows < 0 || T < 0 || F < 0) return SLAYER_EINVAL;
     if (rows == 0 || T == 0) return SLAYER_OK;
-    if (!out || !in || (F > 0 && !filt)) return SLAYER_EINVAL;
+    if (!out || !in || (F > 0 && !filt) || (GATED && !gate.u)) return SLAYER_EINVAL;
     if (T >= (1LL << 30)) return SLAYER_EUNSUPPORTED;
 
-    const bool vec = (T % 4 == 0) && aligned16(out) && aligned16(in);
+    const bool vec = (T % 4 == 0) && aligned16(out) && aligned16(in) && (!GATED || aligned16(gate.u));
     // Register-only kernel: always for short filters (the op is then a stream); up to 81 taps for
     // the correlation, whose input - a gradient - is dense, where it measures 6-9 % faster than
     // the tiled kernel.  The convolution keeps the tiled kernel for longer filters because of its
     // event-driven path for spike trains.
     const int64_t directMax = CAUSAL ? 33 : 81;
-    if (!generic_forced() && vec && F >= 1 && F <= directMax && T < (1LL << 28) && rows * (T / 4) < (1LL << 32)) {
+    // (not with a gate: every lane would evaluate the gate for its whole window).
+    if (!GATED && !generic_forced() && vec && F >= 1 && F <= directMax && T < (1LL << 28) && rows * (T / 4) < (1LL << 32)) {
         const int U = F <= 17 ? 4 : 8;
         const int64_t chunksPerRow = ceil_div(T / 4, U / 4);
         const int64_t chunks = rows * chunksPerRow;
@@ -527,17 +548,17 @@ static int launch_fir(float *out, const float *in, const float *filt, int64_t ro
     }
     FirPlan p;
     if (!generic_forced() && plan_fir(rows, T, F, p) && ceil_div(rows, p.R) < (1LL << 31)) {
-        if (vec && p.U == 16) launch_tiled<CAUSAL, true, 16>(p, out, in, filt, rows, T, F, Ts, stream);
-        else if (vec) launch_tiled<CAUSAL, true, 8>(p, out, in, filt, rows, T, F, Ts, stream);
-        else if (p.U == 16) launch_tiled<CAUSAL, false, 16>(p, out, in, filt, rows, T, F, Ts, stream);
-        else launch_tiled<CAUSAL, false, 8>(p, out, in, filt, rows, T, F, Ts, stream);
+        if (vec && p.U == 16) launch_tiled<CAUSAL, true, 16, GATED>(p, out, in, filt, rows, T, F, Ts, gate, stream);
+        else if (vec) launch_tiled<CAUSAL, true, 8, GATED>(p, out, in, filt, rows, T, F, Ts, gate, stream);
+        else if (p.U == 16) launch_tiled<CAUSAL, false, 16, GATED>(p, out, in, filt, rows, T, F, Ts, gate, stream);
+        else launch_tiled<CAUSAL, false, 8, GATED>(p, out, in, filt, rows, T, F, Ts, gate, stream);
         return launch_status();
     }
     const int64_t tBlocks = ceil_div(T, 256);
     if (tBlocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
     dim3 grid(static_cast<unsigned>(tBlocks), static_cast<unsigned>(rows < 65535 ? rows : 65535));
-    hipLaunchKernelGGL(fir_generic_kernel<CAUSAL>, grid, dim3(256), 0, stream, out, in, filt, rows, T,
-                       F, Ts);
+    hipLaunchKernelGGL((fir_generic_kernel<CAUSAL, GATED>), grid, dim3(256), 0, stream, out, in, filt, rows, T,
+                       F, Ts, gate);
     return launch_status();
 }
 
@@ -546,13 +567,23 @@ static int launch_fir(float *out, const float *in, const float *filt, int64_t ro
 extern "C" int slayer_conv_f32(float *out, const float *in, const float *filt, int64_t nNeurons,
                                int64_t T, int64_t F, float Ts, void *stream)
 {
-    return slayer::launch_fir<true>(out, in, filt, nNeurons, T, F, Ts,
-                                    static_cast<hipStream_t>(stream));
+    return slayer::launch_fir<true, false>(out, in, filt, nNeurons, T, F, Ts, slayer::FirGate{nullptr, 0.0f, 1.0f, 0.0f},
+                                           static_cast<hipStream_t>(stream));
 }
 
 extern "C" int slayer_corr_f32(float *out, const float *in, const float *filt, int64_t nNeurons,
                                int64_t T, int64_t F, float Ts, void *stream)
 {
-    return slayer::launch_fir<false>(out, in, filt, nNeurons, T, F, Ts,
-                                     static_cast<hipStream_t>(stream));
+    return slayer::launch_fir<false, false>(out, in, filt, nNeurons, T, F, Ts, slayer::FirGate{nullptr, 0.0f, 1.0f, 0.0f},
+                                            static_cast<hipStream_t>(stream));
+}
+
+extern "C" int slayer_spike_bwd_corr_f32(float *gradIn, const float *gradOut, const float *u, const float *filt,
+                                         int64_t nNeurons, int64_t T, int64_t F, float theta, float tau,
+                                         float scale, float Ts, void *stream)
+{
+    if (tau == 0.0f) return SLAYER_EINVAL;
+    return slayer::launch_fir<false, true>(gradIn, gradOut, filt, nNeurons, T, F, Ts,
+                                           slayer::FirGate{u, theta, tau, scale / tau},
+                                           static_cast<hipStream_t>(stream));
 }

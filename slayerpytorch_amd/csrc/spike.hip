@@ -318,11 +318,6 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 // runs: one 16-byte vector per lane, one pass per work-group, streaming cache policy.
 typedef float vec4f __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ float spike_pdf(float u, float theta, float tau, float gain)
-{
-    return gain * expf(-fabsf(u - theta) / tau);
-}
-
 __global__ __launch_bounds__(256) void spike_bwd_vec_kernel(float *gradIn, const float *gradOut,
                                                             const float *__restrict__ u, float theta,
                                                             float tau, float gain, int64_t quads)

@@ -191,6 +191,28 @@ def spikeBackward(gradOutput, membranePotential, theta, tau, scale):
     return gradInput
 
 
+def spikeBackwardCorr(gradOutput, membranePotential, filter, theta, tau, scale, Ts):
+    """``corr(spikeBackward(gradOutput, membranePotential, theta, tau, scale), filter, Ts)`` in one
+    kernel, without the intermediate tensor (the backward pass of the Loihi neuron)."""
+    _check_input(gradOutput, "gradOutput")
+    _check_input(membranePotential, "membranePotential")
+    _check_input(filter, "filter")
+    _check_device(gradOutput, membranePotential, "gradOutput", "membranePotential")
+    _check_device(gradOutput, filter, "gradOutput", "filter")
+    if gradOutput.shape != membranePotential.shape:
+        raise RuntimeError("gradOutput and membranePotential must have the same shape")
+    theta, tau, scale, Ts = _scalar(theta, "theta"), _scalar(tau, "tau"), _scalar(scale, "scale"), _scalar(Ts, "Ts")
+    lib = _lib.load()
+    gradInput = torch.empty_like(gradOutput)
+    nNeurons, T = _rows(gradOutput)
+    with _on_device_of(gradOutput) as stream:
+        _lib.check(lib.slayer_spike_bwd_corr_f32(_ptr(gradInput), _ptr(gradOutput), _ptr(membranePotential),
+                                                 _ptr(filter), nNeurons, T, filter.numel(), theta, tau, scale, Ts,
+                                                 stream),
+                   "slayer_spike_bwd_corr_f32")
+    return gradInput
+
+
 def delayGrad(output, gradOutput, Ts):
     """Gradient of ``shift`` with respect to its per-neuron delays: ``Ts * sum over batch and
     time of gradOutput * (output[t-1] - output[t]) / Ts``; shape ``output.shape[1:-1]``."""

@@ -109,6 +109,6 @@ class _spike(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gradOutput):
         voltage, srmKernel = ctx.saved_tensors
-        weighted = slayerCuda.spikeBackward(gradOutput.contiguous(), voltage, ctx.theta,
-                                            ctx.pdfTimeConstant, ctx.pdfScale)
-        return slayerCuda.corr(weighted, srmKernel, ctx.Ts), None, None, None
+        # surrogate gradient and correlation with the PSP kernel in one kernel
+        return slayerCuda.spikeBackwardCorr(gradOutput.contiguous(), voltage, srmKernel, ctx.theta,
+                                            ctx.pdfTimeConstant, ctx.pdfScale, ctx.Ts), None, None, None

@@ -239,6 +239,22 @@ def test_spike_bwd(n):
         assert rel_err(got, ref64) <= REL_TOL
 
 
+@pytest.mark.parametrize("shape,Fl", [((2, 3, 5, 7, 300), 110), ((3, 41, 350), 110), ((2, 9, 64), 8), ((1, 5, 2000), 77),
+                                      ((1, 2, 50), 500), ((4, 7, 1), 3)])
+def test_spike_bwd_corr_is_the_two_ops_in_one(impl, shape, Fl):
+    # the Loihi neuron's backward pass: pdf(voltage) * gradOut, then corr with the PSP kernel
+    rng = np.random.default_rng(shape[-1] + Fl)
+    v = (rng.standard_normal(shape) * 3000 + 3000).astype(np.float32)
+    g = rng.standard_normal(shape).astype(np.float32)
+    f = rng.random(Fl).astype(np.float32) * 100
+    theta, tau, scale, Ts = 5120.0, 5120.0, 1 / 195.0, 0.5
+    got = host(slayerCuda.spikeBackwardCorr(dev(g), dev(v), dev(f), theta, tau, scale, Ts))
+    two = host(slayerCuda.corr(slayerCuda.spikeBackward(dev(g), dev(v), theta, tau, scale), dev(f), Ts))
+    assert np.array_equal(bits(got), bits(two)), "fused kernel differs from spikeBackward followed by corr"
+    want = O.corr(O.spike_bwd(g, v, theta, tau, scale), f, Ts, fused=True)
+    assert rel_err(got, want) <= REL_TOL
+
+
 # ------------------------------------------------------------------------------------------ delay gradient
 @pytest.mark.parametrize("shape,Ts", [((4, 6, 1, 1, 80), 0.1), ((64, 20, 1, 1, 2000), 1.0), ((3, 2, 5, 7, 33), 0.5),
                                       ((1, 1, 1, 1, 1), 1.0)])
