@@ -17,9 +17,10 @@ Python numbers or 0-dim tensors, as with pybind11's float conversion.  Outputs a
 with ``torch.empty_like``; kernels are enqueued on PyTorch's current stream of the tensor's
 device and never synchronise with the host.
 
-``spikeBackward``, ``delayGrad`` and the ``sign`` argument of ``shift`` have no counterpart in
-the reference extension: they are the fused forms of the elementwise chains in
-``_spikeFunction.backward`` / ``_delayFunction.backward`` (src/slayer.py:857-865, 944-957).
+``spikeBackward``, ``spikeBackwardCorr``, ``delayGrad`` and the ``sign`` argument of ``shift``
+have no counterpart in the reference extension: they are the fused forms of the elementwise
+chains in ``_spikeFunction.backward`` / ``_delayFunction.backward`` (src/slayer.py:857-865,
+944-957) and of ``slayerLoihi._spike.backward`` (src/slayerLoihi.py:278-283).
 """
 import numbers
 
@@ -27,7 +28,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "delayGrad"]
+__all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "spikeBackwardCorr", "delayGrad"]
 
 
 def _check_input(x, name):
@@ -70,19 +71,31 @@ def _rows(x):
     return (x.numel() // T if T else 0), T
 
 
+def _raw_stream(index):
+    """Raw handle of PyTorch's current stream on device ``index``."""
+    get = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # skips building a Stream object
+    return get(index) if get is not None else torch.cuda.current_stream(index).cuda_stream
+
+
 class _on_device_of:
     """Makes the tensor's device current (like the reference's cudaSetDevice) and yields the
     raw handle of PyTorch's current stream there."""
+    __slots__ = ("index", "guard")
 
     def __init__(self, x):
-        self.guard = torch.cuda.device(x.device)
+        self.index = x.device.index
+        self.guard = None
 
     def __enter__(self):
-        self.guard.__enter__()
-        return torch.cuda.current_stream().cuda_stream
+        if self.index != torch.cuda.current_device():
+            self.guard = torch.cuda.device(self.index)
+            self.guard.__enter__()
+        return _raw_stream(self.index)
 
     def __exit__(self, *exc):
-        return self.guard.__exit__(*exc)
+        if self.guard is not None:
+            return self.guard.__exit__(*exc)
+        return False
 
 
 def getSpikes(d_u, d_nu, theta, Ts):
