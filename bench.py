@@ -131,7 +131,9 @@ def flip_rate(device, srm_t, ref_t, params):
 
 def other_rows(device):
     """Quick per-op measurements of the scope rows that are not part of the headline chain, each on
-    the largest tensor its BASELINE config gives it (median of 7 event-timed launches)."""
+    the largest tensor its BASELINE config gives it (median of 7 event-timed launches).  hbm_frac
+    counts the algorithmic bytes of the unfused reference sequence (Loihi forward + delayShift:
+    16 + 8 B, Loihi backward: 12 + 8 B), also where one fused kernel moves fewer."""
     from slayerpytorch_amd import slayerCuda, slayerLoihiCuda
     from slayerpytorch_amd.slayer import alphaKernel
     from slayerpytorch_amd.slayerLoihi import loihiPspKernel
@@ -181,6 +183,12 @@ def other_rows(device):
     n = w.numel()
     s, v, u = slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1)
     out.append(row("loihi_forward", 16, n, timed(lambda: slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1)), shape))
+    out.append(row("loihi_forward_spike_and_voltage_delay1_fused", 24, n,
+                   timed(lambda: slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 1, voltage=True, current=False)),
+                   shape))
+    out.append(row("loihi_forward_spike_only_delay1_fused", 24, n,
+                   timed(lambda: slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 1, voltage=False, current=False)),
+                   shape))
     out.append(row("loihi_backward_pdf_plus_corr110", 20, n,
                    timed(lambda: slayerCuda.spikeBackwardCorr(gl, v, psp, 5120.0, 5120.0, 1 / 195.0, 1.0)),
                    shape))

@@ -181,6 +181,23 @@ int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const float *w, in
                                 int64_t T, uint32_t wgtExp, int32_t theta, uint32_t iDecay,
                                 uint32_t vDecay, uint32_t refDelay, void *stream);
 
+/*
+ * The same neuron with the time shift that follows it in Loihi networks fused in, and with
+ * optional outputs.  Replaces the call pair spikeLoihi -> delayShift(spike, 1) of the reference's
+ * network definitions (src/auto/loihi.py:67-69, exampleLoihi/03_IBMGesture/ibmGestureTrain.py:57-81):
+ * slayerLoihiCuda.getSpikes (src/cuda/slayerLoihiKernels.cu:12-46) followed by slayerCuda.shift
+ * (src/cuda/slayerKernels.cu:114-134).
+ *
+ * s[t] = spike[t - delaySteps] (0 for t < delaySteps), 0 <= delaySteps <= 31 (more:
+ * SLAYER_EUNSUPPORTED - shift separately); v and u are as in slayer_loihi_get_spikes_f32 (not
+ * shifted) and either may be NULL when the caller does not need it (the layer engine needs the
+ * voltage for the backward pass only and never the current), which saves its 4 bytes per sample.
+ */
+int slayer_loihi_get_spikes_delayed_f32(float *s, float *v, float *u, const float *w,
+                                        int64_t nNeurons, int64_t T, uint32_t wgtExp, int32_t theta,
+                                        uint32_t iDecay, uint32_t vDecay, uint32_t refDelay,
+                                        int32_t delaySteps, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -34,6 +34,8 @@ SIGNATURES = {
     "slayer_delay_grad_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _i64, _i64, _i64, _f32, _stream]),
     "slayer_loihi_get_spikes_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _i64, _i64, _u32, _i32,
                                                   _u32, _u32, _u32, _stream]),
+    "slayer_loihi_get_spikes_delayed_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _i64, _i64, _u32, _i32,
+                                                          _u32, _u32, _u32, _i32, _stream]),
 }
 
 ABI_VERSION = 1

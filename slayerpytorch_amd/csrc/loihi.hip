@@ -56,7 +56,16 @@ struct LoihiState {
 struct LoihiParams {
     uint32_t weightShift, keepI, keepV, vDecay;
     int refDelay, theta;
+    int delay;  // the spike output is written `delay` samples late (0..31), zeros before: a fused delayShift
 };
+
+// The spike bits of 32 consecutive samples, delayed by p.delay samples: the bits that leave at
+// the top come back at the bottom of the next group of the same row (prev = the previous group's
+// undelayed bits, 0 at the start of a row).
+__device__ __forceinline__ uint32_t loihi_delayed(uint32_t fired, uint32_t prev, int delay)
+{
+    return delay ? ((fired << delay) | (prev >> (32 - delay))) : fired;
+}
 
 // One time step (t >= 1).  Returns the spike (0/1); cOut / vOut are the reported current / voltage.
 __device__ __forceinline__ uint32_t loihi_step(LoihiState &st, const LoihiParams &p, float w,
@@ -86,13 +95,16 @@ __global__ __launch_bounds__(256) void loihi_generic_kernel(float *__restrict__ 
     if (row >= rows) return;
     const int64_t base = row * T;
     LoihiState st = {0, 0, 0};
-    s[base] = 0.0f; v[base] = 0.0f; u[base] = 0.0f;
+    uint32_t history = 0;  // bit k: the spike k samples ago
+    s[base] = 0.0f;
+    if (v) v[base] = 0.0f;
+    if (u) u[base] = 0.0f;
     for (int64_t t = 1; t < T; ++t) {
         float c, vo;
-        const uint32_t spike = loihi_step(st, p, w[base + t], c, vo);
-        s[base + t] = static_cast<float>(spike);
-        u[base + t] = c;
-        v[base + t] = vo;
+        history = (history << 1) | loihi_step(st, p, w[base + t], c, vo);
+        s[base + t] = static_cast<float>((history >> p.delay) & 1u);
+        if (u) u[base + t] = c;
+        if (v) v[base + t] = vo;
     }
 }
 
@@ -114,6 +126,7 @@ __global__ __launch_bounds__(64) void loihi_tile_kernel(float *__restrict__ s, f
 
     const int lane = threadIdx.x;
     LoihiState st = {0, 0, 0};
+    uint32_t prevFired = 0;
 
     float x[NB * V];
     auto rows_of = [&](int64_t t) { return static_cast<int>(min(static_cast<int64_t>(R), rows - t * R)); };
@@ -173,7 +186,7 @@ __global__ __launch_bounds__(64) void loihi_tile_kernel(float *__restrict__ s, f
 
         // ---- sequential update: lane = row
         if (lane < R) {
-            if (tL == 0) st = {0, 0, 0};
+            if (tL == 0) { st = {0, 0, 0}; prevFired = 0; }
             float *mineC = tileC + lane * P;
             float *mineV = tileV + lane * P;
             const int groups = (n + G - 1) / G;
@@ -200,17 +213,18 @@ __global__ __launch_bounds__(64) void loihi_tile_kernel(float *__restrict__ s, f
                     *reinterpret_cast<float4 *>(mineC + c0 + k) = make_float4(cur[k], cur[k + 1], cur[k + 2], cur[k + 3]);
                     *reinterpret_cast<float4 *>(mineV + c0 + k) = make_float4(vol[k], vol[k + 1], vol[k + 2], vol[k + 3]);
                 }
-                masks[lane * MP + g] = fired;
+                masks[lane * MP + g] = loihi_delayed(fired, prevFired, p.delay);
+                prevFired = fired;
             }
         }
         wave_sync();
 
-        // ---- retire
+        // ---- retire (voltage and current only when the caller wants them)
         {
             const int64_t base = t * R * static_cast<int64_t>(T);
             const BufferRsrc bufS = make_buffer(s + base);
-            const BufferRsrc bufV = make_buffer(v + base);
-            const BufferRsrc bufU = make_buffer(u + base);
+            const BufferRsrc bufV = make_buffer((v ? v : s) + base);
+            const BufferRsrc bufU = make_buffer((u ? u : s) + base);
             const int perRow = n / V;
             const int total = nRows * perRow;
             RowCol rc;
@@ -222,14 +236,14 @@ __global__ __launch_bounds__(64) void loihi_tile_kernel(float *__restrict__ s, f
                 const int off = (rc.r * T + tL + col) * 4;
                 const uint32_t m = masks[rc.r * MP + (col >> 5)] >> (col & 31);
                 if (VEC) {
-                    buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + rc.r * P + col));
-                    buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + rc.r * P + col));
+                    if (u) buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + rc.r * P + col));
+                    if (v) buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + rc.r * P + col));
                     buffer_store4(bufS, off, 0,
                                   make_float4((m & 1u) ? 1.0f : 0.0f, (m & 2u) ? 1.0f : 0.0f,
                                               (m & 4u) ? 1.0f : 0.0f, (m & 8u) ? 1.0f : 0.0f));
                 } else {
-                    buffer_store(bufU, off, 0, tileC[rc.r * P + col]);
-                    buffer_store(bufV, off, 0, tileV[rc.r * P + col]);
+                    if (u) buffer_store(bufU, off, 0, tileC[rc.r * P + col]);
+                    if (v) buffer_store(bufV, off, 0, tileV[rc.r * P + col]);
                     buffer_store(bufS, off, 0, (m & 1u) ? 1.0f : 0.0f);
                 }
                 rc.advance(dr, dc, perRow);
@@ -284,6 +298,7 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
     float4 x[NB];
     float headC[MERGE ? G : 1], headV[MERGE ? G : 1];  // results of this row's first line (MERGE)
     uint32_t headFired = 0;
+    uint32_t prevFired = 0;  // undelayed spike bits of this row's previous group
 
     auto rows_of = [&](int64_t t) { return static_cast<int>(min(static_cast<int64_t>(R), rows - t * R)); };
     // samples by which row r of tile t starts after a 128-byte boundary
@@ -331,7 +346,7 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
 
         // ---- sequential update: lane = row; this lane's column c is its sample TC*j - o + c
         if (R == kWave || lane < R) {
-            if (j == 0) st = {0, 0, 0};
+            if (j == 0) { st = {0, 0, 0}; prevFired = 0; }
             float *mineC = tileC + lane * P;
             float *mineV = tileV + lane * P;
             const int tRow = TC * j - ((o0 + lane * T) & 31);
@@ -373,11 +388,19 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
                     *reinterpret_cast<float4 *>(mineC + c0 + k) = make_float4(cur[k], cur[k + 1], cur[k + 2], cur[k + 3]);
                     *reinterpret_cast<float4 *>(mineV + c0 + k) = make_float4(vol[k], vol[k + 1], vol[k + 2], vol[k + 3]);
                 }
-                masks[lane * LPP + g] = fired;
+                // the delayed bits; those that would land beyond the end of the row are dropped
+                // (the end of this row's last line belongs to the next row)
+                uint32_t out = loihi_delayed(fired, prevFired, p.delay);
+                prevFired = fired;
+                if (!inside) {
+                    const int left = T - (tRow + c0);  // samples of the row from this group on
+                    out &= left >= G ? 0xffffffffu : (left > 0 ? (1u << left) - 1u : 0u);
+                }
+                masks[lane * LPP + g] = out;
                 if (MERGE && j == 0) {
 #pragma unroll
                     for (int k = 0; k < G; ++k) { headC[k] = cur[k]; headV[k] = vol[k]; }
-                    headFired = fired;
+                    headFired = out;
                 }
             }
             if (MERGE && j > 0) {
@@ -405,8 +428,8 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
         {
             const int64_t base = t * R * static_cast<int64_t>(T);
             const BufferRsrc bufS = make_buffer(s + base);
-            const BufferRsrc bufV = make_buffer(v + base);
-            const BufferRsrc bufU = make_buffer(u + base);
+            const BufferRsrc bufV = make_buffer((v ? v : s) + base);
+            const BufferRsrc bufU = make_buffer((u ? u : s) + base);
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const int r = b * RPI + subRow;
@@ -421,8 +444,8 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
                 }
                 const int off = masked_offset(ok, (r * T + time) * 4);
                 const uint32_t m = masks[r * LPP + (col >> 5)] >> (col & 31);
-                buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + r * P + col));
-                buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + r * P + col));
+                if (u) buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + r * P + col));
+                if (v) buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + r * P + col));
                 buffer_store4(bufS, off, 0,
                               make_float4((m & 1u) ? 1.0f : 0.0f, (m & 2u) ? 1.0f : 0.0f,
                                           (m & 4u) ? 1.0f : 0.0f, (m & 8u) ? 1.0f : 0.0f));
@@ -437,17 +460,18 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
 
 }  // namespace slayer
 
-extern "C" int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const float *w,
-                                           int64_t nNeurons, int64_t T, uint32_t wgtExp, int32_t theta,
-                                           uint32_t iDecay, uint32_t vDecay, uint32_t refDelay,
-                                           void *stream)
+namespace slayer {
+
+static int launch_loihi(float *s, float *v, float *u, const float *w, int64_t nNeurons, int64_t T,
+                        uint32_t wgtExp, int32_t theta, uint32_t iDecay, uint32_t vDecay, uint32_t refDelay,
+                        int delaySteps, hipStream_t st)
 {
-    using namespace slayer;
     if (nNeurons < 0 || T < 0) return SLAYER_EINVAL;
     if (refDelay == 0 || wgtExp > 25 || refDelay > 0x7fffffffu) return SLAYER_EINVAL;
+    if (delaySteps < 0) return SLAYER_EINVAL;
+    if (delaySteps > 31) return SLAYER_EUNSUPPORTED;
     if (nNeurons == 0 || T == 0) return SLAYER_OK;
-    if (!s || !v || !u || !w) return SLAYER_EINVAL;
-    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (!s || !w) return SLAYER_EINVAL;
 
     LoihiParams p;
     p.weightShift = 6 + wgtExp;  // weight scale 1 << (6 + wgtExp)
@@ -456,6 +480,7 @@ extern "C" int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const f
     p.refDelay = static_cast<int>(refDelay);
     p.vDecay = vDecay;
     p.theta = theta;
+    p.delay = delaySteps;
 
     if (!generic_forced() && T <= kBufferMaxT) {
         constexpr int kRows = 32, kPiece = LOIHI_PIECE;
@@ -468,11 +493,12 @@ extern "C" int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const f
         const size_t lds = (static_cast<size_t>(2 * kRows) * P + kRows * MP) * sizeof(float);
         const int64_t resident = static_cast<int64_t>(compute_units()) * (160 * 1024 / static_cast<int64_t>(lds));
         const unsigned grid = static_cast<unsigned>(tiles < resident ? tiles : resident);
+        // outputs the caller does not want (null) constrain nothing
         const bool vec = (T % 4 == 0) && aligned16(s) && aligned16(v) && aligned16(u) && aligned16(w);
         const uintptr_t phase = reinterpret_cast<uintptr_t>(w) & 127;
         const bool samePhase = (reinterpret_cast<uintptr_t>(s) & 127) == phase &&
-                               (reinterpret_cast<uintptr_t>(v) & 127) == phase &&
-                               (reinterpret_cast<uintptr_t>(u) & 127) == phase;
+                               (!v || (reinterpret_cast<uintptr_t>(v) & 127) == phase) &&
+                               (!u || (reinterpret_cast<uintptr_t>(u) & 127) == phase);
         if (vec && samePhase) {
             constexpr int kR = LOIHI_ROWS, kLpp = LOIHI_LPP;
             const int64_t lineTiles = ceil_div(nNeurons, kR);
@@ -500,4 +526,25 @@ extern "C" int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const f
     hipLaunchKernelGGL(loihi_generic_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, s, v,
                        u, w, nNeurons, T, p);
     return launch_status();
+}
+
+}  // namespace slayer
+
+extern "C" int slayer_loihi_get_spikes_f32(float *s, float *v, float *u, const float *w,
+                                           int64_t nNeurons, int64_t T, uint32_t wgtExp, int32_t theta,
+                                           uint32_t iDecay, uint32_t vDecay, uint32_t refDelay,
+                                           void *stream)
+{
+    if (nNeurons > 0 && T > 0 && (!v || !u)) return SLAYER_EINVAL;
+    return slayer::launch_loihi(s, v, u, w, nNeurons, T, wgtExp, theta, iDecay, vDecay, refDelay, 0,
+                                static_cast<hipStream_t>(stream));
+}
+
+extern "C" int slayer_loihi_get_spikes_delayed_f32(float *s, float *v, float *u, const float *w,
+                                                   int64_t nNeurons, int64_t T, uint32_t wgtExp, int32_t theta,
+                                                   uint32_t iDecay, uint32_t vDecay, uint32_t refDelay,
+                                                   int32_t delaySteps, void *stream)
+{
+    return slayer::launch_loihi(s, v, u, w, nNeurons, T, wgtExp, theta, iDecay, vDecay, refDelay, delaySteps,
+                                static_cast<hipStream_t>(stream));
 }

@@ -73,10 +73,16 @@ class spikeLayer(slayer.spikeLayer):
         return torch.tensor(loihiRefKernel(self.neuron["theta"], self.neuron["vDecay"],
                                            self.neuron["refDelay"], SCALE))
 
-    def spikeLoihi(self, weightedSpikes):
+    def spikeLoihi(self, weightedSpikes, delay=0, delayTs=1):
         """Loihi neuron dynamics on weighted (unfiltered) input spikes -> output spikes, with the
-        SLAYER surrogate gradient attached."""
-        return _spike.apply(weightedSpikes, self.srmKernel, self.neuron, self.simulation["Ts"])
+        SLAYER surrogate gradient attached.  ``delay`` (extension) gives
+        ``delayShift(spikeLoihi(x), delay, delayTs)`` - a shift by ``int(delay / delayTs)`` samples
+        - from the same kernel."""
+        Ts = self.simulation["Ts"]
+        steps = int(float(delay) / float(delayTs))
+        if 0 <= steps <= slayerLoihiCuda.MAX_FUSED_DELAY:
+            return _spike.apply(weightedSpikes, self.srmKernel, self.neuron, Ts, steps)
+        return self.delayShift(_spike.apply(weightedSpikes, self.srmKernel, self.neuron, Ts, 0), delay, delayTs)
 
     def spikeLoihiFull(self, weightedSpikes):
         """Same dynamics without autograd; returns ``(spike, voltage, current)``."""
@@ -88,27 +94,45 @@ class spikeLayer(slayer.spikeLayer):
 
 class _spike(torch.autograd.Function):
     @staticmethod
-    def loihi(weightedSpikes, neuron, Ts):
+    def _scaled(weightedSpikes, Ts):
+        # the reference multiplies by Ts unconditionally; by 1 that is a copy of the tensor
         if weightedSpikes.dtype == torch.int32:
             Ts = 1
-        spike, voltage, current = slayerLoihiCuda.getSpikes(
-            (weightedSpikes * Ts).contiguous(), neuron["wgtExp"], neuron["theta"], neuron["iDecay"],
-            neuron["vDecay"], neuron["refDelay"])
-        return spike / Ts, voltage, current
+        x = weightedSpikes if Ts == 1 else weightedSpikes * Ts
+        return x.contiguous(), Ts
 
     @staticmethod
-    def forward(ctx, weightedSpikes, srmKernel, neuron, Ts):
-        spike, voltage, current = _spike.loihi(weightedSpikes, neuron, Ts)
-        ctx.save_for_backward(voltage, srmKernel.clone().detach())
+    def loihi(weightedSpikes, neuron, Ts):
+        x, Ts = _spike._scaled(weightedSpikes, Ts)
+        spike, voltage, current = slayerLoihiCuda.getSpikes(
+            x, neuron["wgtExp"], neuron["theta"], neuron["iDecay"], neuron["vDecay"], neuron["refDelay"])
+        return (spike if Ts == 1 else spike / Ts), voltage, current
+
+    @staticmethod
+    def forward(ctx, weightedSpikes, srmKernel, neuron, Ts, delaySteps=0):
+        # the layer needs the voltage for the backward pass only, and never the current
+        needVoltage = ctx.needs_input_grad[0]
+        x, scale = _spike._scaled(weightedSpikes, Ts)
+        spike, voltage, _ = slayerLoihiCuda.getSpikesDelayed(
+            x, neuron["wgtExp"], neuron["theta"], neuron["iDecay"], neuron["vDecay"], neuron["refDelay"],
+            delaySteps, voltage=needVoltage, current=False)
+        if scale != 1:
+            spike = spike / scale
+        if needVoltage:
+            ctx.save_for_backward(voltage, srmKernel.clone().detach())
         ctx.theta = float(neuron["theta"])
         ctx.pdfTimeConstant = float(neuron["tauRho"] * neuron["theta"])
         ctx.pdfScale = float(neuron["scaleRho"])
         ctx.Ts = float(Ts)
+        ctx.delaySteps = int(delaySteps)
         return spike
 
     @staticmethod
     def backward(ctx, gradOutput):
         voltage, srmKernel = ctx.saved_tensors
+        gradOutput = gradOutput.contiguous()
+        if ctx.delaySteps:   # adjoint of the fused delay: the gradient moves back by as many samples
+            gradOutput = slayerCuda.shift(gradOutput, float(ctx.delaySteps), 1.0, sign=-1.0)
         # surrogate gradient and correlation with the PSP kernel in one kernel
-        return slayerCuda.spikeBackwardCorr(gradOutput.contiguous(), voltage, srmKernel, ctx.theta,
-                                            ctx.pdfTimeConstant, ctx.pdfScale, ctx.Ts), None, None, None
+        return slayerCuda.spikeBackwardCorr(gradOutput, voltage, srmKernel, ctx.theta,
+                                            ctx.pdfTimeConstant, ctx.pdfScale, ctx.Ts), None, None, None, None

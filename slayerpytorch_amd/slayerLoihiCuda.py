@@ -1,5 +1,9 @@
 """``slayerLoihiCuda`` for MI355X: the one callable of the reference's pybind11 extension
 (src/cuda/slayerLoihiKernels.cu:48-51), implemented over the C ABI of ``libslayer_hip.so``.
+
+``getSpikesDelayed`` has no counterpart in the reference extension: it is ``getSpikes`` with the
+``delayShift`` that follows it in Loihi networks (src/auto/loihi.py:67-69) fused in and with
+optional voltage / current outputs.
 """
 import operator
 
@@ -8,7 +12,9 @@ import torch
 from . import _lib
 from .slayerCuda import _check_input, _on_device_of, _ptr, _rows
 
-__all__ = ["getSpikes"]
+__all__ = ["getSpikes", "getSpikesDelayed", "MAX_FUSED_DELAY"]
+
+MAX_FUSED_DELAY = 31   # longest spike delay (samples) that getSpikesDelayed fuses into the neuron kernel
 
 
 def _unsigned(x, name):
@@ -26,10 +32,7 @@ def _unsigned(x, name):
     return v
 
 
-def getSpikes(weightedSpikes, wgtExp, theta, iDecay, vDecay, refDelay):
-    """Loihi CUBA neuron on ``weightedSpikes`` (any shape, time last).  Returns
-    ``[spike, voltage, current]`` (src/cuda/slayerLoihiKernels.cu:12-46)."""
-    _check_input(weightedSpikes, "weightedSpikes")
+def _neuron_args(wgtExp, theta, iDecay, vDecay, refDelay):
     wgtExp = _unsigned(wgtExp, "wgtExp")
     theta = _unsigned(theta, "theta")
     iDecay = _unsigned(iDecay, "iDecay")
@@ -42,6 +45,14 @@ def getSpikes(weightedSpikes, wgtExp, theta, iDecay, vDecay, refDelay):
         raise ValueError("wgtExp must be at most 25 (weight scale 1 << (6 + wgtExp) is 32 bit)")
     if theta > 0x7FFFFFFF:
         raise ValueError("theta must fit a signed 32 bit integer")
+    return wgtExp, theta, iDecay, vDecay, refDelay
+
+
+def getSpikes(weightedSpikes, wgtExp, theta, iDecay, vDecay, refDelay):
+    """Loihi CUBA neuron on ``weightedSpikes`` (any shape, time last).  Returns
+    ``[spike, voltage, current]`` (src/cuda/slayerLoihiKernels.cu:12-46)."""
+    _check_input(weightedSpikes, "weightedSpikes")
+    wgtExp, theta, iDecay, vDecay, refDelay = _neuron_args(wgtExp, theta, iDecay, vDecay, refDelay)
     lib = _lib.load()
     spike = torch.empty_like(weightedSpikes)
     voltage = torch.empty_like(weightedSpikes)
@@ -53,3 +64,27 @@ def getSpikes(weightedSpikes, wgtExp, theta, iDecay, vDecay, refDelay):
                                                    vDecay, refDelay, stream),
                    "slayer_loihi_get_spikes_f32")
     return [spike, voltage, current]
+
+
+def getSpikesDelayed(weightedSpikes, wgtExp, theta, iDecay, vDecay, refDelay, delaySteps=0, voltage=True,
+                     current=True):
+    """:func:`getSpikes` whose spike output comes ``delaySteps`` samples late (zeros before), i.e.
+    followed by ``shift(spike, delaySteps)``, in one kernel; ``0 <= delaySteps <= MAX_FUSED_DELAY``.
+    Voltage and current are not shifted; with ``voltage=False`` / ``current=False`` they are not
+    computed into memory at all and ``None`` is returned in their place."""
+    _check_input(weightedSpikes, "weightedSpikes")
+    wgtExp, theta, iDecay, vDecay, refDelay = _neuron_args(wgtExp, theta, iDecay, vDecay, refDelay)
+    delaySteps = _unsigned(delaySteps, "delaySteps")
+    if delaySteps > MAX_FUSED_DELAY:
+        raise ValueError("delaySteps must be at most %d; shift separately for longer delays" % MAX_FUSED_DELAY)
+    lib = _lib.load()
+    spike = torch.empty_like(weightedSpikes)
+    volt = torch.empty_like(weightedSpikes) if voltage else None
+    curr = torch.empty_like(weightedSpikes) if current else None
+    n, T = _rows(weightedSpikes)
+    with _on_device_of(weightedSpikes) as stream:
+        _lib.check(lib.slayer_loihi_get_spikes_delayed_f32(
+            _ptr(spike), _ptr(volt) if voltage else None, _ptr(curr) if current else None,
+            _ptr(weightedSpikes), n, T, wgtExp, theta, iDecay, vDecay, refDelay, delaySteps, stream),
+            "slayer_loihi_get_spikes_delayed_f32")
+    return [spike, volt, curr]

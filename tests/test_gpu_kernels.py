@@ -290,6 +290,40 @@ def test_loihi_bit_exact(impl, shape, refDelay):
     assert want[0].sum() > 0 or shape[-1] < 8
 
 
+@pytest.mark.parametrize("shape", [(2, 16, 8, 8, 300), (3, 41, 64), (1, 3, 1, 1, 350), (2, 70, 96), (5, 1), (9, 33),
+                                   (1, 2, 2000), (64, 40)])
+@pytest.mark.parametrize("delay", [0, 1, 5, 31])
+def test_loihi_delayed_spikes_and_optional_outputs(impl, shape, delay):
+    # the fused form is getSpikes followed by a shift of the spike tensor by `delay` samples;
+    # voltage and current are not shifted and may be left out
+    rng = np.random.default_rng(sum(shape) + delay)
+    w = loihi_input(rng, shape, p=0.3)
+    ws, wv, wu = O.loihi_get_spikes(w, 0, 80 * 64, 1024, 128, 2)
+    want_s = O.shift(ws, float(delay), 1.0)
+    s, v, u = slayerLoihiCuda.getSpikesDelayed(dev(w), 0, 80 * 64, 1024, 128, 2, delay)
+    assert np.array_equal(bits(host(s)), bits(want_s)), "spike"
+    assert np.array_equal(bits(host(v)), bits(wv)), "voltage"
+    assert np.array_equal(bits(host(u)), bits(wu)), "current"
+    s2, v2, u2 = slayerLoihiCuda.getSpikesDelayed(dev(w), 0, 80 * 64, 1024, 128, 2, delay, voltage=True, current=False)
+    assert u2 is None and np.array_equal(host(s2), want_s) and np.array_equal(host(v2), wv)
+    s3, v3, u3 = slayerLoihiCuda.getSpikesDelayed(dev(w), 0, 80 * 64, 1024, 128, 2, delay, voltage=False, current=False)
+    assert v3 is None and u3 is None and np.array_equal(host(s3), want_s)
+    # and it is what the two separate calls give
+    two = slayerCuda.shift(slayerLoihiCuda.getSpikes(dev(w), 0, 80 * 64, 1024, 128, 2)[0], float(delay), 1.0)
+    assert torch.equal(s, two)
+
+
+def test_loihi_delay_limits():
+    w = dev(np.zeros((2, 3, 40), np.float32))
+    with pytest.raises(ValueError):
+        slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 32)
+    with pytest.raises(TypeError):
+        slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, -1)
+    lib = _lib.load()
+    assert lib.slayer_loihi_get_spikes_delayed_f32(None, None, None, None, 4, 8, 0, 5120, 1024, 128, 1, 32, None) == 2
+    assert lib.slayer_loihi_get_spikes_delayed_f32(None, None, None, None, 4, 8, 0, 5120, 1024, 128, 1, -1, None) == 1
+
+
 @pytest.mark.parametrize("params", [(1, 10 * 64, 2048, 256, 3), (0, 64, 0, 0, 1), (2, 5000, 4095, 4095, 2),
                                     (0, 1, 4096, 4096, 1), (3, 300000, 100, 10, 500)])
 def test_loihi_parameters_wraparound_and_truncation(impl, params):

@@ -327,6 +327,28 @@ def test_loihi_autograd_backward():
     assert len(psp) == 110 and nd["scaleRho"] == pytest.approx(2.0 / 195.0)
 
 
+@pytest.mark.parametrize("Ts,delay", [(1.0, 1), (1.0, 40), (0.5, 1.0), (1.0, 0)])
+def test_loihi_spike_with_fused_delay_matches_spike_then_delayShift(Ts, delay):
+    # the Loihi network blocks of the reference do delayShift(spikeLoihi(x), 1); the layer offers it as one call
+    nd = loihi_neuron(scaleRho=2.0)
+    layer = snn.loihi(nd, {"Ts": Ts, "tSample": 300}).to(DEV)
+    rng = np.random.default_rng(11)
+    shape = (2, 6, 5, 5, 300)
+    w = ((2 * rng.integers(-64, 64, size=shape) * (rng.random(shape) < 0.3)) / Ts).astype(np.float32)
+    g = rng.standard_normal(shape).astype(np.float32)
+    a = dev(w).requires_grad_(True)
+    fused = layer.spikeLoihi(a, delay)
+    fused.backward(dev(g))
+    b = dev(w).requires_grad_(True)
+    two = layer.delayShift(layer.spikeLoihi(b), delay)
+    two.backward(dev(g))
+    assert torch.equal(fused, two) and float(fused.detach().sum()) > 0
+    assert torch.equal(a.grad, b.grad)
+    # without a gradient to compute the layer asks the kernel for the spikes only
+    with torch.no_grad():
+        assert torch.equal(layer.spikeLoihi(dev(w), delay), two)
+
+
 def test_loihi_Ts_scaling_of_input_and_output():
     layer = snn.loihi(loihi_neuron(), {"Ts": 0.1, "tSample": 20}).to(DEV)
     rng = np.random.default_rng(4)
