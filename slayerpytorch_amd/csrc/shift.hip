@@ -64,6 +64,57 @@ __global__ __launch_bounds__(256) void shift_vec_kernel(float *__restrict__ out,
     if (active) buffer_store4(bufOut, (r * T + (q << 2)) * 4, 0, y);
 }
 
+// Rows that are not whole 16-byte vectors (T % 4 != 0) in a tensor that is (16-byte aligned,
+// rows * T % 4 == 0, T >= 4, fewer than 2^31 samples): lane g still owns the aligned output
+// vector g of the flattened tensor, which now may hold the end of one row and the start of the
+// next.  Each of the (at most two) row parts is assembled like in the kernel above, from the two
+// aligned input vectors that straddle its shifted position; only the lanes whose vector spans
+// two rows, one in T/4, take the second turn.
+__global__ __launch_bounds__(256) void shift_flat_kernel(float *__restrict__ out, const float *__restrict__ in,
+                                                         const float *__restrict__ lut, int mode, float delayValue,
+                                                         float sign, uint32_t quads, uint32_t nPerBatch, int T,
+                                                         FastDiv byT, FastDiv byBatch, float Ts)
+{
+    const uint32_t g = blockIdx.x * 256u + threadIdx.x;
+    if (g >= quads) return;
+    const float4 *vin = reinterpret_cast<const float4 *>(in);
+    const uint32_t e0 = g << 2;                          // first sample of the vector, flat
+    const uint32_t rowA = fastdiv(e0, byT);
+    const int tA = static_cast<int>(e0 - rowA * static_cast<uint32_t>(T));
+    const int nA = min(4, T - tA);                       // samples of the vector that belong to rowA
+
+    float y[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    // samples j0 .. j0+count-1 of the vector are the samples tStart .. of `row`
+    auto part = [&](uint32_t row, int tStart, int j0, int count) {
+        int k;
+        if (mode == kShiftValue) k = delay_steps(delayValue * sign, Ts);
+        else if (mode == kShiftDeviceScalar) k = delay_steps(lut[0] * sign, Ts);
+        else k = delay_steps(lut[row - fastdiv(row, byBatch) * nPerBatch] * sign, Ts);
+        k = max(-T, min(T, k));
+        // the vector's sample j comes from flat position q + j
+        const int q = static_cast<int>(row) * T + tStart - k - j0;
+        const int va = q >> 2, sh = q & 3;               // floor division
+        const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        float4 a = zero, b = zero;
+        if (va >= 0 && va < static_cast<int>(quads)) a = vin[va];
+        if (sh != 0 && va + 1 >= 0 && va + 1 < static_cast<int>(quads)) b = vin[va + 1];
+        float c[4] = {a.x, a.y, a.z, a.w};
+        if (sh == 1) { c[0] = a.y; c[1] = a.z; c[2] = a.w; c[3] = b.x; }
+        if (sh == 2) { c[0] = a.z; c[1] = a.w; c[2] = b.x; c[3] = b.y; }
+        if (sh == 3) { c[0] = a.w; c[1] = b.x; c[2] = b.y; c[3] = b.z; }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int src = tStart + (j - j0) - k;       // source time within the row
+            if (j >= j0 && j < j0 + count && src >= 0 && src < T) y[j] = c[j];
+        }
+    };
+    part(rowA, tA, 0, nA);
+    if (nA < 4) part(rowA + 1, 0, nA, 4 - nA);
+    typedef float vec4f __attribute__((ext_vector_type(4)));
+    const vec4f o = {y[0], y[1], y[2], y[3]};
+    __builtin_nontemporal_store(o, reinterpret_cast<vec4f *>(out) + g);
+}
+
 // Any T, any alignment: one sample per lane, lanes along time (coalesced 256-byte runs).
 __global__ __launch_bounds__(256) void shift_scalar_kernel(float *__restrict__ out,
                                                            const float *__restrict__ in,
@@ -105,6 +156,14 @@ static int launch_shift(float *out, const float *in, const float *lut, int mode,
                            in, lut, mode, delayValue, sign, static_cast<uint32_t>(quads),
                            static_cast<uint32_t>(nPerBatch), static_cast<int>(T),
                            make_fastdiv(static_cast<uint32_t>(T / 4)), Ts);
+        return launch_status();
+    }
+    if (T % 4 != 0 && T >= 4 && aligned16(out) && aligned16(in) && (rows * T) % 4 == 0 && rows * T < (1LL << 31)) {
+        const int64_t quads = rows * T / 4;
+        hipLaunchKernelGGL(shift_flat_kernel, dim3(static_cast<unsigned>(ceil_div(quads, 256))), dim3(256), 0, stream,
+                           out, in, lut, mode, delayValue, sign, static_cast<uint32_t>(quads),
+                           static_cast<uint32_t>(nPerBatch), static_cast<int>(T), make_fastdiv(static_cast<uint32_t>(T)),
+                           make_fastdiv(static_cast<uint32_t>(nPerBatch > 0 ? nPerBatch : 1)), Ts);
         return launch_status();
     }
     const int64_t rowsPerBlock = T >= 256 ? 1 : 256 / T;

@@ -69,6 +69,22 @@ def test_shift_scalar_exact(delay, Ts, T):
         assert np.array_equal(bits(host(slayerCuda.shift(dev(x), delay))), bits(want))      # Ts defaults to 1
 
 
+@pytest.mark.parametrize("shape", [(4, 3, 1, 1, 5), (2, 6, 1, 1, 6), (8, 5, 1, 1, 7), (4, 9, 2, 1, 101), (2, 2, 3, 5, 350),
+                                   (4, 1, 1, 1, 2001), (1, 4, 1, 1, 4097)])
+def test_shift_rows_that_are_not_whole_vectors(shape):
+    # T % 4 != 0 with rows * T % 4 == 0: aligned output vectors span two rows with different delays
+    rng = np.random.default_rng(shape[-1])
+    T = shape[-1]
+    x = rng.standard_normal(shape).astype(np.float32)
+    d = np.round((rng.random(shape[1:4]) * 2 - 1) * (T + 3)).astype(np.float32)     # up to beyond the row length
+    d.reshape(-1)[0] = 0.0
+    for sign in (1.0, -1.0):
+        got = host(slayerCuda.shift(dev(x), dev(d), 1.0, sign=sign))
+        assert np.array_equal(bits(got), bits(O.shift(x, sign * d, 1.0)))
+    for delay in (1.0, -1.0, 3.0, float(T - 1), float(T), -float(T + 5), 0.0):
+        assert np.array_equal(bits(host(slayerCuda.shift(dev(x), delay, 1.0))), bits(O.shift(x, delay, 1.0)))
+
+
 def test_shift_unaligned_storage_offset():
     rng = np.random.default_rng(11)
     base = dev(rng.standard_normal(2 * 3 * 64 + 1).astype(np.float32))
