@@ -153,7 +153,14 @@ constexpr int kTileMaxPiece = 352;  // longest piece (samples per row) a tile st
 // leave a piece are the ones LAG before its end, so with several pieces per row LAG = 32 keeps
 // every run of stores on 128-byte boundaries of the row (partial lines are expensive to write).
 // R: rows per tile (16, or 8 when the tensor has too few rows to fill the GPU with 16-row tiles).
-template <int NU, bool VEC, int LAG, int R>
+// MODE: how global memory is accessed.  kTileVec: rows are whole 16-byte vectors.  kTileFlat:
+// they are not (T % 4 != 0), but the rows of a tile travel whole and an 8-row tile is one
+// contiguous, 16-byte aligned run of whole vectors, so it is still moved with 16-byte accesses;
+// a vector may then hold the end of one row and the start of the next, and its four samples are
+// placed into (gathered from) LDS one by one.  kTileScalar: anything else, one sample per access.
+constexpr int kTileScalar = 0, kTileVec = 1, kTileFlat = 2;
+
+template <int NU, int MODE, int LAG, int R>
 __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, float *u,
                                                         const float *__restrict__ nu, int64_t rows,
                                                         int T, int nuSize, int Tc, int P, int MP,
@@ -161,8 +168,9 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 {
     static_assert(LAG >= NU - 1 && LAG % 4 == 0, "the window must cover the refractory kernel");
     constexpr int G = 32;               // samples per walk group = bits of a spike mask
-    constexpr int V = VEC ? 4 : 1;      // samples per global access
-    constexpr int NB = R * kTileMaxPiece / V / kWave;  // accesses per lane per piece, at most
+    constexpr bool VEC = MODE == kTileVec, FLAT = MODE == kTileFlat;
+    constexpr int V = VEC ? 4 : 1;      // samples per (row-wise) global access
+    constexpr int NB = R * kTileMaxPiece / (FLAT ? 4 : V) / kWave;  // accesses per lane per piece, at most
     extern __shared__ __align__(16) float lds[];
     float *tile = lds;                                                    // [R][P], P = 4 (mod 32)
     uint32_t *masks = reinterpret_cast<uint32_t *>(lds + R * P);  // [R][MP]
@@ -179,10 +187,20 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 
     // A "step" is one piece of one tile.  The global loads of a step are issued one step ahead
     // into x[] and stay in flight while the previous step is walked and retired.
-    float x[NB * V];
+    float x[NB * (FLAT ? 4 : V)];
     auto rows_of = [&](int64_t t) { return static_cast<int>(min(static_cast<int64_t>(R), rows - t * R)); };
+    const float invT = 1.0f / static_cast<float>(T);
     auto issue = [&](int64_t t, int tL) {
         const BufferRsrc bufU = make_buffer(u + t * R * static_cast<int64_t>(T));
+        if constexpr (FLAT) {  // whole rows: the tile is rows_of(t) * T / 4 consecutive vectors
+            const int nVec = (rows_of(t) * T) >> 2;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const float4 q = buffer_load4(bufU, masked_offset(lane + b * kWave < nVec, (lane + b * kWave) * 16), 0);
+                x[4 * b] = q.x; x[4 * b + 1] = q.y; x[4 * b + 2] = q.z; x[4 * b + 3] = q.w;
+            }
+            return;
+        }
         const int n = min(Tc, T - tL);
         const int perRow = n / V;
         const int total = rows_of(t) * perRow;
@@ -204,6 +222,22 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         }
     };
     auto commit = [&](int64_t t, int tL) {  // tile[r][LAG + c] = u[row][tL + c]
+        if constexpr (FLAT) {
+            const int nVec = (rows_of(t) * T) >> 2;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                if (lane + b * kWave < nVec) {
+                    int r, c;
+                    divmod_small((lane + b * kWave) << 2, T, invT, r, c);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        tile[r * P + LAG + c] = x[4 * b + e];
+                        if (++c == T) { c = 0; ++r; }
+                    }
+                }
+            }
+            return;
+        }
         const int n = min(Tc, T - tL);
         const int perRow = n / V;
         const int total = rows_of(t) * perRow;
@@ -282,6 +316,23 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         {
             const BufferRsrc bufU = make_buffer(u + t * R * static_cast<int64_t>(T));
             const BufferRsrc bufS = make_buffer(s + t * R * static_cast<int64_t>(T));
+            if constexpr (FLAT) {
+                const int nVec = (nRows * T) >> 2;
+                for (int vi = lane; vi < nVec; vi += kWave) {
+                    int r, c;
+                    divmod_small(vi << 2, T, invT, r, c);
+                    float uu[4], ss[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int col = LAG + c;   // time c of row r
+                        uu[e] = tile[r * P + col];
+                        ss[e] = ((masks[r * MP + (col >> 5)] >> (col & 31)) & 1u) ? amplitude : 0.0f;
+                        if (++c == T) { c = 0; ++r; }
+                    }
+                    buffer_store4(bufU, vi * 16, 0, make_float4(uu[0], uu[1], uu[2], uu[3]));
+                    buffer_store4(bufS, vi * 16, 0, make_float4(ss[0], ss[1], ss[2], ss[3]));
+                }
+            } else {
             const int first = (tL == 0) ? LAG : 0;  // before the first sample there is nothing to store
             const int perRow = (W - first) / V;
             const int total = nRows * perRow;
@@ -304,6 +355,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                     buffer_store(bufS, off, 0, (m & 1u) ? amplitude : 0.0f);
                 }
                 rc.advance(dr, dc, perRow);
+            }
             }
         }
         wave_sync();
@@ -359,13 +411,18 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
 #define SLAYER_SPIKE_TILE_LAUNCH(NU, LAGV, RV)                                                           \
     do {                                                                                                \
         if (vec)                                                                                        \
-            hipLaunchKernelGGL((spike_tile_kernel<NU, true, LAGV, RV>), dim3(grid), dim3(kWave), lds,   \
-                               st, s, u, nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize),   \
-                               Tc, P, MP, tiles, theta, Ts);                                            \
+            hipLaunchKernelGGL((spike_tile_kernel<NU, kTileVec, LAGV, RV>), dim3(grid), dim3(kWave),    \
+                               lds, st, s, u, nu, nNeurons, static_cast<int>(T),                        \
+                               static_cast<int>(nuSize), Tc, P, MP, tiles, theta, Ts);                  \
+        else if (flat && RV == 8)                                                                       \
+            hipLaunchKernelGGL((spike_tile_kernel<NU, (RV == 8 ? kTileFlat : kTileScalar), LAGV, RV>),  \
+                               dim3(grid), dim3(kWave), lds, st, s, u, nu, nNeurons,                    \
+                               static_cast<int>(T), static_cast<int>(nuSize), Tc, P, MP, tiles, theta,  \
+                               Ts);                                                                     \
         else                                                                                            \
-            hipLaunchKernelGGL((spike_tile_kernel<NU, false, LAGV, RV>), dim3(grid), dim3(kWave), lds,  \
-                               st, s, u, nu, nNeurons, static_cast<int>(T), static_cast<int>(nuSize),   \
-                               Tc, P, MP, tiles, theta, Ts);                                            \
+            hipLaunchKernelGGL((spike_tile_kernel<NU, kTileScalar, LAGV, RV>), dim3(grid), dim3(kWave), \
+                               lds, st, s, u, nu, nNeurons, static_cast<int>(T),                        \
+                               static_cast<int>(nuSize), Tc, P, MP, tiles, theta, Ts);                  \
         return launch_status();                                                                         \
     } while (0)
 #define SLAYER_SPIKE_TILE_LAG(NU, LAGV)                                                                  \
@@ -397,6 +454,8 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
         const bool whole = T <= kTileMaxPiece;
         const int Tc = whole ? static_cast<int>(T) : 256;
         const bool vec = (T % 4 == 0) && aligned16(s) && aligned16(u);
+        // whole rows that are not whole vectors, in a tensor that is: 8-row tiles are aligned runs
+        const bool flat = whole && !vec && T >= 4 && (nNeurons * T) % 4 == 0 && aligned16(s) && aligned16(u);
         const int cus = compute_units();
         if (nuSize <= 4) SLAYER_SPIKE_TILE(4);
         if (nuSize <= 8) SLAYER_SPIKE_TILE(8);

@@ -194,6 +194,9 @@ SPIKE_CASES = [
     ((3, 5, 2, 2, 95), 1), ((3, 5, 2, 2, 96), 0), ((2, 9, 3, 1, 97), 33), ((2, 9, 3, 1, 130), 34),
     ((2, 9, 3, 1, 200), 97), ((1, 70, 1, 1, 500), 110), ((1, 20, 1, 1, 501), 160), ((2, 2, 2, 2, 1), 11),
     ((1, 4, 1, 1, 7), 11),
+    # rows that are not whole 16-byte vectors in tensors that are: 8-row tiles move as flat runs
+    ((2, 4, 3, 1, 350), 11), ((4, 5, 1, 1, 101), 8), ((1, 8, 1, 1, 5), 3), ((1, 12, 1, 1, 351), 24),
+    ((3, 4, 1, 1, 349), 16), ((1, 6, 1, 1, 101), 11),
 ]
 
 
