@@ -273,7 +273,14 @@ __global__ __launch_bounds__(64) void loihi_tile_kernel(float *__restrict__ s, f
 // registers and hands them over when row r reaches that line, so that it goes out once, whole.
 // Only the first and the last row of a tile still write a partial line.
 // R rows per tile (= lanes that update), LPP = 128-byte lines per row and piece.
-template <int R, int LPP, bool MERGE>
+//
+// ELEM (with MERGE): rows that are not whole 16-byte vectors (T % 4 != 0) in tensors that are
+// (16-byte aligned, rows * T % 4 == 0).  Lines and vectors are cut from memory, not from rows, so
+// all accesses stay aligned; what changes is that the vector in which a row ends can also hold
+// the first samples of the next row.  Loads simply fetch such a vector for both rows, and the
+// hand-over of a row's first line to the row above works sample by sample.  R * T * 4 is a
+// multiple of 128 for R = 32, so a tile still begins and ends on a line boundary.
+template <int R, int LPP, bool MERGE, bool ELEM = false>
 __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, float *__restrict__ v,
                                                          float *__restrict__ u, const float *__restrict__ w,
                                                          int64_t rows, int T, int64_t tiles, LoihiParams p)
@@ -294,6 +301,7 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
     const int pieces = (T + G - 1 + TC - 1) / TC;  // enough for the most skewed row
 
     static_assert(!MERGE || (LPP == 1 && R <= kWave), "line merging is written for one line per piece");
+    static_assert(!ELEM || (MERGE && (R * 4) % 128 == 0), "rows that are not whole vectors need merged lines and line-aligned tiles");
     LoihiState st = {0, 0, 0};
     float4 x[NB];
     float headC[MERGE ? G : 1], headV[MERGE ? G : 1];  // results of this row's first line (MERGE)
@@ -313,7 +321,8 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
         for (int b = 0; b < NB; ++b) {
             const int r = b * RPI + subRow;
             const int time = TC * j - ((o0 + r * T) & 31) + col;
-            x[b] = buffer_load4(bufW, masked_offset(r < nRows && time >= 0 && time < T, (r * T + time) * 4), 0);
+            // any sample of the vector inside the row (with whole-vector rows: all or none)
+            x[b] = buffer_load4(bufW, masked_offset(r < nRows && time + 3 >= 0 && time < T, (r * T + time) * 4), 0);
         }
     };
 
@@ -411,11 +420,18 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
                 if (lane > 0 && lane < nRows && skew > 0 && j == lastAbove) {
                     float *aboveC = tileC + (lane - 1) * P;
                     float *aboveV = tileV + (lane - 1) * P;
+                    if (ELEM) {
 #pragma unroll
-                    for (int k = 0; k < G; k += 4) {
-                        if (k >= skew) {
-                            *reinterpret_cast<float4 *>(aboveC + k) = make_float4(headC[k], headC[k + 1], headC[k + 2], headC[k + 3]);
-                            *reinterpret_cast<float4 *>(aboveV + k) = make_float4(headV[k], headV[k + 1], headV[k + 2], headV[k + 3]);
+                        for (int k = 0; k < G; ++k) {
+                            if (k >= skew) { aboveC[k] = headC[k]; aboveV[k] = headV[k]; }
+                        }
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < G; k += 4) {
+                            if (k >= skew) {
+                                *reinterpret_cast<float4 *>(aboveC + k) = make_float4(headC[k], headC[k + 1], headC[k + 2], headC[k + 3]);
+                                *reinterpret_cast<float4 *>(aboveV + k) = make_float4(headV[k], headV[k + 1], headV[k + 2], headV[k + 3]);
+                            }
                         }
                     }
                     masks[lane - 1] |= headFired;
@@ -499,6 +515,18 @@ static int launch_loihi(float *s, float *v, float *u, const float *w, int64_t nN
         const bool samePhase = (reinterpret_cast<uintptr_t>(s) & 127) == phase &&
                                (!v || (reinterpret_cast<uintptr_t>(v) & 127) == phase) &&
                                (!u || (reinterpret_cast<uintptr_t>(u) & 127) == phase);
+        const bool elem = (T % 4 != 0) && T >= 64 && (nNeurons * T) % 4 == 0 && aligned16(s) && aligned16(v) &&
+                          aligned16(u) && aligned16(w) && samePhase && LOIHI_LPP == 1 && LOIHI_ROWS == 32;
+        if (elem) {
+            constexpr int kR = 32;
+            const int64_t lineTiles = ceil_div(nNeurons, kR);
+            const int64_t ldsBytes = (2LL * kR * (32 + 4) + kR) * 4;
+            const int64_t fit = static_cast<int64_t>(compute_units()) * (160 * 1024 / ldsBytes);
+            const dim3 grid(static_cast<unsigned>(lineTiles < fit ? lineTiles : fit));
+            hipLaunchKernelGGL((loihi_lines_kernel<kR, 1, true, true>), grid, dim3(kWave), 0, st, s, v, u, w, nNeurons,
+                               static_cast<int>(T), lineTiles, p);
+            return launch_status();
+        }
         if (vec && samePhase) {
             constexpr int kR = LOIHI_ROWS, kLpp = LOIHI_LPP;
             const int64_t lineTiles = ceil_div(nNeurons, kR);

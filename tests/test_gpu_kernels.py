@@ -371,6 +371,22 @@ def test_loihi_rows_sharing_memory_lines(impl, T, rows):
     assert want[0].sum() > 0
 
 
+@pytest.mark.parametrize("T", [65, 66, 67, 95, 97, 101, 127, 129, 350, 351, 2001])
+@pytest.mark.parametrize("rows", [(4, 1), (4, 33), (8, 8), (2, 2, 3, 5), (12, 3)])
+@pytest.mark.parametrize("delay", [0, 3])
+def test_loihi_rows_that_are_not_whole_vectors(impl, T, rows, delay):
+    # T % 4 != 0 in a tensor of whole vectors: the 16-byte vector in which a row ends also holds the
+    # first samples of the next row; tiles of 32 rows still begin and end on memory lines
+    rng = np.random.default_rng(T + len(rows))
+    w = loihi_input(rng, rows + (T,), p=0.3)
+    ws, wv, wu = O.loihi_get_spikes(w, 0, 20 * 64, 1024, 128, 2)
+    s, v, u = slayerLoihiCuda.getSpikesDelayed(dev(w), 0, 20 * 64, 1024, 128, 2, delay)
+    assert np.array_equal(bits(host(s)), bits(O.shift(ws, float(delay), 1.0))), "spike"
+    assert np.array_equal(bits(host(v)), bits(wv)), "voltage"
+    assert np.array_equal(bits(host(u)), bits(wu)), "current"
+    assert ws.sum() > 0
+
+
 def test_loihi_unaligned_tensors_take_the_general_kernel():
     rng = np.random.default_rng(77)
     w = loihi_input(rng, (2 * 40 * 96 + 1,), p=0.3)
