@@ -28,6 +28,9 @@ namespace slayer {
 constexpr int kFirMaxLdsFloats = 12288;  // 48 KiB of LDS per work-group at most
 constexpr int kFirMaxPitch = 512;     // longest LDS row (samples) the tiled kernel stages
 
+// four floats that need not be 16-byte aligned (the GPU's global memory accesses may be unaligned)
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
+
 // Optional gate on the input: the filter then runs over in[n][t] * gain * exp(-|u[n][t] - theta| / tau),
 // i.e. the spike function's surrogate gradient applied on the way in (u == nullptr: no gate).
 struct FirGate {
@@ -375,14 +378,13 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
             auto at = [&](int t) { return GATED ? gated(src[t], gsrc[t]) : src[t]; };
             const int j = j4 << 2;
             float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            const int tl = CAUSAL ? tHi - j - 3 : t0 + j;  // lowest time of the quad (X order is descending for conv)
             if (CAUSAL) {
-                const int tl = tHi - j - 3;  // lowest time of the quad; X order is descending
                 if (tl + 3 >= 0 && tl + 3 < T) v.x = at(tl + 3);
                 if (tl + 2 >= 0 && tl + 2 < T) v.y = at(tl + 2);
                 if (tl + 1 >= 0 && tl + 1 < T) v.z = at(tl + 1);
                 if (tl >= 0 && tl < T) v.w = at(tl);
             } else {
-                const int tl = t0 + j;
                 if (tl < T) v.x = at(tl);
                 if (tl + 1 < T) v.y = at(tl + 1);
                 if (tl + 2 < T) v.z = at(tl + 2);
@@ -446,8 +448,17 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
         } else {
             float *dst = out + (row0 + r) * static_cast<int64_t>(T);
 #pragma unroll
-            for (int j = 0; j < U; ++j)
-                if (tl + j >= t0 && tl + j < t0 + tt) dst[tl + j] = y[j];
+            for (int v = 0; v < U / 4; ++v) {
+                const int tv = tl + 4 * v;
+                if (tv >= t0 && tv + 3 < t0 + tt) {
+                    const float4u q = {y[4 * v], y[4 * v + 1], y[4 * v + 2], y[4 * v + 3]};
+                    *reinterpret_cast<float4u *>(dst + tv) = q;   // 16 bytes at any alignment
+                } else {
+#pragma unroll
+                    for (int j = 4 * v; j < 4 * v + 4; ++j)
+                        if (tl + j >= t0 && tl + j < t0 + tt) dst[tl + j] = y[j];
+                }
+            }
         }
     }
 }
