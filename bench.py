@@ -175,6 +175,19 @@ def other_rows(device):
     out.append(row("psp_corr_8tap", 8, n, timed(lambda: slayerCuda.corr(grad, srm8, 1.0)), shape))
     out.append(row("spike_T2000", 12, n, timed(lambda: slayerCuda.getSpikes(ub, ref, 10.0, 1.0), lambda: ub.copy_(u0)), shape))
     del x, grad, u0, ub, y
+    # MLP ordering spike(psp(fc(x))): dense input to the 77-tap PSP filter, then the spike function
+    shape = SHAPE
+    a = (torch.randn(shape, generator=g) * 2).to(device)
+    srm77 = torch.tensor(alphaKernel(10.0, 1.0, 300), dtype=torch.float32, device=device)
+    ref11 = torch.tensor(alphaKernel(1.0, 1.0, 300, mult=-20.0), dtype=torch.float32, device=device)
+    out.append(row("psp77_then_spike_fused", 20, a.numel(), timed(lambda: slayerCuda.pspSpike(a, srm77, ref11, 10.0, 1.0)),
+                   shape))
+    out.append(row("psp77_then_spike_two_kernels", 20, a.numel(),
+                   timed(lambda: slayerCuda.getSpikes(slayerCuda.conv(a, srm77, 1.0), ref11, 10.0, 1.0)), shape))
+    gs = torch.randn(shape, generator=g).to(device)
+    out.append(row("spike_pdf_then_corr77_fused", 20, a.numel(),
+                   timed(lambda: slayerCuda.spikeBackwardCorr(gs, a, srm77, 10.0, 10.0, 1.0, 1.0)), shape))
+    del a, gs
     # Loihi config: largest tensor (8, 16, 32, 32, 300)
     shape = (8, 16, 32, 32, 300)
     w = (2 * torch.randint(-128, 128, shape, generator=g) * (torch.rand(shape, generator=g) < 0.05)).float().to(device)

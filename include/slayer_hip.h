@@ -143,6 +143,21 @@ int slayer_spike_bwd_corr_f32(float *gradIn, const float *gradOut, const float *
                               const float *filt, int64_t nNeurons, int64_t T, int64_t F,
                               float theta, float tau, float scale, float Ts, void *stream);
 
+/*
+ * PSP filter followed by the spike function in one kernel, for layers that apply them back to
+ * back: spike(psp(x)), the ordering of the reference's MLP example
+ * (example/02_NMNIST_MLP/nmnistMLP.py:59-60).  Replaces the call pair slayerCuda.conv
+ * (src/cuda/slayerKernels.cu:41-57) -> slayerCuda.getSpikes (src/cuda/slayerKernels.cu:14-39).
+ *
+ * u = Ts * conv(a, srm) as in slayer_conv_f32, then s and the refractory update of u as in
+ * slayer_get_spikes_f32: the same values bit for bit, without the round trip of u through
+ * memory when rows are whole 16-byte vectors of at most 352 samples, nuSize <= 24 and F <= 160;
+ * other shapes run the two kernels one after the other.  u and s must not alias a.
+ */
+int slayer_psp_spike_f32(float *s, float *u, const float *a, const float *srm, const float *nu,
+                         int64_t nNeurons, int64_t T, int64_t F, int64_t nuSize, float theta,
+                         float Ts, void *stream);
+
 /* Bytes of caller-provided device workspace that slayer_delay_grad_f32 needs (may be 0). */
 int64_t slayer_delay_grad_workspace_bytes(int64_t nBatch, int64_t nPerBatch, int64_t T);
 

@@ -22,6 +22,7 @@
 //    is at the FP32 ridge of the machine: on dense input the kernel is FMA-issue bound;
 //  * generic: one lane per output, any shape.
 #include "common.h"
+#include "fir_core.h"
 
 namespace slayer {
 
@@ -144,88 +145,7 @@ __global__ __launch_bounds__(256) void fir_direct_kernel(float *__restrict__ out
 }
 
 // ---- tiled kernel ---------------------------------------------------------------------------------
-// A lane produces U consecutive outputs from a register window of U + 4 samples held as
-// NQ = U/4 + 1 16-byte vectors q[].  ROT says which vector currently holds the oldest samples:
-// window sample e is component e % 4 of q[(ROT + e / 4) % NQ].  After a 4-tap block the oldest
-// vector is replaced by the next one from LDS and ROT advances, so the window slides without any
-// register moves once the loops are unrolled.
-template <int U, int ROT>
-__device__ __forceinline__ void window_of(float (&w)[U + 4], const float4 (&q)[U / 4 + 1])
-{
-    constexpr int NQ = U / 4 + 1;
-#pragma unroll
-    for (int v = 0; v < NQ; ++v) {
-        const float4 &x = q[(ROT + v) % NQ];
-        w[4 * v] = x.x; w[4 * v + 1] = x.y; w[4 * v + 2] = x.z; w[4 * v + 3] = x.w;
-    }
-}
-
-// taps f0..f3 are filter taps i..i+3; output j, tap s uses window sample j + s
-template <int U, int ROT>
-__device__ __forceinline__ void fma_block(float (&acc)[U], const float4 (&q)[U / 4 + 1], float f0, float f1,
-                                          float f2, float f3)
-{
-    float w[U + 4];
-    window_of<U, ROT>(w, q);
-#pragma unroll
-    for (int j = 0; j < U; ++j) {
-        acc[j] = __builtin_fmaf(w[j + 0], f0, acc[j]);
-        acc[j] = __builtin_fmaf(w[j + 1], f1, acc[j]);
-        acc[j] = __builtin_fmaf(w[j + 2], f2, acc[j]);
-        acc[j] = __builtin_fmaf(w[j + 3], f3, acc[j]);
-    }
-}
-
-// the last 1..3 taps of a filter whose length is not a multiple of 4
-template <int U, int ROT>
-__device__ __forceinline__ void fma_rest(float (&acc)[U], const float4 (&q)[U / 4 + 1], const float *__restrict__ f,
-                                         int n)
-{
-    float w[U + 4];
-    window_of<U, ROT>(w, q);
-    const float f0 = f[0];
-    const float f1 = n > 1 ? f[1] : 0.0f;
-    const float f2 = n > 2 ? f[2] : 0.0f;
-#pragma unroll
-    for (int j = 0; j < U; ++j) {
-        acc[j] = __builtin_fmaf(w[j], f0, acc[j]);
-        if (n > 1) acc[j] = __builtin_fmaf(w[j + 1], f1, acc[j]);
-        if (n > 2) acc[j] = __builtin_fmaf(w[j + 2], f2, acc[j]);
-    }
-}
-
-// blocks B, B+1, .., NQ-1 of one trip of the main loop (NQ blocks = 4 NQ taps per trip)
-template <int U, int B>
-struct TripBlocks {
-    static __device__ __forceinline__ void run(float (&acc)[U], float4 (&q)[U / 4 + 1], const float4 *xq, int qi,
-                                               const float *__restrict__ f)
-    {
-        if constexpr (B < U / 4 + 1) {
-            fma_block<U, B>(acc, q, f[4 * B], f[4 * B + 1], f[4 * B + 2], f[4 * B + 3]);
-            q[B] = xq[qi + B];
-            TripBlocks<U, B + 1>::run(acc, q, xq, qi, f);
-        }
-    }
-};
-
-// up to NQ-1 further whole blocks after the main loop, then the rest; B = blocks done so far
-template <int U, int B>
-struct TailBlocks {
-    static __device__ __forceinline__ void run(float (&acc)[U], float4 (&q)[U / 4 + 1], const float4 *xq, int qi,
-                                               const float *__restrict__ f, int left)
-    {
-        if constexpr (B < U / 4 + 1) {
-            if (left >= 4) {
-                fma_block<U, B>(acc, q, f[0], f[1], f[2], f[3]);
-                q[B] = xq[qi];
-                TailBlocks<U, B + 1>::run(acc, q, xq, qi + 1, f + 4, left - 4);
-            } else if (left > 0) {
-                fma_rest<U, B>(acc, q, f, left);
-            }
-        }
-    }
-};
-
+// (the register-window core, window_of .. TailBlocks, is in fir_core.h)
 // true when any of the four samples is not (plus or minus) zero
 __device__ __forceinline__ bool any_nonzero(const float4 &v)
 {

@@ -77,6 +77,12 @@ class spikeLayer(nn.Module):
         updated in place with the refractory response, as in the reference."""
         return _spikeFunction.apply(membranePotential, self.refKernel, self.neuron, self.simulation["Ts"])
 
+    def pspSpike(self, input):
+        """``spike(psp(input))`` - the layer ordering of the reference's MLP example
+        (example/02_NMNIST_MLP/nmnistMLP.py:59-60) - as one forward and one backward kernel
+        (extension; same values as the two calls)."""
+        return _pspSpikeFunction.apply(input, self.srmKernel, self.refKernel, self.neuron, self.simulation["Ts"])
+
     def delayShift(self, input, delay, Ts=1):
         """Delays ``input`` in time by ``delay`` (number, one-element tensor, or one value per
         neuron); the gradient flows to ``input`` only."""
@@ -140,6 +146,30 @@ class _spikeFunction(torch.autograd.Function):
         gradInput = slayerCuda.spikeBackward(gradOutput.contiguous(), membranePotential.contiguous(),
                                              ctx.theta, ctx.pdfTimeConstant, ctx.pdfScale)
         return gradInput, None, None, None
+
+
+class _pspSpikeFunction(torch.autograd.Function):
+    """``_pspFunction`` followed by ``_spikeFunction`` (src/slayer.py:817-899) as one Function:
+    forward is ``slayerCuda.pspSpike``; backward is the spike function's surrogate gradient
+    followed by the correlation with the SRM kernel, also in one kernel."""
+
+    @staticmethod
+    def forward(ctx, input, srmKernel, refractoryResponse, neuron, Ts):
+        spikes, membranePotential = slayerCuda.pspSpike(input.contiguous(), srmKernel, refractoryResponse,
+                                                        neuron["theta"], Ts)
+        ctx.save_for_backward(membranePotential, srmKernel)
+        ctx.theta = float(neuron["theta"])
+        ctx.pdfTimeConstant = float(neuron["tauRho"] * neuron["theta"])
+        ctx.pdfScale = float(neuron["scaleRho"])
+        ctx.Ts = float(Ts)
+        return spikes
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        membranePotential, srmKernel = ctx.saved_tensors
+        gradInput = slayerCuda.spikeBackwardCorr(gradOutput.contiguous(), membranePotential, srmKernel, ctx.theta,
+                                                 ctx.pdfTimeConstant, ctx.pdfScale, ctx.Ts)
+        return gradInput, None, None, None, None
 
 
 class _pspFunction(torch.autograd.Function):

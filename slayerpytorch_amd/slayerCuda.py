@@ -17,10 +17,11 @@ Python numbers or 0-dim tensors, as with pybind11's float conversion.  Outputs a
 with ``torch.empty_like``; kernels are enqueued on PyTorch's current stream of the tensor's
 device and never synchronise with the host.
 
-``spikeBackward``, ``spikeBackwardCorr``, ``delayGrad`` and the ``sign`` argument of ``shift``
-have no counterpart in the reference extension: they are the fused forms of the elementwise
-chains in ``_spikeFunction.backward`` / ``_delayFunction.backward`` (src/slayer.py:857-865,
-944-957) and of ``slayerLoihi._spike.backward`` (src/slayerLoihi.py:278-283).
+``spikeBackward``, ``spikeBackwardCorr``, ``pspSpike``, ``delayGrad`` and the ``sign`` argument
+of ``shift`` have no counterpart in the reference extension: they are the fused forms of the
+elementwise chains in ``_spikeFunction.backward`` / ``_delayFunction.backward``
+(src/slayer.py:857-865, 944-957), of ``slayerLoihi._spike.backward`` (src/slayerLoihi.py:278-283)
+and of the call pair ``spike(psp(x))``.
 """
 import numbers
 
@@ -28,7 +29,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "spikeBackwardCorr", "delayGrad"]
+__all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "spikeBackwardCorr", "pspSpike", "delayGrad"]
 
 
 def _check_input(x, name):
@@ -202,6 +203,29 @@ def spikeBackward(gradOutput, membranePotential, theta, tau, scale):
                                             theta, tau, scale, gradOutput.numel(), stream),
                    "slayer_spike_bwd_f32")
     return gradInput
+
+
+def pspSpike(input, srmKernel, refKernel, theta, Ts):
+    """``conv(input, srmKernel, Ts)`` followed by ``getSpikes`` on the result, in one kernel where
+    the shape allows.  Returns ``(spike, membranePotential)``; the membrane potential is the
+    one after the refractory updates, as ``getSpikes`` leaves it."""
+    _check_input(input, "input")
+    _check_input(srmKernel, "srmKernel")
+    _check_input(refKernel, "refKernel")
+    _check_device(input, srmKernel, "input", "srmKernel")
+    _check_device(input, refKernel, "input", "refKernel")
+    if input.dim() != 5:
+        raise RuntimeError("pspSpike expects a 5 dimensional (N,C,H,W,T) tensor, got %d dimensions" % input.dim())
+    theta, Ts = _scalar(theta, "theta"), _scalar(Ts, "Ts")
+    lib = _lib.load()
+    spike = torch.empty_like(input)
+    u = torch.empty_like(input)
+    n, T = _rows(input)
+    with _on_device_of(input) as stream:
+        _lib.check(lib.slayer_psp_spike_f32(_ptr(spike), _ptr(u), _ptr(input), _ptr(srmKernel), _ptr(refKernel),
+                                            n, T, srmKernel.numel(), refKernel.numel(), theta, Ts, stream),
+                   "slayer_psp_spike_f32")
+    return spike, u
 
 
 def spikeBackwardCorr(gradOutput, membranePotential, filter, theta, tau, scale, Ts):

@@ -274,6 +274,27 @@ def test_spike_bwd_corr_is_the_two_ops_in_one(impl, shape, Fl):
     assert rel_err(got, want) <= REL_TOL
 
 
+@pytest.mark.parametrize("shape,Fl,nuSize", [((2, 6, 5, 3, 300), 77, 11), ((1, 9, 1, 1, 352), 160, 24), ((3, 7, 1, 1, 64), 8, 4),
+                                             ((1, 1, 1, 1, 4), 1, 1), ((2, 5, 1, 1, 100), 130, 16), ((1, 17, 1, 1, 8), 77, 0),
+                                             ((1, 3, 1, 1, 350), 77, 11), ((1, 2, 1, 1, 2000), 8, 11), ((1, 4, 1, 1, 300), 77, 30)])
+def test_psp_spike_is_conv_then_getSpikes(impl, shape, Fl, nuSize):
+    # spike(psp(x)) in one call: bit for bit what the two kernels give, on shapes that take the fused
+    # kernel (whole-vector rows up to 352 samples) and on shapes that do not
+    rng = np.random.default_rng(shape[-1] + Fl + nuSize)
+    a = (rng.standard_normal(shape) * 2).astype(np.float32)
+    srm = rng.random(Fl).astype(np.float32)
+    nu = -(rng.random(nuSize) * 5).astype(np.float32)
+    theta, Ts = 3.0, 0.5
+    s, u = slayerCuda.pspSpike(dev(a), dev(srm), dev(nu), theta, Ts)
+    u2 = slayerCuda.conv(dev(a), dev(srm), Ts)
+    s2 = slayerCuda.getSpikes(u2, dev(nu), theta, Ts)
+    assert torch.equal(s, s2) and np.array_equal(bits(host(u)), bits(host(u2)))
+    wu = O.conv(a, srm, Ts, fused=True)
+    ws, wu = O.get_spikes(wu, nu, theta, Ts)
+    assert np.array_equal(bits(host(s)), bits(ws)) and np.array_equal(bits(host(u)), bits(wu))
+    assert ws.sum() > 0 or shape[-1] < 64
+
+
 # ------------------------------------------------------------------------------------------ delay gradient
 @pytest.mark.parametrize("shape,Ts", [((4, 6, 1, 1, 80), 0.1), ((64, 20, 1, 1, 2000), 1.0), ((3, 2, 5, 7, 33), 0.5),
                                       ((1, 1, 1, 1, 1), 1.0)])

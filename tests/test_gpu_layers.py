@@ -113,6 +113,24 @@ def test_spike_non_contiguous_input_is_left_untouched():
     assert np.array_equal(host(ut), before)          # the kernel worked on a contiguous copy
 
 
+@pytest.mark.parametrize("T", [300, 350])
+def test_pspSpike_layer_call_matches_spike_of_psp(T):
+    # the MLP ordering spike(psp(fc(x))) of the reference's example as one forward and one backward kernel
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": T}).to(DEV)
+    rng = np.random.default_rng(T)
+    shape = (2, 24, 1, 1, T)
+    a = (rng.standard_normal(shape) * 3).astype(np.float32)
+    g = rng.standard_normal(shape).astype(np.float32)
+    x1 = dev(a).requires_grad_(True)
+    s1 = layer.pspSpike(x1)
+    s1.backward(dev(g))
+    x2 = dev(a).requires_grad_(True)
+    s2 = layer.spike(layer.psp(x2))
+    s2.backward(dev(g))
+    assert torch.equal(s1, s2) and float(s1.detach().sum()) > 0
+    assert torch.equal(x1.grad, x2.grad)
+
+
 def test_get_spikes_requires_five_dimensions():
     f = torch.ones(3, device=DEV)
     with pytest.raises(IndexError):
