@@ -2,11 +2,13 @@
 
 ``slayerCuda`` / ``slayerLoihiCuda`` are drop-in replacements of the reference's two extension
 modules, bound to hand-written HIP kernels through the C ABI of ``libslayer_hip.so``;
-``layer`` / ``loihi`` are the host-side layer engines that wrap them in autograd Functions.
+``layer`` / ``loihi`` are the host-side layer engines that wrap them in autograd Functions;
+``loss`` holds the spike-train losses built on the PSP kernel.
 """
 from . import slayerCuda, slayerLoihiCuda            # noqa: F401
 from .slayer import spikeLayer as layer               # noqa: F401
 from .slayerLoihi import spikeLayer as loihi          # noqa: F401
 from .slayerLoihi import quantize                     # noqa: F401
+from .spikeLoss import spikeLoss as loss              # noqa: F401
 
-__all__ = ["slayerCuda", "slayerLoihiCuda", "layer", "loihi", "quantize"]
+__all__ = ["slayerCuda", "slayerLoihiCuda", "layer", "loihi", "quantize", "loss"]

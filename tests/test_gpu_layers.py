@@ -283,13 +283,43 @@ def test_golden_gradients_like_reference_test003():
     des = dev(raster_from_aer(snn_d["spikeOut"], 1, Ns, Ts, 1 / Ts)).reshape(1, 1, 1, 1, Ns)
     s1 = layer.spike(layer.psp(fc1(x)))
     s2 = layer.spike(layer.psp(fc2(s1)))
-    err = layer.psp(s2 - des)
-    loss = 0.5 * torch.sum(err ** 2) * Ts
+    error = snn.loss({"neuron": nd, "simulation": {"Ts": Ts, "tSample": 50}, "training": {"error": {"type": "SpikeTime"}}}).to(DEV)
+    loss = error.spikeTime(s2, des)
+    assert float(loss.detach()) == pytest.approx(float((0.5 * torch.sum(layer.psp(s2 - des) ** 2) * Ts).detach()), rel=1e-6)
     loss.backward()
     g2 = host(fc2.weight.grad).reshape(1, 25)
     g1 = host(fc1.weight.grad).reshape(25, 250)
     assert np.linalg.norm(snn_d["gradW2Initial"] - g2) / g2.size < 1e-4
     assert np.linalg.norm(snn_d["gradW1Initial"] - g1) / g1.size < 1e-4
+
+
+def test_numSpikes_loss_matches_host_side_formulation():
+    # the reference computes the target region, the desired counts and the count error with numpy on
+    # the host (src/spikeLoss.py:84-104); the same numbers, and the gradient, from device tensors
+    Ts, T = 1.0, 300
+    nd = neuron()
+    desc = {"neuron": nd, "simulation": {"Ts": Ts, "tSample": T},
+            "training": {"error": {"type": "NumSpikes", "tgtSpikeRegion": {"start": 50, "stop": 250},
+                                   "tgtSpikeCount": {True: 60, False: 10}}}}
+    error = snn.loss(desc).to(DEV)
+    rng = np.random.default_rng(4)
+    out = ((rng.random((3, 10, 1, 1, T)) < 0.1) / Ts).astype(np.float32)
+    cls = np.zeros((3, 10, 1, 1, 1), np.float32)
+    cls[np.arange(3), rng.integers(0, 10, 3)] = 1
+    x = dev(out).requires_grad_(True)
+    loss = error.numSpikes(x, dev(cls))
+    loss.backward()
+    # host-side formulation with the oracle's PSP filter
+    srm = host(error.slayer.srmKernel)
+    region = np.zeros(out.shape)
+    region[..., 50:250] = 1
+    actual = out[..., 50:250].sum(4, keepdims=True) * Ts
+    desired = np.where(cls == True, 60, 10)      # noqa: E712
+    count_error = (actual - desired) / 200
+    e = O.conv((out - (region * out).astype(np.float32)), srm, Ts) + (count_error * region).astype(np.float32)
+    assert float(loss.detach()) == pytest.approx(0.5 * float((e.astype(np.float64) ** 2).sum()) * Ts, rel=1e-5)
+    want_grad = O.corr((e * np.float32(Ts)).astype(np.float32), srm, Ts)
+    assert rel_err(host(x.grad), want_grad) < REL_TOL
 
 
 # ------------------------------------------------------------------------------------------ Loihi
