@@ -190,20 +190,28 @@ __device__ __forceinline__ void fir_sparse_tile(const BufferRsrc &bufOut, const 
             while (mask) {
                 const int pos = __builtin_ctzll(mask);
                 mask &= mask - 1;
-                const float xv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), pos));
+                const int xbits = __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), pos);
+                const float xv = __builtin_bit_cast(float, xbits);
                 // column j = 64 b + pos is tap i = j - m of output m; it reaches the output blocks
-                // b-2, b-1 and b (F <= 129), each with its own tap; the taps are fetched together
-                float tap[3];
-                bool hit[3];
+                // b, b-1 and b-2 (F <= 129) through the taps 64 d + pos - lane, d = 0, 1, 2.
+                if (((xbits >> 23) & 0xff) != 0xff) {
+                    // finite sample: the filter copy is zero padded on both sides, so lanes that
+                    // the event does not reach simply add xv * 0
+                    // (nor do blocks it does not reach at all: no branches, the three reads go out together)
+                    const float *tp = fL + (pos - lane);
+                    const float t0v = tp[0], t1v = tp[kWave], t2v = tp[2 * kWave];
+                    acc[b] = __builtin_fmaf(xv, t0v, acc[b]);
+                    if (b >= 1) acc[b >= 1 ? b - 1 : 0] = __builtin_fmaf(xv, t1v, acc[b >= 1 ? b - 1 : 0]);
+                    if (b >= 2) acc[b >= 2 ? b - 2 : 0] = __builtin_fmaf(xv, t2v, acc[b >= 2 ? b - 2 : 0]);
+                } else {
+                    // infinite or NaN sample: only the outputs it really reaches may see it
 #pragma unroll
-                for (int d = 0; d < 3; ++d) {
-                    const int i = kWave * d + pos - lane;  // tap for the output block b - d
-                    hit[d] = b - d >= 0 && b - d < nPass && static_cast<unsigned>(i) < static_cast<unsigned>(F);
-                    tap[d] = hit[d] ? fL[i] : 0.0f;
+                    for (int d = 0; d < 3; ++d) {
+                        const int i = kWave * d + pos - lane;  // tap for the output block b - d
+                        const bool hit = b - d >= 0 && b - d < nPass && static_cast<unsigned>(i) < static_cast<unsigned>(F);
+                        if (b - d >= 0 && hit) acc[b - d] = __builtin_fmaf(xv, fL[i], acc[b - d]);
+                    }
                 }
-#pragma unroll
-                for (int d = 0; d < 3; ++d)
-                    if (b - d >= 0 && hit[d]) acc[b - d] = __builtin_fmaf(xv, tap[d], acc[b - d]);
             }
         }
 #pragma unroll
@@ -228,8 +236,9 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
                                                         float Ts, FirGate gate)
 {
     extern __shared__ __align__(16) float X[];
-    float *fL = X + R * LD;                                        // filter copy for the sparse path
-    uint32_t *nzCount = reinterpret_cast<uint32_t *>(fL + F);      // non-zero input vectors, per wavefront
+    // filter copy for the sparse path: taps -63 .. 191, zeros outside [0, F)
+    float *fL = X + R * LD + (kWave - 1);
+    uint32_t *nzCount = reinterpret_cast<uint32_t *>(X + R * LD + 4 * kWave);  // non-zero input vectors, per wavefront
     uint32_t nonZero = 0;                                          // wave-uniform
 
     const int tid = threadIdx.x;
@@ -314,7 +323,10 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
             nonZero += __builtin_popcountll(__ballot(any_nonzero(v)));
         }
     }
-    for (int i = tid; i < F; i += 256) fL[i] = filt[i];
+    {
+        const int i = tid - (kWave - 1);  // 256 lanes, taps -63 .. 192
+        if (i < 3 * kWave) fL[i] = (i >= 0 && i < F) ? filt[i] : 0.0f;
+    }
     if ((tid & (kWave - 1)) == 0) nzCount[tid / kWave] = nonZero;
     __syncthreads();
 
@@ -435,7 +447,8 @@ static void launch_tiled(const FirPlan &p, float *out, const float *in, const fl
                          int64_t F, float Ts, const FirGate &gate, hipStream_t stream)
 {
     dim3 grid(static_cast<unsigned>(ceil_div(rows, p.R)), static_cast<unsigned>(p.nTiles)), block(256);
-    const size_t lds = (static_cast<size_t>(p.R) * p.LD + static_cast<size_t>(F) + 4) * sizeof(float);
+    // rows, the zero-padded filter copy of the sparse path (256 floats) and four counters
+    const size_t lds = (static_cast<size_t>(p.R) * p.LD + 4 * kWave + 4) * sizeof(float);
     hipLaunchKernelGGL((fir_tiled_kernel<CAUSAL, VEC, U, GATED>), grid, block, lds, stream, out, in, filt, rows,
                        static_cast<int>(T), static_cast<int>(F), p.TT, p.LD, p.R, Ts, gate);
 }
