@@ -193,25 +193,19 @@ __device__ __forceinline__ void fir_sparse_tile(const BufferRsrc &bufOut, const 
                 const int xbits = __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), pos);
                 const float xv = __builtin_bit_cast(float, xbits);
                 // column j = 64 b + pos is tap i = j - m of output m; it reaches the output blocks
-                // b, b-1 and b-2 (F <= 129) through the taps 64 d + pos - lane, d = 0, 1, 2.
-                if (((xbits >> 23) & 0xff) != 0xff) {
-                    // finite sample: the filter copy is zero padded on both sides, so lanes that
-                    // the event does not reach simply add xv * 0
-                    // (nor do blocks it does not reach at all: no branches, the three reads go out together)
-                    const float *tp = fL + (pos - lane);
-                    const float t0v = tp[0], t1v = tp[kWave], t2v = tp[2 * kWave];
-                    acc[b] = __builtin_fmaf(xv, t0v, acc[b]);
-                    if (b >= 1) acc[b >= 1 ? b - 1 : 0] = __builtin_fmaf(xv, t1v, acc[b >= 1 ? b - 1 : 0]);
-                    if (b >= 2) acc[b >= 2 ? b - 2 : 0] = __builtin_fmaf(xv, t2v, acc[b >= 2 ? b - 2 : 0]);
-                } else {
-                    // infinite or NaN sample: only the outputs it really reaches may see it
-#pragma unroll
-                    for (int d = 0; d < 3; ++d) {
-                        const int i = kWave * d + pos - lane;  // tap for the output block b - d
-                        const bool hit = b - d >= 0 && b - d < nPass && static_cast<unsigned>(i) < static_cast<unsigned>(F);
-                        if (b - d >= 0 && hit) acc[b - d] = __builtin_fmaf(xv, fL[i], acc[b - d]);
-                    }
-                }
+                // b, b-1 and b-2 (F <= 129) through the taps i_d = 64 d + pos - lane, d = 0, 1, 2.
+                // The filter copy is zero padded on both sides, so the three reads need no checks
+                // and go out together; a lane outside the event's reach multiplies by a zero
+                // sample instead (not by a zero tap: the sample may be infinite).  No branches.
+                const int i0 = pos - lane;
+                const float *tp = fL + i0;
+                const float t0v = tp[0], t1v = tp[kWave], t2v = tp[2 * kWave];
+                const float x0 = static_cast<unsigned>(i0) < static_cast<unsigned>(F) ? xv : 0.0f;
+                const float x1 = static_cast<unsigned>(i0 + kWave) < static_cast<unsigned>(F) ? xv : 0.0f;
+                const float x2 = static_cast<unsigned>(i0 + 2 * kWave) < static_cast<unsigned>(F) ? xv : 0.0f;
+                acc[b] = __builtin_fmaf(x0, t0v, acc[b]);
+                if (b >= 1) acc[b >= 1 ? b - 1 : 0] = __builtin_fmaf(x1, t1v, acc[b >= 1 ? b - 1 : 0]);
+                if (b >= 2) acc[b >= 2 ? b - 2 : 0] = __builtin_fmaf(x2, t2v, acc[b >= 2 ? b - 2 : 0]);
             }
         }
 #pragma unroll
