@@ -64,7 +64,12 @@ def test_cpu_tensors_are_rejected_like_the_reference():
     for call in (lambda: slayerCuda.conv(x, f, 1.0), lambda: slayerCuda.corr(x, f, 1.0),
                  lambda: slayerCuda.shift(x, f, 1.0), lambda: slayerCuda.shift(x, 1.0),
                  lambda: slayerCuda.getSpikes(x, f, 1.0, 1.0),
-                 lambda: slayerLoihiCuda.getSpikes(x, 0, 64, 0, 0, 1)):
+                 lambda: slayerLoihiCuda.getSpikes(x, 0, 64, 0, 0, 1),
+                 lambda: slayerLoihiCuda.getSpikesDelayed(x, 0, 64, 0, 0, 1, 1, voltage=False),
+                 lambda: slayerCuda.pspSpike(x, f, f, 1.0, 1.0),
+                 lambda: slayerCuda.spikeBackward(x, x, 1.0, 1.0, 1.0),
+                 lambda: slayerCuda.spikeBackwardCorr(x, x, f, 1.0, 1.0, 1.0, 1.0),
+                 lambda: slayerCuda.delayGrad(x, x, 1.0)):
         with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
             call()
 
@@ -117,6 +122,17 @@ def test_layer_objects_build_without_gpu():
     w = loihi.dense(8, 4)
     q = w.preHookFx(w.weight)
     assert torch.all(q == torch.round(q / 2) * 2)                        # weights quantised in steps of 2
+
+
+def test_loss_module_builds_without_gpu_and_checks_its_type():
+    neuron = {"theta": 10, "tauSr": 1.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
+    desc = {"neuron": neuron, "simulation": {"Ts": 1.0, "tSample": 100},
+            "training": {"error": {"type": "NumSpikes", "tgtSpikeRegion": {"start": 0, "stop": 100},
+                                   "tgtSpikeCount": {True: 20, False: 5}}}}
+    error = snn.loss(desc)
+    assert error.slayer.srmKernel.numel() == 8
+    with pytest.raises(AssertionError, match="SpikeTime"):
+        error.spikeTime(torch.zeros(1, 1, 1, 1, 100), torch.zeros(1, 1, 1, 1, 100))
 
 
 def test_dropin_modules_re_export_the_extension_api():
