@@ -99,7 +99,8 @@ class spikeLayer(nn.Module):
 
 
 class _denseLayer(nn.Conv3d):
-    """(outFeatures, inFeatures, 1, 1, 1) weight applied at every time step."""
+    """Fully connected synapse: an (outFeatures, C, H, W, 1) weight applied at every time step
+    (src/slayer.py:393-440)."""
 
     def __init__(self, inFeatures, outFeatures, weightScale=1, preHookFx=None):
         if isinstance(inFeatures, int):
@@ -119,6 +120,13 @@ class _denseLayer(nn.Conv3d):
 
     def forward(self, input):
         weight = self.weight if self.preHookFx is None else self.preHookFx(self.weight)
+        # The kernel spans the whole (H, W) extent of the input, so the layer is one matrix product
+        # per batch item, W[O, C*H*W] x X[C*H*W, T], with time innermost as the tensor already is:
+        # a plain library GEMM instead of a 3-D convolution with a degenerate kernel.
+        if input.dim() == 5 and tuple(input.shape[1:4]) == tuple(weight.shape[1:4]) and self.bias is None:
+            N, T = input.shape[0], input.shape[4]
+            O, K = weight.shape[0], weight.shape[1] * weight.shape[2] * weight.shape[3]
+            return torch.matmul(weight.reshape(O, K), input.reshape(N, K, T)).reshape(N, O, 1, 1, T)
         return F.conv3d(input, weight, self.bias, self.stride, self.padding, self.dilation, self.groups)
 
 

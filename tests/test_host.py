@@ -124,6 +124,26 @@ def test_layer_objects_build_without_gpu():
     assert torch.all(q == torch.round(q / 2) * 2)                        # weights quantised in steps of 2
 
 
+def test_dense_layer_as_matrix_product_equals_the_3d_convolution():
+    # the reference's dense layer is a conv3d whose kernel spans the whole (H, W) extent; the same
+    # numbers from one matrix product per batch item (time stays innermost)
+    import torch.nn.functional as F
+    neuron = {"theta": 10, "tauSr": 1.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
+    layer = snn.layer(neuron, {"Ts": 1.0, "tSample": 50})
+    torch.manual_seed(0)
+    for inF, shape in (((3, 4, 2), (2, 2, 4, 3, 17)), (12, (3, 12, 1, 1, 9)), ((5, 2), (1, 1, 2, 5, 4))):
+        fc = layer.dense(inF, 6)
+        x = torch.randn(shape, requires_grad=True)
+        y = fc(x)
+        ref = F.conv3d(x, fc.weight)
+        assert y.shape == ref.shape == (shape[0], 6, 1, 1, shape[-1])
+        assert torch.allclose(y, ref, rtol=1e-5, atol=1e-5)
+        gy = torch.randn_like(y)
+        gx, gw = torch.autograd.grad(y, (x, fc.weight), gy, retain_graph=True)
+        rx, rw = torch.autograd.grad(ref, (x, fc.weight), gy)
+        assert torch.allclose(gx, rx, rtol=1e-5, atol=1e-5) and torch.allclose(gw, rw, rtol=1e-4, atol=1e-4)
+
+
 def test_loss_module_builds_without_gpu_and_checks_its_type():
     neuron = {"theta": 10, "tauSr": 1.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
     desc = {"neuron": neuron, "simulation": {"Ts": 1.0, "tSample": 100},
