@@ -129,6 +129,38 @@ def flip_rate(device, srm_t, ref_t, params):
     return float((s_gpu != s_cpu).mean()), float((s_cpu != 0).mean())
 
 
+def mlp_row(device, timed):
+    """One training step (without the optimiser) of the 2312-512-10 MLP on (12, 2, 34, 34, 350) input
+    spikes at p = 0.015, layer ordering spike(psp(fc(x))), spike-time loss against a random target
+    train; both the separate calls and the fused pspSpike call."""
+    import slayerpytorch_amd as snn
+    params = neuron_params()
+    sim = {"Ts": 1.0, "tSample": 350}
+    net = {"neuron": params, "simulation": sim, "training": {"error": {"type": "SpikeTime"}}}
+    layer = snn.layer(params, sim).to(device)
+    error = snn.loss(net).to(device)
+    torch.manual_seed(0)
+    fc1, fc2 = layer.dense((34, 34, 2), 512).to(device), layer.dense(512, 10).to(device)
+    g = torch.Generator(device="cpu").manual_seed(3)
+    x = (torch.rand((12, 2, 34, 34, 350), generator=g) < 0.015).float().to(device)
+    target = (torch.rand((12, 10, 1, 1, 350), generator=g) < 0.01).float().to(device)
+
+    def step(fused):
+        if fused:
+            s2 = layer.pspSpike(fc2(layer.pspSpike(fc1(x))))
+        else:
+            s2 = layer.spike(layer.psp(fc2(layer.spike(layer.psp(fc1(x))))))
+        loss = error.spikeTime(s2, target)
+        loss.backward()
+        fc1.weight.grad = None
+        fc2.weight.grad = None
+
+    two = timed(lambda: step(False))
+    one = timed(lambda: step(True))
+    return {"op": "nmnist_mlp_2312_512_10_fwd_loss_bwd", "shape": [12, 2, 34, 34, 350], "us": one * 1e6,
+            "us_with_separate_psp_and_spike_calls": two * 1e6, "samples_per_s": 12 / one}
+
+
 def other_rows(device):
     """Quick per-op measurements of the scope rows that are not part of the headline chain, each on
     the largest tensor its BASELINE config gives it (median of 7 event-timed launches).  hbm_frac
@@ -188,6 +220,8 @@ def other_rows(device):
     out.append(row("spike_pdf_then_corr77_fused", 20, a.numel(),
                    timed(lambda: slayerCuda.spikeBackwardCorr(gs, a, srm77, 10.0, 10.0, 1.0, 1.0)), shape))
     del a, gs
+    # NMNIST-shaped MLP end to end (dense layers are library GEMMs): forward, spike-time loss, backward
+    out.append(mlp_row(device, timed))
     # Loihi config: largest tensor (8, 16, 32, 32, 300)
     shape = (8, 16, 32, 32, 300)
     w = (2 * torch.randint(-128, 128, shape, generator=g) * (torch.rand(shape, generator=g) < 0.05)).float().to(device)
