@@ -151,11 +151,18 @@ __global__ __launch_bounds__(64) void psp_spike_kernel(float *__restrict__ s, fl
             }
             uint32_t fired = 0;
 #pragma unroll
-            for (int k = 0; k < G; ++k) {
-                if (v[k] >= theta) {
-                    fired |= 1u << k;
+            for (int k = 0; k < G; k += 2) {  // one scalar branch per two samples, as in spike.hip
+                if (__builtin_amdgcn_ballot_w64((v[k] >= theta) | (v[k + 1] >= theta)) != 0) {
+                    if (v[k] >= theta) {
+                        fired |= 1u << k;
 #pragma unroll
-                    for (int j = 0; j < NU; ++j) v[k + j] += tap[j];
+                        for (int j = 0; j < NU; ++j) v[k + j] += tap[j];
+                    }
+                    if (v[k + 1] >= theta) {
+                        fired |= 2u << k;
+#pragma unroll
+                        for (int j = 0; j < NU; ++j) v[k + 1 + j] += tap[j];
+                    }
                 }
             }
 #pragma unroll

@@ -295,11 +295,20 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                 }
                 uint32_t fired = 0;
 #pragma unroll
-                for (int k = 0; k < G; ++k) {
-                    if (v[k] >= theta) {
-                        fired |= 1u << k;
+                for (int k = 0; k < G; k += 2) {
+                    // One scalar branch per two samples: in most pairs no row spikes.  (The second
+                    // sample is tested again inside, after the first one's refractory response.)
+                    if (__builtin_amdgcn_ballot_w64((v[k] >= theta) | (v[k + 1] >= theta)) != 0) {
+                        if (v[k] >= theta) {
+                            fired |= 1u << k;
 #pragma unroll
-                        for (int j = 0; j < NU; ++j) v[k + j] += tap[j];
+                            for (int j = 0; j < NU; ++j) v[k + j] += tap[j];
+                        }
+                        if (v[k + 1] >= theta) {
+                            fired |= 2u << k;
+#pragma unroll
+                            for (int j = 0; j < NU; ++j) v[k + 1 + j] += tap[j];
+                        }
                     }
                 }
 #pragma unroll
