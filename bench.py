@@ -36,7 +36,7 @@ AB = {"psp_conv": 8, "spike": 12, "shift": 8, "shift_bwd": 8, "spike_bwd": 12, "
 # HBM bytes per launch on SHAPE measured with the FETCH_SIZE and WRITE_SIZE hardware counters
 # (rocprofv3 --pmc, one counter per run, scaled by the reading of a plain copy of known size);
 # the figures and the commands are in profiles/hbm_traffic_counters.txt
-TRAFFIC_BYTES = {"psp_conv": 537.2e6, "spike": 798.8e6, "shift": 540.8e6, "shift_bwd": 540.8e6, "spike_bwd": 798.7e6,
+TRAFFIC_BYTES = {"psp_conv": 537.2e6, "spike": 798.7e6, "shift": 540.8e6, "shift_bwd": 540.8e6, "spike_bwd": 798.7e6,
                  "psp_corr": 545.5e6}
 KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, true, 8, false> (conv, event-driven path)", "spike": "slayer::spike_tile_kernel<12, 1, 12, 8>",
              "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
