@@ -169,3 +169,11 @@ def test_dropin_modules_re_export_the_extension_api():
     for name in ("getSpikes", "conv", "corr", "shift"):
         assert getattr(sc, name) is getattr(slayerCuda, name)
     assert slc.getSpikes is slayerLoihiCuda.getSpikes
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
