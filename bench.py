@@ -163,7 +163,7 @@ def mlp_row(device, timed):
 
 def other_rows(device):
     """Quick per-op measurements of the scope rows that are not part of the headline chain, each on
-    the largest tensor its BASELINE config gives it (median of 7 event-timed launches).  hbm_frac
+    the largest tensor its benchmark configuration gives it (median of 7 event-timed launches).  hbm_frac
     counts the algorithmic bytes of the unfused reference sequence (Loihi forward + delayShift:
     16 + 8 B, Loihi backward: 12 + 8 B), also where one fused kernel moves fewer."""
     from slayerpytorch_amd import slayerCuda, slayerLoihiCuda
