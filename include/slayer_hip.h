@@ -15,8 +15,8 @@
  *     device (the reference bindings call cudaSetDevice on the tensor's device).
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only
  *     enqueue work: no allocation, no free, no host synchronisation, no global state.
- *   - The library never allocates device memory.  Outputs (and the one workspace, see
- *     slayer_delay_grad_f32) are allocated by the caller.
+ *   - The library never allocates device memory.  Outputs (and the workspaces of
+ *     slayer_delay_grad_f32 and slayer_synapse_conv_grad_weight_f32) are allocated by the caller.
  *   - Return value: SLAYER_OK (0) or one of the SLAYER_E* codes; nothing has been launched
  *     when a SLAYER_EINVAL / SLAYER_EUNSUPPORTED code is returned.  Empty tensors
  *     (nNeurons == 0 or T == 0) are a successful no-op.
@@ -212,6 +212,61 @@ int slayer_loihi_get_spikes_delayed_f32(float *s, float *v, float *u, const floa
                                         int64_t nNeurons, int64_t T, uint32_t wgtExp, int32_t theta,
                                         uint32_t iDecay, uint32_t vDecay, uint32_t refDelay,
                                         int32_t delaySteps, void *stream);
+
+/*
+ * ---- Per-timestep synapses ---------------------------------------------------------------------
+ * The reference's conv / pool / convTranspose / unpool layers apply a 2-D filter over (H, W) to
+ * every time sample of an [N][C][H][W][T] tensor by calling torch's conv3d / conv_transpose3d
+ * with a kernel of time extent 1 (src/slayer.py:499-507, :565-575, :631-643, :732-748).  The three
+ * entry points below are that operation and its two gradients on T-innermost tensors; the pooling
+ * layers are the case C = O = 1 on the tensor reshaped to [N][1][C*H][W][T], the transposed layers
+ * use the input gradient as their forward pass.
+ *
+ * Geometry: input [N][C][H][W][T], weights [O][C/groups][KH][KW] (the reference's trailing
+ * time extent of 1 dropped), output [N][O][OH][OW][T] with
+ * OH = (H + 2*padH - dilH*(KH-1) - 1) / strideH + 1 (0 when the filter does not fit), OW alike.
+ * One batch item of the input and of the output must stay below 2 GiB (SLAYER_EUNSUPPORTED).
+ */
+typedef struct slayer_synapse_geom {
+    int32_t N, C, H, W, T;
+    int32_t O, KH, KW;
+    int32_t strideH, strideW, padH, padW, dilH, dilW, groups;
+} slayer_synapse_geom;
+
+/* Validates the geometry and returns the output extents (either pointer may be NULL). */
+int slayer_synapse_out_shape(const slayer_synapse_geom *geom, int32_t *OH, int32_t *OW);
+
+/*
+ * out[n][o][a][b][t] = sum_{c in group(o), i, j} weight[o][c'][i][j] *
+ *                      in[n][c][a*strideH - padH + i*dilH][b*strideW - padW + j*dilW][t]
+ * (samples outside the input count as 0).  Replaces F.conv3d in _convLayer.forward
+ * (src/slayer.py:499-507) and _poolLayer.forward (src/slayer.py:565-575).
+ */
+int slayer_synapse_conv_f32(float *out, const float *in, const float *weight,
+                            const slayer_synapse_geom *geom, void *stream);
+
+/*
+ * Gradient of slayer_synapse_conv_f32 with respect to `in` (every element of gradIn is written).
+ * Replaces the input gradient autograd derives for F.conv3d in those layers, and is the forward
+ * pass F.conv_transpose3d of _convTransposeLayer / _unpoolLayer (src/slayer.py:631-643, :732-748),
+ * whose weight tensor [inChannels][outChannels/groups][KH][KW] is the weight tensor of the
+ * convolution it transposes.
+ */
+int slayer_synapse_conv_grad_input_f32(float *gradIn, const float *gradOut, const float *weight,
+                                       const slayer_synapse_geom *geom, void *stream);
+
+/* Bytes of caller-provided device workspace for slayer_synapse_conv_grad_weight_f32 (may be 0). */
+int64_t slayer_synapse_conv_grad_weight_workspace_bytes(const slayer_synapse_geom *geom);
+
+/*
+ * gradW[o][c'][i][j] = sum_{n,a,b,t} gradOut[n][o][a][b][t] *
+ *                      in[n][c][a*strideH - padH + i*dilH][b*strideW - padW + j*dilW][t]
+ * Replaces the weight gradient autograd derives for F.conv3d / F.conv_transpose3d in the same
+ * layers.  Partial sums go through `workspace` and are added in a fixed order (deterministic).
+ */
+int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gradOut, const float *in,
+                                        float *workspace, const slayer_synapse_geom *geom,
+                                        void *stream);
 
 #ifdef __cplusplus
 }

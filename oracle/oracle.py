@@ -16,6 +16,8 @@ oracle function        reference entry point it restates
 ``loihi_get_spikes``   ``slayerLoihiCuda.getSpikes`` (src/cuda/slayerLoihiKernels.cu:12-46)
 ``spike_bwd``          ``_spikeFunction.backward`` (src/slayer.py:857-865)
 ``delay_grad``         ``_delayFunction.backward`` (src/slayer.py:949-955)
+``synapse_conv*``      ``F.conv3d`` with a (KH, KW, 1) kernel in the synapse layers
+                       (src/slayer.py:499-507, :565-575) and its two gradients
 =====================  ==========================================================
 """
 import ctypes
@@ -30,6 +32,12 @@ _lib = None
 
 _f32p = ctypes.POINTER(ctypes.c_float)
 _i64 = ctypes.c_int64
+
+
+class SynapseGeom(ctypes.Structure):
+    """Geometry of a per-timestep 2-D synapse: input [N][C][H][W][T], weights [O][C/groups][KH][KW]."""
+    _fields_ = [(k, ctypes.c_int32) for k in ("N", "C", "H", "W", "T", "O", "KH", "KW", "sH", "sW",
+                                              "pH", "pW", "dH", "dW", "groups")]
 
 
 def build(force=False):
@@ -59,6 +67,14 @@ def lib():
         L.oracle_loihi_get_spikes_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _i64, _i64,
                                                   ctypes.c_uint32, ctypes.c_int32, ctypes.c_uint32,
                                                   ctypes.c_uint32, ctypes.c_uint32]
+        gp = ctypes.POINTER(SynapseGeom)
+        L.oracle_synapse_out_shape.argtypes = [gp, ctypes.POINTER(_i64), ctypes.POINTER(_i64)]
+        L.oracle_synapse_conv_f32.argtypes = [_f32p, _f32p, _f32p, gp]
+        L.oracle_synapse_conv_grad_input_f32.argtypes = [_f32p, _f32p, _f32p, gp]
+        L.oracle_synapse_conv_grad_weight_f32.argtypes = [_f32p, _f32p, _f32p, gp]
+        for name in ("oracle_synapse_out_shape", "oracle_synapse_conv_f32",
+                     "oracle_synapse_conv_grad_input_f32", "oracle_synapse_conv_grad_weight_f32"):
+            getattr(L, name).restype = None
         for name in ("oracle_get_spikes_f32", "oracle_conv_f32", "oracle_corr_f32",
                      "oracle_shift_f32", "oracle_spike_bwd_f32", "oracle_delay_grad_f32",
                      "oracle_loihi_get_spikes_f32", "oracle_set_threads"):
@@ -177,3 +193,55 @@ def loihi_get_spikes(w, wgtExp, theta, iDecay, vDecay, refDelay):
         lib().oracle_loihi_get_spikes_f32(_p(s), _p(v), _p(u), _p(w), n, T, int(wgtExp), int(theta),
                                           int(iDecay), int(vDecay), int(refDelay))
     return s, v, u
+
+
+def _pair(v):
+    return (int(v), int(v)) if np.isscalar(v) else (int(v[0]), int(v[1]))
+
+
+def synapse_geom(in_shape, w_shape, stride=1, padding=0, dilation=1, groups=1):
+    """Geometry record and output shape of the synapse ``in_shape`` = (N, C, H, W, T),
+    ``w_shape`` = (O, C/groups, KH, KW[, 1])."""
+    N, C, H, W, T = (int(v) for v in in_shape)
+    O, Cg, KH, KW = (int(v) for v in w_shape[:4])
+    if C % groups or O % groups or Cg != C // groups:
+        raise ValueError("channels and groups do not fit the weight shape")
+    (sH, sW), (pH, pW), (dH, dW) = _pair(stride), _pair(padding), _pair(dilation)
+    g = SynapseGeom(N, C, H, W, T, O, KH, KW, sH, sW, pH, pW, dH, dW, int(groups))
+    OH, OW = _i64(), _i64()
+    lib().oracle_synapse_out_shape(ctypes.byref(g), ctypes.byref(OH), ctypes.byref(OW))
+    return g, (N, O, OH.value, OW.value, T)
+
+
+def synapse_conv(x, w, stride=1, padding=0, dilation=1, groups=1):
+    """Per-timestep 2-D cross-correlation of ``x`` [N][C][H][W][T] with ``w`` [O][C/groups][KH][KW]."""
+    x, w = _f32(x), _f32(w)
+    g, oshape = synapse_geom(x.shape, w.shape, stride, padding, dilation, groups)
+    out = np.zeros(oshape, dtype=np.float32)
+    if out.size:
+        lib().oracle_synapse_conv_f32(_p(out), _p(x), _p(w), ctypes.byref(g))
+    return out
+
+
+def synapse_conv_grad_input(grad_out, w, in_shape, stride=1, padding=0, dilation=1, groups=1):
+    """Gradient of :func:`synapse_conv` with respect to ``x`` (shape ``in_shape``)."""
+    go, w = _f32(grad_out), _f32(w)
+    g, oshape = synapse_geom(in_shape, w.shape, stride, padding, dilation, groups)
+    if tuple(go.shape) != oshape:
+        raise ValueError("grad_out has shape %s, expected %s" % (go.shape, oshape))
+    gi = np.zeros(tuple(int(v) for v in in_shape), dtype=np.float32)
+    if gi.size:
+        lib().oracle_synapse_conv_grad_input_f32(_p(gi), _p(go), _p(w), ctypes.byref(g))
+    return gi
+
+
+def synapse_conv_grad_weight(grad_out, x, w_shape, stride=1, padding=0, dilation=1, groups=1):
+    """Gradient of :func:`synapse_conv` with respect to ``w`` (shape ``w_shape[:4]``)."""
+    go, x = _f32(grad_out), _f32(x)
+    g, oshape = synapse_geom(x.shape, w_shape, stride, padding, dilation, groups)
+    if tuple(go.shape) != oshape:
+        raise ValueError("grad_out has shape %s, expected %s" % (go.shape, oshape))
+    gw = np.zeros(tuple(int(v) for v in w_shape[:4]), dtype=np.float32)
+    if gw.size:
+        lib().oracle_synapse_conv_grad_weight_f32(_p(gw), _p(go), _p(x), ctypes.byref(g))
+    return gw

@@ -295,3 +295,123 @@ void oracle_loihi_get_spikes_f32(float *s, float *v, float *u, const float *w, i
         }
     }
 }
+
+/* ------------------------------------------------------------------------------------------
+ * Per-timestep synapse (2-D cross-correlation applied to every time sample of an
+ * [N][C][H][W][T] tensor).  The reference's layers call torch's conv3d / conv_transpose3d with
+ * a kernel of time extent 1 (src/slayer.py:441-449 dense, :499-507 conv, :565-575 pool,
+ * :631-643 convTranspose, :732-748 unpool); this restates that operation's definition:
+ *
+ *   out[n][o][a][b][t] = sum_{c in group(o), i, j} w[o][c'][i][j] *
+ *                        in[n][c][a*sH - pH + i*dH][b*sW - pW + j*dW][t]   (0 outside the tensor)
+ *
+ * with c' = c - group(o)*C/groups.  Sums are accumulated in double and rounded once, so the
+ * result does not depend on a summation order.  geom = {N, C, H, W, T, O, KH, KW, sH, sW, pH, pW,
+ * dH, dW, groups}.
+ * Pins: torch.nn.functional.conv3d / conv_transpose3d and their autograd on the CPU (the very
+ * routine the reference's layers call), the shift-and-add constructions of the reference's
+ * tests (test/test_slayer007.py:36-48, :60-66, test/test_slayer013.py), adjoint identities.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct {
+    int32_t N, C, H, W, T, O, KH, KW, sH, sW, pH, pW, dH, dW, groups;
+} oracle_synapse_geom;
+
+static int64_t syn_out_extent(int64_t in, int64_t k, int64_t s, int64_t p, int64_t d)
+{
+    const int64_t span = in + 2 * p - d * (k - 1) - 1;
+    return span < 0 ? 0 : span / s + 1;
+}
+
+void oracle_synapse_out_shape(const oracle_synapse_geom *g, int64_t *OH, int64_t *OW)
+{
+    *OH = syn_out_extent(g->H, g->KH, g->sH, g->pH, g->dH);
+    *OW = syn_out_extent(g->W, g->KW, g->sW, g->pW, g->dW);
+}
+
+void oracle_synapse_conv_f32(float *out, const float *in, const float *w, const oracle_synapse_geom *g)
+{
+    int64_t OH, OW;
+    oracle_synapse_out_shape(g, &OH, &OW);
+    const int64_t Cg = g->C / g->groups, Og = g->O / g->groups, T = g->T;
+    const int64_t rows = (int64_t)g->N * g->O * OH * OW;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const int64_t b = r % OW, a = (r / OW) % OH, o = (r / (OW * OH)) % g->O, n = r / (OW * OH * g->O);
+        const int64_t grp = o / Og;
+        for (int64_t t = 0; t < T; ++t) {
+            double acc = 0.0;
+            for (int64_t cl = 0; cl < Cg; ++cl)
+                for (int64_t i = 0; i < g->KH; ++i)
+                    for (int64_t j = 0; j < g->KW; ++j) {
+                        const int64_t y = a * g->sH - g->pH + i * g->dH, x = b * g->sW - g->pW + j * g->dW;
+                        if (y < 0 || y >= g->H || x < 0 || x >= g->W) continue;
+                        const int64_t c = grp * Cg + cl;
+                        acc += (double)w[((o * Cg + cl) * g->KH + i) * g->KW + j] *
+                               (double)in[(((n * g->C + c) * g->H + y) * g->W + x) * T + t];
+                    }
+            out[r * T + t] = (float)acc;
+        }
+    }
+}
+
+/* Gradient of oracle_synapse_conv_f32 with respect to its input (= the transposed convolution
+ * of gradOut): every product of the forward sum is sent back to the input sample it read. */
+void oracle_synapse_conv_grad_input_f32(float *gradIn, const float *gradOut, const float *w,
+                                        const oracle_synapse_geom *g)
+{
+    int64_t OH, OW;
+    oracle_synapse_out_shape(g, &OH, &OW);
+    const int64_t Cg = g->C / g->groups, Og = g->O / g->groups, T = g->T;
+    const int64_t rows = (int64_t)g->N * g->C * g->H * g->W;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const int64_t x = r % g->W, y = (r / g->W) % g->H, c = (r / ((int64_t)g->W * g->H)) % g->C,
+                      n = r / ((int64_t)g->W * g->H * g->C);
+        const int64_t grp = c / Cg, cl = c % Cg;
+        for (int64_t t = 0; t < T; ++t) {
+            double acc = 0.0;
+            for (int64_t ol = 0; ol < Og; ++ol)
+                for (int64_t i = 0; i < g->KH; ++i)
+                    for (int64_t j = 0; j < g->KW; ++j) {
+                        const int64_t ya = y + g->pH - i * g->dH, xb = x + g->pW - j * g->dW;
+                        if (ya < 0 || xb < 0 || ya % g->sH || xb % g->sW) continue;
+                        const int64_t a = ya / g->sH, b = xb / g->sW;
+                        if (a >= OH || b >= OW) continue;
+                        const int64_t o = grp * Og + ol;
+                        acc += (double)w[((o * Cg + cl) * g->KH + i) * g->KW + j] *
+                               (double)gradOut[(((n * g->O + o) * OH + a) * OW + b) * T + t];
+                    }
+            gradIn[r * T + t] = (float)acc;
+        }
+    }
+}
+
+/* Gradient of oracle_synapse_conv_f32 with respect to the weights. */
+void oracle_synapse_conv_grad_weight_f32(float *gradW, const float *gradOut, const float *in,
+                                         const oracle_synapse_geom *g)
+{
+    int64_t OH, OW;
+    oracle_synapse_out_shape(g, &OH, &OW);
+    const int64_t Cg = g->C / g->groups, Og = g->O / g->groups, T = g->T;
+    const int64_t nW = (int64_t)g->O * Cg * g->KH * g->KW;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t q = 0; q < nW; ++q) {
+        const int64_t j = q % g->KW, i = (q / g->KW) % g->KH, cl = (q / ((int64_t)g->KW * g->KH)) % Cg,
+                      o = q / ((int64_t)g->KW * g->KH * Cg);
+        const int64_t c = (o / Og) * Cg + cl;
+        double acc = 0.0;
+        for (int64_t n = 0; n < g->N; ++n)
+            for (int64_t a = 0; a < OH; ++a) {
+                const int64_t y = a * g->sH - g->pH + i * g->dH;
+                if (y < 0 || y >= g->H) continue;
+                for (int64_t b = 0; b < OW; ++b) {
+                    const int64_t x = b * g->sW - g->pW + j * g->dW;
+                    if (x < 0 || x >= g->W) continue;
+                    const float *gp = gradOut + (((n * g->O + o) * OH + a) * OW + b) * T;
+                    const float *ip = in + (((n * g->C + c) * g->H + y) * g->W + x) * T;
+                    for (int64_t t = 0; t < T; ++t) acc += (double)gp[t] * (double)ip[t];
+                }
+            }
+        gradW[q] = (float)acc;
+    }
+}

@@ -16,6 +16,17 @@ _u32 = ctypes.c_uint32
 _i32 = ctypes.c_int32
 _stream = ctypes.c_void_p
 
+
+
+class SynapseGeom(ctypes.Structure):
+    """``slayer_synapse_geom``: input [N][C][H][W][T], weights [O][C/groups][KH][KW]."""
+    _fields_ = [(k, ctypes.c_int32) for k in ("N", "C", "H", "W", "T", "O", "KH", "KW", "strideH", "strideW",
+                                              "padH", "padW", "dilH", "dilW", "groups")]
+
+
+_geomp = ctypes.POINTER(SynapseGeom)
+_i32p = ctypes.POINTER(ctypes.c_int32)
+
 # name -> (restype, argtypes); must list every symbol of include/slayer_hip.h
 SIGNATURES = {
     "slayer_hip_abi_version": (ctypes.c_int, []),
@@ -38,6 +49,11 @@ SIGNATURES = {
                                                   _u32, _u32, _u32, _stream]),
     "slayer_loihi_get_spikes_delayed_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _i64, _i64, _u32, _i32,
                                                           _u32, _u32, _u32, _i32, _stream]),
+    "slayer_synapse_out_shape": (ctypes.c_int, [_geomp, _i32p, _i32p]),
+    "slayer_synapse_conv_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _geomp, _stream]),
+    "slayer_synapse_conv_grad_input_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _geomp, _stream]),
+    "slayer_synapse_conv_grad_weight_workspace_bytes": (_i64, [_geomp]),
+    "slayer_synapse_conv_grad_weight_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _geomp, _stream]),
 }
 
 ABI_VERSION = 1

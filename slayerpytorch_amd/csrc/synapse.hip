@@ -1,0 +1,548 @@
+// Per-timestep synapses on [N][C][H][W][T] tensors (time innermost): 2-D cross-correlation over
+// (H, W) applied to every time sample, and its two gradients.  The reference's layers obtain this
+// from conv3d / conv_transpose3d with a kernel of time extent 1 (src/slayer.py:499-507 conv,
+// :565-575 pool, :631-643 convTranspose, :732-748 unpool).
+//
+// With time innermost the filter does not depend on the fastest axis, so every lane owns a run of
+// consecutive time samples (one 16-byte vector) of one pixel: loads and stores are contiguous along
+// T for any stride, padding or dilation, and the weights are wave-uniform.
+#include "common.h"
+
+namespace slayer {
+
+struct SynGeom {
+    int N, C, H, W, T, O, KH, KW, sH, sW, pH, pW, dH, dW, groups, OH, OW;
+};
+
+// ---- gather kernel: forward and input gradient --------------------------------------------------
+// dst[n][m][a][b][t] = sum over the source channels q of m's group and the taps (i, j) of
+//     weight(m, q, i, j) * src[n][q][ya][xb][t]
+// forward  (BACKWARD = false): dst = out, src = in,      ya = a*sH - pH + i*dH
+// gradient (BACKWARD = true):  dst = gradIn, src = gradOut, ya = (a + pH - i*dH) / sH where that
+//                              division is exact (the output rows whose tap i read input row a)
+// A lane owns VEC consecutive time samples of one destination pixel and MB destination channels
+// (accumulators in registers); a work-group of 256 lanes covers 256 consecutive vectors of the
+// (a, b, t) volume, which is also their order in memory, so stores are one contiguous run per
+// channel.  The work-group's MB x K weights sit in LDS, tap-major, and are read as broadcasts.
+struct GatherArgs {
+    const float *src;
+    float *dst;
+    const float *w;
+    int SC, SH, SW, DC, DH, DW, T;
+    int Qg, Mg, mBlocks, groups;  // source / destination channels per group, MB-blocks per group
+    int KH, KW, Cg, Og;
+    int mulH, mulW, offH, offW, stepH, stepW;  // source row numerator = a*mulH + offH + i*stepH
+    FastDiv divH, divW;                        // ... divided by the stride in the gradient
+    int P;                                     // vectors per destination channel plane = DH*DW*T/VEC
+    int chunks;                                // work-groups per (n, group, m-block)
+    FastDiv byChunks, byMBlocks, byGroups, byTV, byDW;
+};
+
+constexpr int kTapChunk = 256;  // taps of weights held in LDS at a time
+
+template <int VEC> struct TimeVec;
+template <> struct TimeVec<4> {
+    float4 v;
+    __device__ __forceinline__ void load(BufferRsrc b, int off) { v = buffer_load4<0>(b, off, 0); }
+    __device__ __forceinline__ void zero() { v = make_float4(0.f, 0.f, 0.f, 0.f); }
+    __device__ __forceinline__ void fma(float w, const TimeVec &x)
+    {
+        v.x = fmaf(w, x.v.x, v.x);
+        v.y = fmaf(w, x.v.y, v.y);
+        v.z = fmaf(w, x.v.z, v.z);
+        v.w = fmaf(w, x.v.w, v.w);
+    }
+    __device__ __forceinline__ void store(BufferRsrc b, int off) const { buffer_store4<kStream>(b, off, 0, v); }
+    __device__ __forceinline__ float dot(const TimeVec &x, float acc) const
+    {
+        acc = fmaf(v.x, x.v.x, acc);
+        acc = fmaf(v.y, x.v.y, acc);
+        acc = fmaf(v.z, x.v.z, acc);
+        return fmaf(v.w, x.v.w, acc);
+    }
+};
+template <> struct TimeVec<1> {
+    float v;
+    __device__ __forceinline__ void load(BufferRsrc b, int off)
+    {
+        v = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(b, off, 0, 0));
+    }
+    __device__ __forceinline__ void zero() { v = 0.f; }
+    __device__ __forceinline__ void fma(float w, const TimeVec &x) { v = fmaf(w, x.v, v); }
+    __device__ __forceinline__ void store(BufferRsrc b, int off) const { buffer_store<kStream>(b, off, 0, v); }
+    __device__ __forceinline__ float dot(const TimeVec &x, float acc) const { return fmaf(v, x.v, acc); }
+};
+
+template <int MB, int VEC, bool BACKWARD, bool STRIDED>
+__global__ __launch_bounds__(256) void synapse_gather_kernel(GatherArgs g)
+{
+    __shared__ __attribute__((aligned(16))) float wl[kTapChunk * MB];
+
+    // work-group -> (batch item, group, block of MB destination channels, chunk of 256 vectors)
+    uint32_t rest = blockIdx.x;
+    const uint32_t nmb = fastdiv(rest, g.byChunks);
+    const int chunk = static_cast<int>(rest - nmb * g.byChunks.d);
+    const uint32_t ng = fastdiv(nmb, g.byMBlocks);
+    const int mb0 = static_cast<int>(nmb - ng * g.byMBlocks.d) * MB;  // first channel of the block, within the group
+    const uint32_t n = fastdiv(ng, g.byGroups);
+    const int grp = static_cast<int>(ng - n * g.byGroups.d);
+
+    const int p = chunk * 256 + static_cast<int>(threadIdx.x);
+    const bool live = p < g.P;
+    const uint32_t pix = fastdiv(static_cast<uint32_t>(live ? p : 0), g.byTV);
+    const int tv = (live ? p : 0) - static_cast<int>(pix * g.byTV.d);
+    const int a = static_cast<int>(fastdiv(pix, g.byDW));
+    const int b = static_cast<int>(pix) - a * g.DW;
+
+    const int64_t srcPlane = static_cast<int64_t>(g.SH) * g.SW * g.T;  // floats per source channel
+    const BufferRsrc srcB = make_buffer(g.src + (static_cast<int64_t>(n) * g.SC + static_cast<int64_t>(grp) * g.Qg) * srcPlane);
+    const int rowBytes = g.SW * g.T * 4, pixBytes = g.T * 4;
+    const int planeBytes = static_cast<int>(srcPlane) * 4;
+    const int laneBytes = tv * VEC * 4;
+    const int yNum0 = a * g.mulH + g.offH, xNum0 = b * g.mulW + g.offW;
+
+    TimeVec<VEC> acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m].zero();
+
+    const int KK = g.KH * g.KW;
+    const int K = g.Qg * KK;
+    for (int k0 = 0; k0 < K; k0 += kTapChunk) {
+        const int kc = min(kTapChunk, K - k0);
+        __syncthreads();
+        for (int e = threadIdx.x; e < kc * MB; e += 256) {
+            const int tap = k0 + e / MB, m = mb0 + e % MB;
+            const int q = tap / KK, ij = tap - q * KK;
+            float v = 0.f;
+            if (m < g.Mg) {
+                const int64_t idx = BACKWARD
+                    ? (static_cast<int64_t>(grp * g.Og + q) * g.Cg + m) * KK + ij
+                    : (static_cast<int64_t>(grp * g.Og + m) * g.Cg + q) * KK + ij;
+                v = g.w[idx];
+            }
+            wl[e] = v;
+        }
+        __syncthreads();
+
+        // taps k0 .. k0+kc in (q, i, j) order; the counters are wave-uniform.  The load of a tap is
+        // issued one tap ahead of the multiply-adds that use it.
+        int q = k0 / KK, ij = k0 - q * KK;
+        int i = ij / g.KW, j = ij - i * g.KW;
+        auto fetch = [&](bool inChunk) {
+            const int yNum = yNum0 + i * g.stepH, xNum = xNum0 + j * g.stepW;
+            int ys, xs;
+            bool ok;
+            if (STRIDED) {
+                const uint32_t yq = fastdiv(static_cast<uint32_t>(yNum), g.divH);
+                const uint32_t xq = fastdiv(static_cast<uint32_t>(xNum), g.divW);
+                ok = yNum >= 0 && xNum >= 0 && static_cast<int>(yq * g.divH.d) == yNum &&
+                     static_cast<int>(xq * g.divW.d) == xNum && static_cast<int>(yq) < g.SH &&
+                     static_cast<int>(xq) < g.SW;
+                ys = static_cast<int>(yq);
+                xs = static_cast<int>(xq);
+            } else {
+                ok = static_cast<unsigned>(yNum) < static_cast<unsigned>(g.SH) &&
+                     static_cast<unsigned>(xNum) < static_cast<unsigned>(g.SW);
+                ys = yNum;
+                xs = xNum;
+            }
+            TimeVec<VEC> x;
+            x.load(srcB, masked_offset(ok && live && inChunk,
+                                       q * planeBytes + ys * rowBytes + xs * pixBytes + laneBytes));
+            if (++j == g.KW) {
+                j = 0;
+                if (++i == g.KH) { i = 0; ++q; }
+            }
+            return x;
+        };
+        TimeVec<VEC> x = fetch(true);
+        for (int t = 0; t < kc; ++t) {
+            const TimeVec<VEC> xn = fetch(t + 1 < kc);
+            const float *wt = wl + t * MB;
+            if constexpr (MB >= 4) {
+#pragma unroll
+                for (int m = 0; m < MB; m += 4) {
+                    const float4 w4 = *reinterpret_cast<const float4 *>(wt + m);
+                    acc[m].fma(w4.x, x);
+                    acc[m + 1].fma(w4.y, x);
+                    acc[m + 2].fma(w4.z, x);
+                    acc[m + 3].fma(w4.w, x);
+                }
+            } else {
+#pragma unroll
+                for (int m = 0; m < MB; ++m) acc[m].fma(wt[m], x);
+            }
+            x = xn;
+        }
+    }
+
+    const int64_t dstPlane = static_cast<int64_t>(g.DH) * g.DW * g.T;
+    const BufferRsrc dstB = make_buffer(g.dst + (static_cast<int64_t>(n) * g.DC + static_cast<int64_t>(grp) * g.Mg) * dstPlane);
+    const int dstPlaneBytes = static_cast<int>(dstPlane) * 4;
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+        acc[m].store(dstB, masked_offset(live && mb0 + m < g.Mg, (mb0 + m) * dstPlaneBytes + p * VEC * 4));
+}
+
+// ---- weight gradient -----------------------------------------------------------------------------
+// gradW[o][c'][i][j] = sum_{n,a,b,t} gradOut[n][o][a][b][t] * in[n][c][a*sH-pH+i*dH][b*sW-pW+j*dW][t]
+// A work-group owns OBW output channels x TAPS taps of one input channel for one slice of one batch
+// item's (a, b, t) volume; a lane walks the slice's vectors with stride 256 keeping OBW x TAPS
+// partial sums in registers.  The 256 lane sums are combined in a fixed tree (wavefront shuffles,
+// then LDS) and written to a workspace row per slice; a second kernel adds the rows in order, so the
+// result does not depend on scheduling.
+struct WgradArgs {
+    const float *gradOut, *in;
+    float *partial;  // [slices][nW]
+    SynGeom s;
+    int Cg, Og, oBlocks, tapBlocks, slicesPerItem, P, perSlice;  // P = OH*OW*T/VEC vectors per plane
+    FastDiv bySlices, byTapBlocks, byCg, byOBlocks, byGroups, byTV, byOW;
+    int nW;
+};
+
+template <int OBW, int TAPS, int VEC>
+__global__ __launch_bounds__(256) void synapse_wgrad_kernel(WgradArgs g)
+{
+    __shared__ float red[4][OBW * TAPS];
+    const SynGeom &s = g.s;
+
+    uint32_t r = blockIdx.x;
+    uint32_t q = fastdiv(r, g.bySlices);
+    const int slice = static_cast<int>(r - q * g.bySlices.d);
+    r = q; q = fastdiv(r, g.byTapBlocks);
+    const int tap0 = static_cast<int>(r - q * g.byTapBlocks.d) * TAPS;
+    r = q; q = fastdiv(r, g.byCg);
+    const int cl = static_cast<int>(r - q * g.byCg.d);
+    r = q; q = fastdiv(r, g.byOBlocks);
+    const int ol0 = static_cast<int>(r - q * g.byOBlocks.d) * OBW;
+    r = q; q = fastdiv(r, g.byGroups);
+    const int grp = static_cast<int>(r - q * g.byGroups.d);
+    const int n = static_cast<int>(q);
+
+    const int KK = s.KH * s.KW;
+    const int64_t goPlane = static_cast<int64_t>(s.OH) * s.OW * s.T, inPlane = static_cast<int64_t>(s.H) * s.W * s.T;
+    const BufferRsrc goB = make_buffer(g.gradOut + (static_cast<int64_t>(n) * s.O + grp * g.Og + ol0) * goPlane);
+    const BufferRsrc inB = make_buffer(g.in + (static_cast<int64_t>(n) * s.C + grp * g.Cg + cl) * inPlane);
+    const int goPlaneBytes = static_cast<int>(goPlane) * 4;
+    const int rowBytes = s.W * s.T * 4, pixBytes = s.T * 4;
+
+    // tap offsets of this block (wave-uniform)
+    int dy[TAPS], dx[TAPS];
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) {
+        const int tap = tap0 + k;
+        const int i = tap / s.KW, j = tap - i * s.KW;
+        dy[k] = tap < KK ? i * s.dH - s.pH : -(1 << 28);  // a tap past the filter never lands inside
+        dx[k] = j * s.dW - s.pW;
+    }
+
+    float acc[OBW][TAPS];
+#pragma unroll
+    for (int o = 0; o < OBW; ++o)
+#pragma unroll
+        for (int k = 0; k < TAPS; ++k) acc[o][k] = 0.f;
+
+    const int pEnd = min(g.P, (slice + 1) * g.perSlice);
+    for (int p = slice * g.perSlice + static_cast<int>(threadIdx.x); p < pEnd; p += 256) {
+        const uint32_t pix = fastdiv(static_cast<uint32_t>(p), g.byTV);
+        const int tv = p - static_cast<int>(pix * g.byTV.d);
+        const int a = static_cast<int>(fastdiv(pix, g.byOW));
+        const int b = static_cast<int>(pix) - a * s.OW;
+        TimeVec<VEC> go[OBW];
+#pragma unroll
+        for (int o = 0; o < OBW; ++o) go[o].load(goB, masked_offset(ol0 + o < g.Og, o * goPlaneBytes + p * VEC * 4));
+        const int y0 = a * s.sH, x0 = b * s.sW, laneBytes = tv * VEC * 4;
+#pragma unroll
+        for (int k = 0; k < TAPS; ++k) {
+            const int y = y0 + dy[k], x = x0 + dx[k];
+            const bool ok = static_cast<unsigned>(y) < static_cast<unsigned>(s.H) &&
+                            static_cast<unsigned>(x) < static_cast<unsigned>(s.W);
+            TimeVec<VEC> xv;
+            xv.load(inB, masked_offset(ok, y * rowBytes + x * pixBytes + laneBytes));
+#pragma unroll
+            for (int o = 0; o < OBW; ++o) acc[o][k] = go[o].dot(xv, acc[o][k]);
+        }
+    }
+
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int o = 0; o < OBW; ++o)
+#pragma unroll
+        for (int k = 0; k < TAPS; ++k) {
+            float v = acc[o][k];
+#pragma unroll
+            for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_down(v, off, kWave);
+            if (lane == 0) red[wave][o * TAPS + k] = v;
+        }
+    __syncthreads();
+    if (threadIdx.x < OBW * TAPS) {
+        const int o = threadIdx.x / TAPS, k = threadIdx.x - o * TAPS;
+        if (ol0 + o < g.Og && tap0 + k < KK) {
+            const float v = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
+            const int64_t widx = (static_cast<int64_t>(grp * g.Og + ol0 + o) * g.Cg + cl) * KK + tap0 + k;
+            g.partial[(static_cast<int64_t>(n) * g.slicesPerItem + slice) * g.nW + widx] = v;
+        }
+    }
+}
+
+// gradW[q] = sum of the workspace rows in row order.
+__global__ __launch_bounds__(256) void synapse_wgrad_sum_kernel(float *__restrict__ gradW,
+                                                                const float *__restrict__ partial, int rows, int nW)
+{
+    const int q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= nW) return;
+    float acc = 0.f;
+    for (int r = 0; r < rows; ++r) acc += partial[static_cast<int64_t>(r) * nW + q];
+    gradW[q] = acc;
+}
+
+// ---- host side -------------------------------------------------------------------------------------
+static int out_extent(int64_t in, int64_t k, int64_t s, int64_t p, int64_t d)
+{
+    const int64_t span = in + 2 * p - d * (k - 1) - 1;
+    return span < 0 ? 0 : static_cast<int>(span / s + 1);
+}
+
+// Validates the caller's geometry and fills the derived output extents.
+static int check_geom(const slayer_synapse_geom *c, SynGeom &s)
+{
+    if (!c) return SLAYER_EINVAL;
+    s = SynGeom{c->N, c->C, c->H, c->W, c->T, c->O, c->KH, c->KW, c->strideH, c->strideW, c->padH,
+                c->padW, c->dilH, c->dilW, c->groups, 0, 0};
+    if (s.N < 0 || s.C < 0 || s.H < 0 || s.W < 0 || s.T < 0 || s.O < 0) return SLAYER_EINVAL;
+    if (s.KH < 1 || s.KW < 1 || s.sH < 1 || s.sW < 1 || s.dH < 1 || s.dW < 1 || s.pH < 0 || s.pW < 0) return SLAYER_EINVAL;
+    if (s.groups < 1 || s.C % s.groups || s.O % s.groups) return SLAYER_EINVAL;
+    s.OH = out_extent(s.H, s.KH, s.sH, s.pH, s.dH);
+    s.OW = out_extent(s.W, s.KW, s.sW, s.pW, s.dW);
+    // the kernels index one batch item with 32-bit byte offsets, and the padded extents with int
+    const int64_t limit = (1LL << 31) - 64;
+    if (static_cast<int64_t>(s.C) * s.H * s.W * s.T * 4 >= limit) return SLAYER_EUNSUPPORTED;
+    if (static_cast<int64_t>(s.O) * s.OH * s.OW * s.T * 4 >= limit) return SLAYER_EUNSUPPORTED;
+    if (static_cast<int64_t>(s.H) + 2LL * s.pH + static_cast<int64_t>(s.dH) * s.KH >= (1 << 24)) return SLAYER_EUNSUPPORTED;
+    if (static_cast<int64_t>(s.W) + 2LL * s.pW + static_cast<int64_t>(s.dW) * s.KW >= (1 << 24)) return SLAYER_EUNSUPPORTED;
+    if (static_cast<int64_t>(s.C / s.groups) * s.KH * s.KW >= (1 << 24)) return SLAYER_EUNSUPPORTED;
+    if (static_cast<int64_t>(s.O) * (s.C / s.groups) * s.KH * s.KW >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+    return SLAYER_OK;
+}
+
+template <int MB, int VEC, bool BACKWARD>
+static void launch_gather_mb(const GatherArgs &g, bool strided, unsigned blocks, hipStream_t st)
+{
+    if (strided)
+        hipLaunchKernelGGL((synapse_gather_kernel<MB, VEC, BACKWARD, true>), dim3(blocks), dim3(256), 0, st, g);
+    else
+        hipLaunchKernelGGL((synapse_gather_kernel<MB, VEC, BACKWARD, false>), dim3(blocks), dim3(256), 0, st, g);
+}
+
+template <bool BACKWARD>
+static int launch_gather(float *dst, const float *src, const float *w, const SynGeom &s, hipStream_t st)
+{
+    GatherArgs g{};
+    g.src = src; g.dst = dst; g.w = w;
+    g.T = s.T; g.groups = s.groups; g.KH = s.KH; g.KW = s.KW;
+    g.Cg = s.C / s.groups; g.Og = s.O / s.groups;
+    bool strided = false;
+    if (!BACKWARD) {
+        g.SC = s.C; g.SH = s.H; g.SW = s.W; g.DC = s.O; g.DH = s.OH; g.DW = s.OW;
+        g.Qg = g.Cg; g.Mg = g.Og;
+        g.mulH = s.sH; g.mulW = s.sW; g.offH = -s.pH; g.offW = -s.pW; g.stepH = s.dH; g.stepW = s.dW;
+        g.divH = make_fastdiv(1); g.divW = make_fastdiv(1);
+    } else {
+        g.SC = s.O; g.SH = s.OH; g.SW = s.OW; g.DC = s.C; g.DH = s.H; g.DW = s.W;
+        g.Qg = g.Og; g.Mg = g.Cg;
+        g.mulH = 1; g.mulW = 1; g.offH = s.pH; g.offW = s.pW; g.stepH = -s.dH; g.stepW = -s.dW;
+        g.divH = make_fastdiv(static_cast<uint32_t>(s.sH)); g.divW = make_fastdiv(static_cast<uint32_t>(s.sW));
+        strided = s.sH > 1 || s.sW > 1;
+    }
+    const int64_t dstElems = static_cast<int64_t>(s.N) * g.DC * g.DH * g.DW * g.T;
+    if (dstElems == 0) return SLAYER_OK;
+    const bool vec = s.T % 4 == 0 && aligned16(src) && aligned16(dst);
+    const int VEC = vec ? 4 : 1;
+    g.P = g.DH * g.DW * (g.T / VEC);
+    g.chunks = static_cast<int>(ceil_div(g.P, 256));
+    // destination channels per lane: as many as the group has, up to 16
+    const int MB = g.Mg >= 12 ? 16 : g.Mg >= 6 ? 8 : g.Mg >= 3 ? 4 : g.Mg == 2 ? 2 : 1;
+    g.mBlocks = static_cast<int>(ceil_div(g.Mg, MB));
+    const int64_t blocks = static_cast<int64_t>(s.N) * s.groups * g.mBlocks * g.chunks;
+    if (blocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+    g.byChunks = make_fastdiv(static_cast<uint32_t>(g.chunks));
+    g.byMBlocks = make_fastdiv(static_cast<uint32_t>(g.mBlocks));
+    g.byGroups = make_fastdiv(static_cast<uint32_t>(s.groups));
+    g.byTV = make_fastdiv(static_cast<uint32_t>(g.T / VEC));
+    g.byDW = make_fastdiv(static_cast<uint32_t>(g.DW));
+    const unsigned nb = static_cast<unsigned>(blocks);
+#define SLAYER_GATHER(MBV)                                                        \
+    do {                                                                          \
+        if (vec) launch_gather_mb<MBV, 4, BACKWARD>(g, strided, nb, st);          \
+        else launch_gather_mb<MBV, 1, BACKWARD>(g, strided, nb, st);              \
+    } while (0)
+    switch (MB) {
+        case 16: SLAYER_GATHER(16); break;
+        case 8: SLAYER_GATHER(8); break;
+        case 4: SLAYER_GATHER(4); break;
+        case 2: SLAYER_GATHER(2); break;
+        default: SLAYER_GATHER(1); break;
+    }
+#undef SLAYER_GATHER
+    return launch_status();
+}
+
+// Slices per batch item for the weight gradient: enough work-groups to fill the GPU a few times
+// over, at least a few trips per lane.
+struct WgradPlan {
+    int OBW, TAPS, oBlocks, tapBlocks, slicesPerItem, perSlice, VEC, P;
+    int64_t groupsOfWork;
+};
+
+static WgradPlan plan_wgrad(const SynGeom &s, bool vec)
+{
+    WgradPlan p{};
+    const int KK = s.KH * s.KW, Og = s.O / s.groups, Cg = s.C / s.groups;
+    p.VEC = vec ? 4 : 1;
+    p.OBW = Og >= 6 ? 8 : Og >= 3 ? 4 : Og == 2 ? 2 : 1;
+    p.TAPS = KK >= 7 ? 9 : KK >= 3 ? 4 : KK;  // 1, 2, 4 or 9 taps per pass
+    p.oBlocks = static_cast<int>(ceil_div(Og, p.OBW));
+    p.tapBlocks = static_cast<int>(ceil_div(KK, p.TAPS));
+    p.P = s.OH * s.OW * (s.T / p.VEC);
+    p.groupsOfWork = static_cast<int64_t>(s.N) * s.groups * p.oBlocks * Cg * p.tapBlocks;
+    const int64_t want = 4096;
+    int64_t slices = p.groupsOfWork > 0 ? ceil_div(want, p.groupsOfWork) : 1;
+    const int64_t maxSlices = ceil_div(p.P, 256 * 4);  // keep at least four trips per lane
+    if (slices > maxSlices) slices = maxSlices;
+    if (slices < 1) slices = 1;
+    p.perSlice = static_cast<int>(ceil_div(ceil_div(p.P, slices), 256) * 256);
+    if (p.perSlice < 256) p.perSlice = 256;  // empty output: one empty slice
+    p.slicesPerItem = static_cast<int>(ceil_div(p.P, p.perSlice));
+    if (p.slicesPerItem < 1) p.slicesPerItem = 1;
+    return p;
+}
+
+template <int OBW, int TAPS>
+static void launch_wgrad_vec(const WgradArgs &g, int VEC, unsigned blocks, hipStream_t st)
+{
+    if (VEC == 4) hipLaunchKernelGGL((synapse_wgrad_kernel<OBW, TAPS, 4>), dim3(blocks), dim3(256), 0, st, g);
+    else hipLaunchKernelGGL((synapse_wgrad_kernel<OBW, TAPS, 1>), dim3(blocks), dim3(256), 0, st, g);
+}
+
+template <int OBW>
+static void launch_wgrad_taps(const WgradArgs &g, const WgradPlan &p, unsigned blocks, hipStream_t st)
+{
+    switch (p.TAPS) {
+        case 9: launch_wgrad_vec<OBW, 9>(g, p.VEC, blocks, st); break;
+        case 4: launch_wgrad_vec<OBW, 4>(g, p.VEC, blocks, st); break;
+        case 2: launch_wgrad_vec<OBW, 2>(g, p.VEC, blocks, st); break;
+        default: launch_wgrad_vec<OBW, 1>(g, p.VEC, blocks, st); break;
+    }
+}
+
+}  // namespace slayer
+
+extern "C" int slayer_synapse_out_shape(const slayer_synapse_geom *geom, int32_t *OH, int32_t *OW)
+{
+    slayer::SynGeom s;
+    const int status = slayer::check_geom(geom, s);
+    if (status != SLAYER_OK) return status;
+    if (OH) *OH = s.OH;
+    if (OW) *OW = s.OW;
+    return SLAYER_OK;
+}
+
+extern "C" int slayer_synapse_conv_f32(float *out, const float *in, const float *weight,
+                                       const slayer_synapse_geom *geom, void *stream)
+{
+    using namespace slayer;
+    SynGeom s;
+    const int status = check_geom(geom, s);
+    if (status != SLAYER_OK) return status;
+    const int64_t outElems = static_cast<int64_t>(s.N) * s.O * s.OH * s.OW * s.T;
+    if (outElems == 0) return SLAYER_OK;
+    if (!out || !in || !weight) return SLAYER_EINVAL;
+    return launch_gather<false>(out, in, weight, s, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int slayer_synapse_conv_grad_input_f32(float *gradIn, const float *gradOut, const float *weight,
+                                                  const slayer_synapse_geom *geom, void *stream)
+{
+    using namespace slayer;
+    SynGeom s;
+    const int status = check_geom(geom, s);
+    if (status != SLAYER_OK) return status;
+    const int64_t inElems = static_cast<int64_t>(s.N) * s.C * s.H * s.W * s.T;
+    if (inElems == 0) return SLAYER_OK;
+    if (!gradIn || !weight) return SLAYER_EINVAL;
+    const int64_t outElems = static_cast<int64_t>(s.N) * s.O * s.OH * s.OW * s.T;
+    if (outElems > 0 && !gradOut) return SLAYER_EINVAL;
+    // with an empty gradOut every tap is out of range and the kernel writes zeros
+    return launch_gather<true>(gradIn, gradOut ? gradOut : gradIn, weight, s, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int64_t slayer_synapse_conv_grad_weight_workspace_bytes(const slayer_synapse_geom *geom)
+{
+    using namespace slayer;
+    SynGeom s;
+    if (check_geom(geom, s) != SLAYER_OK) return 0;
+    const int64_t nW = static_cast<int64_t>(s.O) * (s.C / s.groups) * s.KH * s.KW;
+    if (nW == 0 || s.N == 0) return 0;
+    const WgradPlan p = plan_wgrad(s, s.T % 4 == 0);
+    return static_cast<int64_t>(s.N) * p.slicesPerItem * nW * static_cast<int64_t>(sizeof(float));
+}
+
+extern "C" int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gradOut, const float *in,
+                                                   float *workspace, const slayer_synapse_geom *geom,
+                                                   void *stream)
+{
+    using namespace slayer;
+    SynGeom s;
+    const int status = check_geom(geom, s);
+    if (status != SLAYER_OK) return status;
+    const int64_t nW64 = static_cast<int64_t>(s.O) * (s.C / s.groups) * s.KH * s.KW;
+    if (nW64 == 0) return SLAYER_OK;
+    if (!gradW) return SLAYER_EINVAL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int nW = static_cast<int>(nW64);
+    const int64_t outElems = static_cast<int64_t>(s.N) * s.O * s.OH * s.OW * s.T;
+    int rows = 0;
+    if (outElems > 0) {
+        if (!gradOut || !in || !workspace) return SLAYER_EINVAL;
+        // the slicing must match slayer_synapse_conv_grad_weight_workspace_bytes: vectors only
+        // when T allows them AND the pointers are aligned, otherwise the same slices of samples
+        const bool vecT = s.T % 4 == 0;
+        WgradPlan p = plan_wgrad(s, vecT);
+        const bool vec = vecT && aligned16(gradOut) && aligned16(in);
+        WgradArgs g{};
+        g.gradOut = gradOut; g.in = in; g.partial = workspace; g.s = s;
+        g.Cg = s.C / s.groups; g.Og = s.O / s.groups;
+        g.oBlocks = p.oBlocks; g.tapBlocks = p.tapBlocks; g.slicesPerItem = p.slicesPerItem;
+        g.nW = nW;
+        if (vec) {
+            g.P = p.P; g.perSlice = p.perSlice;
+        } else {
+            // same number of slices, four times the positions when T would have allowed vectors
+            const int scale = vecT ? 4 : 1;
+            p.VEC = 1;
+            g.P = p.P * scale; g.perSlice = p.perSlice * scale;
+        }
+        g.bySlices = make_fastdiv(static_cast<uint32_t>(p.slicesPerItem));
+        g.byTapBlocks = make_fastdiv(static_cast<uint32_t>(p.tapBlocks));
+        g.byCg = make_fastdiv(static_cast<uint32_t>(g.Cg));
+        g.byOBlocks = make_fastdiv(static_cast<uint32_t>(p.oBlocks));
+        g.byGroups = make_fastdiv(static_cast<uint32_t>(s.groups));
+        g.byTV = make_fastdiv(static_cast<uint32_t>(s.T / p.VEC));
+        g.byOW = make_fastdiv(static_cast<uint32_t>(s.OW));
+        const int64_t blocks = p.groupsOfWork * p.slicesPerItem;
+        if (blocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+        const unsigned nb = static_cast<unsigned>(blocks);
+        switch (p.OBW) {
+            case 8: launch_wgrad_taps<8>(g, p, nb, st); break;
+            case 4: launch_wgrad_taps<4>(g, p, nb, st); break;
+            case 2: launch_wgrad_taps<2>(g, p, nb, st); break;
+            default: launch_wgrad_taps<1>(g, p, nb, st); break;
+        }
+        const int st1 = launch_status();
+        if (st1 != SLAYER_OK) return st1;
+        rows = s.N * p.slicesPerItem;
+    }
+    hipLaunchKernelGGL(synapse_wgrad_sum_kernel, dim3(static_cast<unsigned>(ceil_div(nW, 256))), dim3(256), 0, st,
+                       gradW, workspace, rows, nW);
+    return launch_status();
+}

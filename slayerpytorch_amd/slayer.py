@@ -8,8 +8,10 @@ Mirrors, with the same names, signatures and side effects:
 * ``spikeLayer.psp`` / ``spike`` / ``delayShift`` / ``delay`` (src/slayer.py:130-142, 333-391),
 * autograd Functions ``_spikeFunction``, ``_pspFunction``, ``_delayLayer``, ``_delayFunction``,
   ``_delayFunctionNoGradient`` (src/slayer.py:817-979),
-* ``dense`` (src/slayer.py:144-172, 393-437) only as plumbing for end-to-end checks: it is a
-  plain ``conv3d`` and not part of the accelerated path.
+* ``dense`` (src/slayer.py:144-172, 393-437) as one library GEMM per batch item,
+* ``conv`` / ``pool`` / ``convTranspose`` / ``unpool`` (src/slayer.py:207-312, 451-748) over the
+  per-timestep synapse kernels of :mod:`slayerpytorch_amd.synapse` instead of ``F.conv3d`` /
+  ``F.conv_transpose3d`` with a (KH, KW, 1) kernel.
 
 Differences from the reference, all on the host: backward passes use the fused
 ``slayerCuda.spikeBackward`` / ``slayerCuda.delayGrad`` kernels instead of chains of
@@ -24,6 +26,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import slayerCuda
+from . import synapse
 
 
 def alphaKernel(tau, Ts, tSample, mult=1.0, EPSILON=0.01):
@@ -94,8 +97,28 @@ class spikeLayer(nn.Module):
         return _delayLayer(inputSize, self.simulation["Ts"])
 
     def dense(self, inFeatures, outFeatures, weightScale=10, preHookFx=None):
-        """Fully connected synapse applied per time step (plain conv3d, not accelerated here)."""
+        """Fully connected synapse applied per time step."""
         return _denseLayer(inFeatures, outFeatures, weightScale, preHookFx)
+
+    def conv(self, inChannels, outChannels, kernelSize, stride=1, padding=0, dilation=1, groups=1,
+             weightScale=100, preHookFx=None):
+        """Convolution synapse over (H, W), applied per time step (src/slayer.py:207-234)."""
+        return _convLayer(inChannels, outChannels, kernelSize, stride, padding, dilation, groups, weightScale,
+                          preHookFx)
+
+    def pool(self, kernelSize, stride=None, padding=0, dilation=1, preHookFx=None):
+        """Sum-pooling synapse with weights ``1.1 * theta`` (src/slayer.py:236-259)."""
+        return _poolLayer(self.neuron["theta"], kernelSize, stride, padding, dilation, preHookFx)
+
+    def convTranspose(self, inChannels, outChannels, kernelSize, stride=1, padding=0, dilation=1, groups=1,
+                      weightScale=100, preHookFx=None):
+        """Transposed convolution synapse (src/slayer.py:261-288)."""
+        return _convTransposeLayer(inChannels, outChannels, kernelSize, stride, padding, dilation, groups,
+                                   weightScale, preHookFx)
+
+    def unpool(self, kernelSize, stride=None, padding=0, dilation=1, preHookFx=None):
+        """Unpooling synapse with weights ``1.1 * theta`` (src/slayer.py:290-313)."""
+        return _unpoolLayer(self.neuron["theta"], kernelSize, stride, padding, dilation, preHookFx)
 
 
 class _denseLayer(nn.Conv3d):
@@ -128,6 +151,103 @@ class _denseLayer(nn.Conv3d):
             O, K = weight.shape[0], weight.shape[1] * weight.shape[2] * weight.shape[3]
             return torch.matmul(weight.reshape(O, K), input.reshape(N, K, T)).reshape(N, O, 1, 1, T)
         return F.conv3d(input, weight, self.bias, self.stride, self.padding, self.dilation, self.groups)
+
+
+def _hw(value, name, default=None):
+    """An int or a pair as the (h, w, time) triple torch's 3-D modules take, the way the reference's
+    layers expand their arguments (src/slayer.py:456-487)."""
+    if value is None:
+        return default
+    if isinstance(value, int):
+        return (value, value, 1 if name != "padding" else 0)
+    if len(value) == 2:
+        return (value[0], value[1], 1 if name != "padding" else 0)
+    raise Exception("{} can be either int or tuple of size 2. It was: {}".format(name, value))
+
+
+class _convLayer(nn.Conv3d):
+    """Convolution synapse (src/slayer.py:451-507): a (outFeatures, inFeatures/groups, KH, KW, 1)
+    weight applied at every time step by the per-timestep synapse kernel."""
+
+    def __init__(self, inFeatures, outFeatures, kernelSize, stride=1, padding=0, dilation=1, groups=1,
+                 weightScale=1, preHookFx=None):
+        super().__init__(inFeatures, outFeatures, _hw(kernelSize, "kernelSize"), _hw(stride, "stride"),
+                         _hw(padding, "padding"), _hw(dilation, "dilation"), groups, bias=False)
+        if weightScale != 1:
+            self.weight = nn.Parameter(weightScale * self.weight)
+        self.preHookFx = preHookFx
+
+    def forward(self, input):
+        weight = self.weight if self.preHookFx is None else self.preHookFx(self.weight)
+        return synapse.synapseConv(input, weight, self.stride[:2], self.padding[:2], self.dilation[:2],
+                                   self.groups)
+
+
+def _poolWeight(theta, shape):
+    return nn.Parameter(torch.full(shape, 1.1 * theta, dtype=torch.float32), requires_grad=False)
+
+
+class _poolLayer(nn.Conv3d):
+    """Sum pooling as a 1 -> 1 channel synapse with constant weights ``1.1 * theta`` on the tensor
+    viewed as (N, 1, C*H, W, T) (src/slayer.py:509-577).  Like the reference, an extent that is not
+    a multiple of the window is extended by ``extent % window`` rows of zeros."""
+
+    def __init__(self, theta, kernelSize, stride=None, padding=0, dilation=1, preHookFx=None):
+        kernel = _hw(kernelSize, "kernelSize")
+        super().__init__(1, 1, kernel, _hw(stride, "stride", kernel), _hw(padding, "padding"),
+                         _hw(dilation, "dilation"), bias=False)
+        self.weight = _poolWeight(theta, self.weight.shape)
+        self.preHookFx = preHookFx
+
+    def forward(self, input):
+        kH, kW = self.weight.shape[2], self.weight.shape[3]
+        if input.shape[2] % kH != 0:
+            input = torch.cat((input, input.new_zeros((input.shape[0], input.shape[1], input.shape[2] % kH,
+                                                       input.shape[3], input.shape[4]))), 2)
+        if input.shape[3] % kW != 0:
+            input = torch.cat((input, input.new_zeros((input.shape[0], input.shape[1], input.shape[2],
+                                                       input.shape[3] % kW, input.shape[4]))), 3)
+        N, C, H, W, T = input.shape
+        weight = self.weight if self.preHookFx is None else self.preHookFx(self.weight)
+        result = synapse.synapseConv(input.reshape(N, 1, C * H, W, T), weight, self.stride[:2], self.padding[:2],
+                                     self.dilation[:2], 1)
+        return result.reshape(result.shape[0], C, -1, result.shape[3], result.shape[4])
+
+
+class _convTransposeLayer(nn.ConvTranspose3d):
+    """Transposed convolution synapse (src/slayer.py:579-643)."""
+
+    def __init__(self, inFeatures, outFeatures, kernelSize, stride=1, padding=0, dilation=1, groups=1,
+                 weightScale=1, preHookFx=None):
+        super().__init__(inFeatures, outFeatures, _hw(kernelSize, "kernelSize"), _hw(stride, "stride"),
+                         _hw(padding, "padding"), 0, groups, False, _hw(dilation, "dilation"))
+        if weightScale != 1:
+            self.weight = nn.Parameter(weightScale * self.weight)
+        self.preHookFx = preHookFx
+
+    def forward(self, input):
+        weight = self.weight if self.preHookFx is None else self.preHookFx(self.weight)
+        return synapse.synapseConvTranspose(input, weight, self.stride[:2], self.padding[:2], self.dilation[:2],
+                                            self.groups)
+
+
+class _unpoolLayer(nn.ConvTranspose3d):
+    """Unpooling as a 1 -> 1 channel transposed synapse with constant weights ``1.1 * theta`` on the
+    tensor viewed as (N, 1, C*H, W, T) (src/slayer.py:645-748)."""
+
+    def __init__(self, theta, kernelSize, stride=None, padding=0, dilation=1, preHookFx=None):
+        kernel = _hw(kernelSize, "kernelSize")
+        super().__init__(1, 1, kernel, _hw(stride, "stride", kernel), _hw(padding, "padding"), 0, 1, False,
+                         _hw(dilation, "dilation"))
+        self.weight = _poolWeight(theta, self.weight.shape)
+        self.preHookFx = preHookFx
+
+    def forward(self, input):
+        N, C, H, W, T = input.shape
+        weight = self.weight if self.preHookFx is None else self.preHookFx(self.weight)
+        result = synapse.synapseConvTranspose(input.reshape(N, 1, C * H, W, T), weight, self.stride[:2],
+                                              self.padding[:2], self.dilation[:2], 1)
+        return result.reshape(result.shape[0], C, -1, result.shape[3], result.shape[4])
 
 
 class _spikeFunction(torch.autograd.Function):

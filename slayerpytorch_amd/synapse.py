@@ -1,0 +1,177 @@
+"""Per-timestep synapses on (N, C, H, W, T) tensors over the C ABI of ``libslayer_hip.so``.
+
+The reference's ``_convLayer`` / ``_poolLayer`` / ``_convTransposeLayer`` / ``_unpoolLayer`` call
+``F.conv3d`` / ``F.conv_transpose3d`` with a kernel of time extent 1 (src/slayer.py:499-507,
+:565-575, :631-643, :732-748) and leave the gradients to autograd.  Here the operation and its
+two gradients are three extension-level functions on T-innermost tensors, tied together by
+``synapseConv`` / ``synapseConvTranspose`` (autograd Functions with the argument meaning of the
+torch calls they replace).  There is no CPU path: tensors must live on the GPU.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from .slayerCuda import _check_device, _check_input, _on_device_of, _ptr
+
+__all__ = ["conv", "convGradInput", "convGradWeight", "outShape", "synapseConv", "synapseConvTranspose"]
+
+
+def _pair(v, name):
+    if isinstance(v, int):
+        return v, v
+    v = tuple(int(x) for x in v)
+    if len(v) == 3 and name != "kernel":          # torch-style triple with the time entry last
+        v = v[:2]
+    if len(v) != 2:
+        raise ValueError("%s must be an int or a pair, got %r" % (name, v))
+    return v
+
+
+def _geom(inShape, wShape, stride, padding, dilation, groups):
+    if len(inShape) != 5:
+        raise RuntimeError("expected a 5 dimensional (N,C,H,W,T) tensor, got %d dimensions" % len(inShape))
+    if len(wShape) == 5:
+        if wShape[4] != 1:
+            raise RuntimeError("the synapse kernel must have a time extent of 1, got %d" % wShape[4])
+        wShape = wShape[:4]
+    if len(wShape) != 4:
+        raise RuntimeError("expected a weight of shape (O, C/groups, KH, KW[, 1]), got %r" % (tuple(wShape),))
+    N, C, H, W, T = (int(v) for v in inShape)
+    O, Cg, KH, KW = (int(v) for v in wShape)
+    groups = int(groups)
+    if groups < 1 or C % groups or O % groups or Cg * groups != C:
+        raise RuntimeError("weight of shape %r does not fit %d input channels in %d groups"
+                           % (tuple(wShape), C, groups))
+    (sH, sW), (pH, pW), (dH, dW) = _pair(stride, "stride"), _pair(padding, "padding"), _pair(dilation, "dilation")
+    return _lib.SynapseGeom(N, C, H, W, T, O, KH, KW, sH, sW, pH, pW, dH, dW, groups)
+
+
+def outShape(inShape, wShape, stride=1, padding=0, dilation=1, groups=1):
+    """Shape (N, O, OH, OW, T) of ``conv`` for an input of shape ``inShape``."""
+    g = _geom(inShape, wShape, stride, padding, dilation, groups)
+    OH, OW = ctypes.c_int32(), ctypes.c_int32()
+    _lib.check(_lib.load().slayer_synapse_out_shape(ctypes.byref(g), ctypes.byref(OH), ctypes.byref(OW)),
+               "slayer_synapse_out_shape")
+    return (g.N, g.O, OH.value, OW.value, g.T)
+
+
+def conv(input, weight, stride=1, padding=0, dilation=1, groups=1):
+    """``F.conv3d(input, weight, None, (sH,sW,1), (pH,pW,0), (dH,dW,1), groups)`` for a weight of
+    time extent 1."""
+    _check_input(input, "input")
+    _check_input(weight, "weight")
+    _check_device(input, weight, "input", "weight")
+    g = _geom(input.shape, weight.shape, stride, padding, dilation, groups)
+    lib = _lib.load()
+    out = torch.empty(outShape(input.shape, weight.shape, stride, padding, dilation, groups),
+                      dtype=input.dtype, device=input.device)
+    with _on_device_of(input) as stream:
+        _lib.check(lib.slayer_synapse_conv_f32(_ptr(out), _ptr(input), _ptr(weight), ctypes.byref(g), stream),
+                   "slayer_synapse_conv_f32")
+    return out
+
+
+def convGradInput(gradOutput, weight, inShape, stride=1, padding=0, dilation=1, groups=1):
+    """Gradient of ``conv`` with respect to its input of shape ``inShape`` (= the transposed
+    convolution of ``gradOutput``)."""
+    _check_input(gradOutput, "gradOutput")
+    _check_input(weight, "weight")
+    _check_device(gradOutput, weight, "gradOutput", "weight")
+    g = _geom(inShape, weight.shape, stride, padding, dilation, groups)
+    expected = outShape(inShape, weight.shape, stride, padding, dilation, groups)
+    if tuple(gradOutput.shape) != expected:
+        raise RuntimeError("gradOutput has shape %r, expected %r" % (tuple(gradOutput.shape), expected))
+    lib = _lib.load()
+    gradIn = torch.empty(tuple(int(v) for v in inShape), dtype=gradOutput.dtype, device=gradOutput.device)
+    with _on_device_of(gradOutput) as stream:
+        _lib.check(lib.slayer_synapse_conv_grad_input_f32(_ptr(gradIn), _ptr(gradOutput), _ptr(weight),
+                                                          ctypes.byref(g), stream),
+                   "slayer_synapse_conv_grad_input_f32")
+    return gradIn
+
+
+def convGradWeight(gradOutput, input, wShape, stride=1, padding=0, dilation=1, groups=1):
+    """Gradient of ``conv`` with respect to its weight of shape ``wShape``."""
+    _check_input(gradOutput, "gradOutput")
+    _check_input(input, "input")
+    _check_device(gradOutput, input, "gradOutput", "input")
+    g = _geom(input.shape, wShape, stride, padding, dilation, groups)
+    expected = outShape(input.shape, wShape, stride, padding, dilation, groups)
+    if tuple(gradOutput.shape) != expected:
+        raise RuntimeError("gradOutput has shape %r, expected %r" % (tuple(gradOutput.shape), expected))
+    lib = _lib.load()
+    gradW = torch.empty(tuple(int(v) for v in wShape), dtype=input.dtype, device=input.device)
+    nbytes = lib.slayer_synapse_conv_grad_weight_workspace_bytes(ctypes.byref(g))
+    workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=input.device)
+    with _on_device_of(input) as stream:
+        _lib.check(lib.slayer_synapse_conv_grad_weight_f32(_ptr(gradW), _ptr(gradOutput), _ptr(input),
+                                                           _ptr(workspace), ctypes.byref(g), stream),
+                   "slayer_synapse_conv_grad_weight_f32")
+    return gradW
+
+
+class _synapseConvFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, weight, stride, padding, dilation, groups):
+        input = input.contiguous()
+        weight = weight.contiguous()
+        ctx.save_for_backward(input, weight)
+        ctx.args = (stride, padding, dilation, groups)
+        return conv(input, weight, *ctx.args)
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        input, weight = ctx.saved_tensors
+        gradOutput = gradOutput.contiguous()
+        gradInput = gradWeight = None
+        if ctx.needs_input_grad[0]:
+            gradInput = convGradInput(gradOutput, weight, input.shape, *ctx.args)
+        if ctx.needs_input_grad[1]:
+            gradWeight = convGradWeight(gradOutput, input, weight.shape, *ctx.args)
+        return gradInput, gradWeight, None, None, None, None
+
+
+class _synapseConvTransposeFunction(torch.autograd.Function):
+    """The transposed synapse: its forward pass is the input gradient of the convolution whose
+    weight tensor it shares, its input gradient is that convolution."""
+
+    @staticmethod
+    def forward(ctx, input, weight, stride, padding, dilation, groups):
+        input = input.contiguous()
+        weight = weight.contiguous()
+        (sH, sW), (pH, pW), (dH, dW) = _pair(stride, "stride"), _pair(padding, "padding"), _pair(dilation, "dilation")
+        N, Cin, H, W, T = input.shape
+        if weight.shape[0] != Cin:
+            raise RuntimeError("weight of shape %r does not fit %d input channels" % (tuple(weight.shape), Cin))
+        KH, KW = int(weight.shape[2]), int(weight.shape[3])
+        outH = (H - 1) * sH - 2 * pH + dH * (KH - 1) + 1
+        outW = (W - 1) * sW - 2 * pW + dW * (KW - 1) + 1
+        ctx.outShape = (N, int(weight.shape[1]) * groups, outH, outW, T)
+        ctx.save_for_backward(input, weight)
+        ctx.args = (stride, padding, dilation, groups)
+        return convGradInput(input, weight, ctx.outShape, *ctx.args)
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        input, weight = ctx.saved_tensors
+        gradOutput = gradOutput.contiguous()
+        gradInput = gradWeight = None
+        if ctx.needs_input_grad[0]:
+            gradInput = conv(gradOutput, weight, *ctx.args)
+        if ctx.needs_input_grad[1]:
+            gradWeight = convGradWeight(input, gradOutput, weight.shape, *ctx.args)
+        return gradInput, gradWeight, None, None, None, None
+
+
+def synapseConv(input, weight, stride=1, padding=0, dilation=1, groups=1):
+    """Differentiable ``conv``: stands where the reference calls ``F.conv3d(input, weight, None,
+    stride, padding, dilation, groups)`` (src/slayer.py:499-507)."""
+    return _synapseConvFunction.apply(input, weight, stride, padding, dilation, groups)
+
+
+def synapseConvTranspose(input, weight, stride=1, padding=0, dilation=1, groups=1):
+    """Differentiable transposed synapse: stands where the reference calls
+    ``F.conv_transpose3d(input, weight, None, stride, padding, 0, groups, dilation)``
+    (src/slayer.py:631-643)."""
+    return _synapseConvTransposeFunction.apply(input, weight, stride, padding, dilation, groups)

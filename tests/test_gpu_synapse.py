@@ -1,0 +1,255 @@
+"""Parity of the per-timestep synapse kernels (conv / pool / convTranspose / unpool layers and the
+three C-ABI entry points behind them) with the CPU oracle on the same seeded inputs.
+
+Tolerance: fp32 sums in a different order than the oracle's double accumulation, so every element
+must satisfy |gpu - oracle| <= SUM_TOL * sum |terms| (the oracle evaluated on |x|, |w|), which is the
+natural scale of a rounding error of a sum; for unit-scale data this is tighter than 1e-5 relative
+to the largest output.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from slayerpytorch_amd import _lib, synapse
+import slayerpytorch_amd as snn
+
+pytestmark = pytest.mark.gpu
+
+SUM_TOL = 2e-6
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def close(got, ref, scale):
+    assert got.shape == ref.shape
+    err = np.abs(got.astype(np.float64) - ref)
+    bound = SUM_TOL * scale + 1e-30
+    worst = float((err / bound).max()) if err.size else 0.0
+    assert worst <= 1.0, "error is %.2f x the bound" % worst
+
+
+# (N, C, H, W, T, O, (KH, KW), stride, padding, dilation, groups)
+CASES = [
+    (2, 2, 9, 10, 12, 16, (5, 5), 1, 2, 1, 1),        # first CNN layer, small
+    (1, 16, 7, 7, 8, 32, (3, 3), 1, 1, 1, 1),         # 144 taps
+    (1, 32, 5, 5, 4, 20, (3, 3), 1, 1, 1, 1),         # 288 taps: two LDS chunks; 20 = 16 + 4 channels
+    (2, 1, 12, 8, 16, 1, (2, 2), 2, 0, 1, 1),         # pooling geometry
+    (1, 1, 13, 9, 8, 1, (3, 2), (3, 2), 0, 1, 1),     # ragged pooling: windows that do not fit
+    (2, 3, 8, 9, 7, 5, (3, 3), 1, 0, 1, 1),           # T % 4 != 0
+    (1, 4, 10, 11, 6, 8, (3, 2), (2, 1), (1, 0), (1, 2), 2),   # stride, padding, dilation, groups
+    (1, 6, 9, 9, 4, 6, (3, 3), 2, 2, 2, 3),           # all of them, 3 groups of 2
+    (3, 5, 6, 6, 20, 3, (1, 1), 1, 0, 1, 1),          # 1x1
+    (1, 2, 4, 4, 8, 2, (5, 5), 1, 0, 1, 1),           # filter larger than the input: empty output
+    (1, 8, 6, 6, 4, 12, (2, 2), 1, 1, 1, 4),          # 3 output channels per group
+    (2, 2, 34, 34, 300, 16, (5, 5), 1, 2, 1, 1),      # the benchmark's first layer on two samples
+]
+IDS = ["%dx%dx%dx%dx%d-o%d-k%s-s%s-p%s-d%s-g%d" % c for c in CASES]
+
+
+def make(case, seed):
+    N, C, H, W, T, Oc, K, s, p, d, g = case
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((N, C, H, W, T)).astype(np.float32)
+    w = rng.standard_normal((Oc, C // g, K[0], K[1])).astype(np.float32)
+    return x, w, (s, p, d, g)
+
+
+@pytest.mark.parametrize("case", CASES, ids=IDS)
+def test_conv_matches_oracle(case):
+    x, w, a = make(case, 1)
+    ref = O.synapse_conv(x, w, *a).astype(np.float64)
+    got = host(synapse.conv(dev(x), dev(w), *a))
+    close(got, ref, O.synapse_conv(np.abs(x), np.abs(w), *a))
+
+
+@pytest.mark.parametrize("case", CASES, ids=IDS)
+def test_conv_grad_input_matches_oracle(case):
+    x, w, a = make(case, 2)
+    shape = O.synapse_geom(x.shape, w.shape, *a)[1]
+    go = np.random.default_rng(3).standard_normal(shape).astype(np.float32)
+    ref = O.synapse_conv_grad_input(go, w, x.shape, *a).astype(np.float64)
+    got = host(synapse.convGradInput(dev(go), dev(w), x.shape, *a))
+    close(got, ref, O.synapse_conv_grad_input(np.abs(go), np.abs(w), x.shape, *a))
+
+
+@pytest.mark.parametrize("case", CASES, ids=IDS)
+def test_conv_grad_weight_matches_oracle(case):
+    x, w, a = make(case, 4)
+    shape = O.synapse_geom(x.shape, w.shape, *a)[1]
+    go = np.random.default_rng(5).standard_normal(shape).astype(np.float32)
+    ref = O.synapse_conv_grad_weight(go, x, w.shape, *a).astype(np.float64)
+    got = host(synapse.convGradWeight(dev(go), dev(x), w.shape, *a))
+    close(got, ref, O.synapse_conv_grad_weight(np.abs(go), np.abs(x), w.shape, *a))
+
+
+def test_unaligned_storage():
+    """Tensors that start 4 bytes into an allocation take the one-sample-per-lane kernels."""
+    case = (1, 3, 6, 7, 8, 4, (3, 3), 1, 1, 1, 1)
+    x, w, a = make(case, 6)
+    shape = O.synapse_geom(x.shape, w.shape, *a)[1]
+    go = np.random.default_rng(7).standard_normal(shape).astype(np.float32)
+
+    def off(arr):
+        buf = torch.empty(arr.size + 1, dtype=torch.float32, device="cuda")
+        view = buf[1:].view(arr.shape)
+        view.copy_(torch.from_numpy(arr))
+        return view
+
+    close(host(synapse.conv(off(x), dev(w), *a)), O.synapse_conv(x, w, *a).astype(np.float64),
+          O.synapse_conv(np.abs(x), np.abs(w), *a))
+    close(host(synapse.convGradInput(off(go), dev(w), x.shape, *a)),
+          O.synapse_conv_grad_input(go, w, x.shape, *a).astype(np.float64),
+          O.synapse_conv_grad_input(np.abs(go), np.abs(w), x.shape, *a))
+    close(host(synapse.convGradWeight(off(go), off(x), w.shape, *a)),
+          O.synapse_conv_grad_weight(go, x, w.shape, *a).astype(np.float64),
+          O.synapse_conv_grad_weight(np.abs(go), np.abs(x), w.shape, *a))
+
+
+def test_adjoint_identity_full_size():
+    """<conv(x), g> == <x, gradInput(g)> == <w, gradWeight(g, x)> on the benchmark's first layer
+    (12, 2, 34, 34, 300) -> 16 channels: a size-independent check of all three kernels."""
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x = (torch.rand((12, 2, 34, 34, 300), device="cuda", generator=gen) < 0.02).float()
+    w = torch.randn((16, 2, 5, 5), device="cuda", generator=gen)
+    y = synapse.conv(x, w, 1, 2)
+    g = torch.randn(y.shape, device="cuda", generator=gen)
+    lhs = float((y.double() * g.double()).sum())
+    gi = synapse.convGradInput(g, w, x.shape, 1, 2)
+    gw = synapse.convGradWeight(g, x, w.shape, 1, 2)
+    scale = float((y.double().abs() * g.double().abs()).sum())
+    assert abs(lhs - float((gi.double() * x.double()).sum())) <= 1e-6 * scale
+    assert abs(lhs - float((gw.double() * w.double()).sum())) <= 1e-6 * scale
+
+
+def test_argument_errors():
+    lib = _lib.load()
+    g = _lib.SynapseGeom(1, 4, 8, 8, 4, 6, 3, 3, 1, 1, 0, 0, 1, 1, 3)      # 4 channels in 3 groups
+    assert lib.slayer_synapse_out_shape(g, None, None) == 1
+    g = _lib.SynapseGeom(1, 4, 8, 8, 4, 6, 3, 3, 0, 1, 0, 0, 1, 1, 1)      # zero stride
+    assert lib.slayer_synapse_conv_f32(None, None, None, g, None) == 1
+    g = _lib.SynapseGeom(1, 4, 8, 8, 4, 6, 3, 3, 1, 1, 0, 0, 1, 1, 1)
+    assert lib.slayer_synapse_conv_f32(None, None, None, g, None) == 1     # null pointers, non-empty output
+    g = _lib.SynapseGeom(1, 64, 4096, 4096, 4, 6, 3, 3, 1, 1, 0, 0, 1, 1, 1)   # 4 GiB per batch item
+    assert lib.slayer_synapse_out_shape(g, None, None) == 2
+    with pytest.raises(RuntimeError):
+        synapse.conv(torch.zeros((1, 4, 8, 8, 4), device="cuda"), torch.zeros((6, 3, 3, 3), device="cuda"))
+
+
+# ---------------------------------------------------------------------------------------- layers
+NEURON = {"type": "SRMALPHA", "theta": 10, "tauSr": 10.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1,
+          "scaleRho": 1}
+SIM = {"Ts": 1.0, "tSample": 300}
+
+
+def test_conv_layer_shift_and_add():
+    """The construction of the reference's convolution test (test/test_slayer007.py:36-48)."""
+    N, C, H, W, D, K = 2, 8, 20, 22, 24, 5
+    layer = snn.layer(NEURON, SIM).cuda()
+    conv = layer.conv(C, 1, K).cuda()
+    x = torch.randn((N, C, H, W, D), device="cuda")
+    weight = conv.weight.reshape(C, K, K)
+    ref = torch.zeros((N, 1, H - K + 1, W - K + 1, D), device="cuda", dtype=torch.float64)
+    for i in range(K):
+        for j in range(K):
+            for k in range(C):
+                ref += weight[k, j, i].double() * x[:, k:k + 1, j:H - K + 1 + j, i:W - K + 1 + i, :].double()
+    out = conv(x)
+    assert float(torch.norm(out.double() - ref)) / out.numel() < 1e-6      # the reference's criterion
+    assert float((out.double() - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
+
+
+def test_pool_layer_sum_of_four():
+    """The construction of the reference's pooling test (test/test_slayer007.py:60-82), odd extents
+    included."""
+    layer = snn.layer(NEURON, SIM).cuda()
+    pool = layer.pool(2).cuda()
+    x = torch.randn((2, 3, 10, 12, 16), device="cuda")
+    ref = (x[:, :, 0::2, 0::2] + x[:, :, 0::2, 1::2] + x[:, :, 1::2, 0::2] + x[:, :, 1::2, 1::2]) * 1.1 * NEURON["theta"]
+    out = pool(x)
+    assert out.shape == ref.shape
+    assert float((out - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
+    odd = pool(torch.randn((2, 3, 11, 13, 8), device="cuda"))
+    assert odd.shape == (2, 3, 6, 7, 8)
+
+
+def test_conv_transpose_and_unpool_layers():
+    """Transposed layers against their definition (test/test_slayer013.py): every input sample
+    spreads its value, weighted, over the window it maps to."""
+    layer = snn.layer(NEURON, SIM).cuda()
+    Cin, C, K, H, W, D = 3, 4, 3, 6, 7, 8
+    convT = layer.convTranspose(Cin, C, K).cuda()
+    x = torch.randn((2, Cin, H, W, D), device="cuda")
+    weight = convT.weight.reshape(Cin, C, K, K).double()
+    ref = torch.zeros((2, C, H + K - 1, W + K - 1, D), device="cuda", dtype=torch.float64)
+    for i in range(K):
+        for j in range(K):
+            for m in range(Cin):
+                for k in range(C):
+                    ref[:, k, i:i + H, j:j + W, :] += weight[m, k, i, j] * x[:, m].double()
+    out = convT(x)
+    assert out.shape == ref.shape
+    assert float((out.double() - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
+
+    unpool = layer.unpool(2).cuda()
+    x = torch.randn((2, 3, 5, 6, 8), device="cuda")
+    out = unpool(x)
+    ref = x.repeat_interleave(2, 2).repeat_interleave(2, 3) * 1.1 * NEURON["theta"]
+    assert out.shape == ref.shape
+    assert float((out - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("kind", ["conv", "pool", "convTranspose", "unpool"])
+def test_layer_gradients_match_torch_cpu(kind):
+    """Forward and both gradients of every synapse layer against the torch CPU op the reference's
+    layer calls (F.conv3d / F.conv_transpose3d with a time extent of 1)."""
+    import torch.nn.functional as F
+    torch.manual_seed(11)
+    layer = snn.layer(NEURON, SIM)
+    if kind == "conv":
+        mod = layer.conv(4, 6, 3, stride=1, padding=1, groups=2)
+        x = torch.randn((2, 4, 7, 8, 12))
+    elif kind == "pool":
+        mod = layer.pool(2)
+        x = torch.randn((2, 3, 8, 6, 12))
+    elif kind == "convTranspose":
+        mod = layer.convTranspose(4, 6, 3, stride=2, padding=1, groups=2)
+        x = torch.randn((2, 4, 5, 6, 12))
+    else:
+        mod = layer.unpool(2)
+        x = torch.randn((2, 3, 4, 5, 12))
+    w = mod.weight.detach().clone()
+
+    def torch_op(xc, wc):
+        if kind == "conv":
+            return F.conv3d(xc, wc, None, mod.stride, mod.padding, mod.dilation, mod.groups)
+        if kind == "pool":
+            s = xc.shape
+            r = F.conv3d(xc.reshape(s[0], 1, s[1] * s[2], s[3], s[4]), wc, None, mod.stride, mod.padding, mod.dilation)
+            return r.reshape(s[0], s[1], -1, r.shape[3], r.shape[4])
+        if kind == "convTranspose":
+            return F.conv_transpose3d(xc, wc, None, mod.stride, mod.padding, 0, mod.groups, mod.dilation)
+        s = xc.shape
+        r = F.conv_transpose3d(xc.reshape(s[0], 1, -1, s[3], s[4]), wc, None, mod.stride, mod.padding, 0, 1, mod.dilation)
+        return r.reshape(s[0], s[1], -1, r.shape[3], r.shape[4])
+
+    xc = x.clone().double().requires_grad_(True)
+    wc = w.clone().double().requires_grad_(True)
+    yc = torch_op(xc, wc)
+    g = torch.randn(yc.shape)
+    yc.backward(g.double())
+
+    mod = mod.cuda()
+    mod.weight.requires_grad_(True)
+    xg = x.cuda().requires_grad_(True)
+    yg = mod(xg)
+    yg.backward(g.cuda())
+    for got, ref in ((yg, yc), (xg.grad, xc.grad), (mod.weight.grad, wc.grad)):
+        assert got.shape == ref.shape
+        assert float((got.detach().cpu().double() - ref.detach()).abs().max()) <= 1e-5 * float(ref.abs().max())
