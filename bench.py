@@ -161,6 +161,77 @@ def mlp_row(device, timed):
             "us_with_separate_psp_and_spike_calls": two * 1e6, "samples_per_s": 12 / one}
 
 
+def cnn_row(device, timed):
+    """One training step (without the optimiser) of the NMNIST CNN of the reference's example
+    (example/03_NMNIST_CNN/nmnistCNN.py:47-62: conv 2->16 5x5, pool 2, conv 16->32 3x3, pool 2,
+    conv 32->64 3x3, dense 4096->10, every layer as spike(synapse(psp(x)))) on (12, 2, 34, 34, 300)
+    input spikes at p = 0.02 with a spike-time loss against a random target train."""
+    import slayerpytorch_amd as snn
+    params = neuron_params()
+    sim = {"Ts": 1.0, "tSample": 300}
+    net = {"neuron": params, "simulation": sim, "training": {"error": {"type": "SpikeTime"}}}
+    layer = snn.layer(params, sim).to(device)
+    error = snn.loss(net).to(device)
+    torch.manual_seed(0)
+    conv1, conv2, conv3 = layer.conv(2, 16, 5, padding=1), layer.conv(16, 32, 3, padding=1), layer.conv(32, 64, 3, padding=1)
+    pool1, pool2, fc1 = layer.pool(2), layer.pool(2), layer.dense((8, 8, 64), 10)
+    mods = [m.to(device) for m in (conv1, conv2, conv3, pool1, pool2, fc1)]
+    g = torch.Generator(device="cpu").manual_seed(5)
+    x = (torch.rand((12, 2, 34, 34, 300), generator=g) < 0.02).float().to(device)
+    target = (torch.rand((12, 10, 1, 1, 300), generator=g) < 0.01).float().to(device)
+    rates = []
+
+    def step():
+        s = x
+        del rates[:]
+        for syn in (conv1, pool1, conv2, pool2, conv3, fc1):
+            s = layer.spike(syn(layer.psp(s)))
+            rates.append(s)
+        error.spikeTime(s, target).backward()
+        for m in mods:
+            m.weight.grad = None
+
+    t = timed(step)
+    return {"op": "nmnist_cnn_fwd_loss_bwd", "shape": [12, 2, 34, 34, 300], "us": t * 1e6, "samples_per_s": 12 / t,
+            "spike_rate_per_layer": [round(float(r.detach().mean()), 4) for r in rates]}
+
+
+SYNAPSE_LAYERS = (
+    # name, input shape (N, C, H, W, T), weight shape, stride, padding, input spike density
+    ("conv 2->16 5x5", (12, 2, 34, 34, 300), (16, 2, 5, 5), 1, 1, 0.02),
+    ("pool 2x2 on 16x32x32", (12, 1, 16 * 32, 32, 300), (1, 1, 2, 2), 2, 0, 0.05),
+    ("conv 16->32 3x3", (12, 16, 16, 16, 300), (32, 16, 3, 3), 1, 1, 0.05),
+    ("pool 2x2 on 32x16x16", (12, 1, 32 * 16, 16, 300), (1, 1, 2, 2), 2, 0, 0.05),
+    ("conv 32->64 3x3", (12, 32, 8, 8, 300), (64, 32, 3, 3), 1, 1, 0.05),
+)
+
+
+def synapse_rows(device, timed):
+    """The per-timestep synapse kernels on the layer shapes of the NMNIST CNN: forward, input
+    gradient and weight gradient, with the fp32 rate (2 flop per multiply-add) and the fraction of
+    HBM peak that the tensors each kernel must move at least once amount to."""
+    from slayerpytorch_amd import synapse
+    g = torch.Generator(device="cpu").manual_seed(9)
+    rows = []
+    for name, xs, ws, stride, pad, density in SYNAPSE_LAYERS:
+        x = (torch.rand(xs, generator=g) < density).float().to(device)
+        w = torch.randn(ws, generator=g).to(device)
+        y = synapse.conv(x, w, stride, pad)
+        gy = torch.randn(y.shape, generator=g).to(device)
+        flop = 2.0 * y.numel() * ws[1] * ws[2] * ws[3]
+        nbytes = 4.0 * (x.numel() + y.numel())
+        for op, fn in (("forward", lambda: synapse.conv(x, w, stride, pad)),
+                       ("grad_input", lambda: synapse.convGradInput(gy, w, x.shape, stride, pad)),
+                       ("grad_weight", lambda: synapse.convGradWeight(gy, x, w.shape, stride, pad))):
+            if op == "grad_weight" and name.startswith("pool"):
+                continue            # pooling weights are constants
+            t = timed(fn)
+            rows.append({"op": "synapse " + op + " " + name, "shape": list(xs), "us": t * 1e6,
+                         "tflops_fp32": flop / t / 1e12, "hbm_frac": nbytes / t / 1e9 / HBM_PEAK_GBS})
+        del x, w, y, gy
+    return rows
+
+
 def other_rows(device):
     """Quick per-op measurements of the scope rows that are not part of the headline chain, each on
     the largest tensor its benchmark configuration gives it (median of 7 event-timed launches).  hbm_frac
@@ -222,6 +293,9 @@ def other_rows(device):
     del a, gs
     # NMNIST-shaped MLP end to end (dense layers are library GEMMs): forward, spike-time loss, backward
     out.append(mlp_row(device, timed))
+    # NMNIST-shaped CNN end to end (synapses by the per-timestep synapse kernels)
+    out.append(cnn_row(device, timed))
+    out.extend(synapse_rows(device, timed))
     # Loihi config: largest tensor (8, 16, 32, 32, 300)
     shape = (8, 16, 32, 32, 300)
     w = (2 * torch.randint(-128, 128, shape, generator=g) * (torch.rand(shape, generator=g) < 0.05)).float().to(device)

@@ -285,15 +285,25 @@ __global__ __launch_bounds__(256) void synapse_wgrad_kernel(WgradArgs g)
     }
 }
 
-// gradW[q] = sum of the workspace rows in row order.
+// gradW[q] = sum of the workspace rows: lane (q, part) adds rows part, part+16, ... in order, then
+// the 16 parts of a weight are added in order (a fixed association for a given geometry).
 __global__ __launch_bounds__(256) void synapse_wgrad_sum_kernel(float *__restrict__ gradW,
                                                                 const float *__restrict__ partial, int rows, int nW)
 {
-    const int q = blockIdx.x * 256 + threadIdx.x;
-    if (q >= nW) return;
+    __shared__ float part[16][17];
+    const int ql = threadIdx.x & 15, pt = threadIdx.x >> 4;
+    const int q = blockIdx.x * 16 + ql;
     float acc = 0.f;
-    for (int r = 0; r < rows; ++r) acc += partial[static_cast<int64_t>(r) * nW + q];
-    gradW[q] = acc;
+    if (q < nW)
+        for (int r = pt; r < rows; r += 16) acc += partial[static_cast<int64_t>(r) * nW + q];
+    part[pt][ql] = acc;
+    __syncthreads();
+    if (threadIdx.x < 16 && q < nW) {
+        float v = part[0][ql];
+#pragma unroll
+        for (int k = 1; k < 16; ++k) v += part[k][ql];
+        gradW[q] = v;
+    }
 }
 
 // ---- host side -------------------------------------------------------------------------------------
@@ -542,7 +552,7 @@ extern "C" int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gr
         if (st1 != SLAYER_OK) return st1;
         rows = s.N * p.slicesPerItem;
     }
-    hipLaunchKernelGGL(synapse_wgrad_sum_kernel, dim3(static_cast<unsigned>(ceil_div(nW, 256))), dim3(256), 0, st,
+    hipLaunchKernelGGL(synapse_wgrad_sum_kernel, dim3(static_cast<unsigned>(ceil_div(nW, 16))), dim3(256), 0, st,
                        gradW, workspace, rows, nW);
     return launch_status();
 }
