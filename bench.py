@@ -232,6 +232,43 @@ def synapse_rows(device, timed):
     return rows
 
 
+def event_row(device, timed):
+    """A batch of 12 NMNIST-sized samples (5000 events each, the 5-byte layout of the .bs2 files)
+    to a (12, 2, 34, 34, 300) spike tensor: file bytes uploaded and decoded + binned by one kernel
+    into a zeroed tensor, against the host sequence the reference's data loaders run (decode and bin
+    with the CPU oracle, then upload the dense tensor)."""
+    import slayerpytorch_amd as snn
+    from oracle import oracle
+    rng = np.random.default_rng(4)
+    n, shape = 5000, (12, 2, 34, 34, 300)
+    raws = []
+    for _ in range(shape[0]):
+        x, y, p = rng.integers(0, 34, n), rng.integers(0, 34, n), rng.integers(0, 2, n)
+        t = np.sort(rng.integers(0, 300000, n))
+        b = np.zeros((n, 5), dtype=np.uint8)
+        b[:, 0], b[:, 1], b[:, 2] = x, y, ((t >> 16) & 0x7F) | (p << 7)
+        b[:, 3], b[:, 4] = (t >> 8) & 0xFF, t & 0xFF
+        raws.append(b.reshape(-1))
+    events = [snn.io.event._fromBytes(r, 2) for r in raws]
+
+    def on_device():
+        return snn.io.toSpikeTensorBatch(events, torch.zeros(shape, device=device), 1.0)
+
+    def on_host():
+        out = np.zeros(shape, dtype=np.float32)
+        for i, r in enumerate(raws):
+            x, y, p, t = oracle.decode_events(r, 2)
+            out[i] = oracle.bin_events(out[i], x, y, p - p.min(), t / 1000, 1.0)
+        return torch.from_numpy(out).to(device)
+
+    dev_t = timed(on_device)
+    host_t = timed(on_host)
+    same = bool(torch.equal(on_device(), on_host()))
+    return {"op": "event files -> spike tensor (decode + bin, 12 x 5000 events)", "shape": list(shape),
+            "us": dev_t * 1e6, "events_per_s": shape[0] * n / dev_t,
+            "us_host_decode_bin_and_dense_upload": host_t * 1e6, "identical_to_host_result": same}
+
+
 def other_rows(device):
     """Quick per-op measurements of the scope rows that are not part of the headline chain, each on
     the largest tensor its benchmark configuration gives it (median of 7 event-timed launches).  hbm_frac
@@ -296,6 +333,7 @@ def other_rows(device):
     # NMNIST-shaped CNN end to end (synapses by the per-timestep synapse kernels)
     out.append(cnn_row(device, timed))
     out.extend(synapse_rows(device, timed))
+    out.append(event_row(device, timed))
     # Loihi config: largest tensor (8, 16, 32, 32, 300)
     shape = (8, 16, 32, 32, 300)
     w = (2 * torch.randint(-128, 128, shape, generator=g) * (torch.rand(shape, generator=g) < 0.05)).float().to(device)

@@ -268,6 +268,40 @@ int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gradOut, cons
                                         float *workspace, const slayer_synapse_geom *geom,
                                         void *stream);
 
+/*
+ * ---- Spike event files to spike tensors -------------------------------------------------------
+ * Decodes packed spike events and bins them into spike tensors, one launch for a batch of samples.
+ * Replaces spikeFileIO.read1Dspikes / read2Dspikes / read3Dspikes (src/spikeFileIO.py:162-184,
+ * :233-259, :296-321) followed by event.toSpikeTensor (src/spikeFileIO.py:66-144), which the
+ * reference runs with numpy in data-loader workers before copying a dense tensor to the GPU.
+ *
+ * bytes: the samples' file contents back to back on the device (nBytes in all); format 1 = 5-byte
+ * events (16-bit neuron id, polarity bit, 23-bit time in us), 2 = 5-byte events (x, y, polarity bit,
+ * 23-bit time), 3 = 7-byte events (12-bit x, 12-bit y, 8-bit channel, 24-bit time).
+ * sampleTable: device array [nSamples][3] = {first byte of the sample, number of events, time shift
+ * in bins}; an entry that does not lie inside the buffer is skipped.  maxEvents: the largest event
+ * count in the table (sizes the launch).  tensor: [nSamples][C][H][W][T].
+ * Per event: polarity minus the smallest polarity of its sample, bin = rint((time in ms) /
+ * samplingTime) - shift in double precision; events outside the tensor are dropped; mode 0 ("OR")
+ * stores 1/samplingTime, mode 1 ("SUM") stores base[...] + 1/samplingTime, where `base` is a copy of
+ * the tensor from before the call (required and distinct from `tensor` in mode 1, ignored in
+ * mode 0) - once per bin however many events share it, like numpy's indexed +=.
+ */
+int slayer_bin_packed_events_f32(float *tensor, const float *base, const uint8_t *bytes, int64_t nBytes,
+                                 const int64_t *sampleTable, int64_t nSamples, int64_t maxEvents,
+                                 int32_t format, int32_t C, int32_t H, int32_t W, int32_t T,
+                                 double samplingTime, int32_t mode, void *stream);
+
+/*
+ * The binning alone, for one sample whose events are already decoded: x, y (NULL = all 0), p as
+ * int32 and the time in milliseconds as double, tensor [C][H][W][T].  Replaces
+ * event.toSpikeTensor (src/spikeFileIO.py:66-144) for events that did not come from a file.
+ */
+int slayer_bin_events_f32(float *tensor, const float *base, const int32_t *x, const int32_t *y,
+                          const int32_t *p, const double *tMs, int64_t nEvents, int64_t timeShift,
+                          int32_t C, int32_t H, int32_t W, int32_t T, double samplingTime,
+                          int32_t mode, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

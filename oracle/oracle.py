@@ -16,6 +16,8 @@ oracle function        reference entry point it restates
 ``loihi_get_spikes``   ``slayerLoihiCuda.getSpikes`` (src/cuda/slayerLoihiKernels.cu:12-46)
 ``spike_bwd``          ``_spikeFunction.backward`` (src/slayer.py:857-865)
 ``delay_grad``         ``_delayFunction.backward`` (src/slayer.py:949-955)
+``decode_events``      ``spikeFileIO.read1Dspikes/read2Dspikes/read3Dspikes`` (src/spikeFileIO.py:162-321)
+``bin_events``         ``spikeFileIO.event.toSpikeTensor`` (src/spikeFileIO.py:66-144)
 ``synapse_conv*``      ``F.conv3d`` with a (KH, KW, 1) kernel in the synapse layers
                        (src/slayer.py:499-507, :565-575) and its two gradients
 =====================  ==========================================================
@@ -75,6 +77,13 @@ def lib():
         for name in ("oracle_synapse_out_shape", "oracle_synapse_conv_f32",
                      "oracle_synapse_conv_grad_input_f32", "oracle_synapse_conv_grad_weight_f32"):
             getattr(L, name).restype = None
+        i32p, u8p = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_uint8)
+        f64p = ctypes.POINTER(ctypes.c_double)
+        L.oracle_decode_events.argtypes = [i32p, i32p, i32p, i32p, u8p, _i64, ctypes.c_int32]
+        L.oracle_decode_events.restype = None
+        L.oracle_bin_events_f32.argtypes = [_f32p, _f32p, i32p, i32p, i32p, f64p, _i64, _i64] + \
+            [ctypes.c_int32] * 4 + [ctypes.c_double, ctypes.c_int32]
+        L.oracle_bin_events_f32.restype = None
         for name in ("oracle_get_spikes_f32", "oracle_conv_f32", "oracle_corr_f32",
                      "oracle_shift_f32", "oracle_spike_bwd_f32", "oracle_delay_grad_f32",
                      "oracle_loihi_get_spikes_f32", "oracle_set_threads"):
@@ -245,3 +254,36 @@ def synapse_conv_grad_weight(grad_out, x, w_shape, stride=1, padding=0, dilation
     if gw.size:
         lib().oracle_synapse_conv_grad_weight_f32(_p(gw), _p(go), _p(x), ctypes.byref(g))
     return gw
+
+
+def decode_events(data, fmt):
+    """``(x, y, p, tUs)`` int32 arrays of the packed events in ``data`` (bytes / uint8 array);
+    ``fmt`` 1, 2 or 3 for the 1-D, 2-D and 3-D file layouts.  The polarity is the stored one
+    (not yet shifted to start at 0)."""
+    b = np.ascontiguousarray(np.frombuffer(bytes(data), dtype=np.uint8))
+    n = b.size // (7 if fmt == 3 else 5)
+    out = [np.zeros(n, dtype=np.int32) for _ in range(4)]
+    i32p, u8p = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_uint8)
+    if n:
+        lib().oracle_decode_events(*[a.ctypes.data_as(i32p) for a in out], b.ctypes.data_as(u8p), n, int(fmt))
+    return tuple(out)
+
+
+def bin_events(tensor, x, y, p, t_ms, sampling_time=1.0, time_shift=0, mode="OR"):
+    """Returns a copy of the (C, H, W, T) float32 ``tensor`` with the events binned into it."""
+    base = _f32(tensor)
+    out = base.copy()
+    C, H, W, T = out.shape
+    x = np.ascontiguousarray(x, dtype=np.int32)
+    p = np.ascontiguousarray(p, dtype=np.int32)
+    t = np.ascontiguousarray(t_ms, dtype=np.float64)
+    i32p, f64p = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_double)
+    yp = None
+    if y is not None:
+        y = np.ascontiguousarray(y, dtype=np.int32)
+        yp = y.ctypes.data_as(i32p)
+    if x.size:
+        lib().oracle_bin_events_f32(_p(out), _p(base), x.ctypes.data_as(i32p), yp, p.ctypes.data_as(i32p),
+                                    t.ctypes.data_as(f64p), x.size, int(time_shift), C, H, W, T,
+                                    float(sampling_time), {"OR": 0, "SUM": 1}[mode.upper()])
+    return out

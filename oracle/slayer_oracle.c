@@ -415,3 +415,59 @@ void oracle_synapse_conv_grad_weight_f32(float *gradW, const float *gradOut, con
         gradW[q] = (float)acc;
     }
 }
+
+/* ------------------------------------------------------------------------------------------
+ * Spike event files and event binning.  Follows src/spikeFileIO.py:
+ *   read1Dspikes :162-184 (5 bytes: neuron id 16 bit, polarity 1 bit, time 23 bit in us),
+ *   read2Dspikes :233-259 (5 bytes: x 8 bit, y 8 bit, polarity 1 bit, time 23 bit in us),
+ *   read3Dspikes :296-321 (7 bytes: x 12 bit, y 12 bit, channel 8 bit, time 24 bit in us),
+ *   event.__init__ :33 (the polarity is shifted so that its minimum over the events is 0),
+ *   event.toSpikeTensor :66-144 (bin = round-half-even((t in ms) / samplingTime) - shift; events
+ *   outside the tensor are dropped; 'OR' stores 1/samplingTime, 'SUM' stores the value the tensor
+ *   held before the call plus 1/samplingTime - once, however many events share the bin, which is
+ *   what numpy's indexed += does).
+ * Pins: the reference's own sample triple test/test_files/NMNISTsmall/1.bs2 <->
+ * input_validate/1_raw_spikes.csv <-> 1_binned_spikes.csv / 1_binned_spikes_ts2.csv (the csv
+ * tensors were binned by truncation, so they pin decode, layout, validity and value on times
+ * moved to the start of their bin), numpy.round / numpy.rint for the rounding itself.
+ * ------------------------------------------------------------------------------------------ */
+void oracle_decode_events(int32_t *x, int32_t *y, int32_t *p, int32_t *tUs, const uint8_t *bytes,
+                          int64_t nEvents, int32_t format)
+{
+    for (int64_t e = 0; e < nEvents; ++e) {
+        const uint8_t *b = bytes + e * (format == 3 ? 7 : 5);
+        if (format == 1) {
+            x[e] = (b[0] << 8) | b[1];
+            y[e] = 0;
+            p[e] = b[2] >> 7;
+            tUs[e] = ((b[2] << 16) | (b[3] << 8) | b[4]) & 0x7FFFFF;
+        } else if (format == 2) {
+            x[e] = b[0];
+            y[e] = b[1];
+            p[e] = b[2] >> 7;
+            tUs[e] = ((b[2] << 16) | (b[3] << 8) | b[4]) & 0x7FFFFF;
+        } else {
+            x[e] = (b[0] << 4) | (b[1] >> 4);
+            y[e] = b[2] | ((b[1] & 0x0F) << 8);
+            p[e] = b[3];
+            tUs[e] = (b[4] << 16) | (b[5] << 8) | b[6];
+        }
+    }
+}
+
+/* tensor is [C][H][W][T]; base holds the values from before the call (may be tensor itself for
+ * mode 0 = OR; for mode 1 = SUM it must be an untouched copy). */
+void oracle_bin_events_f32(float *tensor, const float *base, const int32_t *x, const int32_t *y,
+                           const int32_t *p, const double *tMs, int64_t nEvents, int64_t timeShift,
+                           int32_t C, int32_t H, int32_t W, int32_t T, double samplingTime, int32_t mode)
+{
+    const float value = (float)(1.0 / samplingTime);
+    for (int64_t e = 0; e < nEvents; ++e) {
+        const double bin = rint(tMs[e] / samplingTime) - (double)timeShift;
+        const int32_t ye = y ? y[e] : 0;
+        if (!(bin >= 0.0 && bin < (double)T)) continue;
+        if (x[e] < 0 || x[e] >= W || ye < 0 || ye >= H || p[e] < 0 || p[e] >= C) continue;
+        const int64_t idx = (((int64_t)p[e] * H + ye) * W + x[e]) * T + (int64_t)bin;
+        tensor[idx] = mode == 0 ? value : base[idx] + value;
+    }
+}

@@ -110,3 +110,21 @@ save(
     binned_ts2_shape=np.array(b2.shape, dtype=np.int32), binned_ts2_events=ev2, binned_ts2_values=val2,
     response_ts2=csv("torch_validate/1_spike_response_signal_ts2.csv")[ROWS].astype(np.float32),
 )
+
+# --- spike event files: the reference's own sample in three forms -------------------------------
+# NMNISTsmall/1.bs2 (packed events) <-> input_validate/1_raw_spikes.csv (x, y, p, t in us, 1-based
+# x/y/p) <-> the binned rasters already read above (b1: 1 ms bins, b2: 2 ms bins; both binned by
+# truncation).  Plus one 1-D file and the head of one 3-D file for the other two byte layouts.
+def raw_bytes(path, limit=None):
+    with open(os.path.join(TF, path), "rb") as f:
+        data = f.read() if limit is None else f.read(limit)
+    return np.frombuffer(data, dtype=np.uint8).copy()
+
+
+save(
+    "spike_events.npz",
+    nmnist_bs2=raw_bytes("NMNISTsmall/1.bs2"),
+    nmnist_raw=np.loadtxt(os.path.join(TF, "input_validate/1_raw_spikes.csv"), delimiter=",", skiprows=1).astype(np.int32),
+    ntidigits_bs1=raw_bytes("binarySpikeTestFiles/NTIDIGITS_1.bs1"),
+    sample_bs3=raw_bytes("binarySpikeTestFiles/1.bs3", 7 * 3000),
+)

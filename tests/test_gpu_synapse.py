@@ -160,8 +160,9 @@ def test_conv_layer_shift_and_add():
         for j in range(K):
             for k in range(C):
                 ref += weight[k, j, i].double() * x[:, k:k + 1, j:H - K + 1 + j, i:W - K + 1 + i, :].double()
-    out = conv(x)
-    assert float(torch.norm(out.detach().double() - ref)) / out.numel() < 1e-6      # the reference's criterion
+    out = conv(x).detach()
+    ref = ref.detach()
+    assert float(torch.norm(out.double() - ref)) / out.numel() < 1e-6      # the reference's criterion
     assert float((out.double() - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
 
 

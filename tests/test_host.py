@@ -6,6 +6,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 import torch
 
@@ -177,3 +178,40 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                        timeout=300)
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+
+
+def test_synapse_and_event_wrappers_need_the_gpu():
+    """No CPU path: the synapse ops and the event binning reject CPU tensors before any launch."""
+    import slayerpytorch_amd as snn
+    from slayerpytorch_amd import synapse
+    x, w = torch.zeros((1, 2, 5, 5, 4)), torch.zeros((3, 2, 3, 3))
+    with pytest.raises(RuntimeError):
+        synapse.conv(x, w)
+    with pytest.raises(RuntimeError):
+        synapse.convGradInput(torch.zeros((1, 3, 3, 3, 4)), w, x.shape)
+    with pytest.raises(RuntimeError):
+        synapse.convGradWeight(torch.zeros((1, 3, 3, 3, 4)), x, w.shape)
+    layer = snn.layer({"theta": 10, "tauSr": 1.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1},
+                      {"Ts": 1.0, "tSample": 10})
+    for mod in (layer.conv(2, 3, 3), layer.pool(2), layer.convTranspose(2, 3, 3), layer.unpool(2)):
+        with pytest.raises(RuntimeError):
+            mod(torch.zeros((1, 2, 6, 6, 4)))
+    assert layer.conv(2, 3, (3, 2), stride=(2, 1), padding=1).weight.shape == (3, 2, 3, 2, 1)
+    assert float(layer.pool(2).weight.flatten()[0]) == pytest.approx(11.0)
+    with pytest.raises(RuntimeError):
+        snn.io.event([1], [1], [0], [1.0]).toSpikeTensor(torch.zeros((1, 4, 4, 8)))
+
+
+def test_event_class_decodes_like_the_oracle():
+    """Host-side members of an event read from file bytes (x, y, p shifted to start at 0, t in ms)."""
+    import os
+    import slayerpytorch_amd as snn
+    from oracle import oracle as O
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "spike_events.npz"))
+    for key, fmt in (("nmnist_bs2", 2), ("ntidigits_bs1", 1), ("sample_bs3", 3)):
+        ev = snn.io.event._fromBytes(g[key], fmt)
+        x, y, p, t = O.decode_events(g[key], fmt)
+        assert np.array_equal(ev.x, x) and np.array_equal(ev.p, p - p.min()) and np.array_equal(ev.t, t / 1000)
+        assert ev.dim == (1 if fmt == 1 else 2)
+        if fmt != 1:
+            assert np.array_equal(ev.y, y)

@@ -2,6 +2,8 @@
 golden vectors held by the reference's own tests, library routines the ops reduce to,
 closed forms, invariants and brute force on small inputs.  Runs without a GPU.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -420,3 +422,138 @@ def test_joint_gradients_golden():
     assert np.linalg.norm(gW2 - snn["gradW2Initial"]) / gW2.size < 1e-4
     assert np.linalg.norm(gW1 - snn["gradW1Initial"]) / gW1.size < 1e-4
     assert np.linalg.norm(snn["gradW1Initial"]) / gW1.size > 1e-3   # the criterion is not vacuous
+
+
+# ------------------------------------------------------------------------ spike event files
+def _spike_events():
+    return np.load(os.path.join(os.path.dirname(__file__), "golden", "spike_events.npz"))
+
+
+def test_event_decoding_matches_reference_sample():
+    """NMNISTsmall/1.bs2 against the reference's listing of the same sample
+    (input_validate/1_raw_spikes.csv: x, y, p one-based, t in us)."""
+    g = _spike_events()
+    x, y, p, t = O.decode_events(g["nmnist_bs2"], 2)
+    raw = g["nmnist_raw"]
+    assert x.size == raw.shape[0] == 4681
+    assert np.array_equal(x, raw[:, 0] - 1) and np.array_equal(y, raw[:, 1] - 1)
+    assert np.array_equal(p, raw[:, 2] - 1) and np.array_equal(t, raw[:, 3])
+
+
+def test_event_decoding_bit_fields():
+    """All three layouts against the shifts and masks written out with numpy integer arithmetic."""
+    g = _spike_events()
+    b = g["ntidigits_bs1"].astype(np.int64).reshape(-1, 5)
+    x, y, p, t = O.decode_events(g["ntidigits_bs1"], 1)
+    assert np.array_equal(x, (b[:, 0] << 8) | b[:, 1]) and not y.any()
+    assert np.array_equal(p, b[:, 2] >> 7)
+    assert np.array_equal(t, ((b[:, 2] << 16) | (b[:, 3] << 8) | b[:, 4]) & 0x7FFFFF)
+    assert x.max() < 64 and np.all(np.diff(t) >= 0)            # 64 cochlea channels, sorted in time
+    b = g["sample_bs3"].astype(np.int64).reshape(-1, 7)
+    x, y, p, t = O.decode_events(g["sample_bs3"], 3)
+    assert np.array_equal(x, (b[:, 0] << 4) | (b[:, 1] >> 4))
+    assert np.array_equal(y, b[:, 2] | ((b[:, 1] & 0x0F) << 8))
+    assert np.array_equal(p, b[:, 3]) and np.array_equal(t, (b[:, 4] << 16) | (b[:, 5] << 8) | b[:, 6])
+    assert np.all(np.diff(t) >= 0)
+
+
+def test_event_binning_matches_reference_rasters():
+    """The reference's binned rasters of the NMNIST sample (1 ms and 2 ms bins; they were binned by
+    truncation, so the times are moved to the start of their bin first): pins layout, validity and
+    value of the binning."""
+    g = _spike_events()
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "nmnist_response.npz"))
+    x, y, p, t = O.decode_events(g["nmnist_bs2"], 2)
+    for Ts, key in ((1, "binned"), (2, "binned_ts2")):
+        shape = tuple(gold[key + "_shape"])
+        raster = np.zeros(shape, np.float32)
+        raster[gold[key + "_events"][:, 0], gold[key + "_events"][:, 1]] = gold[key + "_values"]
+        got = O.bin_events(np.zeros((2, 34, 34, shape[1]), np.float32), x, y, p - p.min(),
+                           np.floor(t / 1000 / Ts) * Ts, Ts)
+        assert np.array_equal(got.reshape(shape), raster)
+
+
+def test_event_binning_rounding_and_modes():
+    """Bin = numpy.round(t / Ts) (half to even) minus the shift; OR stores 1/Ts; SUM adds it once per
+    occupied bin, which is what numpy's indexed += does."""
+    rng = np.random.default_rng(2)
+    n, (C, H, W, T), Ts, shift = 4000, (2, 5, 6, 40), 1.5, 3
+    x, y, p = rng.integers(-1, W + 2, n), rng.integers(-1, H + 2, n), rng.integers(0, C + 1, n)
+    t = rng.random(n) * 80 - 3
+    t[::4] = (np.floor(t[::4] / Ts) + 0.5) * Ts                 # exactly half way
+    base = rng.standard_normal((C, H, W, T)).astype(np.float32)
+    tb = np.round(t / Ts).astype(int) - shift
+    ok = (x >= 0) & (x < W) & (y >= 0) & (y < H) & (p >= 0) & (p < C) & (tb >= 0) & (tb < T)
+    for mode in ("OR", "SUM"):
+        ref = base.copy()
+        if mode == "OR":
+            ref[p[ok], y[ok], x[ok], tb[ok]] = 1 / Ts
+        else:
+            ref[p[ok], y[ok], x[ok], tb[ok]] += 1 / Ts
+        got = O.bin_events(base, x, y, p, t, Ts, shift, mode)
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+
+
+# ------------------------------------------------------------------------ per-timestep synapses
+SYNAPSE_CASES = [
+    # N, C, H, W, T, O, (KH, KW), stride, padding, dilation, groups
+    (2, 4, 9, 8, 5, 6, (3, 3), 1, 1, 1, 1),
+    (1, 4, 10, 11, 3, 8, (3, 2), (2, 1), (1, 0), (1, 2), 2),
+    (2, 1, 8, 8, 4, 1, (2, 2), 2, 0, 1, 1),
+    (1, 6, 7, 7, 2, 6, (3, 3), 2, 2, 2, 3),
+    (1, 2, 4, 4, 3, 2, (5, 5), 1, 0, 1, 1),        # the filter does not fit: empty output
+]
+
+
+@pytest.mark.parametrize("case", SYNAPSE_CASES)
+def test_synapse_oracle_matches_torch_conv3d(case):
+    """The oracle's synapse and both gradients against F.conv3d with a (KH, KW, 1) kernel and its
+    autograd on the CPU - the very call the reference's layers make (src/slayer.py:499-507)."""
+    N, C, H, W, T, Oc, K, s, p, d, g = case
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((N, C, H, W, T)).astype(np.float32)
+    w = rng.standard_normal((Oc, C // g, K[0], K[1])).astype(np.float32)
+    tup = lambda v: (v, v) if isinstance(v, int) else tuple(v)
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    wt = torch.tensor(w[..., None], dtype=torch.float64, requires_grad=True)
+    if O.synapse_geom(x.shape, w.shape, s, p, d, g)[1][2] == 0:
+        assert O.synapse_conv(x, w, s, p, d, g).size == 0
+        return
+    y = F.conv3d(xt, wt, None, tup(s) + (1,), tup(p) + (0,), tup(d) + (1,), g)
+    yo = O.synapse_conv(x, w, s, p, d, g)
+    assert yo.shape == tuple(y.shape)
+    assert rel_err(yo, y.detach().numpy()) < 1e-6
+    go = rng.standard_normal(yo.shape).astype(np.float32)
+    y.backward(torch.tensor(go, dtype=torch.float64))
+    assert rel_err(O.synapse_conv_grad_input(go, w, x.shape, s, p, d, g), xt.grad.numpy()) < 1e-6
+    assert rel_err(O.synapse_conv_grad_weight(go, x, w.shape, s, p, d, g), wt.grad.numpy()[..., 0]) < 1e-6
+
+
+def test_synapse_oracle_shift_and_add():
+    """The constructions of the reference's own tests: convolution as a sum of shifted, weighted
+    copies (test/test_slayer007.py:36-48), pooling as the sum of the four window positions (:60-66),
+    transposed convolution as every input sample spread over its window (test/test_slayer013.py)."""
+    rng = np.random.default_rng(1)
+    N, C, H, W, D, K = 2, 3, 9, 10, 4, 5
+    x = rng.standard_normal((N, C, H, W, D)).astype(np.float32)
+    w = rng.standard_normal((1, C, K, K)).astype(np.float32)
+    ref = np.zeros((N, 1, H - K + 1, W - K + 1, D))
+    for i in range(K):
+        for j in range(K):
+            for k in range(C):
+                ref[:, 0] += w[0, k, j, i].astype(np.float64) * x[:, k, j:H - K + 1 + j, i:W - K + 1 + i, :]
+    assert rel_err(O.synapse_conv(x, w), ref) < 1e-6
+    x = rng.standard_normal((2, 1, 8, 6, 4)).astype(np.float32)
+    ones = np.full((1, 1, 2, 2), 11.0, np.float32)
+    ref = (x[:, :, 0::2, 0::2] + x[:, :, 0::2, 1::2] + x[:, :, 1::2, 0::2] + x[:, :, 1::2, 1::2]) * 11.0
+    assert rel_err(O.synapse_conv(x, ones, 2), ref) < 1e-6
+    Cin, Cout, K, H, W = 2, 3, 3, 4, 5
+    x = rng.standard_normal((1, Cin, H, W, 3)).astype(np.float32)
+    w = rng.standard_normal((Cin, Cout, K, K)).astype(np.float32)
+    ref = np.zeros((1, Cout, H + K - 1, W + K - 1, 3))
+    for i in range(K):
+        for j in range(K):
+            for m in range(Cin):
+                for k in range(Cout):
+                    ref[:, k, i:i + H, j:j + W, :] += w[m, k, i, j].astype(np.float64) * x[:, m]
+    assert rel_err(O.synapse_conv_grad_input(x, w, ref.shape), ref) < 1e-6
