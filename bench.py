@@ -232,13 +232,12 @@ def synapse_rows(device, timed):
     return rows
 
 
-def event_row(device, timed):
+def event_row(device, timed, cpu_leg):
     """A batch of 12 NMNIST-sized samples (5000 events each, the 5-byte layout of the .bs2 files)
     to a (12, 2, 34, 34, 300) spike tensor: file bytes uploaded and decoded + binned by one kernel
-    into a zeroed tensor, against the host sequence the reference's data loaders run (decode and bin
-    with the CPU oracle, then upload the dense tensor)."""
+    into a zeroed tensor.  With the CPU leg: against the host sequence the reference's data loaders run
+    (decode and bin with the CPU oracle, then upload the dense tensor), as part of the CPU baseline."""
     import slayerpytorch_amd as snn
-    from oracle import oracle
     rng = np.random.default_rng(4)
     n, shape = 5000, (12, 2, 34, 34, 300)
     raws = []
@@ -255,6 +254,7 @@ def event_row(device, timed):
         return snn.io.toSpikeTensorBatch(events, torch.zeros(shape, device=device), 1.0)
 
     def on_host():
+        from oracle import oracle
         out = np.zeros(shape, dtype=np.float32)
         for i, r in enumerate(raws):
             x, y, p, t = oracle.decode_events(r, 2)
@@ -262,14 +262,15 @@ def event_row(device, timed):
         return torch.from_numpy(out).to(device)
 
     dev_t = timed(on_device)
-    host_t = timed(on_host)
-    same = bool(torch.equal(on_device(), on_host()))
-    return {"op": "event files -> spike tensor (decode + bin, 12 x 5000 events)", "shape": list(shape),
-            "us": dev_t * 1e6, "events_per_s": shape[0] * n / dev_t,
-            "us_host_decode_bin_and_dense_upload": host_t * 1e6, "identical_to_host_result": same}
+    row = {"op": "event files -> spike tensor (decode + bin, 12 x 5000 events)", "shape": list(shape),
+           "us": dev_t * 1e6, "events_per_s": shape[0] * n / dev_t}
+    if cpu_leg:
+        row["us_host_decode_bin_and_dense_upload"] = timed(on_host) * 1e6
+        row["identical_to_host_result"] = bool(torch.equal(on_device(), on_host()))
+    return row
 
 
-def other_rows(device):
+def other_rows(device, cpu_leg=False):
     """Quick per-op measurements of the scope rows that are not part of the headline chain, each on
     the largest tensor its benchmark configuration gives it (median of 7 event-timed launches).  hbm_frac
     counts the algorithmic bytes of the unfused reference sequence (Loihi forward + delayShift:
@@ -333,7 +334,7 @@ def other_rows(device):
     # NMNIST-shaped CNN end to end (synapses by the per-timestep synapse kernels)
     out.append(cnn_row(device, timed))
     out.extend(synapse_rows(device, timed))
-    out.append(event_row(device, timed))
+    out.append(event_row(device, timed, cpu_leg))
     # Loihi config: largest tensor (8, 16, 32, 32, 300)
     shape = (8, 16, 32, 32, 300)
     w = (2 * torch.randint(-128, 128, shape, generator=g) * (torch.rand(shape, generator=g) < 0.05)).float().to(device)
@@ -364,6 +365,8 @@ def main():
     ap.add_argument("--chain-only", action="store_true",
                     help="only the headline chain (for profiler runs): no per-kernel pass, flip rate, "
                          "other rows or CPU baseline")
+    ap.add_argument("--cnn-only", action="store_true",
+                    help="only the NMNIST CNN training step of the other rows (for profiler runs); prints that row")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain copy of known size (a zero-delay shift of half the tensor: "
                          "%d bytes read, as many written) to scale hardware counters by" % (4 * 6 * 16 * 34 * 34 * 300))
@@ -379,6 +382,18 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.cnn_only:
+        def wall(fn):
+            ts = []
+            for _ in range(args.warmup + args.steps):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                fn()
+                torch.cuda.synchronize()
+                ts.append(time.perf_counter() - t0)
+            return float(np.median(ts[args.warmup:]))
+        print(json.dumps(cnn_row(device, wall)))
+        return
     params = neuron_params()
     srm = np.array(alphaKernel(params["tauSr"], 1.0, SHAPE[-1]), dtype=np.float32)
     ref = np.array(alphaKernel(params["tauRef"], 1.0, SHAPE[-1], mult=-params["scaleRef"] * params["theta"]),
@@ -473,7 +488,7 @@ def main():
     del pool
     if not args.chain_only:
         result["measured_copy_ceiling"] = copy_ceiling(grad)
-        result["other_rows"] = other_rows(device)
+        result["other_rows"] = other_rows(device, cpu_leg=not args.no_cpu_baseline)
         if not args.no_cpu_baseline:
             # the CPU leg: the oracle as the timed baseline and as the checker of the flip rate
             result["cpu_baseline"] = cpu_baseline(SHAPE, srm, ref, params)
