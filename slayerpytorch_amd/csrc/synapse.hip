@@ -285,6 +285,170 @@ __global__ __launch_bounds__(256) void synapse_wgrad_kernel(WgradArgs g)
     }
 }
 
+
+// ---- weight gradient on the matrix cores ------------------------------------------------------
+// For one output pixel (n, a, b) the weight gradient is a matrix product with time as the
+// reduction axis:  gradW[o][col] += sum_t G[o][t] * X[col][t],  G[o][t] = gradOut[n][o][a][b][t],
+// X[col][t] = in[n][c][a*sH-pH+i*dH][b*sW-pW+j*dW][t] for col = (c, i, j).  Both operands are rows
+// that are contiguous in t, which is exactly the register layout of v_mfma_f32_16x16x4_f32: lane
+// (r, h) = (lane % 16, lane / 16) supplies row r at reduction index h of both operands.  A lane
+// loads 16 bytes - four time samples t = 16*step + 4*h + e - and feeds them to four matrix
+// instructions (e = 0..3); the order in which time samples enter the sum does not matter as long
+// as both operands use the same one.  A 16-lane group reads 64 contiguous bytes of each of 16 rows,
+// so every byte a load instruction fetches is used and the operands need no staging in LDS.
+// A wavefront owns MT x NT tiles of 16 output channels x 16 columns; the four wavefronts of a
+// work-group take neighbouring pixels of a slice of one batch item at the same time (their input
+// rows overlap, so they share them through the L1 cache), add their tiles up in LDS in wavefront
+// order and write one workspace row per slice.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+struct WgradMfmaArgs {
+    const float *gradOut, *in;
+    float *partial;
+    SynGeom s;
+    int Cg, Og, CK;          // input channels, output channels and columns (Cg * KH * KW) per group
+    int oGroups, colGroups;  // blocks of 16*MT output channels / 16*NT columns per group
+    int slices, pixPerSlice, nW;
+    FastDiv bySlices, byColGroups, byOGroups, byGroups, byKK, byKW, byOW;
+};
+
+template <int MT, int NT>
+__global__ __launch_bounds__(256) void synapse_wgrad_mfma_kernel(WgradMfmaArgs g)
+{
+    __shared__ float red[MT * NT * 256];
+    const SynGeom &s = g.s;
+    uint32_t rest = blockIdx.x;
+    uint32_t q = fastdiv(rest, g.bySlices);
+    const int slice = static_cast<int>(rest - q * g.bySlices.d);
+    rest = q; q = fastdiv(rest, g.byColGroups);
+    const int cg = static_cast<int>(rest - q * g.byColGroups.d);
+    rest = q; q = fastdiv(rest, g.byOGroups);
+    const int og = static_cast<int>(rest - q * g.byOGroups.d);
+    rest = q; q = fastdiv(rest, g.byGroups);
+    const int grp = static_cast<int>(rest - q * g.byGroups.d);
+    const int n = static_cast<int>(q);
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, h = lane >> 4;
+    const int64_t goPlane = static_cast<int64_t>(s.OH) * s.OW * s.T, inPlane = static_cast<int64_t>(s.H) * s.W * s.T;
+    const BufferRsrc goB = make_buffer(g.gradOut + (static_cast<int64_t>(n) * s.O + grp * g.Og) * goPlane);
+    const BufferRsrc inB = make_buffer(g.in + (static_cast<int64_t>(n) * s.C + grp * g.Cg) * inPlane);
+    const int rowBytes = s.W * s.T * 4, pixBytes = s.T * 4;
+
+    // rows of this lane: output channel of every A tile, (channel, tap) of every B tile
+    int offA[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int o = ((og * MT + mt) << 4) + r;
+        offA[mt] = masked_offset(o < g.Og, o * static_cast<int>(goPlane) * 4);
+    }
+    int baseB[NT], dyB[NT], dxB[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int col = ((cg * NT + nt) << 4) + r;
+        const uint32_t cl = fastdiv(static_cast<uint32_t>(col), g.byKK);
+        const int ij = col - static_cast<int>(cl * g.byKK.d);
+        const int i = static_cast<int>(fastdiv(static_cast<uint32_t>(ij), g.byKW));
+        const int j = ij - i * s.KW;
+        baseB[nt] = col < g.CK ? static_cast<int>(cl) * static_cast<int>(inPlane) * 4 : 0;
+        dyB[nt] = col < g.CK ? i * s.dH - s.pH : -(1 << 28);  // a column past the filter never lands inside
+        dxB[nt] = j * s.dW - s.pW;
+    }
+
+    floatx4 acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const int steps = (s.T + 15) >> 4;
+    const int pixEnd = min(s.OH * s.OW, (slice + 1) * g.pixPerSlice);
+    int offB[NT];
+    auto place = [&](int pixel) {  // byte offsets of this lane's B rows for an output pixel
+        const int a = static_cast<int>(fastdiv(static_cast<uint32_t>(pixel), g.byOW));
+        const int b = pixel - a * s.OW;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int y = a * s.sH + dyB[nt], x = b * s.sW + dxB[nt];
+            const bool ok = static_cast<unsigned>(y) < static_cast<unsigned>(s.H) &&
+                            static_cast<unsigned>(x) < static_cast<unsigned>(s.W);
+            offB[nt] = masked_offset(ok, baseB[nt] + y * rowBytes + x * pixBytes);
+        }
+    };
+    // an offset that is already out of range stays out of range when a small number is added
+    auto issue = [&](float4 (&A)[MT], float4 (&B)[NT], int pixel, int st, bool more) {
+        const int t = (st << 4) + (h << 2);
+        const bool live = more && t < s.T;
+        const int pixA = pixel * pixBytes;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            A[mt] = buffer_load4<0>(goB, live && offA[mt] != kOutOfRange ? offA[mt] + pixA + t * 4 : kOutOfRange, 0);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            B[nt] = buffer_load4<0>(inB, live && offB[nt] != kOutOfRange ? offB[nt] + t * 4 : kOutOfRange, 0);
+    };
+
+    // (pixel, step) pairs in order; the operands of the next pair are loaded while the matrix
+    // instructions of the current one run
+    int pixel = slice * g.pixPerSlice + wave, st = 0;
+    if (pixel < pixEnd) {
+        float4 A[MT], B[NT];
+        place(pixel);
+        issue(A, B, pixel, st, true);
+        for (;;) {
+            int nst = st + 1, npix = pixel;
+            if (nst == steps) {
+                nst = 0;
+                npix += 4;
+                if (npix < pixEnd) place(npix);
+            }
+            const bool more = npix < pixEnd;
+            float4 An[MT], Bn[NT];
+            issue(An, Bn, npix, nst, more);
+            // consecutive matrix instructions go to different accumulators
+#define SLAYER_WGRAD_MFMA(E)                                                                              \
+    _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)     \
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[mt].E, B[nt].E, acc[mt][nt], 0, 0, 0);
+            SLAYER_WGRAD_MFMA(x)
+            SLAYER_WGRAD_MFMA(y)
+            SLAYER_WGRAD_MFMA(z)
+            SLAYER_WGRAD_MFMA(w)
+#undef SLAYER_WGRAD_MFMA
+            if (!more) break;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) A[mt] = An[mt];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) B[nt] = Bn[nt];
+            pixel = npix;
+            st = nst;
+        }
+    }
+
+    // the four wavefronts add their tiles in LDS, in wavefront order
+    for (int w = 0; w < 4; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        float *cell = red + ((mt * NT + nt) * 4 + v) * 64 + lane;
+                        *cell = w == 0 ? acc[mt][nt][v] : *cell + acc[mt][nt][v];
+                    }
+        }
+        __syncthreads();
+    }
+    // element v of a tile's accumulator is row 4*h + v, column r of the tile
+    float *row = g.partial + (static_cast<int64_t>(n) * g.slices + slice) * g.nW;
+    for (int e = threadIdx.x; e < MT * NT * 256; e += 256) {
+        const int tile = e >> 8, v = (e >> 6) & 3, l = e & 63;
+        const int mt = tile / NT, nt = tile - mt * NT;
+        const int o = ((og * MT + mt) << 4) + ((l >> 4) << 2) + v;
+        const int col = ((cg * NT + nt) << 4) + (l & 15);
+        if (o < g.Og && col < g.CK) row[static_cast<int64_t>(grp * g.Og + o) * g.CK + col] = red[e];
+    }
+}
+
 // gradW[q] = sum of the workspace rows: lane (q, part) adds rows part, part+16, ... in order, then
 // the 16 parts of a weight are added in order (a fixed association for a given geometry).
 __global__ __launch_bounds__(256) void synapse_wgrad_sum_kernel(float *__restrict__ gradW,
@@ -427,6 +591,92 @@ static WgradPlan plan_wgrad(const SynGeom &s, bool vec)
     return p;
 }
 
+
+// Tiling of the matrix-core weight gradient: MT x NT tiles of 16 x 16 per wavefront (at most 24
+// tiles = 96 accumulator registers), slices of pixels so that the GPU sees a few thousand wavefronts.
+struct MfmaPlan {
+    bool use;
+    int MT, NT, oGroups, colGroups, slices, pixPerSlice;
+};
+
+static MfmaPlan plan_wgrad_mfma(const SynGeom &s)
+{
+    MfmaPlan p{};
+    const int Og = s.O / s.groups, CK = (s.C / s.groups) * s.KH * s.KW;
+    const int64_t pixels = static_cast<int64_t>(s.OH) * s.OW;
+    // worth it when the 16 x 16 tiles are reasonably full and rows are whole 16-byte vectors
+    p.use = s.T % 4 == 0 && s.T >= 16 && Og >= 8 && CK >= 8 && pixels > 0 && s.N > 0;
+    if (!p.use) return p;
+    const int oTiles = static_cast<int>(ceil_div(Og, 16)), cTiles = static_cast<int>(ceil_div(CK, 16));
+    p.MT = oTiles >= 4 ? 4 : oTiles >= 2 ? 2 : 1;
+    const int ntMax = 24 / p.MT > 9 ? 9 : 24 / p.MT;  // 9, 9 or 6
+    const int options[5] = {1, 2, 4, 6, 9};
+    p.NT = 1;
+    for (int k = 0; k < 5; ++k)
+        if (options[k] <= ntMax) {
+            p.NT = options[k];
+            if (options[k] >= cTiles) break;
+        }
+    // few tiles per wavefront mean little reuse of the operands: the vector kernel is faster then
+    // (measured on 16 channels x 50 columns: 1 x 4 tiles 289 us, vector kernel 221 us)
+    if (p.MT * p.NT < 8) {
+        p.use = false;
+        return p;
+    }
+    p.oGroups = static_cast<int>(ceil_div(oTiles, p.MT));
+    p.colGroups = static_cast<int>(ceil_div(cTiles, p.NT));
+    const int64_t base = static_cast<int64_t>(s.N) * s.groups * p.oGroups * p.colGroups;
+    // four wavefronts per work-group, one pixel each at a time: slices of a multiple of 4 pixels,
+    // enough work-groups for a few per compute unit
+    int64_t slices = ceil_div(1536, base);
+    const int64_t quads = ceil_div(pixels, 4);
+    if (slices > quads) slices = quads;
+    if (slices < 1) slices = 1;
+    p.pixPerSlice = static_cast<int>(ceil_div(quads, slices) * 4);
+    p.slices = static_cast<int>(ceil_div(pixels, p.pixPerSlice));
+    return p;
+}
+
+template <int MT>
+static void launch_wgrad_mfma_nt(const WgradMfmaArgs &g, int NT, unsigned blocks, hipStream_t st)
+{
+    switch (NT) {
+        case 9:
+            if constexpr (MT <= 2) { hipLaunchKernelGGL((synapse_wgrad_mfma_kernel<MT, 9>), dim3(blocks), dim3(256), 0, st, g); break; }
+            [[fallthrough]];
+        case 6: hipLaunchKernelGGL((synapse_wgrad_mfma_kernel<MT, 6>), dim3(blocks), dim3(256), 0, st, g); break;
+        case 4: hipLaunchKernelGGL((synapse_wgrad_mfma_kernel<MT, 4>), dim3(blocks), dim3(256), 0, st, g); break;
+        case 2: hipLaunchKernelGGL((synapse_wgrad_mfma_kernel<MT, 2>), dim3(blocks), dim3(256), 0, st, g); break;
+        default: hipLaunchKernelGGL((synapse_wgrad_mfma_kernel<MT, 1>), dim3(blocks), dim3(256), 0, st, g); break;
+    }
+}
+
+// Returns the number of workspace rows written, or a negative status.
+static int launch_wgrad_mfma(const float *gradOut, const float *in, float *workspace, const SynGeom &s,
+                             const MfmaPlan &p, int nW, hipStream_t st)
+{
+    WgradMfmaArgs g{};
+    g.gradOut = gradOut; g.in = in; g.partial = workspace; g.s = s;
+    g.Cg = s.C / s.groups; g.Og = s.O / s.groups; g.CK = g.Cg * s.KH * s.KW;
+    g.oGroups = p.oGroups; g.colGroups = p.colGroups; g.slices = p.slices; g.pixPerSlice = p.pixPerSlice;
+    g.nW = nW;
+    g.bySlices = make_fastdiv(static_cast<uint32_t>(p.slices));
+    g.byColGroups = make_fastdiv(static_cast<uint32_t>(p.colGroups));
+    g.byOGroups = make_fastdiv(static_cast<uint32_t>(p.oGroups));
+    g.byGroups = make_fastdiv(static_cast<uint32_t>(s.groups));
+    g.byKK = make_fastdiv(static_cast<uint32_t>(s.KH * s.KW));
+    g.byKW = make_fastdiv(static_cast<uint32_t>(s.KW));
+    g.byOW = make_fastdiv(static_cast<uint32_t>(s.OW));
+    const int64_t blocks = static_cast<int64_t>(s.N) * s.groups * p.oGroups * p.colGroups * p.slices;
+    if (blocks >= (1LL << 31)) return -SLAYER_EUNSUPPORTED;
+    const unsigned nb = static_cast<unsigned>(blocks);
+    if (p.MT == 4) launch_wgrad_mfma_nt<4>(g, p.NT, nb, st);
+    else if (p.MT == 2) launch_wgrad_mfma_nt<2>(g, p.NT, nb, st);
+    else launch_wgrad_mfma_nt<1>(g, p.NT, nb, st);
+    const int status = launch_status();
+    return status == SLAYER_OK ? s.N * p.slices : -status;
+}
+
 template <int OBW, int TAPS>
 static void launch_wgrad_vec(const WgradArgs &g, int VEC, unsigned blocks, hipStream_t st)
 {
@@ -494,7 +744,9 @@ extern "C" int64_t slayer_synapse_conv_grad_weight_workspace_bytes(const slayer_
     const int64_t nW = static_cast<int64_t>(s.O) * (s.C / s.groups) * s.KH * s.KW;
     if (nW == 0 || s.N == 0) return 0;
     const WgradPlan p = plan_wgrad(s, s.T % 4 == 0);
-    return static_cast<int64_t>(s.N) * p.slicesPerItem * nW * static_cast<int64_t>(sizeof(float));
+    const MfmaPlan m = plan_wgrad_mfma(s);
+    const int64_t rows = static_cast<int64_t>(s.N) * (m.use && m.slices > p.slicesPerItem ? m.slices : p.slicesPerItem);
+    return rows * nW * static_cast<int64_t>(sizeof(float));
 }
 
 extern "C" int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gradOut, const float *in,
@@ -519,6 +771,14 @@ extern "C" int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gr
         const bool vecT = s.T % 4 == 0;
         WgradPlan p = plan_wgrad(s, vecT);
         const bool vec = vecT && aligned16(gradOut) && aligned16(in);
+        const MfmaPlan m = plan_wgrad_mfma(s);
+        if (m.use && vec && !generic_forced()) {
+            rows = launch_wgrad_mfma(gradOut, in, workspace, s, m, nW, st);
+            if (rows < 0) return -rows;
+            hipLaunchKernelGGL(synapse_wgrad_sum_kernel, dim3(static_cast<unsigned>(ceil_div(nW, 16))), dim3(256), 0, st,
+                               gradW, workspace, rows, nW);
+            return launch_status();
+        }
         WgradArgs g{};
         g.gradOut = gradOut; g.in = in; g.partial = workspace; g.s = s;
         g.Cg = s.C / s.groups; g.Og = s.O / s.groups;

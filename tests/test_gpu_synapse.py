@@ -49,6 +49,12 @@ CASES = [
     (1, 2, 4, 4, 8, 2, (5, 5), 1, 0, 1, 1),           # filter larger than the input: empty output
     (1, 8, 6, 6, 4, 12, (2, 2), 1, 1, 1, 4),          # 3 output channels per group
     (2, 2, 34, 34, 300, 16, (5, 5), 1, 2, 1, 1),      # the benchmark's first layer on two samples
+    # shapes that take the matrix-core weight gradient (T % 4 == 0, T >= 16, at least 8 tiles of 16 x 16)
+    (1, 16, 7, 7, 32, 32, (3, 3), 1, 1, 1, 1),        # 2 x 9 tiles
+    (1, 32, 5, 5, 20, 20, (3, 3), 1, 1, 1, 1),        # T % 16 != 0, 20 = 16 + 4 output channels, 18 column tiles
+    (2, 32, 10, 11, 16, 48, (3, 2), (2, 1), (1, 0), (1, 2), 2),  # groups of 24 channels x 96 columns, stride, dilation
+    (2, 15, 8, 9, 24, 9, (3, 3), 2, 1, 1, 1),         # stride 2, 9 output channels, 135 columns
+    (1, 8, 6, 6, 64, 72, (3, 3), 1, 1, 1, 1),         # 72 output channels: two blocks of four tiles
 ]
 IDS = ["%dx%dx%dx%dx%d-o%d-k%s-s%s-p%s-d%s-g%d" % c for c in CASES]
 
