@@ -184,6 +184,41 @@ __global__ __launch_bounds__(256) void synapse_gather_kernel(GatherArgs g)
         acc[m].store(dstB, masked_offset(live && mb0 + m < g.Mg, (mb0 + m) * dstPlaneBytes + p * VEC * 4));
 }
 
+
+// Input gradient of a one-channel synapse whose windows do not overlap (stride = window, no padding,
+// no dilation: the pooling layers).  Every input pixel belongs to exactly one window, so a lane
+// reads one vector of gradOut, scales it by the weight of its position in the window and writes
+// one vector of gradIn: a plain stream.  The general gather would issue KH*KW masked loads per lane.
+struct WindowArgs {
+    const float *gradOut, *w;
+    float *gradIn;
+    int H, W, OH, OW, T, KW, P;  // P = H*W*T/VEC vectors per batch item
+    int chunks;
+    FastDiv byChunks, byTV, byW, bySH, bySW;
+};
+
+template <int VEC>
+__global__ __launch_bounds__(256) void synapse_window_bwd_kernel(WindowArgs g)
+{
+    const uint32_t n = fastdiv(blockIdx.x, g.byChunks);
+    const int p = static_cast<int>(blockIdx.x - n * g.byChunks.d) * 256 + static_cast<int>(threadIdx.x);
+    if (p >= g.P) return;
+    const uint32_t pix = fastdiv(static_cast<uint32_t>(p), g.byTV);
+    const int tv = p - static_cast<int>(pix * g.byTV.d);
+    const int y = static_cast<int>(fastdiv(pix, g.byW)), x = static_cast<int>(pix) - y * g.W;
+    const int a = static_cast<int>(fastdiv(static_cast<uint32_t>(y), g.bySH));
+    const int b = static_cast<int>(fastdiv(static_cast<uint32_t>(x), g.bySW));
+    const int i = y - a * static_cast<int>(g.bySH.d), j = x - b * static_cast<int>(g.bySW.d);
+    const bool inside = a < g.OH && b < g.OW;  // rows and columns past the last whole window get no gradient
+    const BufferRsrc src = make_buffer(g.gradOut + static_cast<int64_t>(n) * g.OH * g.OW * g.T);
+    const BufferRsrc dst = make_buffer(g.gradIn + static_cast<int64_t>(n) * g.H * g.W * g.T);
+    TimeVec<VEC> v, out;
+    v.load(src, masked_offset(inside, ((a * g.OW + b) * g.T + tv * VEC) * 4));
+    out.zero();
+    out.fma(inside ? g.w[i * g.KW + j] : 0.f, v);
+    out.store(dst, p * VEC * 4);
+}
+
 // ---- weight gradient -----------------------------------------------------------------------------
 // gradW[o][c'][i][j] = sum_{n,a,b,t} gradOut[n][o][a][b][t] * in[n][c][a*sH-pH+i*dH][b*sW-pW+j*dW][t]
 // A work-group owns OBW output channels x TAPS taps of one input channel for one slice of one batch
@@ -532,6 +567,24 @@ static int launch_gather(float *dst, const float *src, const float *w, const Syn
     if (dstElems == 0) return SLAYER_OK;
     const bool vec = s.T % 4 == 0 && aligned16(src) && aligned16(dst);
     const int VEC = vec ? 4 : 1;
+    if (BACKWARD && s.C == 1 && s.O == 1 && s.sH == s.KH && s.sW == s.KW && s.pH == 0 && s.pW == 0 && s.dH == 1 &&
+        s.dW == 1 && s.OH > 0 && s.OW > 0 && !generic_forced()) {
+        WindowArgs a{};
+        a.gradOut = src; a.w = w; a.gradIn = dst;
+        a.H = s.H; a.W = s.W; a.OH = s.OH; a.OW = s.OW; a.T = s.T; a.KW = s.KW;
+        a.P = s.H * s.W * (s.T / VEC);
+        a.chunks = static_cast<int>(ceil_div(a.P, 256));
+        const int64_t nBlocks = static_cast<int64_t>(s.N) * a.chunks;
+        if (nBlocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+        a.byChunks = make_fastdiv(static_cast<uint32_t>(a.chunks));
+        a.byTV = make_fastdiv(static_cast<uint32_t>(s.T / VEC));
+        a.byW = make_fastdiv(static_cast<uint32_t>(s.W));
+        a.bySH = make_fastdiv(static_cast<uint32_t>(s.sH));
+        a.bySW = make_fastdiv(static_cast<uint32_t>(s.sW));
+        if (vec) hipLaunchKernelGGL(synapse_window_bwd_kernel<4>, dim3(static_cast<unsigned>(nBlocks)), dim3(256), 0, st, a);
+        else hipLaunchKernelGGL(synapse_window_bwd_kernel<1>, dim3(static_cast<unsigned>(nBlocks)), dim3(256), 0, st, a);
+        return launch_status();
+    }
     g.P = g.DH * g.DW * (g.T / VEC);
     g.chunks = static_cast<int>(ceil_div(g.P, 256));
     // destination channels per lane: as many as the group has, up to 16

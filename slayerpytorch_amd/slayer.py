@@ -149,7 +149,9 @@ class _denseLayer(nn.Conv3d):
         if input.dim() == 5 and tuple(input.shape[1:4]) == tuple(weight.shape[1:4]) and self.bias is None:
             N, T = input.shape[0], input.shape[4]
             O, K = weight.shape[0], weight.shape[1] * weight.shape[2] * weight.shape[3]
-            return torch.matmul(weight.reshape(O, K), input.reshape(N, K, T)).reshape(N, O, 1, 1, T)
+            # batched product with the weight matrix repeated by a zero stride: torch.matmul of a
+            # 2-D by a 3-D tensor would first copy the input into a (K, N*T) layout
+            return torch.bmm(weight.reshape(1, O, K).expand(N, O, K), input.reshape(N, K, T)).reshape(N, O, 1, 1, T)
         return F.conv3d(input, weight, self.bias, self.stride, self.padding, self.dilation, self.groups)
 
 

@@ -42,6 +42,8 @@ CASES = [
     (1, 32, 5, 5, 4, 20, (3, 3), 1, 1, 1, 1),         # 288 taps: two LDS chunks; 20 = 16 + 4 channels
     (2, 1, 12, 8, 16, 1, (2, 2), 2, 0, 1, 1),         # pooling geometry
     (1, 1, 13, 9, 8, 1, (3, 2), (3, 2), 0, 1, 1),     # ragged pooling: windows that do not fit
+    (2, 1, 6, 8, 7, 1, (2, 2), 2, 0, 1, 1),           # pooling with T % 4 != 0
+    (1, 1, 8, 8, 8, 1, (2, 2), 2, 1, 1, 1),           # padded pooling: overlapping the border, general kernel
     (2, 3, 8, 9, 7, 5, (3, 3), 1, 0, 1, 1),           # T % 4 != 0
     (1, 4, 10, 11, 6, 8, (3, 2), (2, 1), (1, 0), (1, 2), 2),   # stride, padding, dilation, groups
     (1, 6, 9, 9, 4, 6, (3, 3), 2, 2, 2, 3),           # all of them, 3 groups of 2
