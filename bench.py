@@ -247,6 +247,40 @@ def synapse_rows(device, timed):
     return rows
 
 
+def loihi_cnn_row(device, timed):
+    """Inference of the Loihi gesture network of the reference's example
+    (exampleLoihi/03_IBMGesture/ibmGestureTrain.py:44-79, without dropout) on (8, 2, 128, 128, 300) input
+    spikes at p = 0.01: pool 4, conv 2->16 5x5, pool 2, conv 16->32 3x3, pool 2, dense 2048->512->11, weights
+    quantised to even integers, every layer as delayShift(spikeLoihi(synapse(x)), 1) with the shift fused
+    into the neuron kernel; no autograd."""
+    import slayerpytorch_amd as snn
+    desc = {"type": "LOIHI", "vThMant": 80, "vDecay": 128, "iDecay": 1024, "refDelay": 1, "wgtExp": 0,
+            "tauRho": 1, "scaleRho": 1}
+    layer = snn.loihi(desc, {"Ts": 1, "tSample": 300}).to(device)
+    torch.manual_seed(0)
+    mods = [layer.pool(4), layer.conv(2, 16, 5, padding=2, weightScale=10), layer.pool(2),
+            layer.conv(16, 32, 3, padding=1, weightScale=50), layer.pool(2), layer.dense(8 * 8 * 32, 512),
+            layer.dense(512, 11)]
+    mods = [m.to(device) for m in mods]
+    g = torch.Generator(device="cpu").manual_seed(6)
+    x = (torch.rand((8, 2, 128, 128, 300), generator=g) < 0.01).float().to(device)
+    rates = []
+
+    def step():
+        del rates[:]
+        with torch.no_grad():
+            s = x
+            for k, syn in enumerate(mods):
+                if k == 5:
+                    s = s.reshape(s.shape[0], -1, 1, 1, s.shape[-1])
+                s = layer.spikeLoihi(syn(s), delay=1)
+                rates.append(s)
+
+    t = timed(step)
+    return {"op": "loihi_gesture_cnn_inference", "shape": [8, 2, 128, 128, 300], "us": t * 1e6, "samples_per_s": 8 / t,
+            "spike_rate_per_layer": [round(float(r.mean()), 4) for r in rates]}
+
+
 def event_row(device, timed, cpu_leg):
     """A batch of 12 NMNIST-sized samples (5000 events each, the 5-byte layout of the .bs2 files)
     to a (12, 2, 34, 34, 300) spike tensor: file bytes uploaded and decoded + binned by one kernel
@@ -350,6 +384,7 @@ def other_rows(device, cpu_leg=False):
     out.append(cnn_row(device, timed))
     out.extend(synapse_rows(device, timed))
     out.append(event_row(device, timed, cpu_leg))
+    out.append(loihi_cnn_row(device, timed))
     # Loihi config: largest tensor (8, 16, 32, 32, 300)
     shape = (8, 16, 32, 32, 300)
     w = (2 * torch.randint(-128, 128, shape, generator=g) * (torch.rand(shape, generator=g) < 0.05)).float().to(device)

@@ -91,6 +91,31 @@ class spikeLayer(slayer.spikeLayer):
     def dense(self, inFeatures, outFeatures, weightScale=100, preHookFx=lambda x: quantize(x, step=2)):
         return super().dense(inFeatures, outFeatures, weightScale, preHookFx)
 
+    def conv(self, inChannels, outChannels, kernelSize, stride=1, padding=0, dilation=1, groups=1, weightScale=100,
+             preHookFx=lambda x: quantize(x, step=2)):
+        """Convolution synapse with weights quantised in steps of 2 (src/slayerLoihi.py:141-156)."""
+        return super().conv(inChannels, outChannels, kernelSize, stride, padding, dilation, groups, weightScale,
+                            preHookFx)
+
+    def _poolWeight(self):
+        # the pooling weight that makes one input spike cross the threshold, on Loihi's even weight grid
+        # (src/slayerLoihi.py:171-174); the layer multiplies its argument by 1.1 again
+        return float(quantize(torch.tensor(1.1 * self.neuron["theta"] / self.maxPspKernel), 2)) / 1.1
+
+    def pool(self, kernelSize, stride=None, padding=0, dilation=1, preHookFx=None):
+        """Pooling synapse (src/slayerLoihi.py:158-174)."""
+        return slayer._poolLayer(self._poolWeight(), kernelSize, stride, padding, dilation, preHookFx)
+
+    def convTranspose(self, inChannels, outChannels, kernelSize, stride=1, padding=0, dilation=1, groups=1,
+                      weightScale=100, preHookFx=lambda x: quantize(x, step=2)):
+        """Transposed convolution synapse with quantised weights (src/slayerLoihi.py:175-189)."""
+        return super().convTranspose(inChannels, outChannels, kernelSize, stride, padding, dilation, groups,
+                                     weightScale, preHookFx)
+
+    def unpool(self, kernelSize, stride=None, padding=0, dilation=1, preHookFx=None):
+        """Unpooling synapse (src/slayerLoihi.py:191-205)."""
+        return slayer._unpoolLayer(self._poolWeight(), kernelSize, stride, padding, dilation, preHookFx)
+
 
 class _spike(torch.autograd.Function):
     @staticmethod

@@ -494,3 +494,41 @@ def test_delay_stress_config_shapes():
     assert rel_err(host(delay.delay.grad), O.delay_grad(want_y, host(grad), 1.0)) < REL_TOL
     want_gx = O.corr(O.shift(host(grad), -host(delay.delay.data), 1.0), host(layer.srmKernel), 1.0)
     assert np.array_equal(host(x.grad), want_gx)
+
+
+def test_loihi_cnn_inference_is_bit_exact():
+    """A small Loihi network in the ordering of the reference's gesture example
+    (exampleLoihi/03_IBMGesture/ibmGestureTrain.py:55-79): pool, conv, pool, dense with weights on Loihi's even
+    integer grid, every layer followed by a shift of one step.  Sums of small integers are exact in fp32, so the
+    whole pipeline must reproduce the oracle chain (synapse -> integer neuron -> shift) bit for bit."""
+    from oracle import oracle as O
+    desc = {"type": "LOIHI", "vThMant": 80, "vDecay": 128, "iDecay": 1024, "refDelay": 1, "wgtExp": 0,
+            "tauRho": 1, "scaleRho": 1}
+    layer = snn.loihi(desc, {"Ts": 1, "tSample": 64}).cuda()
+    torch.manual_seed(3)
+    pool1, conv1, pool2 = layer.pool(2), layer.conv(2, 8, 3, padding=1, weightScale=30), layer.pool(2)
+    fc = layer.dense(4 * 4 * 8, 5, weightScale=60)
+    mods = [m.cuda() for m in (pool1, conv1, pool2, fc)]
+    rng = np.random.default_rng(12)
+    x = (rng.random((2, 2, 16, 16, 64)) < 0.05).astype(np.float32)
+
+    s = torch.from_numpy(x).cuda()
+    ref = x
+    with torch.no_grad():
+        for k, m in enumerate(mods):
+            w = (m.weight if m.preHookFx is None else m.preHookFx(m.weight)).detach().cpu().numpy()[..., 0]
+            if k == 3:
+                s = s.reshape(2, -1, 1, 1, 64)
+                ref = ref.reshape(2, -1, 1, 1, 64)
+                z = np.einsum("ok,nkt->not", w.reshape(5, -1).astype(np.float64), ref.reshape(2, -1, 64)).reshape(2, 5, 1, 1, 64)
+            elif k == 1:
+                z = O.synapse_conv(ref, w, 1, 1)
+            else:
+                N, C, H, W, T = ref.shape
+                z = O.synapse_conv(ref.reshape(N, 1, C * H, W, T), w, 2).reshape(N, C, H // 2, W // 2, T)
+            assert np.array_equal(z, np.round(z))                      # integer weighted spikes
+            spikes = O.loihi_get_spikes(z.astype(np.float32), 0, desc["theta"], 1024, 128, 1)[0]
+            ref = O.shift(spikes, 1.0, 1.0)
+            s = layer.spikeLoihi(m(s), delay=1)
+            assert np.array_equal(s.cpu().numpy(), ref), "layer %d" % k
+    assert ref.sum() > 0
