@@ -120,6 +120,20 @@ class spikeLayer(nn.Module):
         """Unpooling synapse with weights ``1.1 * theta`` (src/slayer.py:290-313)."""
         return _unpoolLayer(self.neuron["theta"], kernelSize, stride, padding, dilation, preHookFx)
 
+    def dropout(self, p=0.5, inplace=False):
+        """Dropout that keeps a dropped neuron dropped for the whole time axis (src/slayer.py:315-331);
+        a plain PyTorch module, as in the reference."""
+        return _dropoutLayer(p, inplace)
+
+    def replicateInTime(self, input, mode="nearest"):
+        """Repeats an (N, C, H, W) tensor along a new time axis of tSample / Ts samples
+        (src/slayer.py:179-185)."""
+        Ns = int(self.simulation["tSample"] / self.simulation["Ts"])
+        N, C, H, W = input.shape
+        if mode != "nearest":
+            raise Exception("Unsupported mode. It was {}".format(mode))
+        return F.interpolate(input.reshape(N, C, H, W, 1), size=(H, W, Ns), mode="nearest")
+
 
 class _denseLayer(nn.Conv3d):
     """Fully connected synapse: an (outFeatures, C, H, W, 1) weight applied at every time step
@@ -250,6 +264,16 @@ class _unpoolLayer(nn.ConvTranspose3d):
         result = synapse.synapseConvTranspose(input.reshape(N, 1, C * H, W, T), weight, self.stride[:2],
                                               self.padding[:2], self.dilation[:2], 1)
         return result.reshape(result.shape[0], C, -1, result.shape[3], result.shape[4])
+
+
+class _dropoutLayer(nn.Dropout3d):
+    """Dropout over whole neurons: the tensor is viewed as (N, C*H*W, 1, 1, T) so that ``dropout3d``
+    zeroes entire time rows (src/slayer.py:748-759)."""
+
+    def forward(self, input):
+        shape = input.shape
+        return F.dropout3d(input.reshape(shape[0], -1, 1, 1, shape[-1]), self.p, self.training,
+                           self.inplace).reshape(shape)
 
 
 class _spikeFunction(torch.autograd.Function):

@@ -61,6 +61,16 @@ CASES = [
 IDS = ["%dx%dx%dx%dx%d-o%d-k%s-s%s-p%s-d%s-g%d" % c for c in CASES]
 
 
+@pytest.fixture(params=[0, 1], ids=["fast", "generic"])
+def impl(request):
+    """Runs a test with the matrix-core / streaming kernels (default) and with the general vector
+    kernels that serve every geometry."""
+    lib = _lib.load()
+    old = lib.slayer_force_generic_kernels(request.param)
+    yield request.param
+    lib.slayer_force_generic_kernels(old)
+
+
 def make(case, seed):
     N, C, H, W, T, Oc, K, s, p, d, g = case
     rng = np.random.default_rng(seed)
@@ -78,7 +88,7 @@ def test_conv_matches_oracle(case):
 
 
 @pytest.mark.parametrize("case", CASES, ids=IDS)
-def test_conv_grad_input_matches_oracle(case):
+def test_conv_grad_input_matches_oracle(case, impl):
     x, w, a = make(case, 2)
     shape = O.synapse_geom(x.shape, w.shape, *a)[1]
     go = np.random.default_rng(3).standard_normal(shape).astype(np.float32)
@@ -88,7 +98,7 @@ def test_conv_grad_input_matches_oracle(case):
 
 
 @pytest.mark.parametrize("case", CASES, ids=IDS)
-def test_conv_grad_weight_matches_oracle(case):
+def test_conv_grad_weight_matches_oracle(case, impl):
     x, w, a = make(case, 4)
     shape = O.synapse_geom(x.shape, w.shape, *a)[1]
     go = np.random.default_rng(5).standard_normal(shape).astype(np.float32)

@@ -215,3 +215,16 @@ def test_event_class_decodes_like_the_oracle():
         assert ev.dim == (1 if fmt == 1 else 2)
         if fmt != 1:
             assert np.array_equal(ev.y, y)
+
+
+def test_dropout_and_replicate_in_time():
+    """Dropout zeroes whole time rows (src/slayer.py:748-759); replicateInTime repeats along T."""
+    layer = snn.layer({"theta": 10, "tauSr": 1.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1},
+                      {"Ts": 1.0, "tSample": 10})
+    torch.manual_seed(0)
+    y = layer.dropout(0.5)(torch.ones(4, 3, 5, 5, 10))
+    sums = y.sum(-1).flatten()
+    assert set(sums.tolist()) == {0.0, 20.0}
+    x = torch.rand(2, 3, 4, 4)
+    r = layer.replicateInTime(x)
+    assert r.shape == (2, 3, 4, 4, 10) and torch.equal(r[..., 7], x)
