@@ -417,6 +417,8 @@ def main():
                          "other rows or CPU baseline")
     ap.add_argument("--cnn-only", action="store_true",
                     help="only the NMNIST CNN training step of the other rows (for profiler runs); prints that row")
+    ap.add_argument("--synapse-only", action="store_true",
+                    help="only the per-layer synapse kernel rows (for profiler runs); prints those rows")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain copy of known size (a zero-delay shift of half the tensor: "
                          "%d bytes read, as many written) to scale hardware counters by" % (4 * 6 * 16 * 34 * 34 * 300))
@@ -432,7 +434,7 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    if args.cnn_only:
+    if args.cnn_only or args.synapse_only:
         def wall(fn):
             ts = []
             for _ in range(args.warmup + args.steps):
@@ -442,7 +444,7 @@ def main():
                 torch.cuda.synchronize()
                 ts.append(time.perf_counter() - t0)
             return float(np.median(ts[args.warmup:]))
-        print(json.dumps(cnn_row(device, wall)))
+        print(json.dumps(cnn_row(device, wall) if args.cnn_only else {"synapse_rows": synapse_rows(device, wall)}))
         return
     params = neuron_params()
     srm = np.array(alphaKernel(params["tauSr"], 1.0, SHAPE[-1]), dtype=np.float32)

@@ -106,6 +106,19 @@ __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f)
     return (t + ((n - t) >> f.s1)) >> f.s2;
 }
 
+// Work-groups are handed to the GPU's 8 accelerator dies (XCDs, each with its own L2) round-robin by
+// index: group b runs on die b % 8.  Kernels whose neighbouring groups read the same data (filter
+// windows that overlap, operands shared between tiles) would make every die fetch all of it.  This
+// maps the hardware index to a logical one so that each die owns one contiguous range of logical
+// indices: die x gets the k-th index of its range for its k-th group.
+__device__ __forceinline__ uint32_t xcd_contiguous(uint32_t b, uint32_t n)
+{
+    constexpr uint32_t kDies = 8;
+    const uint32_t per = n / kDies, rem = n % kDies;  // die x owns per + (x < rem) indices
+    const uint32_t x = b % kDies, k = b / kDies;
+    return x * per + (x < rem ? x : rem) + k;
+}
+
 // ---- buffer addressing -------------------------------------------------------------------------
 // address = base (128-bit descriptor in scalar registers) + per-lane byte offset (one vector
 // register) + wave-uniform byte offset (scalar register).  Lets a wave touch many rows of a tile

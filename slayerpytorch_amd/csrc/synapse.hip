@@ -78,12 +78,14 @@ __global__ __launch_bounds__(256) void synapse_gather_kernel(GatherArgs g)
 {
     __shared__ __attribute__((aligned(16))) float wl[kTapChunk * MB];
 
-    // work-group -> (batch item, group, block of MB destination channels, chunk of 256 vectors)
-    uint32_t rest = blockIdx.x;
-    const uint32_t nmb = fastdiv(rest, g.byChunks);
-    const int chunk = static_cast<int>(rest - nmb * g.byChunks.d);
-    const uint32_t ng = fastdiv(nmb, g.byMBlocks);
-    const int mb0 = static_cast<int>(nmb - ng * g.byMBlocks.d) * MB;  // first channel of the block, within the group
+    // work-group -> (batch item, group, block of MB destination channels, chunk of 256 vectors);
+    // neighbouring chunks read overlapping source rows, so they are kept on one die
+    // (the blocks of destination channels of one chunk read the same source rows: they are neighbours)
+    uint32_t rest = xcd_contiguous(blockIdx.x, gridDim.x);
+    const uint32_t nc = fastdiv(rest, g.byMBlocks);
+    const int mb0 = static_cast<int>(rest - nc * g.byMBlocks.d) * MB;  // first channel of the block, within the group
+    const uint32_t ng = fastdiv(nc, g.byChunks);
+    const int chunk = static_cast<int>(nc - ng * g.byChunks.d);
     const uint32_t n = fastdiv(ng, g.byGroups);
     const int grp = static_cast<int>(ng - n * g.byGroups.d);
 
@@ -200,8 +202,9 @@ struct WindowArgs {
 template <int VEC>
 __global__ __launch_bounds__(256) void synapse_window_bwd_kernel(WindowArgs g)
 {
-    const uint32_t n = fastdiv(blockIdx.x, g.byChunks);
-    const int p = static_cast<int>(blockIdx.x - n * g.byChunks.d) * 256 + static_cast<int>(threadIdx.x);
+    const uint32_t blk = xcd_contiguous(blockIdx.x, gridDim.x);
+    const uint32_t n = fastdiv(blk, g.byChunks);
+    const int p = static_cast<int>(blk - n * g.byChunks.d) * 256 + static_cast<int>(threadIdx.x);
     if (p >= g.P) return;
     const uint32_t pix = fastdiv(static_cast<uint32_t>(p), g.byTV);
     const int tv = p - static_cast<int>(pix * g.byTV.d);
@@ -241,10 +244,10 @@ __global__ __launch_bounds__(256) void synapse_wgrad_kernel(WgradArgs g)
     __shared__ float red[4][OBW * TAPS];
     const SynGeom &s = g.s;
 
-    uint32_t r = blockIdx.x;
-    uint32_t q = fastdiv(r, g.bySlices);
-    const int slice = static_cast<int>(r - q * g.bySlices.d);
-    r = q; q = fastdiv(r, g.byTapBlocks);
+    // all (channel block, channel, tap block) combinations of one slice are neighbours: they read
+    // the same samples of gradOut and in
+    uint32_t r = xcd_contiguous(blockIdx.x, gridDim.x);
+    uint32_t q = fastdiv(r, g.byTapBlocks);
     const int tap0 = static_cast<int>(r - q * g.byTapBlocks.d) * TAPS;
     r = q; q = fastdiv(r, g.byCg);
     const int cl = static_cast<int>(r - q * g.byCg.d);
@@ -252,6 +255,8 @@ __global__ __launch_bounds__(256) void synapse_wgrad_kernel(WgradArgs g)
     const int ol0 = static_cast<int>(r - q * g.byOBlocks.d) * OBW;
     r = q; q = fastdiv(r, g.byGroups);
     const int grp = static_cast<int>(r - q * g.byGroups.d);
+    r = q; q = fastdiv(r, g.bySlices);
+    const int slice = static_cast<int>(r - q * g.bySlices.d);
     const int n = static_cast<int>(q);
 
     const int KK = s.KH * s.KW;
@@ -352,15 +357,16 @@ __global__ __launch_bounds__(256) void synapse_wgrad_mfma_kernel(WgradMfmaArgs g
 {
     __shared__ float red[MT * NT * 256];
     const SynGeom &s = g.s;
-    uint32_t rest = blockIdx.x;
-    uint32_t q = fastdiv(rest, g.bySlices);
-    const int slice = static_cast<int>(rest - q * g.bySlices.d);
-    rest = q; q = fastdiv(rest, g.byColGroups);
+    // the tile groups of one slice of pixels are neighbours: they read the same operand rows
+    uint32_t rest = xcd_contiguous(blockIdx.x, gridDim.x);
+    uint32_t q = fastdiv(rest, g.byColGroups);
     const int cg = static_cast<int>(rest - q * g.byColGroups.d);
     rest = q; q = fastdiv(rest, g.byOGroups);
     const int og = static_cast<int>(rest - q * g.byOGroups.d);
     rest = q; q = fastdiv(rest, g.byGroups);
     const int grp = static_cast<int>(rest - q * g.byGroups.d);
+    rest = q; q = fastdiv(rest, g.bySlices);
+    const int slice = static_cast<int>(rest - q * g.bySlices.d);
     const int n = static_cast<int>(q);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, h = lane >> 4;
@@ -484,25 +490,38 @@ __global__ __launch_bounds__(256) void synapse_wgrad_mfma_kernel(WgradMfmaArgs g
     }
 }
 
-// gradW[q] = sum of the workspace rows: lane (q, part) adds rows part, part+16, ... in order, then
-// the 16 parts of a weight are added in order (a fixed association for a given geometry).
+// gradW[q] = sum of the workspace rows: lane (q, part) adds rows part, part+PARTS, ... in order, then
+// the PARTS sums of a weight are added in order (a fixed association for a given geometry).  A group
+// handles 256 / PARTS weights; few weights take more parts so that the launch still fills the GPU.
+template <int PARTS>
 __global__ __launch_bounds__(256) void synapse_wgrad_sum_kernel(float *__restrict__ gradW,
                                                                 const float *__restrict__ partial, int rows, int nW)
 {
-    __shared__ float part[16][17];
-    const int ql = threadIdx.x & 15, pt = threadIdx.x >> 4;
-    const int q = blockIdx.x * 16 + ql;
+    constexpr int kWeights = 256 / PARTS;
+    __shared__ float part[PARTS][kWeights + 1];
+    const int ql = threadIdx.x % kWeights, pt = threadIdx.x / kWeights;
+    const int q = blockIdx.x * kWeights + ql;
     float acc = 0.f;
     if (q < nW)
-        for (int r = pt; r < rows; r += 16) acc += partial[static_cast<int64_t>(r) * nW + q];
+        for (int r = pt; r < rows; r += PARTS) acc += partial[static_cast<int64_t>(r) * nW + q];
     part[pt][ql] = acc;
     __syncthreads();
-    if (threadIdx.x < 16 && q < nW) {
+    if (threadIdx.x < kWeights && q < nW) {
         float v = part[0][ql];
 #pragma unroll
-        for (int k = 1; k < 16; ++k) v += part[k][ql];
+        for (int k = 1; k < PARTS; ++k) v += part[k][ql];
         gradW[q] = v;
     }
+}
+
+static void launch_wgrad_sum(float *gradW, const float *workspace, int rows, int nW, hipStream_t st)
+{
+    if (nW < 8192)
+        hipLaunchKernelGGL(synapse_wgrad_sum_kernel<64>, dim3(static_cast<unsigned>(ceil_div(nW, 4))), dim3(256), 0, st,
+                           gradW, workspace, rows, nW);
+    else
+        hipLaunchKernelGGL(synapse_wgrad_sum_kernel<16>, dim3(static_cast<unsigned>(ceil_div(nW, 16))), dim3(256), 0, st,
+                           gradW, workspace, rows, nW);
 }
 
 // ---- host side -------------------------------------------------------------------------------------
@@ -828,8 +847,7 @@ extern "C" int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gr
         if (m.use && vec && !generic_forced()) {
             rows = launch_wgrad_mfma(gradOut, in, workspace, s, m, nW, st);
             if (rows < 0) return -rows;
-            hipLaunchKernelGGL(synapse_wgrad_sum_kernel, dim3(static_cast<unsigned>(ceil_div(nW, 16))), dim3(256), 0, st,
-                               gradW, workspace, rows, nW);
+            launch_wgrad_sum(gradW, workspace, rows, nW, st);
             return launch_status();
         }
         WgradArgs g{};
@@ -865,7 +883,6 @@ extern "C" int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gr
         if (st1 != SLAYER_OK) return st1;
         rows = s.N * p.slicesPerItem;
     }
-    hipLaunchKernelGGL(synapse_wgrad_sum_kernel, dim3(static_cast<unsigned>(ceil_div(nW, 16))), dim3(256), 0, st,
-                       gradW, workspace, rows, nW);
+    launch_wgrad_sum(gradW, workspace, rows, nW, st);
     return launch_status();
 }
