@@ -516,7 +516,7 @@ __global__ __launch_bounds__(256) void synapse_wgrad_sum_kernel(float *__restric
 
 static void launch_wgrad_sum(float *gradW, const float *workspace, int rows, int nW, hipStream_t st)
 {
-    if (nW < 8192)
+    if (nW < 2048)
         hipLaunchKernelGGL(synapse_wgrad_sum_kernel<64>, dim3(static_cast<unsigned>(ceil_div(nW, 4))), dim3(256), 0, st,
                            gradW, workspace, rows, nW);
     else
