@@ -689,9 +689,9 @@ static MfmaPlan plan_wgrad_mfma(const SynGeom &s)
             p.NT = options[k];
             if (options[k] >= cTiles) break;
         }
-    // few tiles per wavefront mean little reuse of the operands: the vector kernel is faster then
-    // (measured on 16 channels x 50 columns: 1 x 4 tiles 289 us, vector kernel 221 us)
-    if (p.MT * p.NT < 8) {
+    // very few tiles per wavefront mean little reuse of the operands: left to the vector kernel
+    // (1 x 4 tiles on 16 channels x 50 columns: 172 us against 212 us for the vector kernel)
+    if (p.MT * p.NT < 4) {
         p.use = false;
         return p;
     }
