@@ -161,6 +161,60 @@ def mlp_row(device, timed):
             "us_with_separate_psp_and_spike_calls": two * 1e6, "samples_per_s": 12 / one}
 
 
+def scale_weights_to_rate(weight, rate, target=0.04):
+    """Scales a random weight tensor in place until ``rate()`` (the fraction of output samples that
+    are spikes) is within 25 % of ``target``: random weights at the default scale leave a layer
+    silent or saturated, a trained network fires a few per cent of the time."""
+    with torch.no_grad():
+        for _ in range(16):
+            r = rate()
+            if 0.75 * target <= r <= 1.25 * target:
+                break
+            weight.mul_(min(3.0, max(0.3, (target / max(r, 1e-4)) ** 0.7)))
+
+
+def delay_mlp_row(device, timed):
+    """One training step (without the optimiser) of the long-sequence delay network: 200 input neurons
+    with Poisson spikes at 0.005 per step, batch 64, T = 2000, dense 200 -> 256 -> 200 with a learnable
+    axonal delay per neuron (U[0, 62]) after every layer, SRM tauSr = tauRef = 1, spike-time loss against
+    a random raster at p = 0.01; layer ordering delay(spike(psp(fc(x))))."""
+    import slayerpytorch_amd as snn
+    params = {"type": "SRMALPHA", "theta": 10, "tauSr": 1.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
+    sim = {"Ts": 1.0, "tSample": 2000}
+    net = {"neuron": params, "simulation": sim, "training": {"error": {"type": "SpikeTime"}}}
+    layer = snn.layer(params, sim).to(device)
+    error = snn.loss(net).to(device)
+    torch.manual_seed(0)
+    fc1, fc2 = layer.dense(200, 256).to(device), layer.dense(256, 200).to(device)
+    d1, d2 = layer.delay(256).to(device), layer.delay(200).to(device)
+    with torch.no_grad():
+        d1.delay.mul_(62.0)
+        d2.delay.mul_(62.0)
+    g = torch.Generator(device="cpu").manual_seed(7)
+    x = (torch.rand((64, 200, 1, 1, 2000), generator=g) < 0.005).float().to(device)
+    target = (torch.rand((64, 200, 1, 1, 2000), generator=g) < 0.01).float().to(device)
+    rates = []
+    with torch.no_grad():
+        scale_weights_to_rate(fc1.weight, lambda: float(layer.spike(layer.psp(fc1(x))).mean()))
+        s1 = d1(layer.spike(layer.psp(fc1(x))))
+        scale_weights_to_rate(fc2.weight, lambda: float(layer.spike(layer.psp(fc2(s1))).mean()))
+
+    def step():
+        s1 = d1(layer.spike(layer.psp(fc1(x))))
+        s2 = d2(layer.spike(layer.psp(fc2(s1))))
+        del rates[:]
+        rates.extend((s1, s2))
+        error.spikeTime(s2, target).backward()
+        for m in (fc1, fc2):
+            m.weight.grad = None
+        for m in (d1, d2):
+            m.delay.grad = None
+
+    t = timed(step)
+    return {"op": "delay_mlp_200_256_200_fwd_loss_bwd", "shape": [64, 200, 1, 1, 2000], "us": t * 1e6,
+            "samples_per_s": 64 / t, "spike_rate_per_layer": [round(float(r.detach().mean()), 4) for r in rates]}
+
+
 def cnn_row(device, timed):
     """One training step (without the optimiser) of the NMNIST CNN of the reference's example
     (example/03_NMNIST_CNN/nmnistCNN.py:47-62: conv 2->16 5x5, pool 2, conv 16->32 3x3, pool 2,
@@ -181,19 +235,13 @@ def cnn_row(device, timed):
     x = (torch.rand((12, 2, 34, 34, 300), generator=g) < 0.02).float().to(device)
     target = (torch.rand((12, 10, 1, 1, 300), generator=g) < 0.01).float().to(device)
     rates = []
-    # Random weights at the default scale drive every layer into saturation (20-80 % of all samples
-    # spike); a trained network fires a few per cent of the time.  Scale each trainable layer's random
-    # weights, front to back, until about 4 % of its output samples are spikes.
+    # random weights scaled, front to back, until about 4 % of a trainable layer's output samples are spikes
     with torch.no_grad():
         s = x
         for syn in (conv1, pool1, conv2, pool2, conv3, fc1):
             a = layer.psp(s)
             if syn.weight.requires_grad:
-                for _ in range(12):
-                    rate = float(layer.spike(syn(a)).mean())
-                    if 0.03 <= rate <= 0.05:
-                        break
-                    syn.weight.mul_(min(3.0, max(0.3, (0.04 / max(rate, 1e-4)) ** 0.7)))
+                scale_weights_to_rate(syn.weight, lambda: float(layer.spike(syn(a)).mean()))
             s = layer.spike(syn(a))
 
     def step():
@@ -382,6 +430,7 @@ def other_rows(device, cpu_leg=False):
     out.append(mlp_row(device, timed))
     # NMNIST-shaped CNN end to end (synapses by the per-timestep synapse kernels)
     out.append(cnn_row(device, timed))
+    out.append(delay_mlp_row(device, timed))
     out.extend(synapse_rows(device, timed))
     out.append(event_row(device, timed, cpu_leg))
     out.append(loihi_cnn_row(device, timed))
