@@ -588,6 +588,35 @@ def main():
         result["per_kernel_pass"] = "%d untimed steps before the timed region, an event pair around every launch" % probe
     del pool
     if not args.chain_only:
+        # The same step with the shift fused into the spike kernel (forward) and into the surrogate
+        # gradient (backward): four launches, 40 instead of 56 bytes per element, same results.
+        pool = [u0.clone() for _ in range(args.warmup + args.steps + 2)]
+
+        def fused_step(u):
+            slayerCuda.conv(spikes, srm_t, 1.0)
+            slayerCuda.getSpikesDelayed(u, ref_t, theta, 1.0, 1.0, 1.0)
+            gs = slayerCuda.spikeBackwardDelayed(grad, u, theta, tau, scale, 1.0, 1.0)
+            slayerCuda.corr(gs, srm_t, 1.0)
+
+        for i in range(args.warmup):
+            fused_step(pool[i])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            fused_step(pool[args.warmup + i])
+        torch.cuda.synchronize()
+        fused = (time.perf_counter() - t0) / args.steps
+        ua, ub = pool[-1], pool[-2]
+        same = bool(torch.equal(slayerCuda.getSpikesDelayed(ua, ref_t, theta, 1.0, 1.0, 1.0),
+                                slayerCuda.shift(slayerCuda.getSpikes(ub, ref_t, theta, 1.0), 1.0, 1.0))
+                    and torch.equal(slayerCuda.spikeBackwardDelayed(grad, ua, theta, tau, scale, 1.0, 1.0),
+                                    slayerCuda.spikeBackward(slayerCuda.shift(grad, 1.0, 1.0, sign=-1.0), ub, theta, tau,
+                                                             scale)))
+        result["fused_shift_chain"] = {
+            "launches": "psp conv, spike+shift | shift+spike pdf, psp corr", "ms_per_step": fused * 1e3,
+            "value": numel / fused, "unit": "neuron-timesteps/s", "algorithmic_bytes_per_element": 40,
+            "hbm_frac": 40 * numel / fused / 1e9 / HBM_PEAK_GBS, "identical_to_unfused_results": same}
+        del pool
         result["measured_copy_ceiling"] = copy_ceiling(grad)
         result["other_rows"] = other_rows(device, cpu_leg=not args.no_cpu_baseline)
         if not args.no_cpu_baseline:

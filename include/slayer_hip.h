@@ -158,6 +158,34 @@ int slayer_psp_spike_f32(float *s, float *u, const float *a, const float *srm, c
                          int64_t nNeurons, int64_t T, int64_t F, int64_t nuSize, float theta,
                          float Ts, void *stream);
 
+/*
+ * Spike generation with the time shift that follows it fused into the store of the spikes.
+ * Replaces the call pair slayerCuda.getSpikes (src/cuda/slayerKernels.cu:14-39) -> slayerCuda.shift
+ * (src/cuda/slayerKernels.cu:77-134) that `delayShift(spike(u), d)` / `delay(spike(u))` make
+ * (src/slayer.py:333-391, 901-979): 8 of the 20 bytes per sample of the two kernels are not moved.
+ *
+ * s[t] = spike[t - k] with k = (int)(d / delayTs) (0 where t - k is outside the row); d is
+ * delayLut[neuron % lutSize] when delayLut is given (one delay per neuron of a batch item, nNeurons a
+ * multiple of lutSize) and `delay` otherwise.  `u` is updated in place and NOT shifted, exactly as by
+ * slayer_get_spikes_f32.  Only rows that the tile kernel moves whole are fused (T <= 352, nuSize <= 24);
+ * other shapes return SLAYER_EUNSUPPORTED with nothing launched - call the two functions then.
+ */
+int slayer_get_spikes_delayed_f32(float *s, float *u, const float *nu, const float *delayLut,
+                                  int64_t lutSize, float delay, float delayTs, int64_t nNeurons,
+                                  int64_t T, int64_t nuSize, float theta, float Ts, void *stream);
+
+/*
+ * Backward pass of the above in one kernel: gradIn[t] = gradOut[t + k] * scale/tau * exp(-|u[t]-theta|/tau)
+ * (0 where t + k is outside the row), i.e. the backward shift of _delayFunction / delayShift
+ * (src/slayer.py:944-979) followed by the surrogate gradient of _spikeFunction.backward
+ * (src/slayer.py:857-865), bit-identical to slayer_shift_*_f32 with the negated delay followed by
+ * slayer_spike_bwd_f32.  Any T.
+ */
+int slayer_spike_bwd_delayed_f32(float *gradIn, const float *gradOut, const float *u,
+                                 const float *delayLut, int64_t lutSize, float delay, float delayTs,
+                                 int64_t nNeurons, int64_t T, float theta, float tau, float scale,
+                                 void *stream);
+
 /* Bytes of caller-provided device workspace that slayer_delay_grad_f32 needs (may be 0). */
 int64_t slayer_delay_grad_workspace_bytes(int64_t nBatch, int64_t nPerBatch, int64_t T);
 

@@ -160,11 +160,23 @@ constexpr int kTileMaxPiece = 352;  // longest piece (samples per row) a tile st
 // placed into (gathered from) LDS one by one.  kTileScalar: anything else, one sample per access.
 constexpr int kTileScalar = 0, kTileVec = 1, kTileFlat = 2;
 
+// Optional time shift of the spike output (the delayShift that follows spike() in networks with
+// axonal delays, fused into the store of the spikes): s[t] = spike[t - k], k = (int)(delay / Ts),
+// with one delay for all rows or one per neuron of a batch item (row % lutSize).  The membrane
+// potential is not shifted.  Only tiles whose rows travel whole support it.
+struct SpikeDelay {
+    const float *lut;   // per-neuron delays, or NULL
+    int64_t lutSize;    // neurons per batch item when lut is given
+    float delay;        // the one delay when lut is NULL
+    float Ts;
+    int on;
+};
+
 template <int NU, int MODE, int LAG, int R>
 __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, float *u,
                                                         const float *__restrict__ nu, int64_t rows,
                                                         int T, int nuSize, int Tc, int P, int MP,
-                                                        int64_t tiles, float theta, float Ts)
+                                                        int64_t tiles, float theta, float Ts, SpikeDelay dl)
 {
     static_assert(LAG >= NU - 1 && LAG % 4 == 0, "the window must cover the refractory kernel");
     constexpr int G = 32;               // samples per walk group = bits of a spike mask
@@ -174,6 +186,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     extern __shared__ __align__(16) float lds[];
     float *tile = lds;                                                    // [R][P], P = 4 (mod 32)
     uint32_t *masks = reinterpret_cast<uint32_t *>(lds + R * P);  // [R][MP]
+    int *rowShift = reinterpret_cast<int *>(masks + R * MP);      // [R], used when the output is shifted
 
     const int lane = threadIdx.x;
     const float amplitude = 1.0f / Ts;
@@ -325,6 +338,24 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         {
             const BufferRsrc bufU = make_buffer(u + t * R * static_cast<int64_t>(T));
             const BufferRsrc bufS = make_buffer(s + t * R * static_cast<int64_t>(T));
+            if (dl.on) {  // whole rows only (the launcher sees to it): every row's shift in samples
+                if (lane < R) {
+                    const int64_t row = t * R + lane;
+                    const float d = dl.lut ? dl.lut[row < rows ? row % dl.lutSize : 0] : dl.delay;
+                    rowShift[lane] = delay_steps(d, dl.Ts);
+                }
+                wave_sync();
+            }
+            // the spike bit of the sample `shift` steps before column `col` (0 outside the row)
+            const int nCols = (MP - 1) << 5;
+            auto bits_from = [&](int r, int col) -> uint32_t {
+                const int c2 = col - rowShift[r];
+                if (c2 < 0 || c2 >= nCols) return 0u;
+                const int w = c2 >> 5, sh = c2 & 31;
+                uint32_t m = masks[r * MP + w] >> sh;
+                if (sh > 28 && w + 1 < MP - 1) m |= masks[r * MP + w + 1] << (32 - sh);
+                return m;
+            };
             if constexpr (FLAT) {
                 const int nVec = (nRows * T) >> 2;
                 for (int vi = lane; vi < nVec; vi += kWave) {
@@ -335,7 +366,8 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                     for (int e = 0; e < 4; ++e) {
                         const int col = LAG + c;   // time c of row r
                         uu[e] = tile[r * P + col];
-                        ss[e] = ((masks[r * MP + (col >> 5)] >> (col & 31)) & 1u) ? amplitude : 0.0f;
+                        const uint32_t bit = dl.on ? bits_from(r, col) : masks[r * MP + (col >> 5)] >> (col & 31);
+                        ss[e] = (bit & 1u) ? amplitude : 0.0f;
                         if (++c == T) { c = 0; ++r; }
                     }
                     buffer_store4(bufU, vi * 16, 0, make_float4(uu[0], uu[1], uu[2], uu[3]));
@@ -353,7 +385,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                 const int col = first + rc.c * V;
                 const int off = (rc.r * T + tW + col) * 4;
                 const float *src = tile + rc.r * P + col;
-                const uint32_t m = masks[rc.r * MP + (col >> 5)] >> (col & 31);
+                const uint32_t m = dl.on ? bits_from(rc.r, col) : masks[rc.r * MP + (col >> 5)] >> (col & 31);
                 if (VEC) {
                     buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(src));
                     buffer_store4(bufS, off, 0,
@@ -395,6 +427,40 @@ __global__ __launch_bounds__(256) void spike_bwd_vec_kernel(float *gradIn, const
     __builtin_nontemporal_store(o, reinterpret_cast<vec4f *>(gradIn) + i);
 }
 
+// The same gradient behind a shifted output: with s_out[t] = spike[t - k] the gradient that reaches
+// the spike at time t is gradOut[t + k].  One lane per VEC output samples; the row's shift comes from
+// the per-neuron table or the one delay, like in the forward pass.
+template <int VEC>
+__global__ __launch_bounds__(256) void spike_bwd_delayed_kernel(float *gradIn, const float *gradOut,
+                                                                const float *__restrict__ u, SpikeDelay dl,
+                                                                int T, FastDiv byTV, float theta, float tau,
+                                                                float gain, int64_t vectors)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= vectors) return;
+    // rows are addressed relative to the work-group's first row so that offsets stay 32 bit
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * 256;
+    const int64_t row0 = first / byTV.d;
+    const uint32_t local = static_cast<uint32_t>(i - row0 * byTV.d);
+    const uint32_t rl = fastdiv(local, byTV);
+    const int t = static_cast<int>(local - rl * byTV.d) * VEC;
+    const int64_t row = row0 + rl;
+    const int k = delay_steps(dl.lut ? dl.lut[row % dl.lutSize] : dl.delay, dl.Ts);
+    const BufferRsrc gB = make_buffer(gradOut + row0 * T);
+    const int rowBytes = static_cast<int>(rl) * T * 4;
+    float g[VEC], x[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        // t + k + e computed without overflow for any k
+        const int64_t src = static_cast<int64_t>(t) + k + e;
+        g[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+            gB, masked_offset(src >= 0 && src < T, rowBytes + static_cast<int>(src < T && src >= 0 ? src : 0) * 4), 0, 0));
+        x[e] = u[row * T + t + e];
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) gradIn[row * T + t + e] = g[e] * spike_pdf(x[e], theta, tau, gain);
+}
+
 __global__ __launch_bounds__(256) void spike_bwd_scalar_kernel(float *gradIn, const float *gradOut,
                                                                const float *__restrict__ u, float theta,
                                                                float tau, float gain, int64_t numel)
@@ -405,14 +471,13 @@ __global__ __launch_bounds__(256) void spike_bwd_scalar_kernel(float *gradIn, co
 
 }  // namespace slayer
 
-extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_t nNeurons,
-                                     int64_t T, int64_t nuSize, float theta, float Ts, void *stream)
+namespace slayer {
+
+// Picks and launches the spike kernel.  With a shift of the output (dl.on) only the tile kernel with
+// whole rows qualifies; other shapes return SLAYER_EUNSUPPORTED before anything is launched.
+static int launch_get_spikes(float *s, float *u, const float *nu, int64_t nNeurons, int64_t T, int64_t nuSize,
+                             float theta, float Ts, hipStream_t st, const SpikeDelay &dl)
 {
-    using namespace slayer;
-    if (nNeurons < 0 || T < 0 || nuSize < 0) return SLAYER_EINVAL;
-    if (nNeurons == 0 || T == 0) return SLAYER_OK;
-    if (!s || !u || (nuSize > 0 && !nu)) return SLAYER_EINVAL;
-    hipStream_t st = static_cast<hipStream_t>(stream);
 
     const int64_t groups = ceil_div(nNeurons, kWave);
     const bool stream_ok = !generic_forced() && T < (1LL << 30) && groups < (1LL << 31);
@@ -422,16 +487,16 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
         if (vec)                                                                                        \
             hipLaunchKernelGGL((spike_tile_kernel<NU, kTileVec, LAGV, RV>), dim3(grid), dim3(kWave),    \
                                lds, st, s, u, nu, nNeurons, static_cast<int>(T),                        \
-                               static_cast<int>(nuSize), Tc, P, MP, tiles, theta, Ts);                  \
+                               static_cast<int>(nuSize), Tc, P, MP, tiles, theta, Ts, dl);              \
         else if (flat && RV == 8)                                                                       \
             hipLaunchKernelGGL((spike_tile_kernel<NU, (RV == 8 ? kTileFlat : kTileScalar), LAGV, RV>),  \
                                dim3(grid), dim3(kWave), lds, st, s, u, nu, nNeurons,                    \
                                static_cast<int>(T), static_cast<int>(nuSize), Tc, P, MP, tiles, theta,  \
-                               Ts);                                                                     \
+                               Ts, dl);                                                                 \
         else                                                                                            \
             hipLaunchKernelGGL((spike_tile_kernel<NU, kTileScalar, LAGV, RV>), dim3(grid), dim3(kWave), \
                                lds, st, s, u, nu, nNeurons, static_cast<int>(T),                        \
-                               static_cast<int>(nuSize), Tc, P, MP, tiles, theta, Ts);                  \
+                               static_cast<int>(nuSize), Tc, P, MP, tiles, theta, Ts, dl);              \
         return launch_status();                                                                         \
     } while (0)
 #define SLAYER_SPIKE_TILE_LAG(NU, LAGV)                                                                  \
@@ -445,7 +510,7 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
            wavefront slots of the GPU empty. */                                                         \
         const int64_t slots16 = static_cast<int64_t>(cus) * (160 * 1024 / ((16LL * P + 16 * MP) * 4));  \
         const int rowsPerTile = (!whole && ceil_div(nNeurons, 16) >= slots16) ? 16 : 8;                 \
-        const size_t lds = (static_cast<size_t>(rowsPerTile) * P + rowsPerTile * MP) * sizeof(float);   \
+        const size_t lds = (static_cast<size_t>(rowsPerTile) * P + rowsPerTile * MP + rowsPerTile) * sizeof(float); \
         const int64_t tiles = ceil_div(nNeurons, rowsPerTile);                                          \
         const int64_t resident = static_cast<int64_t>(cus) * (160 * 1024 / static_cast<int64_t>(lds));  \
         if (tiles >= (1LL << 31)) return SLAYER_EUNSUPPORTED;                                           \
@@ -458,6 +523,7 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
         if (whole) SLAYER_SPIKE_TILE_LAG(NU, ((NU + 2) & ~3));                                          \
         SLAYER_SPIKE_TILE_LAG(NU, 32);                                                                  \
     } while (0)
+    if (dl.on && !(window_ok && nuSize <= 24 && T <= kTileMaxPiece)) return SLAYER_EUNSUPPORTED;
     if (window_ok && nuSize <= 24) {
         // short rows travel whole; long rows in pieces of 256 samples (1 KiB per row)
         const bool whole = T <= kTileMaxPiece;
@@ -494,6 +560,32 @@ extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_
     return launch_status();
 }
 
+}  // namespace slayer
+
+extern "C" int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_t nNeurons,
+                                     int64_t T, int64_t nuSize, float theta, float Ts, void *stream)
+{
+    using namespace slayer;
+    if (nNeurons < 0 || T < 0 || nuSize < 0) return SLAYER_EINVAL;
+    if (nNeurons == 0 || T == 0) return SLAYER_OK;
+    if (!s || !u || (nuSize > 0 && !nu)) return SLAYER_EINVAL;
+    return launch_get_spikes(s, u, nu, nNeurons, T, nuSize, theta, Ts, static_cast<hipStream_t>(stream),
+                             SpikeDelay{nullptr, 0, 0.0f, 1.0f, 0});
+}
+
+extern "C" int slayer_get_spikes_delayed_f32(float *s, float *u, const float *nu, const float *delayLut,
+                                             int64_t lutSize, float delay, float delayTs, int64_t nNeurons,
+                                             int64_t T, int64_t nuSize, float theta, float Ts, void *stream)
+{
+    using namespace slayer;
+    if (nNeurons < 0 || T < 0 || nuSize < 0 || lutSize < 0) return SLAYER_EINVAL;
+    if (delayLut && (lutSize == 0 || nNeurons % lutSize != 0)) return SLAYER_EINVAL;
+    if (nNeurons == 0 || T == 0) return SLAYER_OK;
+    if (!s || !u || (nuSize > 0 && !nu)) return SLAYER_EINVAL;
+    return launch_get_spikes(s, u, nu, nNeurons, T, nuSize, theta, Ts, static_cast<hipStream_t>(stream),
+                             SpikeDelay{delayLut, lutSize, delay, delayTs, 1});
+}
+
 extern "C" int slayer_spike_bwd_f32(float *gradIn, const float *gradOut, const float *u, float theta,
                                     float tau, float scale, int64_t numel, void *stream)
 {
@@ -513,5 +605,32 @@ extern "C" int slayer_spike_bwd_f32(float *gradIn, const float *gradOut, const f
     else
         hipLaunchKernelGGL(spike_bwd_scalar_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
                            gradIn, gradOut, u, theta, tau, gain, lanes);
+    return launch_status();
+}
+
+extern "C" int slayer_spike_bwd_delayed_f32(float *gradIn, const float *gradOut, const float *u,
+                                            const float *delayLut, int64_t lutSize, float delay, float delayTs,
+                                            int64_t nNeurons, int64_t T, float theta, float tau, float scale,
+                                            void *stream)
+{
+    using namespace slayer;
+    if (nNeurons < 0 || T < 0 || lutSize < 0) return SLAYER_EINVAL;
+    if (delayLut && (lutSize == 0 || nNeurons % lutSize != 0)) return SLAYER_EINVAL;
+    if (nNeurons == 0 || T == 0) return SLAYER_OK;
+    if (!gradIn || !gradOut || !u) return SLAYER_EINVAL;
+    if (T > kBufferMaxT) return SLAYER_EUNSUPPORTED;  // 256 vectors of a work-group must stay below 2 GiB
+    const SpikeDelay dl{delayLut, lutSize, delay, delayTs, 1};
+    const bool vec = T % 4 == 0;
+    const int64_t vectors = nNeurons * (vec ? T / 4 : T);
+    const int64_t blocks = ceil_div(vectors, 256);
+    if (blocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const FastDiv byTV = make_fastdiv(static_cast<uint32_t>(vec ? T / 4 : T));
+    if (vec)
+        hipLaunchKernelGGL(spike_bwd_delayed_kernel<4>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, gradIn,
+                           gradOut, u, dl, static_cast<int>(T), byTV, theta, tau, scale / tau, vectors);
+    else
+        hipLaunchKernelGGL(spike_bwd_delayed_kernel<1>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, gradIn,
+                           gradOut, u, dl, static_cast<int>(T), byTV, theta, tau, scale / tau, vectors);
     return launch_status();
 }

@@ -80,6 +80,22 @@ class spikeLayer(nn.Module):
         updated in place with the refractory response, as in the reference."""
         return _spikeFunction.apply(membranePotential, self.refKernel, self.neuron, self.simulation["Ts"])
 
+    def spikeDelayed(self, membranePotential, delay, Ts=None):
+        """``delayShift(spike(membranePotential), delay, Ts)`` or, with a ``_delayLayer`` as ``delay``,
+        ``delay(spike(membranePotential))`` (src/slayer.py:333-391) from one kernel: the spikes are
+        shifted while they are stored, and the backward pass shifts the gradient while it applies the
+        surrogate gradient.  A delay layer's delays receive their gradient as in the reference."""
+        Ts = self.simulation["Ts"] if Ts is None else Ts
+        if isinstance(delay, _delayLayer):
+            N, C, H, W, Ns = membranePotential.shape
+            table = delay.delay
+            if membranePotential.numel() != table.numel() * Ns * N:
+                table = table.repeat((1, H, W))
+            return _spikeDelayedFunction.apply(membranePotential, self.refKernel, self.neuron, self.simulation["Ts"],
+                                               table, delay.Ts)
+        return _spikeDelayedFunction.apply(membranePotential, self.refKernel, self.neuron, self.simulation["Ts"],
+                                           delay, Ts)
+
     def pspSpike(self, input):
         """``spike(psp(input))`` - the layer ordering of the reference's MLP example
         (example/02_NMNIST_MLP/nmnistMLP.py:59-60) - as one forward and one backward kernel
@@ -300,6 +316,41 @@ class _spikeFunction(torch.autograd.Function):
         gradInput = slayerCuda.spikeBackward(gradOutput.contiguous(), membranePotential.contiguous(),
                                              ctx.theta, ctx.pdfTimeConstant, ctx.pdfScale)
         return gradInput, None, None, None
+
+
+class _spikeDelayedFunction(torch.autograd.Function):
+    """``_spikeFunction`` followed by ``_delayFunction`` / ``_delayFunctionNoGradient``
+    (src/slayer.py:817-865, 930-979) as one Function over ``slayerCuda.getSpikesDelayed`` and
+    ``slayerCuda.spikeBackwardDelayed``.  ``delay`` is a number or a tensor; a tensor that requires
+    grad gets the delay gradient of ``_delayFunction.backward``."""
+
+    @staticmethod
+    def forward(ctx, membranePotential, refractoryResponse, neuron, Ts, delay, delayTs):
+        theta = neuron["theta"]
+        table = delay.detach().to(device=membranePotential.device, dtype=membranePotential.dtype).contiguous() \
+            if isinstance(delay, torch.Tensor) else delay
+        spikes = slayerCuda.getSpikesDelayed(membranePotential.contiguous(), refractoryResponse, theta, Ts, table,
+                                             delayTs)
+        ctx.learn = isinstance(delay, torch.Tensor) and delay.requires_grad
+        ctx.save_for_backward(membranePotential, *((spikes,) if ctx.learn else ()))
+        ctx.delay = table
+        ctx.delayShape = tuple(delay.shape) if isinstance(delay, torch.Tensor) else None
+        ctx.delayTs = float(delayTs)
+        ctx.theta = float(theta)
+        ctx.pdfTimeConstant = float(neuron["tauRho"] * neuron["theta"])
+        ctx.pdfScale = float(neuron["scaleRho"])
+        return spikes
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        membranePotential = ctx.saved_tensors[0]
+        gradOutput = gradOutput.contiguous()
+        gradDelay = None
+        if ctx.learn:
+            gradDelay = slayerCuda.delayGrad(ctx.saved_tensors[1], gradOutput, ctx.delayTs).reshape(ctx.delayShape)
+        gradInput = slayerCuda.spikeBackwardDelayed(gradOutput, membranePotential.contiguous(), ctx.theta,
+                                                    ctx.pdfTimeConstant, ctx.pdfScale, ctx.delay, ctx.delayTs)
+        return gradInput, None, None, None, gradDelay, None
 
 
 class _pspSpikeFunction(torch.autograd.Function):

@@ -17,11 +17,12 @@ Python numbers or 0-dim tensors, as with pybind11's float conversion.  Outputs a
 with ``torch.empty_like``; kernels are enqueued on PyTorch's current stream of the tensor's
 device and never synchronise with the host.
 
-``spikeBackward``, ``spikeBackwardCorr``, ``pspSpike``, ``delayGrad`` and the ``sign`` argument
+``spikeBackward``, ``spikeBackwardCorr``, ``pspSpike``, ``getSpikesDelayed``, ``spikeBackwardDelayed``,
+``delayGrad`` and the ``sign`` argument
 of ``shift`` have no counterpart in the reference extension: they are the fused forms of the
 elementwise chains in ``_spikeFunction.backward`` / ``_delayFunction.backward``
 (src/slayer.py:857-865, 944-957), of ``slayerLoihi._spike.backward`` (src/slayerLoihi.py:278-283)
-and of the call pair ``spike(psp(x))``.
+and of the call pairs ``spike(psp(x))`` and ``delayShift(spike(u), d)``.
 """
 import numbers
 
@@ -29,7 +30,8 @@ import torch
 
 from . import _lib
 
-__all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "spikeBackwardCorr", "pspSpike", "delayGrad"]
+__all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "spikeBackwardCorr", "pspSpike", "delayGrad",
+           "getSpikesDelayed", "spikeBackwardDelayed"]
 
 
 def _check_input(x, name):
@@ -185,6 +187,66 @@ def shift(input, shiftLUT, Ts=1.0, sign=1.0):
         _lib.check(lib.slayer_shift_f32(_ptr(output), _ptr(input), delay * sign, n, T, Ts, stream),
                    "slayer_shift_f32")
     return output
+
+
+def _delay_args(delay, x, n):
+    """(table pointer, table size, scalar delay) of a delay given as a number, a one-element tensor
+    or a tensor with one entry per neuron of a batch item."""
+    if isinstance(delay, torch.Tensor):
+        _check_input(delay, "delay")
+        _check_device(x, delay, "input", "delay")
+        if delay.numel() != 1:
+            nBatch = x.shape[0]
+            if nBatch == 0 or delay.numel() != n // nBatch:
+                raise RuntimeError("shift and number of neurons must be same")
+        return _ptr(delay), delay.numel(), 0.0
+    return None, 0, _scalar(delay, "delay")
+
+
+def getSpikesDelayed(d_u, d_nu, theta, Ts, delay, delayTs=1.0):
+    """``shift(getSpikes(d_u, d_nu, theta, Ts), delay, delayTs)`` with the shift done while the spikes
+    are stored (``d_u`` is updated in place and not shifted).  ``delay`` as in :func:`shift`.  Shapes
+    the fused kernel does not serve run the two kernels."""
+    _check_input(d_u, "d_u")
+    _check_input(d_nu, "d_nu")
+    _check_device(d_u, d_nu, "d_u", "d_nu")
+    if d_u.dim() != 5:
+        raise RuntimeError("getSpikesDelayed expects a 5 dimensional (N,C,H,W,T) tensor, got %d dimensions"
+                           % d_u.dim())
+    theta, Ts, delayTs = _scalar(theta, "theta"), _scalar(Ts, "Ts"), _scalar(delayTs, "delayTs")
+    n, T = _rows(d_u)
+    lut, lutSize, scalar = _delay_args(delay, d_u, n)
+    lib = _lib.load()
+    d_s = torch.empty_like(d_u)
+    nuSize = d_nu.shape[-1] if d_nu.dim() else 1
+    with _on_device_of(d_u) as stream:
+        status = lib.slayer_get_spikes_delayed_f32(_ptr(d_s), _ptr(d_u), _ptr(d_nu), lut, lutSize, scalar, delayTs,
+                                                   n, T, nuSize, theta, Ts, stream)
+    if status == 2:      # not a shape of the fused kernel; nothing was launched
+        return shift(getSpikes(d_u, d_nu, theta, Ts), delay, delayTs)
+    _lib.check(status, "slayer_get_spikes_delayed_f32")
+    return d_s
+
+
+def spikeBackwardDelayed(gradOutput, membranePotential, theta, tau, scale, delay, delayTs=1.0):
+    """``spikeBackward(shift(gradOutput, delay, delayTs, sign=-1), membranePotential, ...)`` in one
+    pass: the backward of :func:`getSpikesDelayed` with respect to the membrane potential."""
+    _check_input(gradOutput, "gradOutput")
+    _check_input(membranePotential, "membranePotential")
+    _check_device(gradOutput, membranePotential, "gradOutput", "membranePotential")
+    if gradOutput.shape != membranePotential.shape:
+        raise RuntimeError("gradOutput and membranePotential must have the same shape")
+    theta, tau, scale = _scalar(theta, "theta"), _scalar(tau, "tau"), _scalar(scale, "scale")
+    delayTs = _scalar(delayTs, "delayTs")
+    n, T = _rows(gradOutput)
+    lut, lutSize, scalar = _delay_args(delay, gradOutput, n)
+    lib = _lib.load()
+    gradInput = torch.empty_like(gradOutput)
+    with _on_device_of(gradOutput) as stream:
+        _lib.check(lib.slayer_spike_bwd_delayed_f32(_ptr(gradInput), _ptr(gradOutput), _ptr(membranePotential), lut,
+                                                    lutSize, scalar, delayTs, n, T, theta, tau, scale, stream),
+                   "slayer_spike_bwd_delayed_f32")
+    return gradInput
 
 
 def spikeBackward(gradOutput, membranePotential, theta, tau, scale):

@@ -432,3 +432,48 @@ def test_empty_tensors():
     assert slayerCuda.getSpikes(z, f, 1.0, 1.0).shape == z.shape
     assert host(slayerCuda.delayGrad(z, z, 1.0)).tolist() == [[[0.0]]] * 3
     torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------ spike with the shift fused in
+@pytest.mark.parametrize("shape", [(3, 5, 4, 4, 300), (2, 3, 2, 2, 352), (2, 7, 1, 1, 100), (2, 3, 1, 1, 7),
+                                   (4, 3, 2, 2, 350), (1, 9, 1, 1, 33), (2, 4, 1, 1, 2000)])
+@pytest.mark.parametrize("delay", ["scalar", "negative", "zero", "huge", "table", "one-element"])
+def test_spike_delayed_equals_spike_then_shift(shape, delay, impl):
+    """getSpikesDelayed against the two kernels it fuses (both already pinned to the oracle), and
+    against the oracle itself: bit-exact, membrane potential included.  (2, 4, 1, 1, 2000) and the
+    generic kernels are shapes the fused kernel declines: the wrapper then runs the two kernels.)"""
+    rng = np.random.default_rng(31)
+    Ts, dTs = 1.0, 0.5
+    u = (rng.standard_normal(shape) * 6 + 4).astype(np.float32)
+    nu = np.array(alphaKernel(1.0, Ts, shape[-1], mult=-20.0), dtype=np.float32)
+    d = {"scalar": 3.4, "negative": -2.6, "zero": 0.0, "huge": 1e9,
+         "table": (rng.random(shape[1:4]) * 12 - 2).astype(np.float32),
+         "one-element": np.array([5.0], dtype=np.float32)}[delay]
+    dd = dev(d) if isinstance(d, np.ndarray) else d
+    ua, ub = dev(u), dev(u)
+    got = slayerCuda.getSpikesDelayed(ua, dev(nu), 10.0, Ts, dd, dTs)
+    ref = slayerCuda.shift(slayerCuda.getSpikes(ub, dev(nu), 10.0, Ts), dd, dTs)
+    assert np.array_equal(bits(host(got)), bits(host(ref)))
+    assert np.array_equal(bits(host(ua)), bits(host(ub)))
+    s_ref, u_ref = O.get_spikes(u, nu, 10.0, Ts)
+    assert np.array_equal(bits(host(got)), bits(O.shift(s_ref, d, dTs)))
+    assert np.array_equal(bits(host(ua)), bits(u_ref))
+    assert s_ref.sum() > 0
+
+
+@pytest.mark.parametrize("shape", [(3, 5, 4, 4, 300), (2, 3, 1, 1, 7), (4, 3, 2, 2, 350), (2, 4, 1, 1, 2000)])
+@pytest.mark.parametrize("delay", ["scalar", "negative", "huge", "table"])
+def test_spike_backward_delayed_equals_shift_then_spike_backward(shape, delay):
+    rng = np.random.default_rng(32)
+    dTs = 0.5
+    u = (rng.standard_normal(shape) * 6 + 4).astype(np.float32)
+    g = rng.standard_normal(shape).astype(np.float32)
+    d = {"scalar": 3.4, "negative": -2.6, "huge": 1e9,
+         "table": (rng.random(shape[1:4]) * 12 - 2).astype(np.float32)}[delay]
+    dd = dev(d) if isinstance(d, np.ndarray) else d
+    got = slayerCuda.spikeBackwardDelayed(dev(g), dev(u), 10.0, 10.0, 1.0, dd, dTs)
+    ref = slayerCuda.spikeBackward(slayerCuda.shift(dev(g), dd, dTs, sign=-1.0), dev(u), 10.0, 10.0, 1.0)
+    assert np.array_equal(bits(host(got)), bits(host(ref)))
+    neg = -d if isinstance(d, np.ndarray) else -d
+    want = O.spike_bwd(O.shift(g, neg, dTs), u, 10.0, 10.0, 1.0)
+    assert rel_err(host(got), want) <= REL_TOL

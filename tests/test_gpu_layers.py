@@ -532,3 +532,36 @@ def test_loihi_cnn_inference_is_bit_exact():
             s = layer.spikeLoihi(m(s), delay=1)
             assert np.array_equal(s.cpu().numpy(), ref), "layer %d" % k
     assert ref.sum() > 0
+
+
+@pytest.mark.parametrize("learnable", [True, False])
+def test_spike_delayed_layer_matches_spike_then_delay(learnable):
+    """spikeLayer.spikeDelayed against delay(spike(u)) / delayShift(spike(u), d): same spikes, same
+    gradient with respect to the membrane potential and, for a delay layer, the delays."""
+    params = {"type": "SRMALPHA", "theta": 10, "tauSr": 2.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
+    layer = snn.layer(params, {"Ts": 1.0, "tSample": 120}).cuda()
+    torch.manual_seed(4)
+    u0 = (torch.randn((3, 6, 2, 2, 120)) * 6 + 4).cuda()
+    g = torch.randn_like(u0)
+    if learnable:
+        dl = layer.delay((6, 2, 2)).cuda()
+        with torch.no_grad():
+            dl.delay.mul_(9.0)
+        dl2 = layer.delay((6, 2, 2)).cuda()
+        with torch.no_grad():
+            dl2.delay.copy_(dl.delay)
+    ua = u0.clone().requires_grad_(True)
+    ub = u0.clone().requires_grad_(True)
+    # the spike function updates its input in place: give each path its own copy inside the graph
+    if learnable:
+        sa = dl(layer.spike(ua * 1.0))
+        sb = layer.spikeDelayed(ub * 1.0, dl2)
+    else:
+        sa = layer.delayShift(layer.spike(ua * 1.0), 4.0, 1.0)
+        sb = layer.spikeDelayed(ub * 1.0, 4.0, 1.0)
+    assert torch.equal(sa, sb) and float(sa.sum()) > 0
+    sa.backward(g)
+    sb.backward(g)
+    assert torch.equal(ua.grad, ub.grad)
+    if learnable:
+        assert torch.equal(dl.delay.grad, dl2.delay.grad) and float(dl.delay.grad.abs().sum()) > 0
