@@ -186,6 +186,10 @@ def test_synapse_and_event_wrappers_need_the_gpu():
     from slayerpytorch_amd import synapse
     x, w = torch.zeros((1, 2, 5, 5, 4)), torch.zeros((3, 2, 3, 3))
     with pytest.raises(RuntimeError):
+        slayerCuda.getSpikesDelayed(torch.zeros((1, 2, 1, 1, 8)), torch.zeros(3), 10.0, 1.0, 2.0)
+    with pytest.raises(RuntimeError):
+        slayerCuda.spikeBackwardDelayed(torch.zeros((1, 2, 1, 1, 8)), torch.zeros((1, 2, 1, 1, 8)), 10.0, 10.0, 1.0, 2.0)
+    with pytest.raises(RuntimeError):
         synapse.conv(x, w)
     with pytest.raises(RuntimeError):
         synapse.convGradInput(torch.zeros((1, 3, 3, 3, 4)), w, x.shape)
