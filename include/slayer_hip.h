@@ -16,7 +16,8 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only
  *     enqueue work: no allocation, no free, no host synchronisation, no global state.
  *   - The library never allocates device memory.  Outputs (and the workspaces of
- *     slayer_delay_grad_f32 and slayer_synapse_conv_grad_weight_f32) are allocated by the caller.
+ *     slayer_delay_grad_f32, slayer_synapse_conv_grad_weight_f32 and slayer_spike_loss_f32) are allocated by
+ *     the caller.
  *   - Return value: SLAYER_OK (0) or one of the SLAYER_E* codes; nothing has been launched
  *     when a SLAYER_EINVAL / SLAYER_EUNSUPPORTED code is returned.  Empty tensors
  *     (nNeurons == 0 or T == 0) are a successful no-op.
@@ -329,6 +330,21 @@ int slayer_bin_events_f32(float *tensor, const float *base, const int32_t *x, co
                           const int32_t *p, const double *tMs, int64_t nEvents, int64_t timeShift,
                           int32_t C, int32_t H, int32_t W, int32_t T, double samplingTime,
                           int32_t mode, void *stream);
+
+/*
+ * ---- Spike-train loss ---------------------------------------------------------------------------
+ * error = psp(out - desired) [+ addend], loss = 1/2 * sum(error^2) * Ts in two launches.
+ * Replaces the tensor expressions of spikeLoss.spikeTime (src/spikeLoss.py:56-58) and of the last
+ * two statements of spikeLoss.numSpikes (src/spikeLoss.py:100-104, where `addend` is the spike count
+ * error inside the target region).  out, desired, error and the optional addend are [rows][T]; psp
+ * is the causal filter of slayer_conv_f32 with the same arithmetic; `loss` is one float.  The sum
+ * has a fixed association (deterministic).  `workspace` holds slayer_spike_loss_workspace_bytes(rows)
+ * bytes.  Rows whose T + 2 F floats exceed 60 KB return SLAYER_EUNSUPPORTED (nothing launched).
+ */
+int64_t slayer_spike_loss_workspace_bytes(int64_t rows);
+int slayer_spike_loss_f32(float *loss, float *error, const float *out, const float *desired,
+                          const float *addend, const float *srm, float *workspace, int64_t rows,
+                          int64_t T, int64_t F, float Ts, void *stream);
 
 #ifdef __cplusplus
 }

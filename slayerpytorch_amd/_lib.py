@@ -57,6 +57,9 @@ SIGNATURES = {
                                                     _i32, ctypes.c_double, _i32, _stream]),
     "slayer_bin_events_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _i64, _i64, _i32, _i32, _i32,
                                              _i32, ctypes.c_double, _i32, _stream]),
+    "slayer_spike_loss_workspace_bytes": (_i64, [_i64]),
+    "slayer_spike_loss_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _i64, _i64, _i64, _f32,
+                                             _stream]),
     "slayer_synapse_out_shape": (ctypes.c_int, [_geomp, _i32p, _i32p]),
     "slayer_synapse_conv_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _geomp, _stream]),
     "slayer_synapse_conv_grad_input_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _geomp, _stream]),

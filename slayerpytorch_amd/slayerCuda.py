@@ -31,7 +31,7 @@ import torch
 from . import _lib
 
 __all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "spikeBackwardCorr", "pspSpike", "delayGrad",
-           "getSpikesDelayed", "spikeBackwardDelayed"]
+           "getSpikesDelayed", "spikeBackwardDelayed", "spikeLoss"]
 
 
 def _check_input(x, name):
@@ -338,3 +338,35 @@ def delayGrad(output, gradOutput, Ts):
                                              workspace.data_ptr(), nBatch, nPerBatch, T, Ts, stream),
                    "slayer_delay_grad_f32")
     return gradDelay
+
+
+def spikeLoss(spikeOut, spikeDesired, srmKernel, Ts, addend=None):
+    """``error = conv(spikeOut - spikeDesired, srmKernel, Ts) [+ addend]`` and
+    ``loss = 1/2 * sum(error**2) * Ts`` in two launches.  Returns ``(loss, error)`` (``loss`` is a
+    0-dim tensor), or ``None`` when a row does not fit the kernel (nothing was launched)."""
+    _check_input(spikeOut, "spikeOut")
+    _check_input(spikeDesired, "spikeDesired")
+    _check_input(srmKernel, "srmKernel")
+    _check_device(spikeOut, spikeDesired, "spikeOut", "spikeDesired")
+    _check_device(spikeOut, srmKernel, "spikeOut", "srmKernel")
+    if spikeOut.shape != spikeDesired.shape:
+        raise RuntimeError("spikeOut and spikeDesired must have the same shape")
+    if addend is not None:
+        _check_input(addend, "addend")
+        _check_device(spikeOut, addend, "spikeOut", "addend")
+        if addend.shape != spikeOut.shape:
+            raise RuntimeError("addend and spikeOut must have the same shape")
+    Ts = _scalar(Ts, "Ts")
+    lib = _lib.load()
+    rows, T = _rows(spikeOut)
+    loss = torch.empty((), dtype=spikeOut.dtype, device=spikeOut.device)
+    error = torch.empty_like(spikeOut)
+    workspace = torch.empty((max(rows, 1),), dtype=torch.float32, device=spikeOut.device)
+    with _on_device_of(spikeOut) as stream:
+        status = lib.slayer_spike_loss_f32(loss.data_ptr(), _ptr(error), _ptr(spikeOut), _ptr(spikeDesired),
+                                           _ptr(addend) if addend is not None else None, _ptr(srmKernel),
+                                           workspace.data_ptr(), rows, T, srmKernel.numel(), Ts, stream)
+    if status == 2:
+        return None
+    _lib.check(status, "slayer_spike_loss_f32")
+    return loss, error

@@ -1,6 +1,8 @@
 """Spike-train losses on top of the PSP kernel (src/spikeLoss.py:7-104), computed on the device.
 
-``spikeTime``: half the squared van Rossum distance between output and desired spike trains.
+``spikeTime``: half the squared van Rossum distance between output and desired spike trains, from the
+fused error + squared-sum kernels of ``slayerCuda.spikeLoss`` (rows too long for them take the tensor
+expression of the reference).
 ``numSpikes``: spike count inside a target region against a desired count, spike-time loss
 outside it.  The reference builds the target region, the desired counts and the count error on
 the host (numpy round trips, src/spikeLoss.py:91-102); here every step is a tensor operation on
@@ -8,7 +10,35 @@ the device of ``spikeOut``, so the loss never synchronises with the host.
 """
 import torch
 
+from . import slayerCuda
 from .slayer import spikeLayer
+
+
+class _spikeLossFunction(torch.autograd.Function):
+    """``1/2 * sum((psp(out - desired) + addend)**2) * Ts`` over ``slayerCuda.spikeLoss``; the backward
+    pass is the correlation of the saved error signal, as autograd derives it for the reference's
+    expression (src/spikeLoss.py:56-58)."""
+
+    @staticmethod
+    def forward(ctx, spikeOut, spikeDesired, addend, srmKernel, Ts):
+        result = slayerCuda.spikeLoss(spikeOut.contiguous(), spikeDesired.contiguous(), srmKernel, Ts,
+                                      None if addend is None else addend.contiguous())
+        loss, error = result
+        ctx.save_for_backward(error, srmKernel)
+        ctx.Ts = float(Ts)
+        return loss
+
+    @staticmethod
+    def backward(ctx, gradLoss):
+        error, srmKernel = ctx.saved_tensors
+        grad = slayerCuda.corr(error * (gradLoss * ctx.Ts), srmKernel, ctx.Ts)
+        return (grad if ctx.needs_input_grad[0] else None, -grad if ctx.needs_input_grad[1] else None,
+                None, None, None)
+
+
+def _fits(spike, srmKernel):
+    # the fused loss keeps one row and the filter in the LDS of a work-group
+    return spike.is_cuda and spike.dtype == torch.float32 and (spike.shape[-1] + 2 * srmKernel.numel()) * 4 <= 60 * 1024
 
 
 class spikeLoss(torch.nn.Module):
@@ -26,8 +56,11 @@ class spikeLoss(torch.nn.Module):
     def spikeTime(self, spikeOut, spikeDesired):
         """``1/2 * sum(psp(spikeOut - spikeDesired)^2) * Ts`` (src/spikeLoss.py:37-58)."""
         assert self.errorDescriptor["type"] == "SpikeTime", "Error type is not SpikeTime"
+        Ts = self.simulation["Ts"]
+        if _fits(spikeOut, self.slayer.srmKernel):
+            return _spikeLossFunction.apply(spikeOut, spikeDesired, None, self.slayer.srmKernel, Ts)
         error = self.slayer.psp(spikeOut - spikeDesired)
-        return 1 / 2 * torch.sum(error ** 2) * self.simulation["Ts"]
+        return 1 / 2 * torch.sum(error ** 2) * Ts
 
     def numSpikes(self, spikeOut, desiredClass, numSpikesScale=1):
         """Spike-count loss (src/spikeLoss.py:60-104).  ``desiredClass`` is one-hot with a time
@@ -52,6 +85,8 @@ class spikeLoss(torch.nn.Module):
             errorSpikeCount = (actualSpikes.double() - desiredSpikes) / (stopID - startID) * numSpikesScale
             spikeDesired = out * inRegion                 # the output's own spikes inside the region
             countError = (errorSpikeCount * inRegion.double()).to(out.dtype)
+        if _fits(spikeOut, self.slayer.srmKernel):
+            return _spikeLossFunction.apply(spikeOut, spikeDesired, countError, self.slayer.srmKernel, Ts)
         error = self.slayer.psp(spikeOut - spikeDesired)
         error = error + countError
         return 1 / 2 * torch.sum(error ** 2) * Ts

@@ -620,3 +620,28 @@ def test_training_step_replayed_from_a_hip_graph():
         again = eager()                      # the program's own eager work between replays
         for a, b in zip(again, ref):
             assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("Ts,T,shape", [(1.0, 300, (4, 10, 1, 1)), (0.5, 128, (2, 3, 2, 2)), (1.0, 20000, (1, 2, 1, 1))])
+def test_spike_time_loss_kernel_matches_tensor_expression(Ts, T, shape):
+    """The fused loss (error signal + squared sum in two launches) against the reference's expression
+    1/2 * sum(psp(out - desired)^2) * Ts evaluated with torch ops on the same psp kernel: the loss to
+    rounding of the sum, the gradient bit for bit (the error signal is the same arithmetic).  T = 20000
+    does not fit the fused kernel and takes the tensor expression."""
+    params = {"type": "SRMALPHA", "theta": 10, "tauSr": 5.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
+    sim = {"Ts": Ts, "tSample": int(T * Ts)}
+    error = snn.loss({"neuron": params, "simulation": sim, "training": {"error": {"type": "SpikeTime"}}}).cuda()
+    torch.manual_seed(5)
+    out = ((torch.rand(shape + (T,)) < 0.05).float() / Ts).cuda().requires_grad_(True)
+    des = ((torch.rand(shape + (T,)) < 0.05).float() / Ts).cuda()
+    loss = error.spikeTime(out, des)
+    loss.backward()
+    out2 = out.detach().clone().requires_grad_(True)
+    e = error.slayer.psp(out2 - des)
+    ref = 1 / 2 * torch.sum(e ** 2) * Ts
+    ref.backward()
+    assert abs(float(loss) - float(ref)) <= 1e-5 * abs(float(ref)) and float(ref) > 0
+    assert torch.equal(out.grad, out2.grad)
+    # against the oracle's psp
+    eo = O.conv((out.detach() - des).cpu().numpy(), error.slayer.srmKernel.cpu().numpy(), Ts)
+    assert abs(float(loss) - 0.5 * float((eo.astype(np.float64) ** 2).sum()) * Ts) <= 1e-5 * abs(float(ref))
