@@ -664,8 +664,8 @@ static WgradPlan plan_wgrad(const SynGeom &s, bool vec)
 }
 
 
-// Tiling of the matrix-core weight gradient: MT x NT tiles of 16 x 16 per wavefront (at most 24
-// tiles = 96 accumulator registers), slices of pixels so that the GPU sees a few thousand wavefronts.
+// Tiling of the matrix-core weight gradient: MT x NT tiles of 16 x 16 per wavefront (at most 18
+// tiles = 72 accumulator registers), slices of pixels so that the GPU sees a few thousand wavefronts.
 struct MfmaPlan {
     bool use;
     int MT, NT, oGroups, colGroups, slices, pixPerSlice;
@@ -680,8 +680,10 @@ static MfmaPlan plan_wgrad_mfma(const SynGeom &s)
     p.use = s.T % 4 == 0 && s.T >= 16 && Og >= 8 && CK >= 8 && pixels > 0 && s.N > 0;
     if (!p.use) return p;
     const int oTiles = static_cast<int>(ceil_div(Og, 16)), cTiles = static_cast<int>(ceil_div(CK, 16));
-    p.MT = oTiles >= 4 ? 4 : oTiles >= 2 ? 2 : 1;
-    const int ntMax = 24 / p.MT > 9 ? 9 : 24 / p.MT;  // 9, 9 or 6
+    // two tiles of output channels at most: 4 x 6 tiles (one wavefront per SIMD) measured 132 us on
+    // 64 channels x 288 columns, 2 x 9 tiles (two per SIMD, fewer operand loads per tile) 111 us
+    p.MT = oTiles >= 2 ? 2 : 1;
+    const int ntMax = 9;
     const int options[5] = {1, 2, 4, 6, 9};
     p.NT = 1;
     for (int k = 0; k < 5; ++k)
@@ -713,9 +715,7 @@ template <int MT>
 static void launch_wgrad_mfma_nt(const WgradMfmaArgs &g, int NT, unsigned blocks, hipStream_t st)
 {
     switch (NT) {
-        case 9:
-            if constexpr (MT <= 2) { hipLaunchKernelGGL((synapse_wgrad_mfma_kernel<MT, 9>), dim3(blocks), dim3(256), 0, st, g); break; }
-            [[fallthrough]];
+        case 9: hipLaunchKernelGGL((synapse_wgrad_mfma_kernel<MT, 9>), dim3(blocks), dim3(256), 0, st, g); break;
         case 6: hipLaunchKernelGGL((synapse_wgrad_mfma_kernel<MT, 6>), dim3(blocks), dim3(256), 0, st, g); break;
         case 4: hipLaunchKernelGGL((synapse_wgrad_mfma_kernel<MT, 4>), dim3(blocks), dim3(256), 0, st, g); break;
         case 2: hipLaunchKernelGGL((synapse_wgrad_mfma_kernel<MT, 2>), dim3(blocks), dim3(256), 0, st, g); break;
@@ -742,8 +742,7 @@ static int launch_wgrad_mfma(const float *gradOut, const float *in, float *works
     const int64_t blocks = static_cast<int64_t>(s.N) * s.groups * p.oGroups * p.colGroups * p.slices;
     if (blocks >= (1LL << 31)) return -SLAYER_EUNSUPPORTED;
     const unsigned nb = static_cast<unsigned>(blocks);
-    if (p.MT == 4) launch_wgrad_mfma_nt<4>(g, p.NT, nb, st);
-    else if (p.MT == 2) launch_wgrad_mfma_nt<2>(g, p.NT, nb, st);
+    if (p.MT == 2) launch_wgrad_mfma_nt<2>(g, p.NT, nb, st);
     else launch_wgrad_mfma_nt<1>(g, p.NT, nb, st);
     const int status = launch_status();
     return status == SLAYER_OK ? s.N * p.slices : -status;
