@@ -129,6 +129,28 @@ def flip_rate(device, srm_t, ref_t, params):
     return float((s_gpu != s_cpu).mean()), float((s_cpu != 0).mean())
 
 
+def layer_flip_rate(device, srm_t, ref_t, params):
+    """Part of the CPU leg.  The same for a whole layer of the NMNIST CNN: spike(conv 2->16 5x5 (psp(x))) on
+    (4, 2, 34, 34, 300) input spikes, the GPU chain (event-driven psp, fp32 synapse kernel, spike kernel)
+    against the CPU oracle chain (separately rounded psp, synapse accumulated in double, spike loop)."""
+    from oracle import oracle as O
+    from slayerpytorch_amd import slayerCuda, synapse
+    rng = np.random.default_rng(1)
+    x = (rng.random((4, 2, 34, 34, 300)) < 0.02).astype(np.float32)
+    w = (rng.standard_normal((16, 2, 5, 5)) * 1.5).astype(np.float32)     # about 3 % of the output samples spike
+    a = slayerCuda.conv(torch.from_numpy(x).to(device), srm_t, 1.0)
+    u = synapse.conv(a, torch.from_numpy(w).to(device), 1, 1)
+    s_gpu = slayerCuda.getSpikes(u, ref_t, params["theta"], 1.0).cpu().numpy()
+    threads = O.lib().oracle_get_threads()
+    O.set_threads(O.max_threads())
+    try:
+        u_cpu = O.synapse_conv(O.conv(x, srm_t.cpu().numpy(), 1.0, fused=False), w, 1, 1)
+        s_cpu, _ = O.get_spikes(u_cpu, ref_t.cpu().numpy(), params["theta"], 1.0)
+    finally:
+        O.set_threads(threads)
+    return float((s_gpu != s_cpu).mean()), float((s_cpu != 0).mean())
+
+
 def mlp_row(device, timed):
     """One training step (without the optimiser) of the 2312-512-10 MLP on (12, 2, 34, 34, 350) input
     spikes at p = 0.015, layer ordering spike(psp(fc(x))), spike-time loss against a random target
@@ -639,6 +661,9 @@ def main():
             flips, rate = flip_rate(device, srm_t, ref_t, params)
             result["spike_flip_rate"] = flips
             result["spike_rate"] = rate
+            lflips, lrate = layer_flip_rate(device, srm_t, ref_t, params)
+            result["cnn_layer_spike_flip_rate"] = lflips
+            result["cnn_layer_spike_rate"] = lrate
     print(json.dumps(result))
 
 
