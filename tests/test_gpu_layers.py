@@ -645,3 +645,35 @@ def test_spike_time_loss_kernel_matches_tensor_expression(Ts, T, shape):
     # against the oracle's psp
     eo = O.conv((out.detach() - des).cpu().numpy(), error.slayer.srmKernel.cpu().numpy(), Ts)
     assert abs(float(loss) - 0.5 * float((eo.astype(np.float64) ** 2).sum()) * Ts) <= 1e-5 * abs(float(ref))
+
+
+def test_cpu_plumbing_configuration():
+    """The reference's CPU-runnable case: Bernoulli(0.02) spikes (4, 2, 34, 34, 300), dense 2312 -> 512 as a
+    conv3d with N(0,1) weights, a pspLayer-style conv3d PSP (left-padded, flipped SRM kernel, tauSr = 10) on the
+    CPU with torch, threshold / refractory spikes by the oracle - against dense -> psp -> spike of this package on
+    the GPU.  The membrane potentials agree to fp32 rounding; spikes may flip only where the potential sits
+    within that rounding of the threshold."""
+    params = {"type": "SRMALPHA", "theta": 10, "tauSr": 10.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
+    layer = snn.layer(params, {"Ts": 1.0, "tSample": 300})
+    torch.manual_seed(0)
+    x = (torch.rand((4, 2, 34, 34, 300)) < 0.02).float()
+    fc = layer.dense((34, 34, 2), 512)
+    with torch.no_grad():
+        fc.weight.copy_(torch.randn(fc.weight.shape) * 0.5)
+    srm = layer.srmKernel.clone()
+    # CPU: conv3d dense, then the PSP as a conv3d over time with the flipped kernel (src/slayer.py:760-791)
+    with torch.no_grad():
+        z = F.conv3d(x, fc.weight)
+        pad = F.pad(z, (srm.numel() - 1, 0)).reshape(4 * 512, 1, 1, 1, -1)
+        a_cpu = F.conv3d(pad, srm.flip(0).reshape(1, 1, 1, 1, -1)).reshape(z.shape)
+    s_cpu, u_cpu = O.get_spikes(a_cpu.numpy(), layer.refKernel.numpy(), params["theta"], 1.0)
+    # GPU
+    layer = layer.cuda()
+    fc = fc.cuda()
+    with torch.no_grad():
+        a_gpu = layer.psp(fc(x.cuda()))
+        assert rel_err(a_gpu.cpu().numpy(), a_cpu.numpy()) <= 1e-5
+        s_gpu = layer.spike(a_gpu)
+    flips = float((s_gpu.cpu().numpy() != s_cpu).mean())
+    assert 0.005 < float(s_cpu.mean()) < 0.5
+    assert flips <= 1e-4, "spike flip rate %g" % flips
