@@ -5,7 +5,11 @@
 //
 // With time innermost the filter does not depend on the fastest axis, so every lane owns a run of
 // consecutive time samples (one 16-byte vector) of one pixel: loads and stores are contiguous along
-// T for any stride, padding or dilation, and the weights are wave-uniform.
+// T for any stride, padding or dilation, and the weights are wave-uniform.  Forward and input
+// gradient are one gather kernel on the vector ALUs; the weight gradient, a matrix product with time
+// as the reduction axis, runs on the matrix cores (with a vector kernel for small or unaligned
+// shapes); pooling has a streaming input gradient.  Work-groups that read the same rows are kept
+// on the same die (xcd_contiguous).
 #include "common.h"
 
 namespace slayer {
