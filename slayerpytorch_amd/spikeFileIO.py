@@ -118,12 +118,19 @@ def toSpikeTensorBatch(events, emptyTensor, samplingTime=1, randomShift=False, b
             for i, ev in enumerate(events):
                 table[i] = (first, ev._raw.size // _EVENT_BYTES[fmt], shifts[i])
                 first += ev._raw.size
-            raw = np.concatenate([ev._raw for ev in events]) if first else np.zeros(0, dtype=np.uint8)
-            d_raw = torch.from_numpy(raw).to(emptyTensor.device, non_blocking=False)
-            d_table = torch.from_numpy(table).to(emptyTensor.device)
+            # one upload: the sample table followed by the files' bytes, staged in pinned host memory
+            # (allocated pinned by PyTorch's caching host allocator) so that the copy is asynchronous
+            staging = torch.empty(table.nbytes + first, dtype=torch.uint8, pin_memory=True)
+            host = staging.numpy()
+            host[:table.nbytes] = table.reshape(-1).view(np.uint8)
+            at = table.nbytes
+            for ev in events:
+                host[at:at + ev._raw.size] = ev._raw
+                at += ev._raw.size
+            d_staging = staging.to(emptyTensor.device, non_blocking=True)
             _lib.check(lib.slayer_bin_packed_events_f32(
-                _ptr(emptyTensor), _ptr(base) if base is not None else None, _ptr(d_raw), raw.size, _ptr(d_table), N,
-                int(table[:, 1].max()), fmt, C, H, W, T, float(samplingTime), mode, stream),
+                _ptr(emptyTensor), _ptr(base) if base is not None else None, d_staging.data_ptr() + table.nbytes, first,
+                d_staging.data_ptr(), N, int(table[:, 1].max()), fmt, C, H, W, T, float(samplingTime), mode, stream),
                 "slayer_bin_packed_events_f32")
             return emptyTensor
         for i, ev in enumerate(events):
