@@ -137,3 +137,20 @@ def test_argument_errors():
     assert float(t.abs().sum()) == 0.0
     with pytest.raises(RuntimeError):
         snn.io.event([1], [1], [0], [1.0]).toSpikeTensor(torch.zeros((2, 4, 4, 8)))
+
+
+def test_binning_on_a_side_stream():
+    """Upload and binning run on PyTorch's current stream: under a side stream they can overlap other
+    work, and the result is the same once that stream is waited for."""
+    raw = GOLD["nmnist_bs2"]
+    events = [snn.io.event._fromBytes(raw, 2) for _ in range(3)]
+    side = torch.cuda.Stream()
+    busy = torch.randn((2048, 2048), device="cuda")
+    with torch.cuda.stream(side):
+        out = snn.io.toSpikeTensorBatch(events, torch.zeros((3, 2, 34, 34, 350), device="cuda"), 1.0)
+    for _ in range(4):
+        busy = busy @ busy * 1e-3                     # work on the default stream meanwhile
+    torch.cuda.current_stream().wait_stream(side)
+    ref = oracle_tensor(raw, 2, (2, 34, 34, 350), 1.0)
+    for k in range(3):
+        assert np.array_equal(out[k].cpu().numpy(), ref)
