@@ -361,8 +361,27 @@ def loihi_cnn_row(device, timed):
                 rates.append(s)
 
     t = timed(step)
-    return {"op": "loihi_gesture_cnn_inference", "shape": [8, 2, 128, 128, 300], "us": t * 1e6, "samples_per_s": 8 / t,
-            "spike_rate_per_layer": [round(float(r.mean()), 4) for r in rates]}
+    row = {"op": "loihi_gesture_cnn_inference", "shape": [8, 2, 128, 128, 300], "us": t * 1e6, "samples_per_s": 8 / t,
+           "spike_rate_per_layer": [round(float(r.mean()), 4) for r in rates]}
+
+    # the same network trained: forward with autograd, spike-time loss against a random target, backward
+    # (surrogate gradient fused into the 110-tap correlation, quantised weights with straight-through gradient)
+    error = snn.loss({"neuron": desc, "simulation": {"Ts": 1, "tSample": 300},
+                      "training": {"error": {"type": "SpikeTime"}}}, snn.loihi).to(device)
+    target = (torch.rand((8, 11, 1, 1, 300), generator=g) < 0.02).float().to(device)
+
+    def train_step():
+        s = x
+        for k, syn in enumerate(mods):
+            if k == 5:
+                s = s.reshape(s.shape[0], -1, 1, 1, s.shape[-1])
+            s = layer.spikeLoihi(syn(s), delay=1)
+        error.spikeTime(s, target).backward()
+        for m in mods:
+            m.weight.grad = None
+
+    row["us_training_step"] = timed(train_step) * 1e6
+    return row
 
 
 def event_row(device, timed, cpu_leg):
