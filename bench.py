@@ -29,7 +29,7 @@ sys.path.insert(0, ROOT)
 
 SHAPE = (12, 16, 34, 34, 300)
 HBM_PEAK_GBS = 8000.0                     # MI355X HBM3E, published
-FP32_PEAK_TFLOPS = 157.3                  # MI355X FP32 vector, published (with packed FP32; this build issues scalar FMAs: 78.6)
+FP32_PEAK_TFLOPS = 157.3                  # MI355X FP32, published: vector (with packed FP32; scalar FMAs: 78.6) and matrix alike
 SRM_TAPS = 77
 # algorithmic bytes per neuron-timestep (fp32 tensors read + written once)
 AB = {"psp_conv": 8, "spike": 12, "shift": 8, "shift_bwd": 8, "spike_bwd": 12, "psp_corr": 8}
@@ -37,10 +37,10 @@ AB = {"psp_conv": 8, "spike": 12, "shift": 8, "shift_bwd": 8, "spike_bwd": 12, "
 # (rocprofv3 --pmc, one counter per run, scaled by the reading of a plain copy of known size);
 # the figures and the commands are in profiles/hbm_traffic_counters.txt
 TRAFFIC_BYTES = {"psp_conv": 537.2e6, "spike": 798.7e6, "shift": 540.8e6, "shift_bwd": 540.8e6, "spike_bwd": 798.7e6,
-                 "psp_corr": 545.5e6}
+                 "psp_corr": 532.5e6}
 KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, true, 8, false> (conv, event-driven path)", "spike": "slayer::spike_tile_kernel<12, 1, 12, 8>",
              "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
-             "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_direct_kernel<false, 22, 8> (corr)"}
+             "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_mfma_kernel<6, 20, true> (corr, matrix cores)"}
 
 
 def neuron_params():

@@ -127,6 +127,12 @@ __device__ __forceinline__ uint32_t xcd_contiguous(uint32_t b, uint32_t n)
 typedef __amdgpu_buffer_rsrc_t BufferRsrc;
 constexpr int64_t kBufferMaxT = 1 << 22;
 
+// The same with a range check: accesses at byte offsets >= bytes read zeros / are dropped.
+__device__ __forceinline__ BufferRsrc make_buffer(const void *base, int bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+
 __device__ __forceinline__ BufferRsrc make_buffer(const void *base)
 {
     // raw buffer, no stride/swizzle, 32-bit data format; range = the whole 32-bit offset space

@@ -32,13 +32,6 @@ constexpr int kFirMaxPitch = 512;     // longest LDS row (samples) the tiled ker
 // four floats that need not be 16-byte aligned (the GPU's global memory accesses may be unaligned)
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
 
-// Optional gate on the input: the filter then runs over in[n][t] * gain * exp(-|u[n][t] - theta| / tau),
-// i.e. the spike function's surrogate gradient applied on the way in (u == nullptr: no gate).
-struct FirGate {
-    const float *u;
-    float theta, tau, gain;
-};
-
 // ---- generic kernel: one lane per output sample (any F, any T) ---------------------------------
 template <bool CAUSAL, bool GATED>
 __global__ __launch_bounds__(256) void fir_generic_kernel(float *__restrict__ out,
@@ -457,6 +450,12 @@ static int launch_fir(float *out, const float *in, const float *filt, int64_t ro
     if (T >= (1LL << 30)) return SLAYER_EUNSUPPORTED;
 
     const bool vec = (T % 4 == 0) && aligned16(out) && aligned16(in) && (!GATED || aligned16(gate.u));
+    // The correlation's input is a gradient, i.e. dense: from 34 taps on, where the chain kernels are bound by
+    // FMA issue, it runs on the matrix cores.  The convolution does not: its input is mostly spike trains, which
+    // the tiled kernel's event-driven path serves at the speed of a copy and with the bits of the chain.  Nor does
+    // the gated correlation, which measured no faster there (the gate is as much work as the filter).
+    if (!CAUSAL && !GATED && !generic_forced() && launch_fir_corr_mfma(out, in, filt, rows, T, F, Ts, stream))
+        return launch_status();
     // Register-only kernel: always for short filters (the op is then a stream); up to 81 taps for
     // the correlation, whose input - a gradient - is dense, where it measures 6-9 % faster than
     // the tiled kernel.  The convolution keeps the tiled kernel for longer filters because of its

@@ -7,6 +7,17 @@
 
 namespace slayer {
 
+// Optional gate on the input: the filter then runs over in[n][t] * gain * exp(-|u[n][t] - theta| / tau),
+// i.e. the spike function's surrogate gradient applied on the way in (u == nullptr: no gate).
+struct FirGate {
+    const float *u;
+    float theta, tau, gain;
+};
+
+// Matrix-core correlation (fir_mfma.hip).  Returns false, launching nothing, for shapes it does not serve.
+bool launch_fir_corr_mfma(float *out, const float *in, const float *filt, int64_t rows, int64_t T, int64_t F, float Ts,
+                          hipStream_t stream);
+
 // A lane produces U consecutive outputs from a register window of U + 4 samples held as
 // NQ = U/4 + 1 16-byte vectors q[].  ROT says which vector currently holds the oldest samples:
 // window sample e is component e % 4 of q[(ROT + e / 4) % NQ].  After a 4-tap block the oldest
