@@ -150,6 +150,11 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
         return __builtin_amdgcn_ballot_w64(bad) != 0;
     };
 
+    // 64 bytes of zeros: behind the 16 rows, where the linear copy leaves zeros with every tile (the range check of
+    // its loads; nv KiB hold at least 256 bytes more than 16 rows whose T / 4 is odd), else an extra block
+    const int zeroOff = LINEAR ? 16 * T : 16 * P;
+    if (!LINEAR && lane < 4) *reinterpret_cast<float4 *>(X + zeroOff + 4 * lane) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+
     uint32_t i = blockIdx.x;
     if (i >= p.nItems) return;
     Tile cur = tile_of(i);
@@ -180,13 +185,13 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
         } else {
             // walk: step j makes output block j from input blocks j .. j + D - 1 and writes it over input block j
             float *col = X + c * P + 4 * h;
+            const float *zeros = X + zeroOff + 4 * h;
             const int nIn = cur.nIn;
-            auto block = [&](int q) {  // block q of the lane's row; zeros behind the row
-                const float4 x = *reinterpret_cast<const float4 *>(col + 16 * min(q, nIn - 1));
+            // block q of the lane's row; behind the row, 16 bytes of zeros (choosing the address instead of masking
+            // the data leaves nothing to do when the read returns, so it can stay in flight during the step)
+            auto block = [&](int q) {
                 const bool keep = q < nIn && (!LINEAR || 16 * q + 4 * h < T);
-                const uint32_t m = keep ? 0xffffffffu : 0u;
-                auto bits = [&](float f) { return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, f) & m); };
-                return make_float4(bits(x.x), bits(x.y), bits(x.z), bits(x.w));
+                return *reinterpret_cast<const float4 *>(keep ? col + 16 * q : zeros);
             };
             float4 w[W];
 #pragma unroll
@@ -197,6 +202,7 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
                     const int j = j0 + u;
                     if (j < cur.nb) {
                         w[(u + D) % W] = block(j + D);  // the block the next step adds
+                        __builtin_amdgcn_sched_barrier(0);  // (issued here, not after the step's matrix work)
                         f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                         for (int d = 0; d < D; ++d) {
@@ -259,7 +265,7 @@ static MfmaFirPlan plan_mfma(int nBlk, int D, int ldsBytes)
         const int staged = nb + (timeTiles > 1 ? D - 1 : 0);
         int pitch = 16 * staged;
         if ((pitch / 4) % 2 == 0) pitch += 4;
-        if (16 * pitch * 4 <= ldsBytes) return MfmaFirPlan{nb, timeTiles, pitch};
+        if ((16 * pitch + 16) * 4 <= ldsBytes) return MfmaFirPlan{nb, timeTiles, pitch};
         if (nb <= D) break;  // more halo than tile
     }
     return MfmaFirPlan{0, 0, 0};
@@ -307,7 +313,7 @@ bool launch_fir_corr_mfma(float *out, const float *in, const float *filt, int64_
                      nv, static_cast<uint32_t>(items), Ts};
     const dim3 grid(static_cast<unsigned>(waves));
     // (the linear layout writes whole vectors per lane: nv KiB)
-    const size_t lds = linear ? static_cast<size_t>(nv) * 1024 : static_cast<size_t>(16) * plan.pitch * sizeof(float);
+    const size_t lds = linear ? static_cast<size_t>(nv) * 1024 : (static_cast<size_t>(16) * plan.pitch + 16) * sizeof(float);
     if (linear) {
         if (nv <= 12) launch_mfma<12, true>(D, grid, lds, stream, args);
         else if (nv <= 16) launch_mfma<16, true>(D, grid, lds, stream, args);
