@@ -7,7 +7,8 @@
 // then one multiply by Ts, exactly like the sequential loop; samples outside [0,T) enter as
 // zeros, which leaves the chain's value unchanged.
 //
-// Three kernels share that definition:
+// Three kernels share that definition (the plain correlation with 34 to 129 taps on rows of whole 16-byte
+// vectors goes to the matrix-core kernel of fir_mfma.hip instead, which agrees with it to rounding):
 //  * direct: rows of whole 16-byte vectors and filters of at most 33 taps (81 for the
 //    correlation): everything in registers, addressing of a plain copy;
 //  * tiled: the convolution is the correlation on a reversed time axis, so both share one core
