@@ -40,7 +40,7 @@ TRAFFIC_BYTES = {"psp_conv": 537.2e6, "spike": 798.7e6, "shift": 540.8e6, "shift
                  "psp_corr": 532.5e6}
 KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, true, 8, false> (conv, event-driven path)", "spike": "slayer::spike_tile_kernel<12, 1, 12, 8>",
              "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
-             "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_mfma_kernel<6, 20, true> (corr, matrix cores)"}
+             "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_mfma_kernel<6, 20, true, false> (corr, matrix cores)"}
 
 
 def neuron_params():

@@ -452,10 +452,10 @@ static int launch_fir(float *out, const float *in, const float *filt, int64_t ro
 
     const bool vec = (T % 4 == 0) && aligned16(out) && aligned16(in) && (!GATED || aligned16(gate.u));
     // The correlation's input is a gradient, i.e. dense: from 34 taps on, where the chain kernels are bound by
-    // FMA issue, it runs on the matrix cores.  The convolution does not: its input is mostly spike trains, which
-    // the tiled kernel's event-driven path serves at the speed of a copy and with the bits of the chain.  Nor does
-    // the gated correlation, which measured no faster there (the gate is as much work as the filter).
-    if (!CAUSAL && !GATED && !generic_forced() && launch_fir_corr_mfma(out, in, filt, rows, T, F, Ts, stream))
+    // FMA issue, it runs on the matrix cores (the gated one too when its rows fit that kernel's linear layout).
+    // The convolution does not: its input is mostly spike trains, which the tiled kernel's event-driven path
+    // serves at the speed of a copy and with the bits of the chain.
+    if (!CAUSAL && !generic_forced() && launch_fir_corr_mfma(out, in, filt, rows, T, F, Ts, gate, stream))
         return launch_status();
     // Register-only kernel: always for short filters (the op is then a stream); up to 81 taps for
     // the correlation, whose input - a gradient - is dense, where it measures 6-9 % faster than

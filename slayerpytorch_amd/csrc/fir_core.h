@@ -16,7 +16,7 @@ struct FirGate {
 
 // Matrix-core correlation (fir_mfma.hip).  Returns false, launching nothing, for shapes it does not serve.
 bool launch_fir_corr_mfma(float *out, const float *in, const float *filt, int64_t rows, int64_t T, int64_t F, float Ts,
-                          hipStream_t stream);
+                          const FirGate &gate, hipStream_t stream);
 
 // A lane produces U consecutive outputs from a register window of U + 4 samples held as
 // NQ = U/4 + 1 16-byte vectors q[].  ROT says which vector currently holds the oldest samples:

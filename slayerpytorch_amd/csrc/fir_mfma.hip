@@ -1,7 +1,8 @@
 // Temporal FIR of neuron rows on the matrix cores, for dense input and filters of 34 to 129 taps, where the
 // register-window kernels of fir.hip are bound by FMA issue (an FIR of 77 taps needs 154 flop per 8 bytes).
-// Correlation only: the convolution's input is mostly spike trains, which the tiled kernel of fir.hip serves
-// through its event-driven path.
+// Correlation only (plain, or with the spike function's surrogate gradient applied to the samples on their way
+// into LDS): the convolution's input is mostly spike trains, which the tiled kernel of fir.hip serves through
+// its event-driven path.
 //
 // The rows are cut into blocks of 16 samples.  For Y[m] = sum_t X[m+t] * filt[t], the 16 outputs of block b of
 // 16 rows are the 16x16 product
@@ -47,13 +48,14 @@ struct MfmaFirArgs {
     int nv;         // 16-byte vectors per lane and tile that are in use (<= NV)
     uint32_t nItems;
     float Ts;
+    FirGate gate;  // GATED: the samples are in * gain * exp(-|u - theta| / tau), applied on the way into LDS
 };
 
 // NV: 16-byte vectors per lane and tile, NV * 64 >= 16 rows * (staged blocks * 4)
 // LINEAR: the tile is 16 whole rows kept in LDS exactly as they lie in memory (pitch == T): vector e of the tile
 // is vector e of LDS, no index arithmetic, and the range check of the buffers masks what lies behind the last row.
 // The last block of a row then ends in the first samples of the next row, which the walk masks.
-template <int D, int NV, bool LINEAR>
+template <int D, int NV, bool LINEAR, bool GATED>
 __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
 {
     extern __shared__ __align__(16) float X[];
@@ -98,7 +100,7 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
         return q;
     };
     // vector e = lane + 64 k of a tile is vector e % lenIn of row e / lenIn; samples outside the row read as zeros
-    float4 pre[NV];
+    float4 pre[NV], preU[GATED ? NV : 1];
     // the lane index behind a barrier for the optimiser: the (row, vector) sequences below do not depend on the
     // tile, and kept across the walk they would cost 2 registers per vector
     auto lane_again = [&]() {
@@ -109,15 +111,18 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
     auto fetch = [&](const Tile &q) {
         if (LINEAR) {
             const BufferRsrc bufIn = make_buffer(p.in + q.row0 * T, q.nRows * T * 4);
+            const BufferRsrc bufU = make_buffer(GATED ? p.gate.u + q.row0 * T : p.in, q.nRows * T * 4);
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
                 if (k < p.nv) {
                     pre[k] = buffer_load4(bufIn, (lane + kWave * k) * 16, 0);
+                    if (GATED) preU[k] = buffer_load4(bufU, (lane + kWave * k) * 16, 0);
                 }
             }
             return;
         }
         const BufferRsrc bufIn = make_buffer(p.in + q.row0 * T);
+        const BufferRsrc bufU = make_buffer(GATED ? p.gate.u + q.row0 * T : p.in);
         RowCol rc;
         rc.init(lane_again(), lenIn, 1.0f / static_cast<float>(lenIn));
         const int dr = kWave / lenIn, dc = kWave % lenIn;
@@ -126,6 +131,7 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
             const int t = q.t0 + (rc.c << 2);
             const int off = masked_offset(rc.r < q.nRows && t < T, (rc.r * T + t) * 4);
             pre[k] = buffer_load4(bufIn, off, 0);
+            if (GATED) preU[k] = buffer_load4(bufU, off, 0);
             rc.advance(dr, dc, lenIn);
         }
     };
@@ -137,7 +143,12 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             if (LINEAR && k >= p.nv) continue;
-            const float4 x = pre[k];
+            float4 x = pre[k];
+            if (GATED)
+                x = make_float4(x.x * spike_pdf(preU[k].x, p.gate.theta, p.gate.tau, p.gate.gain),
+                                x.y * spike_pdf(preU[k].y, p.gate.theta, p.gate.tau, p.gate.gain),
+                                x.z * spike_pdf(preU[k].z, p.gate.theta, p.gate.tau, p.gate.gain),
+                                x.w * spike_pdf(preU[k].w, p.gate.theta, p.gate.tau, p.gate.gain));
             // infinite or NaN (or four samples that add up to more than fp32 holds, which only costs time)
             bad |= ((x.x + x.y) + (x.z + x.w)) * 0.0f != 0.0f;
             if (LINEAR) {
@@ -175,10 +186,12 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
             for (int e = lane; e < cur.nRows * width; e += kWave) {
                 const int r = e / width, t = cur.t0 + (e - r * width);
                 const float *x = p.in + (cur.row0 + r) * T;
+                const float *gu = GATED ? p.gate.u + (cur.row0 + r) * T : nullptr;
                 const int taps = min(T - t, F);
                 float acc = 0.0f;
                 for (int k = 0; k < taps; ++k) {
-                    acc = __builtin_fmaf(x[t + k], p.filt[k], acc);
+                    acc = __builtin_fmaf(GATED ? x[t + k] * spike_pdf(gu[t + k], p.gate.theta, p.gate.tau, p.gate.gain) : x[t + k],
+                                         p.filt[k], acc);
                 }
                 p.out[(cur.row0 + r) * T + t] = acc * p.Ts;
             }
@@ -271,12 +284,12 @@ static MfmaFirPlan plan_mfma(int nBlk, int D, int ldsBytes)
     return MfmaFirPlan{0, 0, 0};
 }
 
-template <int NV, bool LINEAR>
+template <int NV, bool LINEAR, bool GATED>
 static void launch_mfma(int D, dim3 grid, size_t lds, hipStream_t st, const MfmaFirArgs &args)
 {
 #define SLAYER_FIR_MFMA(DD)                                                                                            \
     case DD:                                                                                                           \
-        hipLaunchKernelGGL((fir_mfma_kernel<DD, NV, LINEAR>), grid, dim3(64), lds, st, args);                         \
+        hipLaunchKernelGGL((fir_mfma_kernel<DD, NV, LINEAR, GATED>), grid, dim3(64), lds, st, args);                  \
         break
     switch (D) {
         SLAYER_FIR_MFMA(4);
@@ -291,16 +304,18 @@ static void launch_mfma(int D, dim3 grid, size_t lds, hipStream_t st, const Mfma
 }
 
 bool launch_fir_corr_mfma(float *out, const float *in, const float *filt, int64_t rows, int64_t T, int64_t F, float Ts,
-                          hipStream_t stream)
+                          const FirGate &gate, hipStream_t stream)
 {
     if (F < kMfmaMinTaps || F > kMfmaMaxTaps || T % 4 != 0 || T < 16 || T > kBufferMaxT) return false;
-    if (!aligned16(out) || !aligned16(in)) return false;
+    if (!aligned16(out) || !aligned16(in) || (gate.u && !aligned16(gate.u))) return false;
     const int D = static_cast<int>((F + 14) / 16 + 1);
     const int nBlk = static_cast<int>(ceil_div(T, 16));
     MfmaFirPlan plan = plan_mfma(nBlk, D, kMfmaLdsBytes);
     if (plan.nb < 1) return false;
     // whole rows whose length spreads the 16 rows over the LDS banks as it is: the tile as it lies in memory
     const bool linear = plan.timeTiles == 1 && (T / 4) % 2 == 1;
+    // the gated correlation only in that layout (elsewhere it measured no faster than the tiled kernel)
+    if (gate.u && !linear) return false;
     if (linear) plan.pitch = static_cast<int>(T);
     const int64_t items = ceil_div(rows, 16) * plan.timeTiles;
     if (items >= (1LL << 31) || 16 * T >= (1LL << 28)) return false;
@@ -310,18 +325,22 @@ bool launch_fir_corr_mfma(float *out, const float *in, const float *filt, int64_
     const int64_t waves = ceil_div(ceil_div(items, trips), 8) * 8;  // a multiple of 8: one range of tiles per die
     const int nv = plan.nb + (plan.timeTiles > 1 ? D - 1 : 0);      // vectors per lane = staged blocks per row
     MfmaFirArgs args{out, in, filt, rows, static_cast<int>(T), static_cast<int>(F), plan.nb, plan.timeTiles, plan.pitch,
-                     nv, static_cast<uint32_t>(items), Ts};
+                     nv, static_cast<uint32_t>(items), Ts, gate};
     const dim3 grid(static_cast<unsigned>(waves));
     // (the linear layout writes whole vectors per lane: nv KiB)
     const size_t lds = linear ? static_cast<size_t>(nv) * 1024 : (static_cast<size_t>(16) * plan.pitch + 16) * sizeof(float);
-    if (linear) {
-        if (nv <= 12) launch_mfma<12, true>(D, grid, lds, stream, args);
-        else if (nv <= 16) launch_mfma<16, true>(D, grid, lds, stream, args);
-        else launch_mfma<20, true>(D, grid, lds, stream, args);
+    if (gate.u) {
+        if (nv <= 12) launch_mfma<12, true, true>(D, grid, lds, stream, args);
+        else if (nv <= 16) launch_mfma<16, true, true>(D, grid, lds, stream, args);
+        else launch_mfma<20, true, true>(D, grid, lds, stream, args);
+    } else if (linear) {
+        if (nv <= 12) launch_mfma<12, true, false>(D, grid, lds, stream, args);
+        else if (nv <= 16) launch_mfma<16, true, false>(D, grid, lds, stream, args);
+        else launch_mfma<20, true, false>(D, grid, lds, stream, args);
     } else {
-        if (nv <= 12) launch_mfma<12, false>(D, grid, lds, stream, args);
-        else if (nv <= 16) launch_mfma<16, false>(D, grid, lds, stream, args);
-        else launch_mfma<20, false>(D, grid, lds, stream, args);
+        if (nv <= 12) launch_mfma<12, false, false>(D, grid, lds, stream, args);
+        else if (nv <= 16) launch_mfma<16, false, false>(D, grid, lds, stream, args);
+        else launch_mfma<20, false, false>(D, grid, lds, stream, args);
     }
     return true;
 }

@@ -193,6 +193,24 @@ def test_fir_sparse_input_edges(impl, T, Fl, op):
     check(x)
 
 
+def test_gated_corr_on_the_matrix_cores_keeps_non_finite_samples_in_place():
+    # an infinite gradient sample reaches exactly the outputs within Fl taps before it, as in the chain; so does an
+    # infinite membrane potential (gate 0 times a finite sample is 0, times an infinite one NaN)
+    rng = np.random.default_rng(12)
+    g = rng.standard_normal((40, 300)).astype(np.float32)
+    v = (rng.standard_normal((40, 300)) * 3 + 8).astype(np.float32)
+    g[3, 150] = np.inf
+    g[20, 7] = -np.inf
+    v[20, 7] = np.inf
+    f = rng.standard_normal(77).astype(np.float32)
+    got = host(slayerCuda.spikeBackwardCorr(dev(g), dev(v), dev(f), 10.0, 5.0, 1.0, 0.5))
+    want = O.corr(O.spike_bwd(g, v, 10.0, 5.0, 1.0), f, 0.5, fused=True)
+    fin = np.isfinite(want)
+    assert not fin.all()
+    assert np.array_equal(np.isfinite(got), fin) and np.array_equal(got[~fin], want[~fin], equal_nan=True)
+    assert rel_err(np.where(fin, got, 0), np.where(fin, want, 0)) <= REL_TOL
+
+
 def test_fir_is_left_padded_conv3d(impl):
     # the identity the reference's test_slayer011 asserts: psp == pspLayer, ||diff|| / numel < 1e-6
     rng = np.random.default_rng(6)
@@ -285,7 +303,9 @@ def test_spike_bwd(n):
 
 
 @pytest.mark.parametrize("shape,Fl", [((2, 3, 5, 7, 300), 110), ((3, 41, 350), 110), ((2, 9, 64), 8), ((1, 5, 2000), 77),
-                                      ((1, 2, 50), 500), ((4, 7, 1), 3)])
+                                      ((1, 2, 50), 500), ((4, 7, 1), 3),
+                                      # the fused kernel on the matrix cores (rows kept as they lie in memory: T / 4 odd)
+                                      ((37, 300), 77), ((3, 44), 40), ((18, 76), 113), ((100, 28), 45), ((5, 316), 129)])
 def test_spike_bwd_corr_is_the_two_ops_in_one(impl, shape, Fl):
     # the Loihi neuron's backward pass: pdf(voltage) * gradOut, then corr with the PSP kernel
     rng = np.random.default_rng(shape[-1] + Fl)
@@ -298,7 +318,8 @@ def test_spike_bwd_corr_is_the_two_ops_in_one(impl, shape, Fl):
     want = O.corr(O.spike_bwd(g, v, theta, tau, scale), f, Ts, fused=True)
     assert rel_err(got, want) <= REL_TOL
     if on_matrix_cores("corr", shape[-1], Fl, impl):
-        # the plain correlation of this shape runs on the matrix cores, the fused kernel as a chain
+        # the plain correlation of this shape runs on the matrix cores (and so does the fused kernel where the rows fit
+        # its linear layout), which add the terms in another order than the chain
         assert rel_err(two, want) <= REL_TOL and rel_err(got, two) <= REL_TOL
     else:
         assert np.array_equal(bits(got), bits(two)), "fused kernel differs from spikeBackward followed by corr"
