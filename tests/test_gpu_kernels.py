@@ -211,6 +211,37 @@ def test_gated_corr_on_the_matrix_cores_keeps_non_finite_samples_in_place():
     assert rel_err(np.where(fin, got, 0), np.where(fin, want, 0)) <= REL_TOL
 
 
+def test_matrix_core_corr_replayed_from_a_hip_graph():
+    # the persistent matrix-core kernels (plain and gated) captured in a HIP graph: every replay, with eager work and
+    # synchronisations in between, gives the bits of the eager launch
+    rng = np.random.default_rng(13)
+    g, v = dev(rng.standard_normal((70, 300)).astype(np.float32)), dev((rng.standard_normal((70, 300)) * 3 + 8).astype(np.float32))
+    f = dev(rng.standard_normal(77).astype(np.float32))
+
+    def both():
+        return slayerCuda.corr(g, f, 1.0), slayerCuda.spikeBackwardCorr(g, v, f, 10.0, 5.0, 1.0, 1.0)
+
+    ref = [t.clone() for t in both()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        both()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = both()
+    for _ in range(3):
+        for t in outs:
+            t.fill_(-1.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(outs, ref))
+        assert all(torch.equal(a, b) for a, b in zip(both(), ref))     # eager work between the replays
+        torch.cuda.synchronize()
+
+
 def test_fir_is_left_padded_conv3d(impl):
     # the identity the reference's test_slayer011 asserts: psp == pspLayer, ||diff|| / numel < 1e-6
     rng = np.random.default_rng(6)
