@@ -208,6 +208,21 @@ int slayer_delay_grad_f32(float *gradDelay, const float *out, const float *gradO
                           void *stream);
 
 /*
+ * slayer_delay_grad_f32 for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): it has no counterpart in the reference.  Same
+ * arguments and bit-identical results, but the partial sums live in a fixed array inside the library's
+ * device image (4 bytes per neuron row, slayer_delay_grad_static_max_rows() = 262144 rows = 1 MiB, held
+ * by every GPU the library runs on until the process ends) instead of a caller workspace, so the call
+ * allocates and frees nothing.  nBatch * nPerBatch beyond that maximum: SLAYER_EUNSUPPORTED, nothing
+ * launched.  The array's device address is looked up on the first call on each device (make that call
+ * outside a graph capture).  All calls on one GPU share the array: calls that overlap on one GPU (two
+ * streams, two threads) race - serialise them.  Nothing needs clearing between calls.
+ */
+int64_t slayer_delay_grad_static_max_rows(void);
+int slayer_delay_grad_static_f32(float *gradDelay, const float *out, const float *gradOut,
+                                 int64_t nBatch, int64_t nPerBatch, int64_t T, float Ts, void *stream);
+
+/*
  * Loihi CUBA (current based) integer neuron.
  * Replaces slayerLoihiCuda.getSpikes -> getSpikesCuda (src/cuda/slayerLoihiKernels.cu:12-46),
  * kernel and launcher src/cuda/spikeLoihiKernels.h:9-96.

@@ -11,6 +11,8 @@
 // are reproducible from run to run.
 #include "common.h"
 
+#include <atomic>
+
 namespace slayer {
 
 // VEC: rows are whole 16-byte vectors (T % 4 == 0, 16-byte aligned tensors): a lane takes four
@@ -102,11 +104,68 @@ extern "C" int64_t slayer_delay_grad_workspace_bytes(int64_t nBatch, int64_t nPe
     return nBatch * nPerBatch * static_cast<int64_t>(sizeof(float));
 }
 
+namespace slayer {
+
+// Partial sums of slayer_delay_grad_static_f32: one float per neuron row.  Every GPU the library runs on
+// holds its own copy of this array at its own address until the process ends.
+constexpr int64_t kStaticRows = 262144;  // 1 MiB
+static __device__ __align__(256) float scratch[kStaticRows];
+
+// The array's address on each device, looked up once per device; host code uses these pointers, never
+// the array's name (which is only a handle for the lookup on the host side).
+constexpr int kMaxDevices = 64;
+static std::atomic<float *> g_scratch_ptr[kMaxDevices];
+
+static int scratch_of_current_device(float **ptr)
+{
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return note_hip_error(err);
+    if (device < 0 || device >= kMaxDevices) return SLAYER_EUNSUPPORTED;
+    float *p = g_scratch_ptr[device].load(std::memory_order_acquire);
+    if (!p) {
+        void *sym = nullptr;
+        err = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return note_hip_error(err);
+        if (!sym) return SLAYER_ELAUNCH;
+        p = static_cast<float *>(sym);
+        g_scratch_ptr[device].store(p, std::memory_order_release);  // (two racing threads store the same address)
+    }
+    *ptr = p;
+    return SLAYER_OK;
+}
+
+static int launch_delay_grad(float *gradDelay, const float *out, const float *gradOut, float *workspace, int64_t nBatch,
+                             int64_t nPerBatch, int64_t T, float Ts, void *stream);
+
+}  // namespace slayer
+
 extern "C" int slayer_delay_grad_f32(float *gradDelay, const float *out, const float *gradOut,
                                      float *workspace, int64_t nBatch, int64_t nPerBatch, int64_t T,
                                      float Ts, void *stream)
 {
+    return slayer::launch_delay_grad(gradDelay, out, gradOut, workspace, nBatch, nPerBatch, T, Ts, stream);
+}
+
+extern "C" int64_t slayer_delay_grad_static_max_rows(void) { return slayer::kStaticRows; }
+
+extern "C" int slayer_delay_grad_static_f32(float *gradDelay, const float *out, const float *gradOut, int64_t nBatch,
+                                            int64_t nPerBatch, int64_t T, float Ts, void *stream)
+{
     using namespace slayer;
+    if (nBatch < 0 || nPerBatch < 0 || T < 0) return SLAYER_EINVAL;
+    // (checked before the product is formed, so that it cannot overflow)
+    if (nBatch > kStaticRows || nPerBatch > kStaticRows || nBatch * nPerBatch > kStaticRows) return SLAYER_EUNSUPPORTED;
+    float *partial = nullptr;
+    const int status = scratch_of_current_device(&partial);
+    if (status != SLAYER_OK) return status;
+    // every partial sum that pass 2 reads has been written by pass 1 of the same call: nothing to clear
+    return launch_delay_grad(gradDelay, out, gradOut, partial, nBatch, nPerBatch, T, Ts, stream);
+}
+
+static int slayer::launch_delay_grad(float *gradDelay, const float *out, const float *gradOut, float *workspace,
+                                     int64_t nBatch, int64_t nPerBatch, int64_t T, float Ts, void *stream)
+{
     if (nBatch < 0 || nPerBatch < 0 || T < 0) return SLAYER_EINVAL;
     if (nPerBatch == 0) return SLAYER_OK;
     if (!gradDelay) return SLAYER_EINVAL;

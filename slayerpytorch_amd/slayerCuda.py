@@ -340,6 +340,43 @@ def delayGrad(output, gradOutput, Ts):
     return gradDelay
 
 
+def delayGradStatic(output, gradOutput, Ts, out=None):
+    """``delayGrad`` without any device allocation inside the library call: the partial sums live in a
+    fixed array of the library (at most ``slayer_delay_grad_static_max_rows()`` neuron rows), and the
+    result goes into ``out`` when given (shape ``output.shape[1:-1]``).  For callers that must not
+    allocate (graph capture, serving loops).  Calls that overlap on one GPU share the array and race."""
+    _check_input(output, "output")
+    _check_input(gradOutput, "gradOutput")
+    _check_device(output, gradOutput, "output", "gradOutput")
+    if output.shape != gradOutput.shape:
+        raise RuntimeError("output and gradOutput must have the same shape")
+    if output.dim() < 2:
+        raise RuntimeError("delayGradStatic expects at least (batch, time) dimensions")
+    Ts = _scalar(Ts, "Ts")
+    lib = _lib.load()
+    T = output.shape[-1]
+    nBatch = output.shape[0]
+    shape = tuple(output.shape[1:-1])
+    nPerBatch = 1
+    for d in shape:
+        nPerBatch *= d
+    limit = lib.slayer_delay_grad_static_max_rows()
+    if nBatch * nPerBatch > limit:
+        raise RuntimeError("delayGradStatic serves at most %d neuron rows (got %d); use delayGrad"
+                           % (limit, nBatch * nPerBatch))
+    if out is None:
+        out = torch.empty(shape, dtype=output.dtype, device=output.device)
+    else:
+        _check_input(out, "out")
+        _check_device(output, out, "output", "out")
+        if tuple(out.shape) != shape:
+            raise RuntimeError("out must have shape %s" % (shape,))
+    with _on_device_of(output) as stream:
+        _lib.check(lib.slayer_delay_grad_static_f32(_ptr(out), _ptr(output), _ptr(gradOutput), nBatch, nPerBatch,
+                                                    T, Ts, stream), "slayer_delay_grad_static_f32")
+    return out
+
+
 def spikeLoss(spikeOut, spikeDesired, srmKernel, Ts, addend=None):
     """``error = conv(spikeOut - spikeDesired, srmKernel, Ts) [+ addend]`` and
     ``loss = 1/2 * sum(error**2) * Ts`` in two launches.  Returns ``(loss, error)`` (``loss`` is a
