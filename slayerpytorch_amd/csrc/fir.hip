@@ -216,7 +216,9 @@ __device__ __forceinline__ void fir_sparse_tile(const BufferRsrc &bufOut, const 
 
 // VEC: rows are whole 16-byte vectors (T % 4 == 0, pointers 16-byte aligned)
 // GATED: the staged samples are in * pdf(gate.u), computed once per staged sample
-template <bool CAUSAL, bool VEC, int U, bool GATED>
+// DM: 0 = dense tiles run the register-window chains; 4..9 = dense tiles run on the matrix cores with a window
+//     of DM blocks of 16 samples (VEC, U = 16, R = 16 rows, LD >= tile + 16 (DM - 1))
+template <bool CAUSAL, bool VEC, int U, bool GATED, int DM>
 __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
                                                         const float *__restrict__ in,
                                                         const float *__restrict__ filt,
@@ -322,10 +324,82 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
     {
         const uint32_t nz = nzCount[0] + nzCount[1] + nzCount[2] + nzCount[3];
         const uint32_t vectors = static_cast<uint32_t>(nRows) * static_cast<uint32_t>(LD >> 2);
-        if (F <= kSparseMaxTaps && LD <= kSparseBlocks * kWave && nz * 8u <= vectors) {
+        // (dense tiles cost less on the matrix cores, so the event-driven path pays up to a lower density there)
+        if (F <= kSparseMaxTaps && LD <= kSparseBlocks * kWave && nz * (DM > 0 ? 5u : 8u) <= vectors) {
             fir_sparse_tile<CAUSAL>(bufOut, X, fL, nRows, LD, ttp, t0, tt, tHi, T, F, Ts);
             return;
         }
+    }
+
+    // ---- dense input on the matrix cores.  The tile's rows are cut into blocks of 16 outputs; the blocks of all rows
+    // are the "columns", and a wavefront takes 16 consecutive columns at a time.  The 16 outputs of a column are the
+    // product of a banded Toeplitz matrix of the filter with the DM blocks of X that start where the column does:
+    //     Y[16b + i] = sum_{d < DM} sum_{kk < 16} filt[16d + kk - i] * X[16(b + d) + kk].
+    // v_mfma_f32_16x16x4_f32 takes 4 of the 16 kk per instruction: lane (c = lane % 16, h = lane / 16) supplies
+    // X[16(b + d) + 4h + v] of column c for instruction v = 0..3 - one 16-byte LDS read per d, 64 d bytes on from
+    // the first, an offset that sits in the instruction - and filt[16d + 4h + v - i] for i = lane % 16 (from the
+    // zero-padded filter copy, kept in 4 DM registers); its accumulator holds outputs 4h..4h+3 of column c, which
+    // it stores straight to memory.  The rows' zero padding in LDS ends every window where its row ends.  The
+    // matrix instruction adds 4 products per step in its own order: results agree with the chain to rounding,
+    // not bit for bit.  A structural zero times a non-finite sample would be NaN where the chain has no such
+    // term: columns whose results contain a NaN are computed again as sequential chains.
+    if constexpr (DM > 0) {
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        const int lane = tid & (kWave - 1), wave = tid / kWave;
+        const int c = lane & 15, h = lane >> 4;
+        float a[DM][4];
+        {
+            const float *fa = fL + (4 * h - c);
+#pragma unroll
+            for (int d = 0; d < DM; ++d)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) a[d][v] = fa[16 * d + v];
+        }
+        const int nb = ttp >> 4;  // columns per row
+        const int cols = nRows * nb;
+        // (a wavefront's columns beyond the last row fall into rows of LDS that were not staged: their results
+        // are not stored)
+        RowCol rb;
+        rb.init(16 * wave + c, nb, 1.0f / static_cast<float>(nb));
+        const int stepR = 64 / nb, stepB = 64 % nb;
+        for (int g0 = 16 * wave; g0 < cols; g0 += 64, rb.advance(stepR, stepB, nb)) {
+            const bool on = g0 + c < cols;
+            const int r = rb.r, b = rb.c;
+            const int m0 = 16 * b + 4 * h;
+            const float *xp = X + r * LD + m0;
+            float4 w[DM];
+#pragma unroll
+            for (int d = 0; d < DM; ++d) w[d] = *reinterpret_cast<const float4 *>(xp + 16 * d);
+            f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int d = 0; d < DM; ++d) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[d][0], w[d].x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[d][1], w[d].y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[d][2], w[d].z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[d][3], w[d].w, acc, 0, 0, 0);
+            }
+            // (only in columns that are part of the tile: the others hold whatever LDS held)
+            const bool nan = on & (__builtin_isunordered(acc.x, acc.y) | __builtin_isunordered(acc.z, acc.w));
+            if (__builtin_amdgcn_ballot_w64(nan) != 0) {
+                float y[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float sum = 0.0f;
+                    for (int i = 0; i < F; ++i) sum = __builtin_fmaf(xp[j + i], fL[i], sum);
+                    y[j] = sum;
+                }
+                acc = f32x4{y[0], y[1], y[2], y[3]};
+            }
+            // times t0 + m0 .. (correlation) or tHi - m0 - 3 .. tHi - m0 (convolution); both are multiples of 4 and so
+            // is the tile's end, so the vector is all in or all out
+            const int tl = CAUSAL ? (tHi - m0 - 3) : (t0 + m0);
+            const bool valid = on && tl >= t0 && tl + 3 < t0 + tt;
+            const float4 y = CAUSAL ? make_float4(acc.w * Ts, acc.z * Ts, acc.y * Ts, acc.x * Ts)
+                                    : make_float4(acc.x * Ts, acc.y * Ts, acc.z * Ts, acc.w * Ts);
+            // the columns of a wavefront are consecutive in memory: neighbouring stores complete each other's lines
+            buffer_store4<0>(bufOut, masked_offset(valid, (r * T + tl) * 4), 0, y);
+        }
+        return;
     }
 
     // ---- compute: work item = (row, chunk of 8 outputs), row-major over lanes
@@ -430,14 +504,36 @@ static bool plan_fir(int64_t rows, int64_t T, int64_t F, FirPlan &best)
     return true;
 }
 
-template <bool CAUSAL, bool VEC, int U, bool GATED>
+// The plan of the matrix-core variant: tiles of 16 rows, whole blocks of 16 outputs, and a row pitch that holds
+// the window of the tile's last block.
+static bool plan_fir_mfma(int64_t rows, int64_t T, int64_t F, FirPlan &best)
+{
+    if (F < kFirMfmaMinTaps || F > kFirMfmaMaxTaps || T > kBufferMaxT || T < 16) return false;
+    const int64_t D = (F + 14) / 16 + 1;
+    const int64_t halo = (F + 4 > 16 * (D - 1) ? F + 4 : 16 * (D - 1));
+    const int64_t ttMax = (kFirMaxPitch - 4 - halo) & ~static_cast<int64_t>(15);
+    if (ttMax < 64) return false;
+    const int64_t nTiles = ceil_div(T, ttMax);
+    if (nTiles > 65535) return false;
+    int64_t TT = ceil_div(ceil_div(T, nTiles), 16) * 16;
+    if (nTiles == 1) TT = T;
+    const int64_t ttp = ceil_div(TT, 16) * 16;
+    best.U = 16;
+    best.TT = static_cast<int>(TT);
+    best.LD = static_cast<int>((ttp + halo + 3) & ~static_cast<int64_t>(3));
+    best.R = 16;
+    best.nTiles = static_cast<int>(nTiles);
+    return true;
+}
+
+template <bool CAUSAL, bool VEC, int U, bool GATED, int DM = 0>
 static void launch_tiled(const FirPlan &p, float *out, const float *in, const float *filt, int64_t rows, int64_t T,
                          int64_t F, float Ts, const FirGate &gate, hipStream_t stream)
 {
     dim3 grid(static_cast<unsigned>(ceil_div(rows, p.R)), static_cast<unsigned>(p.nTiles)), block(256);
     // rows, the zero-padded filter copy of the sparse path (256 floats) and four counters
     const size_t lds = (static_cast<size_t>(p.R) * p.LD + 4 * kWave + 4) * sizeof(float);
-    hipLaunchKernelGGL((fir_tiled_kernel<CAUSAL, VEC, U, GATED>), grid, block, lds, stream, out, in, filt, rows,
+    hipLaunchKernelGGL((fir_tiled_kernel<CAUSAL, VEC, U, GATED, DM>), grid, block, lds, stream, out, in, filt, rows,
                        static_cast<int>(T), static_cast<int>(F), p.TT, p.LD, p.R, Ts, gate);
 }
 
@@ -457,11 +553,24 @@ static int launch_fir(float *out, const float *in, const float *filt, int64_t ro
     // serves at the speed of a copy and with the bits of the chain.
     if (!CAUSAL && !generic_forced() && launch_fir_corr_mfma(out, in, filt, rows, T, F, Ts, gate, stream))
         return launch_status();
-    // Register-only kernel: always for short filters (the op is then a stream); up to 81 taps for
-    // the correlation, whose input - a gradient - is dense, where it measures 6-9 % faster than
-    // the tiled kernel.  The convolution keeps the tiled kernel for longer filters because of its
-    // event-driven path for spike trains.
-    const int64_t directMax = CAUSAL ? 33 : 81;
+    {
+    FirPlan p;
+    // Longer filters on rows of whole vectors: the tiled kernel whose dense tiles run on the matrix cores (its
+    // sparse tiles, spike trains, keep the event-driven path and the bits of the chain).
+    if (!generic_forced() && vec && plan_fir_mfma(rows, T, F, p) && ceil_div(rows, p.R) < (1LL << 31)) {
+        switch ((F + 14) / 16 + 1) {
+            case 4: launch_tiled<CAUSAL, true, 16, GATED, 4>(p, out, in, filt, rows, T, F, Ts, gate, stream); break;
+            case 5: launch_tiled<CAUSAL, true, 16, GATED, 5>(p, out, in, filt, rows, T, F, Ts, gate, stream); break;
+            case 6: launch_tiled<CAUSAL, true, 16, GATED, 6>(p, out, in, filt, rows, T, F, Ts, gate, stream); break;
+            case 7: launch_tiled<CAUSAL, true, 16, GATED, 7>(p, out, in, filt, rows, T, F, Ts, gate, stream); break;
+            case 8: launch_tiled<CAUSAL, true, 16, GATED, 8>(p, out, in, filt, rows, T, F, Ts, gate, stream); break;
+            default: launch_tiled<CAUSAL, true, 16, GATED, 9>(p, out, in, filt, rows, T, F, Ts, gate, stream); break;
+        }
+        return launch_status();
+    }
+    }
+    // Register-only kernel for short filters (the op is then a stream).
+    const int64_t directMax = 33;
     // (not with a gate: every lane would evaluate the gate for its whole window).
     if (!GATED && !generic_forced() && vec && F >= 1 && F <= directMax && T < (1LL << 28) && rows * (T / 4) < (1LL << 32)) {
         const int U = F <= 17 ? 4 : 8;
@@ -477,10 +586,7 @@ static int launch_fir(float *out, const float *in, const float *filt, int64_t ro
         else if (F <= 13) SLAYER_FIR_DIRECT(4, 4);
         else if (F <= 17) SLAYER_FIR_DIRECT(5, 4);
         else if (F <= 25) SLAYER_FIR_DIRECT(8, 8);
-        else if (F <= 33) SLAYER_FIR_DIRECT(10, 8);
-        else if (F <= 49) SLAYER_FIR_DIRECT(14, 8);
-        else if (F <= 65) SLAYER_FIR_DIRECT(18, 8);
-        else SLAYER_FIR_DIRECT(22, 8);
+        else SLAYER_FIR_DIRECT(10, 8);
 #undef SLAYER_FIR_DIRECT
         return launch_status();
     }

@@ -18,6 +18,10 @@ struct FirGate {
 bool launch_fir_corr_mfma(float *out, const float *in, const float *filt, int64_t rows, int64_t T, int64_t F, float Ts,
                           const FirGate &gate, hipStream_t stream);
 
+// Filter lengths that the matrix-core paths serve (the correlation kernel of fir_mfma.hip and the dense tiles of
+// the tiled kernel of fir.hip).
+constexpr int kFirMfmaMinTaps = 34, kFirMfmaMaxTaps = 129;
+
 // A lane produces U consecutive outputs from a register window of U + 4 samples held as
 // NQ = U/4 + 1 16-byte vectors q[].  ROT says which vector currently holds the oldest samples:
 // window sample e is component e % 4 of q[(ROT + e / 4) % NQ].  After a 4-tap block the oldest

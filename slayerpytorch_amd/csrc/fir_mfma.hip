@@ -34,7 +34,6 @@ namespace slayer {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kMfmaMinTaps = 34, kMfmaMaxTaps = 129;
 constexpr int kMfmaLdsBytes = 160 * 1024 / 8;  // per wavefront: 8 of them on a compute unit
 
 struct MfmaFirArgs {
@@ -306,7 +305,7 @@ static void launch_mfma(int D, dim3 grid, size_t lds, hipStream_t st, const Mfma
 bool launch_fir_corr_mfma(float *out, const float *in, const float *filt, int64_t rows, int64_t T, int64_t F, float Ts,
                           const FirGate &gate, hipStream_t stream)
 {
-    if (F < kMfmaMinTaps || F > kMfmaMaxTaps || T % 4 != 0 || T < 16 || T > kBufferMaxT) return false;
+    if (F < kFirMfmaMinTaps || F > kFirMfmaMaxTaps || T % 4 != 0 || T < 16 || T > kBufferMaxT) return false;
     if (!aligned16(out) || !aligned16(in) || (gate.u && !aligned16(gate.u))) return false;
     const int D = static_cast<int>((F + 14) / 16 + 1);
     const int nBlk = static_cast<int>(ceil_div(T, 16));

@@ -645,7 +645,13 @@ def test_spike_time_loss_kernel_matches_tensor_expression(Ts, T, shape):
     ref = 1 / 2 * torch.sum(e ** 2) * Ts
     ref.backward()
     assert abs(float(loss) - float(ref)) <= 1e-5 * abs(float(ref)) and float(ref) > 0
-    assert torch.equal(out.grad, out2.grad)
+    Fl = error.slayer.srmKernel.numel()
+    if 34 <= Fl <= 129 and T % 4 == 0 and T <= 60000 // 4:
+        # the tensor expression's psp of this dense difference runs on the matrix cores, the fused kernel filters
+        # with the chain: equal to rounding
+        assert rel_err(out.grad.cpu().numpy(), out2.grad.cpu().numpy()) <= 1e-5
+    else:
+        assert torch.equal(out.grad, out2.grad)
     # against the oracle's psp
     eo = O.conv((out.detach() - des).cpu().numpy(), error.slayer.srmKernel.cpu().numpy(), Ts)
     assert abs(float(loss) - 0.5 * float((eo.astype(np.float64) ** 2).sum()) * Ts) <= 1e-5 * abs(float(ref))
