@@ -38,7 +38,7 @@ AB = {"psp_conv": 8, "spike": 12, "shift": 8, "shift_bwd": 8, "spike_bwd": 12, "
 # the figures and the commands are in profiles/hbm_traffic_counters.txt
 TRAFFIC_BYTES = {"psp_conv": 537.2e6, "spike": 798.7e6, "shift": 540.8e6, "shift_bwd": 540.8e6, "spike_bwd": 798.7e6,
                  "psp_corr": 532.5e6}
-KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, true, 8, false> (conv, event-driven path)", "spike": "slayer::spike_tile_kernel<12, 1, 12, 8>",
+KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, true, 16, false, 6> (conv; spike trains: event-driven path)", "spike": "slayer::spike_tile_kernel<12, 1, 12, 8>",
              "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
              "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_mfma_kernel<6, 20, true, false> (corr, matrix cores)"}
 
@@ -86,6 +86,55 @@ def cpu_baseline(shape, srm, ref, params, rows_fraction=1):
     return {"value": spikes.size / best, "unit": "neuron-timesteps/s", "cores": threads, "kind": "port",
             "sample": "oracle chain (conv77+spike+shift, shift+spike_bwd+corr77) on %s, median of %d passes, %.2f s each"
                       % (str(sub), len(times), best)}
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_plumbing_baseline(srm, ref, params):
+    """The reference's own CPU-runnable case, timed on the host cores: Bernoulli(0.02) spikes (4, 2, 34, 34, 300),
+    dense 2312 -> 512 as torch's conv3d with a (34, 34, 1) kernel (src/slayer.py:393-449), the PSP as a left-padded
+    conv3d with the flipped SRM kernel like pspLayer (src/slayer.py:760-791), torch on all host threads; then the
+    threshold / refractory loop by the CPU oracle.  Reported beside the GPU figures, not a target."""
+    import torch.nn.functional as F
+    from oracle import oracle as O
+    threads = os.cpu_count() or 1
+    old = torch.get_num_threads()
+    torch.set_num_threads(threads)
+    O.set_threads(O.max_threads())
+    try:
+        g = torch.Generator().manual_seed(0)
+        x = (torch.rand((4, 2, 34, 34, 300), generator=g) < 0.02).float()
+        w = torch.randn((512, 2, 34, 34, 1), generator=g) * (100.0 / 2312)
+        k = torch.from_numpy(srm[::-1].copy()).reshape(1, 1, 1, 1, -1)
+        times = {"dense_conv3d": [], "psp_conv3d": [], "spike_oracle": []}
+        for _ in range(6):
+            t0 = time.perf_counter()
+            a = F.conv3d(x, w)                                               # (4, 512, 1, 1, 300)
+            t1 = time.perf_counter()
+            u = F.conv3d(F.pad(a.reshape(4, 1, 512, 1, 300), (len(srm) - 1, 0)), k).reshape(a.shape)
+            t2 = time.perf_counter()
+            O.get_spikes(u.numpy().copy(), ref, params["theta"], 1.0)
+            t3 = time.perf_counter()
+            for name, dt in zip(times, (t1 - t0, t2 - t1, t3 - t2)):
+                times[name].append(dt)
+        med = {n: float(np.median(v[1:])) for n, v in times.items()}
+        total = sum(med.values())
+        return {"value": u.numel() / total, "unit": "neuron-timesteps/s", "cores": threads, "kind": "port",
+                "sample": "CPU plumbing case: torch conv3d dense 2312->512 + pspLayer-style conv3d PSP (77 taps) + oracle "
+                          "spike loop on (4, 2, 34, 34, 300) -> (4, 512, 1, 1, 300), median of 5 passes",
+                "seconds": med, "torch_threads": torch.get_num_threads()}
+    finally:
+        torch.set_num_threads(old)
+        O.set_threads(1)
 
 
 def copy_ceiling(x):
@@ -445,9 +494,13 @@ def other_rows(device, cpu_leg=False):
                 ts.append(a.elapsed_time(b) * 1e-3)
         return float(np.median(ts))
 
-    def row(name, ab, numel, seconds, shape):
-        return {"op": name, "shape": list(shape), "us": seconds * 1e6, "neuron_timesteps_per_s": numel / seconds,
-                "hbm_frac": ab * numel / seconds / 1e9 / HBM_PEAK_GBS}
+    def row(name, ab, numel, seconds, shape, moved=None):
+        r = {"op": name, "shape": list(shape), "us": seconds * 1e6, "neuron_timesteps_per_s": numel / seconds,
+             "hbm_frac": ab * numel / seconds / 1e9 / HBM_PEAK_GBS}
+        if moved is not None:       # a fused kernel: the bytes it really moves, next to the unfused sequence's
+            r["bytes_per_element_moved"] = moved
+            r["hbm_frac_of_bytes_moved"] = moved * numel / seconds / 1e9 / HBM_PEAK_GBS
+        return r
 
     out = []
     g = torch.Generator(device="cpu").manual_seed(2)
@@ -468,18 +521,26 @@ def other_rows(device, cpu_leg=False):
     out.append(row("psp_corr_8tap", 8, n, timed(lambda: slayerCuda.corr(grad, srm8, 1.0)), shape))
     out.append(row("spike_T2000", 12, n, timed(lambda: slayerCuda.getSpikes(ub, ref, 10.0, 1.0), lambda: ub.copy_(u0)), shape))
     del x, grad, u0, ub, y
+    # the 77-tap PSP filter over the density of its input: spike trains take the event-driven path tile by tile,
+    # denser tiles the matrix cores
+    shape = SHAPE
+    srm77 = torch.tensor(alphaKernel(10.0, 1.0, 300), dtype=torch.float32, device=device)
+    for p in (0.02, 0.05, 0.10, 0.40, None):
+        xin = (torch.randn(shape, generator=g) if p is None else (torch.rand(shape, generator=g) < p).float()).to(device)
+        out.append(row("psp_conv77_input_density_%s" % ("dense" if p is None else "%.2f" % p), 8, xin.numel(),
+                       timed(lambda: slayerCuda.conv(xin, srm77, 1.0)), shape))
+        del xin
     # MLP ordering spike(psp(fc(x))): dense input to the 77-tap PSP filter, then the spike function
     shape = SHAPE
     a = (torch.randn(shape, generator=g) * 2).to(device)
-    srm77 = torch.tensor(alphaKernel(10.0, 1.0, 300), dtype=torch.float32, device=device)
     ref11 = torch.tensor(alphaKernel(1.0, 1.0, 300, mult=-20.0), dtype=torch.float32, device=device)
     out.append(row("psp77_then_spike_fused", 20, a.numel(), timed(lambda: slayerCuda.pspSpike(a, srm77, ref11, 10.0, 1.0)),
-                   shape))
+                   shape, moved=12))
     out.append(row("psp77_then_spike_two_kernels", 20, a.numel(),
                    timed(lambda: slayerCuda.getSpikes(slayerCuda.conv(a, srm77, 1.0), ref11, 10.0, 1.0)), shape))
     gs = torch.randn(shape, generator=g).to(device)
     out.append(row("spike_pdf_then_corr77_fused", 20, a.numel(),
-                   timed(lambda: slayerCuda.spikeBackwardCorr(gs, a, srm77, 10.0, 10.0, 1.0, 1.0)), shape))
+                   timed(lambda: slayerCuda.spikeBackwardCorr(gs, a, srm77, 10.0, 10.0, 1.0, 1.0)), shape, moved=12))
     del a, gs
     # NMNIST-shaped MLP end to end (dense layers are library GEMMs): forward, spike-time loss, backward
     out.append(mlp_row(device, timed))
@@ -499,13 +560,13 @@ def other_rows(device, cpu_leg=False):
     out.append(row("loihi_forward", 16, n, timed(lambda: slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1)), shape))
     out.append(row("loihi_forward_spike_and_voltage_delay1_fused", 24, n,
                    timed(lambda: slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 1, voltage=True, current=False)),
-                   shape))
+                   shape, moved=12))
     out.append(row("loihi_forward_spike_only_delay1_fused", 24, n,
                    timed(lambda: slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 1, voltage=False, current=False)),
-                   shape))
+                   shape, moved=8))
     out.append(row("loihi_backward_pdf_plus_corr110", 20, n,
                    timed(lambda: slayerCuda.spikeBackwardCorr(gl, v, psp, 5120.0, 5120.0, 1 / 195.0, 1.0)),
-                   shape))
+                   shape, moved=12))
     return out
 
 
@@ -521,6 +582,10 @@ def main():
                          "other rows or CPU baseline")
     ap.add_argument("--cnn-only", action="store_true",
                     help="only the NMNIST CNN training step of the other rows (for profiler runs); prints that row")
+    ap.add_argument("--delay-only", action="store_true",
+                    help="only the long-sequence delay network's training step (for profiler runs); prints that row")
+    ap.add_argument("--loihi-only", action="store_true",
+                    help="only the Loihi gesture network's inference and training steps (for profiler runs); prints that row")
     ap.add_argument("--synapse-only", action="store_true",
                     help="only the per-layer synapse kernel rows (for profiler runs); prints those rows")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -538,7 +603,7 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    if args.cnn_only or args.synapse_only:
+    if args.cnn_only or args.synapse_only or args.delay_only or args.loihi_only:
         def wall(fn):
             ts = []
             for _ in range(args.warmup + args.steps):
@@ -548,7 +613,14 @@ def main():
                 torch.cuda.synchronize()
                 ts.append(time.perf_counter() - t0)
             return float(np.median(ts[args.warmup:]))
-        print(json.dumps(cnn_row(device, wall) if args.cnn_only else {"synapse_rows": synapse_rows(device, wall)}))
+        if args.cnn_only:
+            print(json.dumps(cnn_row(device, wall)))
+        elif args.delay_only:
+            print(json.dumps(delay_mlp_row(device, wall)))
+        elif args.loihi_only:
+            print(json.dumps(loihi_cnn_row(device, wall)))
+        else:
+            print(json.dumps({"synapse_rows": synapse_rows(device, wall)}))
         return
     params = neuron_params()
     srm = np.array(alphaKernel(params["tauSr"], 1.0, SHAPE[-1]), dtype=np.float32)
@@ -677,6 +749,9 @@ def main():
         if not args.no_cpu_baseline:
             # the CPU leg: the oracle as the timed baseline and as the checker of the flip rate
             result["cpu_baseline"] = cpu_baseline(SHAPE, srm, ref, params)
+            result["cpu_baseline"]["cpu_model"] = cpu_model()
+            result["cpu_baseline"]["host_cpu_count"] = os.cpu_count()
+            result["cpu_baseline_plumbing_case"] = cpu_plumbing_baseline(srm, ref, params)
             flips, rate = flip_rate(device, srm_t, ref_t, params)
             result["spike_flip_rate"] = flips
             result["spike_rate"] = rate

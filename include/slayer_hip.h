@@ -14,7 +14,9 @@
  *   - Pointers are device pointers valid on the CURRENT HIP device; the caller selects the
  *     device (the reference bindings call cudaSetDevice on the tensor's device).
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only
- *     enqueue work: no allocation, no free, no host synchronisation, no global state.
+ *     enqueue work: no allocation, no free, no host synchronisation, and no state kept between
+ *     calls - with two exceptions, both stated where they are declared: the process-wide test knob
+ *     slayer_force_generic_kernels, and the fixed device array of slayer_delay_grad_static_f32.
  *   - The library never allocates device memory.  Outputs (and the workspaces of
  *     slayer_delay_grad_f32, slayer_synapse_conv_grad_weight_f32 and slayer_spike_loss_f32) are allocated by
  *     the caller.
@@ -78,6 +80,12 @@ int slayer_get_spikes_f32(float *s, float *u, const float *nu, int64_t nNeurons,
  * out[n][t] = Ts * sum_{i=0..F-1, t-i>=0} in[n][t-i] * filt[i], accumulated in fp32 by
  * fused multiply-add in tap order i = 0,1,...  `out` must not alias `in`.  F >= 1... F == 0
  * yields zeros.
+ *
+ * Rows of whole 16-byte vectors with 34 to 129 taps: tiles of 16 rows whose input is dense (more than one
+ * 16-byte vector in five holds a non-zero sample) are computed on the matrix cores, which add the terms in
+ * another order than the sequential loop: those results agree with it to rounding (every output within
+ * 1e-5 of the sum of the magnitudes of its own terms; measured about 1e-7 of the largest output).  Tiles of
+ * spike trains (almost all zeros) and all other shapes match the fused-multiply-add loop bit for bit.
  */
 int slayer_conv_f32(float *out, const float *in, const float *filt, int64_t nNeurons, int64_t T,
                     int64_t F, float Ts, void *stream);
@@ -141,8 +149,10 @@ int slayer_spike_bwd_f32(float *gradIn, const float *gradOut, const float *u, fl
  *
  * gradIn[n][t] = Ts * sum_{i<F} [t+i < T] w[n][t+i] * filt[i],
  * w[n][t]      = gradOut[n][t] * (scale / tau) * exp(-|u[n][t] - theta| / tau).
- * The values of slayer_spike_bwd_f32 followed by the sequential correlation loop (bit for bit, always
- * as a fused-multiply-add chain), without the intermediate tensor.  gradIn must not alias the inputs.  tau must be non-zero.
+ * The values of slayer_spike_bwd_f32 followed by slayer_corr_f32, without the intermediate tensor: rows of
+ * whole 16-byte vectors with 34 to 129 taps are summed on the matrix cores and agree with the sequential
+ * fused-multiply-add loop to rounding (1e-5, as for slayer_corr_f32), all other shapes bit for bit.
+ * gradIn must not alias the inputs.  tau must be non-zero.
  */
 int slayer_spike_bwd_corr_f32(float *gradIn, const float *gradOut, const float *u,
                               const float *filt, int64_t nNeurons, int64_t T, int64_t F,
@@ -154,10 +164,12 @@ int slayer_spike_bwd_corr_f32(float *gradIn, const float *gradOut, const float *
  * (example/02_NMNIST_MLP/nmnistMLP.py:59-60).  Replaces the call pair slayerCuda.conv
  * (src/cuda/slayerKernels.cu:41-57) -> slayerCuda.getSpikes (src/cuda/slayerKernels.cu:14-39).
  *
- * u = Ts * conv(a, srm) as in slayer_conv_f32, then s and the refractory update of u as in
- * slayer_get_spikes_f32: the same values bit for bit, without the round trip of u through
- * memory when rows are whole 16-byte vectors of at most 352 samples, nuSize <= 24 and F <= 160;
- * other shapes run the two kernels one after the other.  u and s must not alias a.
+ * u = Ts * conv(a, srm), then s and the refractory update of u as in slayer_get_spikes_f32, without
+ * the round trip of u through memory when rows are whole 16-byte vectors of at most 352 samples,
+ * nuSize <= 24 and F <= 160: the filter then runs as the sequential fused-multiply-add loop for every
+ * input (the reference's bits; slayer_conv_f32 on its own may sum a dense input on the matrix cores and
+ * differ in the last bit).  Other shapes run the two kernels one after the other.  u and s must not
+ * alias a.
  */
 int slayer_psp_spike_f32(float *s, float *u, const float *a, const float *srm, const float *nu,
                          int64_t nNeurons, int64_t T, int64_t F, int64_t nuSize, float theta,

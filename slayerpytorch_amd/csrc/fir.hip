@@ -219,7 +219,7 @@ __device__ __forceinline__ void fir_sparse_tile(const BufferRsrc &bufOut, const 
 // DM: 0 = dense tiles run the register-window chains; 4..9 = dense tiles run on the matrix cores with a window
 //     of DM blocks of 16 samples (VEC, U = 16, R = 16 rows, LD >= tile + 16 (DM - 1))
 template <bool CAUSAL, bool VEC, int U, bool GATED, int DM>
-__global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
+__global__ __launch_bounds__(256, DM > 0 ? 2 : 1) void fir_tiled_kernel(float *__restrict__ out,
                                                         const float *__restrict__ in,
                                                         const float *__restrict__ filt,
                                                         int64_t rows, int T, int F, int TT, int LD, int R,
@@ -255,22 +255,30 @@ __global__ __launch_bounds__(256) void fir_tiled_kernel(float *__restrict__ out,
         const int nq = (tB - tA) >> 2;               // source vectors per row
         const int jA = CAUSAL ? (tHi + 1 - tB) : 0;  // X columns [jA, jA + 4 nq) receive them
         {
-            RowCol rc;
-            rc.init(tid, nq, 1.0f / static_cast<float>(nq));
+            // vector g of the tile is vector g % nq of row g / nq; a lane's vectors are 256 apart, so its source and
+            // destination offsets move by a fixed step plus a correction whenever the column wraps into the next row
+            int r, col;
+            divmod_small(tid, nq, 1.0f / static_cast<float>(nq), r, col);
             const int dr = 256 / nq, dc = 256 % nq;
             const int total = nRows * nq;
-            for (int g = tid; g < total; g += 256, rc.advance(dr, dc, nq)) {
-                float4 v = buffer_load4(bufIn, (rc.r * T + tA + (rc.c << 2)) * 4, 0);
+            int src = (r * T + tA + (col << 2)) * 4;
+            int dst = (r * LD + (CAUSAL ? jA + ((nq - 1 - col) << 2) : (col << 2))) * 4;
+            const int srcStep = (dr * T + dc * 4) * 4, srcWrap = srcStep + (T - nq * 4) * 4;
+            const int dstStep = (dr * LD + (CAUSAL ? -dc : dc) * 4) * 4, dstWrap = dstStep + (LD + (CAUSAL ? nq : -nq) * 4) * 4;
+            for (int g = tid; g < total; g += 256) {
+                float4 v = buffer_load4(bufIn, src, 0);
                 if (GATED) {
-                    const float4 g = buffer_load4(bufGate, (rc.r * T + tA + (rc.c << 2)) * 4, 0);
+                    const float4 g = buffer_load4(bufGate, src, 0);
                     v = make_float4(gated(v.x, g.x), gated(v.y, g.y), gated(v.z, g.z), gated(v.w, g.w));
                 }
                 nonZero += __builtin_popcountll(__ballot(any_nonzero(v)));
-                if (CAUSAL)  // descending time: the vector lands mirrored
-                    *reinterpret_cast<float4 *>(X + rc.r * LD + (jA + ((nq - 1 - rc.c) << 2))) =
-                        make_float4(v.w, v.z, v.y, v.x);
-                else
-                    *reinterpret_cast<float4 *>(X + rc.r * LD + (rc.c << 2)) = v;
+                // (convolution: descending time, the vector lands mirrored)
+                *reinterpret_cast<float4 *>(reinterpret_cast<char *>(X) + dst) = CAUSAL ? make_float4(v.w, v.z, v.y, v.x) : v;
+                col += dc;
+                const bool wrap = col >= nq;
+                if (wrap) col -= nq;
+                src += wrap ? srcWrap : srcStep;
+                dst += wrap ? dstWrap : dstStep;
             }
         }
         // zero padding: columns [0, jA) and [jA + 4 nq, LD)
