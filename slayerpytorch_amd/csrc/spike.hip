@@ -138,20 +138,27 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
 // The fast path.  A wavefront owns R consecutive rows and moves them through LDS in
 // pieces of Tc samples per row (the whole row when it is short enough), so that global memory
 // is read and written as long contiguous runs with 16-byte accesses per lane - the access
-// pattern of a plain copy.  Lanes 0..R-1 then walk their row in LDS order:
-// 32 samples at a time are pulled into a register window v[0 .. 32+LAG), a spike adds
-// nu[0..NU) onto v[k .. k+NU) (the same fp32 additions, in the same order, as the sequential
-// loop), and the 32 oldest samples go back to LDS together with a 32-bit spike mask.  The last
-// LAG samples of a piece are not final until the next piece arrives; they wait in v[0..LAG).
-// Taps beyond nuSize are -0.0f, whose addition changes no value; slots before the first and
-// after the last sample hold NaN, which never reaches the threshold.
+// pattern of a plain copy.  The sequential part then works in LDS, lane = row:
+//  * a refractory kernel without positive taps (the normal case) can only lower the potential, so a sample
+//    that arrives below the threshold never fires.  All 64 lanes mark the samples at or above it
+//    ("candidates", a few per cent) while the piece is staged, one bit per sample, and the walking lanes go from
+//    candidate to candidate: test the sample's current value and, on a spike, add nu[0..NU) onto the NU samples
+//    from it on, in place - the same fp32 additions in the same order as the sequential loop;
+//  * any other kernel: every sample in turn, also in place.
+// The last LAG samples of a piece are not final until the next piece arrives: they (and their candidate bits)
+// are copied to the front of the tile and open the next piece.  Taps beyond nuSize are -0.0f, whose addition
+// changes no value; a response may reach past the row's end into padding that is never stored.
 // Leaving most lanes idle during the walk is deliberate: the kernel is bound by HBM traffic,
 // not by the vector ALU, and short tiles keep many wavefronts (and bytes) in flight per CU.
-constexpr int kTileMaxPiece = 352;  // longest piece (samples per row) a tile stages at once
+constexpr int kTileMaxPiece = 352;  // longest row (samples) that travels whole
+// Rows in pieces: samples per piece and row.  With 8-row tiles - tensors of few, long rows - the bytes in flight
+// per compute unit are what the rows in LDS amount to, so those pieces are longer.
+constexpr int kTilePiece16 = 256, kTilePiece8 = 512;
 
-// LAG: look-ahead of the walk in samples (>= NU - 1, whole 16-byte vectors).  The samples that
-// leave a piece are the ones LAG before its end, so with several pieces per row LAG = 32 keeps
-// every run of stores on 128-byte boundaries of the row (partial lines are expensive to write).
+// LAG: samples of a piece that stay behind for the next one (>= NU - 1, whole 16-byte vectors; 32 = one word of
+// candidate bits for rows in pieces).  The samples that leave a piece are the ones LAG before its end, so with
+// several pieces per row LAG = 32 keeps every run of stores on 128-byte boundaries of the row (partial lines
+// are expensive to write).
 // R: rows per tile (16, or 8 when the tensor has too few rows to fill the GPU with 16-row tiles).
 // MODE: how global memory is accessed.  kTileVec: rows are whole 16-byte vectors.  kTileFlat:
 // they are not (T % 4 != 0), but the rows of a tile travel whole and an 8-row tile is one
@@ -182,11 +189,14 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     constexpr int G = 32;               // samples per walk group = bits of a spike mask
     constexpr bool VEC = MODE == kTileVec, FLAT = MODE == kTileFlat;
     constexpr int V = VEC ? 4 : 1;      // samples per (row-wise) global access
-    constexpr int NB = R * kTileMaxPiece / (FLAT ? 4 : V) / kWave;  // accesses per lane per piece, at most
+    // longest piece this instance stages (LAG = 32 marks the instances for rows in pieces)
+    constexpr int kPiece = (LAG == 32 && VEC) ? (R == 8 ? kTilePiece8 : kTilePiece16) : kTileMaxPiece;
+    constexpr int NB = R * kPiece / (FLAT ? 4 : V) / kWave;  // accesses per lane per piece, at most
     extern __shared__ __align__(16) float lds[];
     float *tile = lds;                                                    // [R][P], P = 4 (mod 32)
     uint32_t *masks = reinterpret_cast<uint32_t *>(lds + R * P);  // [R][MP]
     int *rowShift = reinterpret_cast<int *>(masks + R * MP);      // [R], used when the output is shifted
+    uint32_t *cand = reinterpret_cast<uint32_t *>(rowShift + R);  // [R][MP], candidate samples (see below)
 
     const int lane = threadIdx.x;
     const float amplitude = 1.0f / Ts;
@@ -195,8 +205,17 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     float tap[NU];
 #pragma unroll
     for (int j = 0; j < NU; ++j) tap[j] = (j < nuSize) ? nu[j] : -0.0f;
-
-    float v[G + LAG];
+    // The normal refractory kernel only lowers the potential (every tap <= 0; a NaN tap fails the test).  A sample
+    // below the threshold as it arrives can then never fire, so the sequential part need only visit the samples
+    // at or above it ("candidates", a few per cent): all 64 lanes mark them while the tile is staged, and the
+    // walking lanes go from candidate to candidate, test the sample's current value and add the refractory
+    // response in place in LDS - the same fp32 additions in the same order as the sequential loop.
+    bool monotone = true;
+#pragma unroll
+    for (int j = 0; j < NU; ++j) monotone = monotone && tap[j] <= 0.0f;
+    auto mark = [&](int r, int col, float x) {  // one sample
+        if (x >= theta) atomicOr(cand + r * MP + (col >> 5), 1u << (col & 31));
+    };
 
     // A "step" is one piece of one tile.  The global loads of a step are issued one step ahead
     // into x[] and stay in flight while the previous step is walked and retired.
@@ -222,14 +241,14 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         const int dr = kWave / perRow, dc = kWave % perRow;
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            if (lane + b * kWave < total) {
-                const int off = (rc.r * T + tL + rc.c * V) * 4;
-                if (VEC) {
-                    const float4 q = buffer_load4(bufU, off, 0);
-                    x[4 * b] = q.x; x[4 * b + 1] = q.y; x[4 * b + 2] = q.z; x[4 * b + 3] = q.w;
-                } else {
-                    x[b] = buffer_load(bufU, off, 0);
-                }
+            const int off = (rc.r * T + tL + rc.c * V) * 4;
+            if constexpr (VEC) {
+                // (masked, not skipped: a fixed number of loads lets the wait for them leave the stores that
+                // are issued behind them in flight)
+                const float4 q = buffer_load4(bufU, masked_offset(lane + b * kWave < total, off), 0);
+                x[4 * b] = q.x; x[4 * b + 1] = q.y; x[4 * b + 2] = q.z; x[4 * b + 3] = q.w;
+            } else if (lane + b * kWave < total) {
+                x[b] = buffer_load(bufU, off, 0);
             }
             rc.advance(dr, dc, perRow);
         }
@@ -245,6 +264,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         tile[r * P + LAG + c] = x[4 * b + e];
+                        if (monotone) mark(r, LAG + c, x[4 * b + e]);
                         if (++c == T) { c = 0; ++r; }
                     }
                 }
@@ -261,8 +281,18 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         for (int b = 0; b < NB; ++b) {
             if (lane + b * kWave < total) {
                 float *dst = tile + rc.r * P + LAG + rc.c * V;
-                if (VEC) *reinterpret_cast<float4 *>(dst) = make_float4(x[4 * b], x[4 * b + 1], x[4 * b + 2], x[4 * b + 3]);
-                else *dst = x[b];
+                if (VEC) {
+                    *reinterpret_cast<float4 *>(dst) = make_float4(x[4 * b], x[4 * b + 1], x[4 * b + 2], x[4 * b + 3]);
+                    if (monotone) {  // (the column is a multiple of 4: the four bits lie in one word)
+                        const uint32_t bits = (x[4 * b] >= theta ? 1u : 0u) | (x[4 * b + 1] >= theta ? 2u : 0u) |
+                                              (x[4 * b + 2] >= theta ? 4u : 0u) | (x[4 * b + 3] >= theta ? 8u : 0u);
+                        const int col = LAG + rc.c * V;
+                        if (bits) atomicOr(cand + rc.r * MP + (col >> 5), bits << (col & 31));
+                    }
+                } else {
+                    *dst = x[b];
+                    if (monotone) mark(rc.r, LAG + rc.c, x[b]);
+                }
             }
             rc.advance(dr, dc, perRow);
         }
@@ -271,65 +301,75 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     int64_t t = blockIdx.x;
     int tL = 0;
     if (t < tiles) issue(t, tL);
+    for (int i = lane; i < R * MP; i += kWave) cand[i] = 0u;
+    wave_sync();
+    if (t < tiles) commit(t, tL);
+    // One trip = one step.  The next step's loads are issued first, this step's stores follow, and the next step's
+    // samples are committed to LDS at the end of the same trip: loads, stores and the wait for the loads lie in one
+    // straight line, so that wait can leave the younger stores in flight (their number is fixed: masked, never
+    // skipped).  issue() and commit() of a step beyond the last tile do nothing.
     while (t < tiles) {
         const int nRows = rows_of(t);
         const int n = min(Tc, T - tL);  // new samples per row in this piece
         const bool last = tL + n == T;
         const int tW = tL - LAG;        // time of tile column 0 (columns [0, LAG) are carried over)
+        const int64_t tn = last ? t + gridDim.x : t;  // next step: next piece of this tile, or first piece of the next
+        const int tLn = last ? 0 : tL + Tc;
 
-        commit(t, tL);
         wave_sync();
-        {   // next step: next piece of this tile, or first piece of this group's next tile
-            const int64_t tn = last ? t + gridDim.x : t;
-            const int tLn = last ? 0 : tL + Tc;
-            if (tn < tiles) issue(tn, tLn);
-        }
+        issue(tn, tLn);
 
         // ---- walk: lane = row.  Columns [0, W) become final in this step.
         const int W = last ? n + LAG : n;
-        if (lane < R) {
-            float *mine = tile + lane * P;
-            if (tL == 0) {
+        if (monotone) {
+            // lane = row; every lane keeps its own place in its row's candidate words (lanes without a row have none)
+            const int words = lane < R ? (W + 31) >> 5 : 0;
+            const uint32_t *cw = cand + (lane < R ? lane : 0) * MP;
+            uint32_t *mw = masks + (lane < R ? lane : 0) * MP;
+            float *mine = tile + (lane < R ? lane : 0) * P;
+            int w = 0;
+            uint32_t cm = words > 0 ? cw[0] : 0u, fired = 0u;
+            for (;;) {
+                while (cm == 0u && w + 1 < words) {
+                    mw[w] = fired;
+                    fired = 0u;
+                    ++w;
+                    cm = cw[w];
+                }
+                if (__builtin_amdgcn_ballot_w64(cm != 0u) == 0) break;
+                if (cm != 0u) {
+                    const int k = __builtin_ctz(cm);
+                    cm &= cm - 1u;
+                    float *q = mine + (w << 5) + k;
+                    if (q[0] >= theta) {
+                        fired |= 1u << k;
 #pragma unroll
-                for (int k = 0; k < LAG; ++k) v[k] = quiet;
+                        for (int j = 0; j < NU; ++j) q[j] += tap[j];
+                    }
+                }
             }
-            const int groups = (W + G - 1) / G;
-            for (int g = 0; g < groups; ++g) {
-                const int c0 = g * G;
-                if (c0 + G <= n) {
-#pragma unroll
-                    for (int k = 0; k < G; k += 4) {
-                        const float4 q = *reinterpret_cast<const float4 *>(mine + LAG + c0 + k);
-                        v[LAG + k] = q.x; v[LAG + k + 1] = q.y; v[LAG + k + 2] = q.z; v[LAG + k + 3] = q.w;
-                    }
-                } else {
-#pragma unroll
-                    for (int k = 0; k < G; ++k) v[LAG + k] = (c0 + k < n) ? mine[LAG + c0 + k] : quiet;
-                }
+            if (words > 0) mw[w] = fired;
+        } else if (lane < R) {
+            // a refractory kernel that can raise the potential: every sample in turn, in place in LDS
+            float *mine = tile + lane * P;
+            const int begin = (tL == 0) ? LAG : 0;  // (before the first sample lies nothing)
+            for (int c0 = 0; c0 < W; c0 += G) {
                 uint32_t fired = 0;
+                for (int k = 0; k < G; k += 4) {
+                    float4 q = *reinterpret_cast<const float4 *>(mine + c0 + k);
 #pragma unroll
-                for (int k = 0; k < G; k += 2) {
-                    // One scalar branch per two samples: in most pairs no row spikes.  (The second
-                    // sample is tested again inside, after the first one's refractory response.)
-                    if (__builtin_amdgcn_ballot_w64((v[k] >= theta) | (v[k + 1] >= theta)) != 0) {
-                        if (v[k] >= theta) {
-                            fired |= 1u << k;
+                    for (int e = 0; e < 4; ++e) {
+                        const int col = c0 + k + e;
+                        const float val = e == 0 ? q.x : e == 1 ? q.y : e == 2 ? q.z : q.w;
+                        if (col >= begin && col < W && val >= theta) {
+                            fired |= 1u << (k + e);
 #pragma unroll
-                            for (int j = 0; j < NU; ++j) v[k + j] += tap[j];
-                        }
-                        if (v[k + 1] >= theta) {
-                            fired |= 2u << k;
-#pragma unroll
-                            for (int j = 0; j < NU; ++j) v[k + 1 + j] += tap[j];
+                            for (int j = 0; j < NU; ++j) mine[col + j] += tap[j];
+                            q = *reinterpret_cast<const float4 *>(mine + c0 + k);
                         }
                     }
                 }
-#pragma unroll
-                for (int k = 0; k < G; k += 4)
-                    *reinterpret_cast<float4 *>(mine + c0 + k) = make_float4(v[k], v[k + 1], v[k + 2], v[k + 3]);
-                masks[lane * MP + g] = fired;
-#pragma unroll
-                for (int k = 0; k < LAG; ++k) v[k] = v[G + k];
+                masks[lane * MP + (c0 >> 5)] = fired;
             }
         }
         wave_sync();
@@ -380,29 +420,53 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
             RowCol rc;
             rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
             const int dr = kWave / perRow, dc = kWave % perRow;
-#pragma unroll 4
-            for (int g0 = lane; g0 < total; g0 += kWave) {
-                const int col = first + rc.c * V;
-                const int off = (rc.r * T + tW + col) * 4;
-                const float *src = tile + rc.r * P + col;
-                const uint32_t m = dl.on ? bits_from(rc.r, col) : masks[rc.r * MP + (col >> 5)] >> (col & 31);
-                if (VEC) {
+            if constexpr (VEC) {
+                // a fixed number of (masked) stores, see above
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    const bool on = lane + b * kWave < total;
+                    const int r = on ? rc.r : 0, col = on ? first + rc.c * V : first;
+                    const float *src = tile + r * P + col;
+                    const uint32_t m = dl.on ? bits_from(r, col) : masks[r * MP + (col >> 5)] >> (col & 31);
+                    const int off = masked_offset(on, (r * T + tW + col) * 4);
                     buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(src));
                     buffer_store4(bufS, off, 0,
                                   make_float4((m & 1u) ? amplitude : 0.0f, (m & 2u) ? amplitude : 0.0f,
                                               (m & 4u) ? amplitude : 0.0f, (m & 8u) ? amplitude : 0.0f));
-                } else {
+                    rc.advance(dr, dc, perRow);
+                }
+            } else {
+#pragma unroll 4
+                for (int g0 = lane; g0 < total; g0 += kWave) {
+                    const int col = first + rc.c * V;
+                    const int off = (rc.r * T + tW + col) * 4;
+                    const float *src = tile + rc.r * P + col;
+                    const uint32_t m = dl.on ? bits_from(rc.r, col) : masks[rc.r * MP + (col >> 5)] >> (col & 31);
                     buffer_store(bufU, off, 0, src[0]);
                     buffer_store(bufS, off, 0, (m & 1u) ? amplitude : 0.0f);
+                    rc.advance(dr, dc, perRow);
                 }
-                rc.advance(dr, dc, perRow);
             }
             }
         }
         wave_sync();
 
-        if (last) { t += gridDim.x; tL = 0; }
-        else tL += Tc;
+        // rows in pieces: the LAG columns behind this piece's final ones, and their candidates, open the next
+        // piece (LAG is one word of candidates then); every other word of candidates starts empty
+        if (!last) {
+            for (int i = lane; i < R * (LAG / 4); i += kWave) {
+                const int r = i / (LAG / 4), c4 = i - r * (LAG / 4);
+                *reinterpret_cast<float4 *>(tile + r * P + 4 * c4) = *reinterpret_cast<const float4 *>(tile + r * P + n + 4 * c4);
+            }
+            if (lane < R) cand[lane * MP] = cand[lane * MP + (n >> 5)];
+            wave_sync();
+        }
+        for (int i = lane; i < R * MP; i += kWave)
+            if (last || i % MP != 0) cand[i] = 0u;
+        wave_sync();
+        commit(tn, tLn);
+        t = tn;
+        tL = tLn;
     }
 }
 
@@ -501,16 +565,28 @@ static int launch_get_spikes(float *s, float *u, const float *nu, int64_t nNeuro
     } while (0)
 #define SLAYER_SPIKE_TILE_LAG(NU, LAGV)                                                                  \
     do {                                                                                                \
-        const int cols = (LAGV + Tc + 31) & ~31; /* the walk goes in groups of 32 columns */            \
-        const int P = cols + 4; /* 4 (mod 32): rows are 16-byte aligned and start in different banks */ \
-        const int MP = cols / 32 + 1;                                                                   \
         /* Rows that travel whole: 8-row tiles, one work-group per tile - many short-lived groups per   \
            CU overlap the memory phases of some with the walks of others better than a loop does.       \
-           Rows in pieces: the group loops over the pieces; 16 rows per tile unless that would leave    \
-           wavefront slots of the GPU empty. */                                                         \
-        const int64_t slots16 = static_cast<int64_t>(cus) * (160 * 1024 / ((16LL * P + 16 * MP) * 4));  \
+           Rows in pieces: the group loops over the pieces; 16 rows per tile and pieces of 256 samples  \
+           unless that would leave wavefront slots of the GPU empty: then 8 rows and, for rows of whole \
+           vectors, pieces of 512 samples, which doubles the bytes in flight per wavefront. */          \
+        int Tc = whole ? static_cast<int>(T) : kTilePiece16;                                            \
+        int cols, P, MP;                                                                                \
+        auto layout = [&]() {                                                                           \
+            cols = (LAGV + Tc + 31) & ~31; /* the walk goes in groups of 32 columns */                  \
+            /* 4 (mod 32): rows are 16-byte aligned and start in different banks; a refractory response \
+               that is added in place may reach NU - 1 columns past the last one */                    \
+            P = cols + 4 + ((cols + 4 - (LAGV + Tc) < NU - 1) ? 32 : 0);                                \
+            MP = cols / 32 + 1;                                                                         \
+        };                                                                                              \
+        layout();                                                                                       \
+        const int64_t slots16 = static_cast<int64_t>(cus) * (160 * 1024 / ((16LL * P + 32 * MP + 16) * 4)); \
         const int rowsPerTile = (!whole && ceil_div(nNeurons, 16) >= slots16) ? 16 : 8;                 \
-        const size_t lds = (static_cast<size_t>(rowsPerTile) * P + rowsPerTile * MP + rowsPerTile) * sizeof(float); \
+        if (!whole && rowsPerTile == 8 && vec) {                                                        \
+            Tc = kTilePiece8;                                                                           \
+            layout();                                                                                   \
+        }                                                                                               \
+        const size_t lds = (static_cast<size_t>(rowsPerTile) * P + 2 * rowsPerTile * MP + rowsPerTile) * sizeof(float); \
         const int64_t tiles = ceil_div(nNeurons, rowsPerTile);                                          \
         const int64_t resident = static_cast<int64_t>(cus) * (160 * 1024 / static_cast<int64_t>(lds));  \
         if (tiles >= (1LL << 31)) return SLAYER_EUNSUPPORTED;                                           \
@@ -525,9 +601,8 @@ static int launch_get_spikes(float *s, float *u, const float *nu, int64_t nNeuro
     } while (0)
     if (dl.on && !(window_ok && nuSize <= 24 && T <= kTileMaxPiece)) return SLAYER_EUNSUPPORTED;
     if (window_ok && nuSize <= 24) {
-        // short rows travel whole; long rows in pieces of 256 samples (1 KiB per row)
+        // short rows travel whole; long rows in pieces
         const bool whole = T <= kTileMaxPiece;
-        const int Tc = whole ? static_cast<int>(T) : 256;
         const bool vec = (T % 4 == 0) && aligned16(s) && aligned16(u);
         // whole rows that are not whole vectors, in a tensor that is: 8-row tiles are aligned runs
         const bool flat = whole && !vec && T >= 4 && (nNeurons * T) % 4 == 0 && aligned16(s) && aligned16(u);
