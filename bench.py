@@ -284,9 +284,13 @@ def delay_mlp_row(device, timed):
         s1 = d1(layer.spike(layer.psp(fc1(x))))
         scale_weights_to_rate(fc2.weight, lambda: float(layer.spike(layer.psp(fc2(s1))).mean()))
 
-    def step():
-        s1 = d1(layer.spike(layer.psp(fc1(x))))
-        s2 = d2(layer.spike(layer.psp(fc2(s1))))
+    def step(fused=True):
+        if fused:   # delay(spike(u)) from one kernel each way (the spikes are shifted while they are stored)
+            s1 = layer.spikeDelayed(layer.psp(fc1(x)), d1)
+            s2 = layer.spikeDelayed(layer.psp(fc2(s1)), d2)
+        else:
+            s1 = d1(layer.spike(layer.psp(fc1(x))))
+            s2 = d2(layer.spike(layer.psp(fc2(s1))))
         del rates[:]
         rates.extend((s1, s2))
         error.spikeTime(s2, target).backward()
@@ -295,8 +299,10 @@ def delay_mlp_row(device, timed):
         for m in (d1, d2):
             m.delay.grad = None
 
+    two = timed(lambda: step(False))
     t = timed(step)
     return {"op": "delay_mlp_200_256_200_fwd_loss_bwd", "shape": [64, 200, 1, 1, 2000], "us": t * 1e6,
+            "us_with_separate_spike_and_delay_calls": two * 1e6,
             "samples_per_s": 64 / t, "spike_rate_per_layer": [round(float(r.detach().mean()), 4) for r in rates]}
 
 
@@ -473,26 +479,34 @@ def event_row(device, timed, cpu_leg):
 
 def other_rows(device, cpu_leg=False):
     """Quick per-op measurements of the scope rows that are not part of the headline chain, each on
-    the largest tensor its benchmark configuration gives it (median of 7 event-timed launches).  hbm_frac
+    the largest tensor its benchmark configuration gives it (kernel rows: median of 7 event-timed passes of 8
+    launches back to back; network steps: median of 7 event-timed steps).  hbm_frac
     counts the algorithmic bytes of the unfused reference sequence (Loihi forward + delayShift:
     16 + 8 B, Loihi backward: 12 + 8 B), also where one fused kernel moves fewer."""
     from slayerpytorch_amd import slayerCuda, slayerLoihiCuda
     from slayerpytorch_amd.slayer import alphaKernel
     from slayerpytorch_amd.slayerLoihi import loihiPspKernel
 
-    def timed(fn, setup=None):
+    def timed(fn, burst=1, args=None):
+        """Median over 7 event-timed passes of the time per call; a pass is `burst` calls back to back (kernel rows:
+        8, so that the few microseconds an event pair costs do not count as kernel time), each with its own
+        argument from `args` when the op works in place."""
         ts = []
         for i in range(10):
-            if setup:
-                setup()
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            if args is not None:
+                args[1]()                      # restore the in-place operands (untimed)
+                torch.cuda.synchronize()
             a.record()
-            fn()
+            for k in range(burst):
+                fn(args[0][k]) if args is not None else fn()
             b.record()
             torch.cuda.synchronize()
             if i >= 3:
-                ts.append(a.elapsed_time(b) * 1e-3)
+                ts.append(a.elapsed_time(b) * 1e-3 / burst)
         return float(np.median(ts))
+
+    K = 8
 
     def row(name, ab, numel, seconds, shape, moved=None):
         r = {"op": name, "shape": list(shape), "us": seconds * 1e6, "neuron_timesteps_per_s": numel / seconds,
@@ -515,12 +529,16 @@ def other_rows(device, cpu_leg=False):
     ub = u0.clone()
     n = x.numel()
     y = slayerCuda.shift(x, lut, 1.0)
-    out.append(row("shift_per_neuron_table", 8, n, timed(lambda: slayerCuda.shift(x, lut, 1.0)), shape))
-    out.append(row("delay_gradient", 8, n, timed(lambda: slayerCuda.delayGrad(y, grad, 1.0)), shape))
-    out.append(row("psp_conv_8tap", 8, n, timed(lambda: slayerCuda.conv(x, srm8, 1.0)), shape))
-    out.append(row("psp_corr_8tap", 8, n, timed(lambda: slayerCuda.corr(grad, srm8, 1.0)), shape))
-    out.append(row("spike_T2000", 12, n, timed(lambda: slayerCuda.getSpikes(ub, ref, 10.0, 1.0), lambda: ub.copy_(u0)), shape))
-    del x, grad, u0, ub, y
+    out.append(row("shift_per_neuron_table", 8, n, timed(lambda: slayerCuda.shift(x, lut, 1.0), K), shape))
+    out.append(row("delay_gradient", 8, n, timed(lambda: slayerCuda.delayGrad(y, grad, 1.0), K), shape))
+    out.append(row("psp_conv_8tap", 8, n, timed(lambda: slayerCuda.conv(x, srm8, 1.0), K), shape))
+    out.append(row("psp_corr_8tap", 8, n, timed(lambda: slayerCuda.corr(grad, srm8, 1.0), K), shape))
+    pool = [u0.clone() for _ in range(K)]
+    restore = lambda: [p.copy_(u0) for p in pool]
+    out.append(row("spike_T2000", 12, n, timed(lambda u: slayerCuda.getSpikes(u, ref, 10.0, 1.0), K, (pool, restore)), shape))
+    out.append(row("spike_T2000_then_per_neuron_delay_fused", 20, n,
+                   timed(lambda u: slayerCuda.getSpikesDelayed(u, ref, 10.0, 1.0, lut, 1.0), K, (pool, restore)), shape, moved=12))
+    del x, grad, u0, ub, y, pool
     # the 77-tap PSP filter over the density of its input: spike trains take the event-driven path tile by tile,
     # denser tiles the matrix cores
     shape = SHAPE
@@ -528,19 +546,19 @@ def other_rows(device, cpu_leg=False):
     for p in (0.02, 0.05, 0.10, 0.40, None):
         xin = (torch.randn(shape, generator=g) if p is None else (torch.rand(shape, generator=g) < p).float()).to(device)
         out.append(row("psp_conv77_input_density_%s" % ("dense" if p is None else "%.2f" % p), 8, xin.numel(),
-                       timed(lambda: slayerCuda.conv(xin, srm77, 1.0)), shape))
+                       timed(lambda: slayerCuda.conv(xin, srm77, 1.0), K), shape))
         del xin
     # MLP ordering spike(psp(fc(x))): dense input to the 77-tap PSP filter, then the spike function
     shape = SHAPE
     a = (torch.randn(shape, generator=g) * 2).to(device)
     ref11 = torch.tensor(alphaKernel(1.0, 1.0, 300, mult=-20.0), dtype=torch.float32, device=device)
-    out.append(row("psp77_then_spike_fused", 20, a.numel(), timed(lambda: slayerCuda.pspSpike(a, srm77, ref11, 10.0, 1.0)),
+    out.append(row("psp77_then_spike_fused", 20, a.numel(), timed(lambda: slayerCuda.pspSpike(a, srm77, ref11, 10.0, 1.0), K),
                    shape, moved=12))
     out.append(row("psp77_then_spike_two_kernels", 20, a.numel(),
-                   timed(lambda: slayerCuda.getSpikes(slayerCuda.conv(a, srm77, 1.0), ref11, 10.0, 1.0)), shape))
+                   timed(lambda: slayerCuda.getSpikes(slayerCuda.conv(a, srm77, 1.0), ref11, 10.0, 1.0), K), shape))
     gs = torch.randn(shape, generator=g).to(device)
     out.append(row("spike_pdf_then_corr77_fused", 20, a.numel(),
-                   timed(lambda: slayerCuda.spikeBackwardCorr(gs, a, srm77, 10.0, 10.0, 1.0, 1.0)), shape, moved=12))
+                   timed(lambda: slayerCuda.spikeBackwardCorr(gs, a, srm77, 10.0, 10.0, 1.0, 1.0), K), shape, moved=12))
     del a, gs
     # NMNIST-shaped MLP end to end (dense layers are library GEMMs): forward, spike-time loss, backward
     out.append(mlp_row(device, timed))
@@ -557,15 +575,15 @@ def other_rows(device, cpu_leg=False):
     psp = torch.tensor(loihiPspKernel(1024, 128, 0), dtype=torch.float32, device=device)
     n = w.numel()
     s, v, u = slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1)
-    out.append(row("loihi_forward", 16, n, timed(lambda: slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1)), shape))
+    out.append(row("loihi_forward", 16, n, timed(lambda: slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1), K), shape))
     out.append(row("loihi_forward_spike_and_voltage_delay1_fused", 24, n,
-                   timed(lambda: slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 1, voltage=True, current=False)),
+                   timed(lambda: slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 1, voltage=True, current=False), K),
                    shape, moved=12))
     out.append(row("loihi_forward_spike_only_delay1_fused", 24, n,
-                   timed(lambda: slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 1, voltage=False, current=False)),
+                   timed(lambda: slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 1, voltage=False, current=False), K),
                    shape, moved=8))
     out.append(row("loihi_backward_pdf_plus_corr110", 20, n,
-                   timed(lambda: slayerCuda.spikeBackwardCorr(gl, v, psp, 5120.0, 5120.0, 1 / 195.0, 1.0)),
+                   timed(lambda: slayerCuda.spikeBackwardCorr(gl, v, psp, 5120.0, 5120.0, 1 / 195.0, 1.0), K),
                    shape, moved=12))
     return out
 

@@ -183,9 +183,11 @@ int slayer_psp_spike_f32(float *s, float *u, const float *a, const float *srm, c
  *
  * s[t] = spike[t - k] with k = (int)(d / delayTs) (0 where t - k is outside the row); d is
  * delayLut[neuron % lutSize] when delayLut is given (one delay per neuron of a batch item, nNeurons a
- * multiple of lutSize) and `delay` otherwise.  `u` is updated in place and NOT shifted, exactly as by
- * slayer_get_spikes_f32.  Only rows that the tile kernel moves whole are fused (T <= 352, nuSize <= 24);
- * other shapes return SLAYER_EUNSUPPORTED with nothing launched - call the two functions then.
+ * multiple of lutSize) and `delay` otherwise, of any size and sign.  `u` is updated in place and NOT shifted,
+ * exactly as by slayer_get_spikes_f32.  Fused shapes: nuSize <= 24 and rows of at most 352 samples, or longer
+ * rows of whole 16-byte vectors up to 16384 samples (those travel in pieces: the kernel keeps the spike bits
+ * of the whole row and stores the shifted spikes behind the row's last piece).  Other shapes return
+ * SLAYER_EUNSUPPORTED with nothing launched - call the two functions then.
  */
 int slayer_get_spikes_delayed_f32(float *s, float *u, const float *nu, const float *delayLut,
                                   int64_t lutSize, float delay, float delayTs, int64_t nNeurons,

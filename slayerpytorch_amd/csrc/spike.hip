@@ -154,6 +154,7 @@ constexpr int kTileMaxPiece = 352;  // longest row (samples) that travels whole
 // Rows in pieces: samples per piece and row.  With 8-row tiles - tensors of few, long rows - the bytes in flight
 // per compute unit are what the rows in LDS amount to, so those pieces are longer.
 constexpr int kTilePiece16 = 256, kTilePiece8 = 512;
+constexpr int kSpikeRecordMaxT = 16384;  // longest row in pieces whose spikes can be stored shifted (2 KiB of spike bits)
 
 // LAG: samples of a piece that stay behind for the next one (>= NU - 1, whole 16-byte vectors; 32 = one word of
 // candidate bits for rows in pieces).  The samples that leave a piece are the ones LAG before its end, so with
@@ -182,21 +183,28 @@ struct SpikeDelay {
 template <int NU, int MODE, int LAG, int R>
 __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, float *u,
                                                         const float *__restrict__ nu, int64_t rows,
-                                                        int T, int nuSize, int Tc, int P, int MP,
+                                                        int T, int nuSize, int Tc, int P, int MP, int MPT,
                                                         int64_t tiles, float theta, float Ts, SpikeDelay dl)
 {
     static_assert(LAG >= NU - 1 && LAG % 4 == 0, "the window must cover the refractory kernel");
-    constexpr int G = 32;               // samples per walk group = bits of a spike mask
     constexpr bool VEC = MODE == kTileVec, FLAT = MODE == kTileFlat;
     constexpr int V = VEC ? 4 : 1;      // samples per (row-wise) global access
     // longest piece this instance stages (LAG = 32 marks the instances for rows in pieces)
     constexpr int kPiece = (LAG == 32 && VEC) ? (R == 8 ? kTilePiece8 : kTilePiece16) : kTileMaxPiece;
     constexpr int NB = R * kPiece / (FLAT ? 4 : V) / kWave;  // accesses per lane per piece, at most
+    // vectors per lane that leave in one step, at most: a row's last piece also retires the LAG columns behind it
+    constexpr int NBR = (R * (kPiece + (LAG == 32 ? LAG : 0)) / 4 + kWave - 1) / kWave;
     extern __shared__ __align__(16) float lds[];
     float *tile = lds;                                                    // [R][P], P = 4 (mod 32)
     uint32_t *masks = reinterpret_cast<uint32_t *>(lds + R * P);  // [R][MP]
     int *rowShift = reinterpret_cast<int *>(masks + R * MP);      // [R], used when the output is shifted
     uint32_t *cand = reinterpret_cast<uint32_t *>(rowShift + R);  // [R][MP], candidate samples (see below)
+    // [R][MPT], MPT > 0: rows in pieces whose spikes are stored shifted.  A shift may reach any distance back and
+    // (negative delays) forward, so the spike bits of the whole row are kept - bit LAG + t for time t - and the
+    // shifted spikes of a tile's rows leave in one go after the rows' last piece.
+    uint32_t *rowMasks = cand + R * MP + 4;
+    uint32_t *candCount = cand + R * MP;  // candidates among the samples staged in this step
+    const bool record = MPT > 0;
 
     const int lane = threadIdx.x;
     const float amplitude = 1.0f / Ts;
@@ -210,12 +218,17 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     // at or above it ("candidates", a few per cent): all 64 lanes mark them while the tile is staged, and the
     // walking lanes go from candidate to candidate, test the sample's current value and add the refractory
     // response in place in LDS - the same fp32 additions in the same order as the sequential loop.
-    bool monotone = true;
+    bool monotone = VEC;  // (rows of whole vectors only: elsewhere marking sample by sample costs what it saves)
 #pragma unroll
     for (int j = 0; j < NU; ++j) monotone = monotone && tap[j] <= 0.0f;
     auto mark = [&](int r, int col, float x) {  // one sample
-        if (x >= theta) atomicOr(cand + r * MP + (col >> 5), 1u << (col & 31));
+        if (x >= theta) {
+            atomicOr(cand + r * MP + (col >> 5), 1u << (col & 31));
+            atomicAdd(candCount, 1u);
+        }
     };
+    constexpr int G = 32;               // samples per group of the window walk = bits of a spike mask
+    float v[G + LAG];                   // its register window
 
     // A "step" is one piece of one tile.  The global loads of a step are issued one step ahead
     // into x[] and stay in flight while the previous step is walked and retired.
@@ -287,7 +300,10 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                         const uint32_t bits = (x[4 * b] >= theta ? 1u : 0u) | (x[4 * b + 1] >= theta ? 2u : 0u) |
                                               (x[4 * b + 2] >= theta ? 4u : 0u) | (x[4 * b + 3] >= theta ? 8u : 0u);
                         const int col = LAG + rc.c * V;
-                        if (bits) atomicOr(cand + rc.r * MP + (col >> 5), bits << (col & 31));
+                        if (bits) {
+                            atomicOr(cand + rc.r * MP + (col >> 5), bits << (col & 31));
+                            atomicAdd(candCount, static_cast<uint32_t>(__builtin_popcount(bits)));
+                        }
                     }
                 } else {
                     *dst = x[b];
@@ -301,7 +317,8 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     int64_t t = blockIdx.x;
     int tL = 0;
     if (t < tiles) issue(t, tL);
-    for (int i = lane; i < R * MP; i += kWave) cand[i] = 0u;
+    for (int i = lane; i < R * MP + 1; i += kWave) cand[i] = 0u;
+    if (record && lane < R) rowMasks[lane * MPT + MPT - 1] = 0u;  // the word behind a row's spike bits
     wave_sync();
     if (t < tiles) commit(t, tL);
     // One trip = one step.  The next step's loads are issued first, this step's stores follow, and the next step's
@@ -317,15 +334,28 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         const int tLn = last ? 0 : tL + Tc;
 
         wave_sync();
-        issue(tn, tLn);
+        // a shifted output: the rows' delays, read with the tile's first piece and ahead of the next step's loads
+        // (the wait for this value then leaves those in flight)
+        float rowDelay = dl.delay;
+        if (dl.on && tL == 0 && dl.lut && lane < R) {
+            const int64_t row = t * R + lane;
+            rowDelay = dl.lut[row < rows ? (rows <= 0xffffffffLL && dl.lutSize <= 0xffffffffLL
+                                                ? static_cast<int64_t>(static_cast<uint32_t>(row) % static_cast<uint32_t>(dl.lutSize))
+                                                : row % dl.lutSize)
+                                         : 0];
+        }
+        // (whole rows: one tile per work-group, nothing follows, and the walk may use the registers)
+        if constexpr (LAG == 32) issue(tn, tLn);
 
         // ---- walk: lane = row.  Columns [0, W) become final in this step.
         const int W = last ? n + LAG : n;
-        if (monotone) {
+        // going from candidate to candidate costs a round trip through LDS each: it pays while candidates are few
+        const bool hop = monotone && *candCount * 32u <= static_cast<uint32_t>(nRows * n);
+        if (hop) {
             // lane = row; every lane keeps its own place in its row's candidate words (lanes without a row have none)
             const int words = lane < R ? (W + 31) >> 5 : 0;
             const uint32_t *cw = cand + (lane < R ? lane : 0) * MP;
-            uint32_t *mw = masks + (lane < R ? lane : 0) * MP;
+            uint32_t *mw = record ? rowMasks + (lane < R ? lane : 0) * MPT + (tL >> 5) : masks + (lane < R ? lane : 0) * MP;
             float *mine = tile + (lane < R ? lane : 0) * P;
             int w = 0;
             uint32_t cm = words > 0 ? cw[0] : 0u, fired = 0u;
@@ -350,26 +380,54 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
             }
             if (words > 0) mw[w] = fired;
         } else if (lane < R) {
-            // a refractory kernel that can raise the potential: every sample in turn, in place in LDS
+            // every sample in turn: 32 samples at a time are pulled into a register window v[0 .. 32+LAG), a spike
+            // adds nu[0..NU) onto v[k .. k+NU), and the 32 oldest samples go back to LDS with their spike mask
             float *mine = tile + lane * P;
-            const int begin = (tL == 0) ? LAG : 0;  // (before the first sample lies nothing)
-            for (int c0 = 0; c0 < W; c0 += G) {
+            uint32_t *mw = record ? rowMasks + lane * MPT + (tL >> 5) : masks + lane * MP;
+#pragma unroll
+            for (int k = 0; k < LAG; ++k) v[k] = (tL == 0) ? quiet : mine[k];
+            const int groups = (W + G - 1) / G;
+            for (int g = 0; g < groups; ++g) {
+                const int c0 = g * G;
+                if (c0 + G <= n) {
+#pragma unroll
+                    for (int k = 0; k < G; k += 4) {
+                        const float4 q = *reinterpret_cast<const float4 *>(mine + LAG + c0 + k);
+                        v[LAG + k] = q.x; v[LAG + k + 1] = q.y; v[LAG + k + 2] = q.z; v[LAG + k + 3] = q.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < G; ++k) v[LAG + k] = (c0 + k < n) ? mine[LAG + c0 + k] : quiet;
+                }
                 uint32_t fired = 0;
-                for (int k = 0; k < G; k += 4) {
-                    float4 q = *reinterpret_cast<const float4 *>(mine + c0 + k);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int col = c0 + k + e;
-                        const float val = e == 0 ? q.x : e == 1 ? q.y : e == 2 ? q.z : q.w;
-                        if (col >= begin && col < W && val >= theta) {
-                            fired |= 1u << (k + e);
+                for (int k = 0; k < G; k += 2) {
+                    // One scalar branch per two samples: in most pairs no row spikes.  (The second
+                    // sample is tested again inside, after the first one's refractory response.)
+                    if (__builtin_amdgcn_ballot_w64((v[k] >= theta) | (v[k + 1] >= theta)) != 0) {
+                        if (v[k] >= theta) {
+                            fired |= 1u << k;
 #pragma unroll
-                            for (int j = 0; j < NU; ++j) mine[col + j] += tap[j];
-                            q = *reinterpret_cast<const float4 *>(mine + c0 + k);
+                            for (int j = 0; j < NU; ++j) v[k + j] += tap[j];
+                        }
+                        if (v[k + 1] >= theta) {
+                            fired |= 2u << k;
+#pragma unroll
+                            for (int j = 0; j < NU; ++j) v[k + 1 + j] += tap[j];
                         }
                     }
                 }
-                masks[lane * MP + (c0 >> 5)] = fired;
+#pragma unroll
+                for (int k = 0; k < G; k += 4)
+                    *reinterpret_cast<float4 *>(mine + c0 + k) = make_float4(v[k], v[k + 1], v[k + 2], v[k + 3]);
+                mw[g] = fired;
+#pragma unroll
+                for (int k = 0; k < LAG; ++k) v[k] = v[G + k];
+            }
+            // the LAG columns behind the final ones have taken part of the responses: back to LDS for the next piece
+            if (!last) {
+#pragma unroll
+                for (int k = 0; k < LAG; ++k) mine[W + k] = v[k];
             }
         }
         wave_sync();
@@ -378,12 +436,9 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         {
             const BufferRsrc bufU = make_buffer(u + t * R * static_cast<int64_t>(T));
             const BufferRsrc bufS = make_buffer(s + t * R * static_cast<int64_t>(T));
-            if (dl.on) {  // whole rows only (the launcher sees to it): every row's shift in samples
-                if (lane < R) {
-                    const int64_t row = t * R + lane;
-                    const float d = dl.lut ? dl.lut[row < rows ? row % dl.lutSize : 0] : dl.delay;
-                    rowShift[lane] = delay_steps(d, dl.Ts);
-                }
+            if (dl.on && tL == 0) {  // every row's shift in samples (kept for the row's further pieces)
+                // (a shift of more than the longest row moves everything out, whatever its size)
+                if (lane < R) rowShift[lane] = max(-(1 << 24), min(1 << 24, delay_steps(rowDelay, dl.Ts)));
                 wave_sync();
             }
             // the spike bit of the sample `shift` steps before column `col` (0 outside the row)
@@ -395,6 +450,17 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                 uint32_t m = masks[r * MP + w] >> sh;
                 if (sh > 28 && w + 1 < MP - 1) m |= masks[r * MP + w + 1] << (32 - sh);
                 return m;
+            };
+            // the same from the record of the whole row (rows in pieces): the four bits from bit c2 on
+            const int nBits = T + LAG, nWords = (nBits + 31) >> 5;
+            auto bits_of_row = [&](int r, int c2) -> uint32_t {
+                // no branches: the LDS reads of all vectors of a step go out together.  Bits before LAG and from
+                // nBits on are never set, and the word behind a row's last is kept at zero.
+                const bool in = c2 >= 0 && c2 < nBits;
+                const int cc = in ? c2 : 0;
+                const uint32_t *rm = rowMasks + r * MPT + (cc >> 5);
+                const uint64_t both = (static_cast<uint64_t>(rm[1]) << 32) | rm[0];
+                return in ? static_cast<uint32_t>(both >> (cc & 31)) : 0u;
             };
             if constexpr (FLAT) {
                 const int nVec = (nRows * T) >> 2;
@@ -423,14 +489,18 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
             if constexpr (VEC) {
                 // a fixed number of (masked) stores, see above
 #pragma unroll
-                for (int b = 0; b < NB; ++b) {
+                for (int b = 0; b < NBR; ++b) {
                     const bool on = lane + b * kWave < total;
                     const int r = on ? rc.r : 0, col = on ? first + rc.c * V : first;
                     const float *src = tile + r * P + col;
-                    const uint32_t m = dl.on ? bits_from(r, col) : masks[r * MP + (col >> 5)] >> (col & 31);
+                    // rows in pieces with a shifted output: a shift towards later times only needs spikes that are
+                    // final by now; the rows with a negative shift wait for their last piece
+                    const int shift = record ? rowShift[r] : 0;
+                    const uint32_t m = record ? bits_of_row(r, tL + col - shift)
+                                              : dl.on ? bits_from(r, col) : masks[r * MP + (col >> 5)] >> (col & 31);
                     const int off = masked_offset(on, (r * T + tW + col) * 4);
                     buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(src));
-                    buffer_store4(bufS, off, 0,
+                    buffer_store4(bufS, shift < 0 ? kOutOfRange : off, 0,
                                   make_float4((m & 1u) ? amplitude : 0.0f, (m & 2u) ? amplitude : 0.0f,
                                               (m & 4u) ? amplitude : 0.0f, (m & 8u) ? amplitude : 0.0f));
                     rc.advance(dr, dc, perRow);
@@ -451,6 +521,40 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         }
         wave_sync();
 
+        if constexpr (VEC) {
+            bool early = false;  // a row of this tile takes its spikes from later times
+            if (record && last) early = __builtin_amdgcn_ballot_w64(lane < nRows && rowShift[lane < R ? lane : 0] < 0) != 0;
+            if (early) {
+                // the rows are complete: the spikes of those rows, shifted, from the record of the whole row
+                const BufferRsrc bufS = make_buffer(s + t * R * static_cast<int64_t>(T));
+                const int nBits = T + LAG, nWords = (nBits + 31) >> 5;
+                const int perRow = T >> 2;
+                const int total = nRows * perRow;
+                RowCol rc;
+                rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
+                const int dr = kWave / perRow, dc = kWave % perRow;
+                for (int g0 = lane; g0 < total; g0 += kWave, rc.advance(dr, dc, perRow)) {
+                    if (rowShift[rc.r] >= 0) continue;
+                    const int c2 = LAG + 4 * rc.c - rowShift[rc.r];
+                    uint32_t m = 0u;
+                    if (c2 > -4 && c2 < nBits) {
+                        // (bits before LAG and from nBits on are never set; c2 may be up to 3 below zero)
+                        const int w = c2 >> 5, sh = c2 & 31;
+                        const uint32_t *rm = rowMasks + rc.r * MPT;
+                        if (c2 >= 0) {
+                            m = rm[w] >> sh;
+                            if (sh > 28 && w + 1 < nWords) m |= rm[w + 1] << (32 - sh);
+                        } else {
+                            m = rm[0] << -c2;
+                        }
+                    }
+                    buffer_store4(bufS, (rc.r * T + 4 * rc.c) * 4, 0,
+                                  make_float4((m & 1u) ? amplitude : 0.0f, (m & 2u) ? amplitude : 0.0f,
+                                              (m & 4u) ? amplitude : 0.0f, (m & 8u) ? amplitude : 0.0f));
+                }
+                wave_sync();
+            }
+        }
         // rows in pieces: the LAG columns behind this piece's final ones, and their candidates, open the next
         // piece (LAG is one word of candidates then); every other word of candidates starts empty
         if (!last) {
@@ -461,10 +565,14 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
             if (lane < R) cand[lane * MP] = cand[lane * MP + (n >> 5)];
             wave_sync();
         }
-        for (int i = lane; i < R * MP; i += kWave)
-            if (last || i % MP != 0) cand[i] = 0u;
+        for (int i = lane; i < R * MP + 1; i += kWave)
+            if (last || i % MP != 0 || i == R * MP) cand[i] = 0u;
         wave_sync();
-        commit(tn, tLn);
+        if constexpr (LAG == 32) commit(tn, tLn);
+        else if (tn < tiles) {  // (not reached: whole rows are launched with one work-group per tile)
+            issue(tn, tLn);
+            commit(tn, tLn);
+        }
         t = tn;
         tL = tLn;
     }
@@ -551,16 +659,16 @@ static int launch_get_spikes(float *s, float *u, const float *nu, int64_t nNeuro
         if (vec)                                                                                        \
             hipLaunchKernelGGL((spike_tile_kernel<NU, kTileVec, LAGV, RV>), dim3(grid), dim3(kWave),    \
                                lds, st, s, u, nu, nNeurons, static_cast<int>(T),                        \
-                               static_cast<int>(nuSize), Tc, P, MP, tiles, theta, Ts, dl);              \
+                               static_cast<int>(nuSize), Tc, P, MP, MPT, tiles, theta, Ts, dl);         \
         else if (flat && RV == 8)                                                                       \
             hipLaunchKernelGGL((spike_tile_kernel<NU, (RV == 8 ? kTileFlat : kTileScalar), LAGV, RV>),  \
                                dim3(grid), dim3(kWave), lds, st, s, u, nu, nNeurons,                    \
-                               static_cast<int>(T), static_cast<int>(nuSize), Tc, P, MP, tiles, theta,  \
-                               Ts, dl);                                                                 \
+                               static_cast<int>(T), static_cast<int>(nuSize), Tc, P, MP, MPT, tiles,    \
+                               theta, Ts, dl);                                                          \
         else                                                                                            \
             hipLaunchKernelGGL((spike_tile_kernel<NU, kTileScalar, LAGV, RV>), dim3(grid), dim3(kWave), \
                                lds, st, s, u, nu, nNeurons, static_cast<int>(T),                        \
-                               static_cast<int>(nuSize), Tc, P, MP, tiles, theta, Ts, dl);              \
+                               static_cast<int>(nuSize), Tc, P, MP, MPT, tiles, theta, Ts, dl);         \
         return launch_status();                                                                         \
     } while (0)
 #define SLAYER_SPIKE_TILE_LAG(NU, LAGV)                                                                  \
@@ -574,9 +682,10 @@ static int launch_get_spikes(float *s, float *u, const float *nu, int64_t nNeuro
         int cols, P, MP;                                                                                \
         auto layout = [&]() {                                                                           \
             cols = (LAGV + Tc + 31) & ~31; /* the walk goes in groups of 32 columns */                  \
-            /* 4 (mod 32): rows are 16-byte aligned and start in different banks; a refractory response \
-               that is added in place may reach NU - 1 columns past the last one */                    \
-            P = cols + 4 + ((cols + 4 - (LAGV + Tc) < NU - 1) ? 32 : 0);                                \
+            /* 4 (mod 8): rows are 16-byte aligned and 8 of them start in different banks; a refractory \
+               response that is added in place may reach NU - 1 columns past the last one */           \
+            P = cols + 4;                                                                               \
+            while (P - (LAGV + Tc) < NU - 1) P += 8;                                                    \
             MP = cols / 32 + 1;                                                                         \
         };                                                                                              \
         layout();                                                                                       \
@@ -586,7 +695,19 @@ static int launch_get_spikes(float *s, float *u, const float *nu, int64_t nNeuro
             Tc = kTilePiece8;                                                                           \
             layout();                                                                                   \
         }                                                                                               \
-        const size_t lds = (static_cast<size_t>(rowsPerTile) * P + 2 * rowsPerTile * MP + rowsPerTile) * sizeof(float); \
+        /* shifted spikes of rows in pieces: the spike bits of whole rows stay in LDS */                \
+        const int MPT = (dl.on && !whole) ? static_cast<int>((T + LAGV + 31) / 32 + 1) : 0;             \
+        auto lds_bytes = [&]() {                                                                        \
+            return (static_cast<size_t>(rowsPerTile) * P + 2 * rowsPerTile * MP + rowsPerTile + 4 +     \
+                    static_cast<size_t>(rowsPerTile) * MPT) * sizeof(float);                            \
+        };                                                                                              \
+        /* eight wavefronts per compute unit are what the 8-row tiles of a small tensor need to be      \
+           resident all at once: shorter pieces if the tile does not fit an eighth of the LDS */        \
+        while (!whole && rowsPerTile == 8 && vec && Tc > kTilePiece16 && lds_bytes() > 160 * 1024 / 8) { \
+            Tc -= 32;                                                                                   \
+            layout();                                                                                   \
+        }                                                                                               \
+        const size_t lds = lds_bytes();                                                                 \
         const int64_t tiles = ceil_div(nNeurons, rowsPerTile);                                          \
         const int64_t resident = static_cast<int64_t>(cus) * (160 * 1024 / static_cast<int64_t>(lds));  \
         if (tiles >= (1LL << 31)) return SLAYER_EUNSUPPORTED;                                           \
@@ -599,7 +720,10 @@ static int launch_get_spikes(float *s, float *u, const float *nu, int64_t nNeuro
         if (whole) SLAYER_SPIKE_TILE_LAG(NU, ((NU + 2) & ~3));                                          \
         SLAYER_SPIKE_TILE_LAG(NU, 32);                                                                  \
     } while (0)
-    if (dl.on && !(window_ok && nuSize <= 24 && T <= kTileMaxPiece)) return SLAYER_EUNSUPPORTED;
+    // a shifted output: rows that travel whole, or rows of whole vectors whose spike bits fit into LDS
+    if (dl.on && !(window_ok && nuSize <= 24 &&
+                   (T <= kTileMaxPiece || (T <= kSpikeRecordMaxT && T % 4 == 0 && aligned16(s) && aligned16(u)))))
+        return SLAYER_EUNSUPPORTED;
     if (window_ok && nuSize <= 24) {
         // short rows travel whole; long rows in pieces
         const bool whole = T <= kTileMaxPiece;

@@ -320,6 +320,10 @@ SPIKE_CASES = [
     # rows that are not whole 16-byte vectors in tensors that are: 8-row tiles move as flat runs
     ((2, 4, 3, 1, 350), 11), ((4, 5, 1, 1, 101), 8), ((1, 8, 1, 1, 5), 3), ((1, 12, 1, 1, 351), 24),
     ((3, 4, 1, 1, 349), 16), ((1, 6, 1, 1, 101), 11),
+    # rows in pieces of 512 samples: a last piece that retires more columns than a full one (488 + 32), a last
+    # piece of one vector, exactly one and two pieces, a piece boundary right behind a row of 352
+    ((1, 21, 1, 1, 1000), 11), ((1, 9, 1, 1, 516), 24), ((2, 5, 1, 1, 512), 11), ((1, 17, 1, 1, 1024), 16),
+    ((1, 9, 1, 1, 356), 4), ((1, 3, 1, 1, 1056), 11),
 ]
 
 
@@ -438,6 +442,22 @@ def test_psp_spike_is_conv_then_getSpikes(impl, shape, Fl, nuSize):
         if not one_kernel:
             assert torch.equal(s, s2) and np.array_equal(bits(host(u)), bits(host(u2)))
     assert ws.sum() > 0 or shape[-1] < 64
+
+
+def test_spikes_many_long_rows_use_16_row_tiles():
+    # enough long rows to fill the GPU with 16-row tiles (pieces of 256 samples): sampled rows against the oracle
+    rng = np.random.default_rng(77)
+    rows, T = 70000, 400
+    u = (rng.standard_normal((1, rows, 1, 1, T)) * 6).astype(np.float32)
+    nu = np.array(alphaKernel(1.0, 1.0, T, mult=-20.0), dtype=np.float32)
+    ud = dev(u)
+    s = host(slayerCuda.getSpikes(ud, dev(nu), 10.0, 1.0)).reshape(rows, T)
+    un = host(ud).reshape(rows, T)
+    pick = np.concatenate([np.arange(40), rng.integers(0, rows, 400), np.arange(rows - 40, rows)])
+    ws, wu = O.get_spikes(u.reshape(rows, T)[pick].reshape(1, len(pick), 1, 1, T), nu, 10.0, 1.0)
+    assert np.array_equal(bits(s[pick]), bits(ws.reshape(len(pick), T)))
+    assert np.array_equal(bits(un[pick]), bits(wu.reshape(len(pick), T)))
+    assert ws.sum() > 0
 
 
 # ------------------------------------------------------------------------------------------ delay gradient
@@ -581,18 +601,23 @@ def test_empty_tensors():
 
 # ------------------------------------------------------------------ spike with the shift fused in
 @pytest.mark.parametrize("shape", [(3, 5, 4, 4, 300), (2, 3, 2, 2, 352), (2, 7, 1, 1, 100), (2, 3, 1, 1, 7),
-                                   (4, 3, 2, 2, 350), (1, 9, 1, 1, 33), (2, 4, 1, 1, 2000)])
-@pytest.mark.parametrize("delay", ["scalar", "negative", "zero", "huge", "table", "one-element"])
+                                   (4, 3, 2, 2, 350), (1, 9, 1, 1, 33), (2, 4, 1, 1, 2000), (3, 21, 1, 1, 1000),
+                                   (1, 9, 1, 1, 356), (2, 40, 1, 1, 512), (1, 3, 1, 1, 2002)])
+@pytest.mark.parametrize("delay", ["scalar", "negative", "zero", "huge", "table", "one-element", "far", "far-negative",
+                                   "long-table"])
 def test_spike_delayed_equals_spike_then_shift(shape, delay, impl):
     """getSpikesDelayed against the two kernels it fuses (both already pinned to the oracle), and
-    against the oracle itself: bit-exact, membrane potential included.  (2, 4, 1, 1, 2000) and the
-    generic kernels are shapes the fused kernel declines: the wrapper then runs the two kernels.)"""
+    against the oracle itself: bit-exact, membrane potential included.  Rows longer than 352 samples travel in
+    pieces: the fused kernel keeps their spike bits and stores the shifted spikes after the last piece, for
+    shifts of any size and sign ("far": beyond a piece).  (1, 3, 1, 1, 2002) and the generic kernels are shapes
+    the fused kernel declines: the wrapper then runs the two kernels."""
     rng = np.random.default_rng(31)
     Ts, dTs = 1.0, 0.5
     u = (rng.standard_normal(shape) * 6 + 4).astype(np.float32)
     nu = np.array(alphaKernel(1.0, Ts, shape[-1], mult=-20.0), dtype=np.float32)
-    d = {"scalar": 3.4, "negative": -2.6, "zero": 0.0, "huge": 1e9,
+    d = {"scalar": 3.4, "negative": -2.6, "zero": 0.0, "huge": 1e9, "far": 300.3, "far-negative": -170.0,
          "table": (rng.random(shape[1:4]) * 12 - 2).astype(np.float32),
+         "long-table": ((rng.random(shape[1:4]) * 2 - 1) * shape[-1] * 0.3).astype(np.float32),
          "one-element": np.array([5.0], dtype=np.float32)}[delay]
     dd = dev(d) if isinstance(d, np.ndarray) else d
     ua, ub = dev(u), dev(u)
