@@ -202,8 +202,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     // [R][MPT], MPT > 0: rows in pieces whose spikes are stored shifted.  A shift may reach any distance back and
     // (negative delays) forward, so the spike bits of the whole row are kept - bit LAG + t for time t - and the
     // shifted spikes of a tile's rows leave in one go after the rows' last piece.
-    uint32_t *rowMasks = cand + R * MP + 4;
-    uint32_t *candCount = cand + R * MP;  // candidates among the samples staged in this step
+    uint32_t *rowMasks = cand + R * MP;
     const bool record = MPT > 0;
 
     const int lane = threadIdx.x;
@@ -222,10 +221,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 #pragma unroll
     for (int j = 0; j < NU; ++j) monotone = monotone && tap[j] <= 0.0f;
     auto mark = [&](int r, int col, float x) {  // one sample
-        if (x >= theta) {
-            atomicOr(cand + r * MP + (col >> 5), 1u << (col & 31));
-            atomicAdd(candCount, 1u);
-        }
+        if (x >= theta) atomicOr(cand + r * MP + (col >> 5), 1u << (col & 31));
     };
     constexpr int G = 32;               // samples per group of the window walk = bits of a spike mask
     float v[G + LAG];                   // its register window
@@ -300,10 +296,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                         const uint32_t bits = (x[4 * b] >= theta ? 1u : 0u) | (x[4 * b + 1] >= theta ? 2u : 0u) |
                                               (x[4 * b + 2] >= theta ? 4u : 0u) | (x[4 * b + 3] >= theta ? 8u : 0u);
                         const int col = LAG + rc.c * V;
-                        if (bits) {
-                            atomicOr(cand + rc.r * MP + (col >> 5), bits << (col & 31));
-                            atomicAdd(candCount, static_cast<uint32_t>(__builtin_popcount(bits)));
-                        }
+                        if (bits) atomicOr(cand + rc.r * MP + (col >> 5), bits << (col & 31));
                     }
                 } else {
                     *dst = x[b];
@@ -317,7 +310,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     int64_t t = blockIdx.x;
     int tL = 0;
     if (t < tiles) issue(t, tL);
-    for (int i = lane; i < R * MP + 1; i += kWave) cand[i] = 0u;
+    for (int i = lane; i < R * MP; i += kWave) cand[i] = 0u;
     if (record && lane < R) rowMasks[lane * MPT + MPT - 1] = 0u;  // the word behind a row's spike bits
     wave_sync();
     if (t < tiles) commit(t, tL);
@@ -349,8 +342,15 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 
         // ---- walk: lane = row.  Columns [0, W) become final in this step.
         const int W = last ? n + LAG : n;
-        // going from candidate to candidate costs a round trip through LDS each: it pays while candidates are few
-        const bool hop = monotone && *candCount * 32u <= static_cast<uint32_t>(nRows * n);
+        // going from candidate to candidate costs a round trip through LDS each, and the wavefront stays as long as
+        // its busiest row: it pays while no row of the tile has more than a candidate per 24 samples
+        bool hop = monotone;
+        if (monotone) {
+            int mine = 0;
+            if (lane < R)
+                for (int w = 0; w < ((W + 31) >> 5); ++w) mine += __builtin_popcount(cand[lane * MP + w]);
+            hop = __builtin_amdgcn_ballot_w64(mine * 24 > W) == 0;
+        }
         if (hop) {
             // lane = row; every lane keeps its own place in its row's candidate words (lanes without a row have none)
             const int words = lane < R ? (W + 31) >> 5 : 0;
@@ -565,8 +565,8 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
             if (lane < R) cand[lane * MP] = cand[lane * MP + (n >> 5)];
             wave_sync();
         }
-        for (int i = lane; i < R * MP + 1; i += kWave)
-            if (last || i % MP != 0 || i == R * MP) cand[i] = 0u;
+        for (int i = lane; i < R * MP; i += kWave)
+            if (last || i % MP != 0) cand[i] = 0u;
         wave_sync();
         if constexpr (LAG == 32) commit(tn, tLn);
         else if (tn < tiles) {  // (not reached: whole rows are launched with one work-group per tile)
@@ -698,7 +698,7 @@ static int launch_get_spikes(float *s, float *u, const float *nu, int64_t nNeuro
         /* shifted spikes of rows in pieces: the spike bits of whole rows stay in LDS */                \
         const int MPT = (dl.on && !whole) ? static_cast<int>((T + LAGV + 31) / 32 + 1) : 0;             \
         auto lds_bytes = [&]() {                                                                        \
-            return (static_cast<size_t>(rowsPerTile) * P + 2 * rowsPerTile * MP + rowsPerTile + 4 +     \
+            return (static_cast<size_t>(rowsPerTile) * P + 2 * rowsPerTile * MP + rowsPerTile +         \
                     static_cast<size_t>(rowsPerTile) * MPT) * sizeof(float);                            \
         };                                                                                              \
         /* eight wavefronts per compute unit are what the 8-row tiles of a small tensor need to be      \
