@@ -79,9 +79,14 @@ class spikeLayer(slayer.spikeLayer):
         ``delayShift(spikeLoihi(x), delay, delayTs)`` - a shift by ``int(delay / delayTs)`` samples
         - from the same kernel."""
         Ts = self.simulation["Ts"]
-        steps = int(float(delay) / float(delayTs))
-        if 0 <= steps <= slayerLoihiCuda.MAX_FUSED_DELAY:
-            return _spike.apply(weightedSpikes, self.srmKernel, self.neuron, Ts, steps)
+        scalar = not isinstance(delay, torch.Tensor) and not isinstance(delayTs, torch.Tensor) and np.ndim(delay) == 0
+        if scalar:
+            # the shift kernel's own arithmetic: the fp32 quotient, truncated toward zero
+            quotient = np.float32(delay) / np.float32(delayTs)
+            steps = int(quotient) if np.isfinite(quotient) else -1
+            if 0 <= steps <= slayerLoihiCuda.MAX_FUSED_DELAY:
+                return _spike.apply(weightedSpikes, self.srmKernel, self.neuron, Ts, steps)
+        # a delay per neuron, a tensor, a negative or a long delay: the separate shift
         return self.delayShift(_spike.apply(weightedSpikes, self.srmKernel, self.neuron, Ts, 0), delay, delayTs)
 
     def spikeLoihiFull(self, weightedSpikes):

@@ -44,6 +44,14 @@ class event():
     and time stamps ``t`` in ms (src/spikeFileIO.py:6-34).  As in the reference the polarity is
     shifted so that its minimum is 0."""
 
+    def __setattr__(self, name, value):
+        # the file bytes stand for the events only as long as nobody reassigns them (a flip, a time offset, any
+        # augmentation): after that the members are binned, as in the reference
+        if name in ("x", "y", "p", "t"):
+            object.__setattr__(self, "_raw", None)
+            object.__setattr__(self, "_format", None)
+        object.__setattr__(self, name, value)
+
     def __init__(self, xEvent, yEvent, pEvent, tEvent):
         self._raw = None
         self._format = None
@@ -67,6 +75,11 @@ class event():
         raw = raw[:n * _EVENT_BYTES[fmt]]
         x, y, p, t = _decode(raw, fmt)
         self = cls(x, y, p, t / 1000)          # spike times in ms
+        # the decoded arrays are handed out read-only: an in-place edit would not be seen by the packed path (assign
+        # a new array, e.g. ev.t = ev.t + 5, to change the events)
+        for a in (self.x, self.y, self.p, self.t):
+            if a is not None:
+                a.setflags(write=False)
         self._raw, self._format = raw, fmt
         return self
 

@@ -14,7 +14,7 @@ import torch
 from . import _lib
 from .slayerCuda import _check_device, _check_input, _on_device_of, _ptr
 
-__all__ = ["conv", "convGradInput", "convGradWeight", "outShape", "synapseConv", "synapseConvTranspose"]
+__all__ = ["conv", "convGradInput", "convGradWeight", "outShape", "supported", "synapseConv", "synapseConvTranspose"]
 
 
 def _pair(v, name):
@@ -54,6 +54,25 @@ def outShape(inShape, wShape, stride=1, padding=0, dilation=1, groups=1):
     _lib.check(_lib.load().slayer_synapse_out_shape(ctypes.byref(g), ctypes.byref(OH), ctypes.byref(OW)),
                "slayer_synapse_out_shape")
     return (g.N, g.O, OH.value, OW.value, g.T)
+
+
+def supported(inShape, wShape, stride=1, padding=0, dilation=1, groups=1):
+    """Whether the synapse kernels index this geometry: one batch item of the input and of the output below
+    2 GiB, and a filter window - (padH + dilH * KH) rows plus (padW + dilW * KW) columns of the input - below
+    16 MiB.  Decided on the host from the sizes alone (no GPU involved).  Beyond these limits the differentiable
+    ``synapseConv`` / ``synapseConvTranspose`` fall back to torch's conv3d / conv_transpose3d, which the
+    reference calls for every geometry."""
+    g = _geom(inShape, wShape, stride, padding, dilation, groups)
+    status = _lib.load().slayer_synapse_out_shape(ctypes.byref(g), None, None)
+    if status == 2:
+        return False
+    _lib.check(status, "slayer_synapse_out_shape")
+    return True
+
+
+def _triple(v, last):
+    a, b = _pair(v, "argument")
+    return (a, b, last)
 
 
 def conv(input, weight, stride=1, padding=0, dilation=1, groups=1):
@@ -167,6 +186,10 @@ class _synapseConvTransposeFunction(torch.autograd.Function):
 def synapseConv(input, weight, stride=1, padding=0, dilation=1, groups=1):
     """Differentiable ``conv``: stands where the reference calls ``F.conv3d(input, weight, None,
     stride, padding, dilation, groups)`` (src/slayer.py:499-507)."""
+    if not supported(input.shape, weight.shape, stride, padding, dilation, groups):
+        w5 = weight if weight.dim() == 5 else weight.unsqueeze(-1)
+        return torch.nn.functional.conv3d(input, w5, None, _triple(stride, 1), _triple(padding, 0), _triple(dilation, 1),
+                                          groups)
     return _synapseConvFunction.apply(input, weight, stride, padding, dilation, groups)
 
 
@@ -174,4 +197,14 @@ def synapseConvTranspose(input, weight, stride=1, padding=0, dilation=1, groups=
     """Differentiable transposed synapse: stands where the reference calls
     ``F.conv_transpose3d(input, weight, None, stride, padding, 0, groups, dilation)``
     (src/slayer.py:631-643)."""
+    (sH, sW), (pH, pW), (dH, dW) = _pair(stride, "stride"), _pair(padding, "padding"), _pair(dilation, "dilation")
+    KH, KW = int(weight.shape[2]), int(weight.shape[3])
+    N, Cin, H, W, T = (int(v) for v in input.shape)
+    # (the geometry of the convolution that this transposes: its input is this op's output)
+    conv_in = (N, int(weight.shape[1]) * groups, (H - 1) * sH - 2 * pH + dH * (KH - 1) + 1,
+               (W - 1) * sW - 2 * pW + dW * (KW - 1) + 1, T)
+    if min(conv_in) >= 0 and not supported(conv_in, weight.shape[:4], stride, padding, dilation, groups):
+        w5 = weight if weight.dim() == 5 else weight.unsqueeze(-1)
+        return torch.nn.functional.conv_transpose3d(input, w5, None, _triple(stride, 1), _triple(padding, 0), 0, groups,
+                                                    _triple(dilation, 1))
     return _synapseConvTransposeFunction.apply(input, weight, stride, padding, dilation, groups)

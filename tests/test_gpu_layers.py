@@ -13,7 +13,7 @@ from oracle import oracle as O
 from slayerpytorch_amd import slayerCuda, slayerLoihiCuda
 from slayerpytorch_amd.slayer import alphaKernel
 
-from _util import golden, raster_from_aer, rel_err
+from _util import golden, raster_from_aer, raster_from_events, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -297,6 +297,37 @@ def test_golden_gradients_like_reference_test003():
     assert np.linalg.norm(snn_d["gradW1Initial"] - g1) / g1.size < 1e-4
 
 
+def test_golden_output_layer_and_gradients_torch_validate():
+    """The legacy traces of the 250-25-1 network at Ts = 0.1 through the layer engine and autograd: hidden and
+    output spikes (266 and 11), the output neuron's potential, the error signal of the spike-time loss and both
+    weight gradients (Wgrad1, Wgrad2: a second joint pin of psp, spike, the surrogate gradient and corr next to
+    the gradW*Initial files).  The files carry 5 digits."""
+    tv = golden("torch_validate.npz")
+    Ts, Ns = 0.1, 501
+    nd = neuron(tauSr=1.0, tauRho=0.43429)                         # pdf tau = tauRho * theta = 4.3429
+    layer = snn.layer(nd, {"Ts": Ts, "tSample": 50}, fullRefKernel=True).to(DEV)
+    fc1, fc2 = layer.dense(250, 25).to(DEV), layer.dense(25, 1).to(DEV)
+    fc1.weight = torch.nn.Parameter(dev(tv["W12"]).reshape(25, 250, 1, 1, 1))
+    fc2.weight = torch.nn.Parameter(dev(tv["W23"]).reshape(1, 25, 1, 1, 1))
+    s1 = dev(raster_from_events(tv["s1_shape"], tv["s1_events"], tv["s1_values"])).reshape(1, 250, 1, 1, Ns)
+    a1 = layer.psp(s1)
+    assert np.abs(host(a1).reshape(250, Ns) - tv["a1"]).max() < 1e-4
+    u2 = fc1(a1)
+    s2 = layer.spike(u2)
+    assert np.array_equal(host(s2).reshape(25, Ns), tv["s2"]) and float((s2 > 0).sum()) == 266
+    u3 = fc2(layer.psp(s2))
+    s3 = layer.spike(u3)
+    assert np.array_equal(host(s3).reshape(1, Ns), tv["s3"]) and float((s3 > 0).sum()) == 11
+    assert np.abs(host(u3).reshape(1, Ns) - tv["u3"]).max() < 2e-2   # (the potential after the refractory response)
+    des = dev(tv["des_s"]).reshape(1, 1, 1, 1, Ns)
+    e3 = layer.psp(s3 - des)
+    assert np.abs(host(e3).reshape(1, Ns) - tv["e3"]).max() < 2e-4
+    error = snn.loss({"neuron": nd, "simulation": {"Ts": Ts, "tSample": 50}, "training": {"error": {"type": "SpikeTime"}}}).to(DEV)
+    error.spikeTime(s3, des).backward()
+    assert rel_err(host(fc2.weight.grad).reshape(1, 25), tv["Wgrad2"]) < 2e-3
+    assert rel_err(host(fc1.weight.grad).reshape(25, 250), tv["Wgrad1"]) < 2e-3
+
+
 def test_numSpikes_loss_matches_host_side_formulation():
     # the reference computes the target region, the desired counts and the count error with numpy on
     # the host (src/spikeLoss.py:84-104); the same numbers, and the gradient, from device tensors
@@ -399,6 +430,35 @@ def test_loihi_spike_with_fused_delay_matches_spike_then_delayShift(Ts, delay):
     # without a gradient to compute the layer asks the kernel for the spikes only
     with torch.no_grad():
         assert torch.equal(layer.spikeLoihi(dev(w), delay), two)
+
+
+@pytest.mark.parametrize("delay,delayTs", [(0.3, 0.1), (0.7, 0.1), (2.9999999, 1.0), (5.0, 2.5), (-0.3, 0.1), (4.0, 0.1)])
+def test_loihi_fused_delay_uses_the_shift_kernels_quotient(delay, delayTs):
+    # delay / delayTs in fp32, truncated toward zero, like the shift kernel: 0.3 / 0.1 is 3 steps there (2 in double
+    # precision); negative and long delays, a delay per neuron and tensors take the separate shift
+    layer = snn.loihi(loihi_neuron(scaleRho=2.0), {"Ts": 1.0, "tSample": 120}).to(DEV)
+    rng = np.random.default_rng(13)
+    shape = (2, 3, 2, 2, 120)
+    w = (2 * rng.integers(-64, 64, size=shape) * (rng.random(shape) < 0.3)).astype(np.float32)
+    with torch.no_grad():
+        plain = layer.spikeLoihi(dev(w))
+        want = layer.delayShift(plain, delay, delayTs)
+        assert torch.equal(layer.spikeLoihi(dev(w), delay, delayTs), want)
+        assert torch.equal(want, dev(O.shift(host(plain), delay, delayTs)))
+    assert float(plain.sum()) > 0
+
+
+def test_loihi_delay_per_neuron_or_tensor_takes_the_separate_shift():
+    layer = snn.loihi(loihi_neuron(scaleRho=2.0), {"Ts": 1.0, "tSample": 120}).to(DEV)
+    rng = np.random.default_rng(14)
+    shape = (2, 3, 2, 2, 120)
+    w = (2 * rng.integers(-64, 64, size=shape) * (rng.random(shape) < 0.3)).astype(np.float32)
+    table = dev((rng.random((3, 2, 2)) * 6).astype(np.float32))
+    with torch.no_grad():
+        plain = layer.spikeLoihi(dev(w))
+        assert torch.equal(layer.spikeLoihi(dev(w), table), layer.delayShift(plain, table))
+        one = torch.tensor([2.0], device=DEV)
+        assert torch.equal(layer.spikeLoihi(dev(w), one), layer.delayShift(plain, one))
 
 
 def test_loihi_Ts_scaling_of_input_and_output():

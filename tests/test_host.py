@@ -232,3 +232,32 @@ def test_dropout_and_replicate_in_time():
     x = torch.rand(2, 3, 4, 4)
     r = layer.replicateInTime(x)
     assert r.shape == (2, 3, 4, 4, 10) and torch.equal(r[..., 7], x)
+
+
+def test_synapse_geometries_beyond_the_kernels_fall_back_to_torch():
+    """The synapse kernels index a filter window of less than 16 MiB and batch items below 2 GiB; the decision is
+    made on the host from the sizes alone, and the differentiable ops then call torch's conv3d /
+    conv_transpose3d like the reference's layers do (here on CPU tensors: the fallback never reaches the
+    library).  Geometries within the limits keep the kernels - and reject CPU tensors."""
+    import torch.nn.functional as F
+    from slayerpytorch_amd import synapse
+    assert synapse.supported((12, 2, 34, 34, 300), (16, 2, 5, 5), 1, 2)
+    assert not synapse.supported((1, 2, 346, 260, 5000), (8, 2, 5, 5), 1, 2)          # 5 rows of 346 x 5000 samples
+    assert not synapse.supported((1, 16, 128, 128, 8192), (16, 16, 3, 3), 1, 1)       # 4 GiB per batch item
+    # a small tensor whose dilated, padded window is 24.6 MB
+    geo = dict(stride=1, padding=(1000, 0), dilation=(1000, 1), groups=1)
+    x = torch.randn((1, 1, 4, 64, 32), requires_grad=True)
+    w = torch.randn((2, 1, 2, 3, 1), requires_grad=True)
+    assert not synapse.supported(x.shape, w.shape, **geo)
+    y = synapse.synapseConv(x, w, **geo)
+    want = F.conv3d(x, w, None, (1, 1, 1), (1000, 0, 0), (1000, 1, 1), 1)
+    assert torch.equal(y, want) and y.shape == (1, 2, 1004, 62, 32)
+    y.sum().backward()
+    assert x.grad is not None and w.grad is not None and float(w.grad.abs().sum()) > 0
+    # the transposed op of the same geometry
+    z = torch.randn((1, 2, 1004, 62, 32))
+    t = synapse.synapseConvTranspose(z, w.detach(), **geo)
+    assert torch.equal(t, F.conv_transpose3d(z, w.detach(), None, (1, 1, 1), (1000, 0, 0), 0, 1, (1000, 1, 1)))
+    assert t.shape == x.shape
+    with pytest.raises(RuntimeError, match="CUDA"):
+        synapse.synapseConv(torch.zeros((1, 2, 5, 5, 4)), torch.zeros((3, 2, 3, 3)), 1, 1)

@@ -220,6 +220,34 @@ def test_spike_chain_golden_torch_validate():
     assert np.abs(u2r.reshape(25, -1) - tv["u2"]).max() < 2e-2      # a1 itself carries 5 digits
 
 
+def test_output_layer_and_gradients_golden_torch_validate():
+    """The rest of the legacy traces of the 250-25-1 network (Ts = 0.1): the output neuron's potential and spikes
+    (u3, s3: 11 spikes) from the hidden spikes, its filtered spikes a3, the error signal e3 against the desired
+    response, and both weight gradients - a second joint pin of conv, spike, spike pdf and corr:
+    delta3 = pdf(u3) * corr(e3), Wgrad2 = Ts * delta3 a2^T, delta2 = pdf(u2) * corr(W23^T delta3),
+    Wgrad1 = Ts * delta2 a1^T.  Tolerances are those of 5-digit CSV files."""
+    tv = golden("torch_validate.npz")
+    Ts, theta, tau = 0.1, 10.0, 4.3429
+    srm = np.array(alphaKernel(1.0, Ts, 50), dtype=np.float32)
+    ref = tv["refractory_kernel"]
+    a2 = O.conv(tv["s2"].reshape(1, 25, 1, 1, -1), srm, Ts).reshape(25, -1)
+    pre3 = (tv["W23"].astype(np.float64) @ a2.astype(np.float64)).astype(np.float32)
+    s3, u3 = O.get_spikes(pre3.reshape(1, 1, 1, 1, -1), ref, theta, Ts)
+    assert np.array_equal(s3.reshape(1, -1), tv["s3"]) and (tv["s3"] > 0).sum() == 11
+    assert np.abs(u3.reshape(1, -1) - tv["u3"]).max() < 2e-2
+    a3 = O.conv(s3, srm, Ts).reshape(1, -1)
+    assert np.abs(a3 - tv["a3"]).max() < 1e-4
+    assert np.abs((a3 - tv["des_a"]) - tv["e3"]).max() < 2e-4
+    d3 = O.spike_bwd(O.corr(tv["e3"].reshape(1, 1, 1, 1, -1), srm, Ts), tv["u3"].reshape(1, 1, 1, 1, -1), theta, tau, 1.0)
+    d3 = d3.reshape(1, -1)
+    g2 = (d3.astype(np.float64) @ a2.astype(np.float64).T) * Ts
+    assert rel_err(g2, tv["Wgrad2"]) < 1e-4
+    e2 = (tv["W23"].astype(np.float64).T @ d3.astype(np.float64)).astype(np.float32)
+    d2 = O.spike_bwd(O.corr(e2.reshape(1, 25, 1, 1, -1), srm, Ts), tv["u2"].reshape(1, 25, 1, 1, -1), theta, tau, 1.0)
+    g1 = (d2.reshape(25, -1).astype(np.float64) @ tv["a1"].astype(np.float64).T) * Ts
+    assert rel_err(g1, tv["Wgrad1"]) < 2e-4
+
+
 # ------------------------------------------------------------------------------------------
 # spike pdf backward
 # ------------------------------------------------------------------------------------------
