@@ -34,10 +34,21 @@ SRM_TAPS = 77
 # algorithmic bytes per neuron-timestep (fp32 tensors read + written once)
 AB = {"psp_conv": 8, "spike": 12, "shift": 8, "shift_bwd": 8, "spike_bwd": 12, "psp_corr": 8}
 # HBM bytes per launch on SHAPE measured with the FETCH_SIZE and WRITE_SIZE hardware counters
-# (rocprofv3 --pmc, one counter per run, scaled by the reading of a plain copy of known size);
-# the figures and the commands are in profiles/hbm_traffic_counters.txt
-TRAFFIC_BYTES = {"psp_conv": 537.2e6, "spike": 798.7e6, "shift": 540.8e6, "shift_bwd": 540.8e6, "spike_bwd": 798.7e6,
-                 "psp_corr": 532.5e6}
+# (rocprofv3 --pmc, one counter per run, scaled by the reading of a plain copy of known size):
+# profiles/hbm_traffic_counters.json holds the figures, profiles/hbm_traffic_counters.txt the commands
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_counters.json")
+
+
+def measured_traffic(op):
+    """HBM bytes per launch of `op` on SHAPE from the committed counter run, and where they come from (the file
+    names the commit of the library the counters were read on)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+        return rec["bytes_per_launch"].get(op), {"file": "profiles/hbm_traffic_counters.json", "library_commit": rec.get("commit"),
+                                                 "kernel": rec.get("kernels", {}).get(op)}
+    except (OSError, ValueError, KeyError):
+        return None, None
 KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, true, 16, false, 6> (conv; spike trains: event-driven path)", "spike": "slayer::spike_tile_kernel<12, 1, 12, 8>",
              "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
              "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_mfma_kernel<6, 20, true, false> (corr, matrix cores)"}
@@ -606,6 +617,9 @@ def main():
                     help="only the Loihi gesture network's inference and training steps (for profiler runs); prints that row")
     ap.add_argument("--synapse-only", action="store_true",
                     help="only the per-layer synapse kernel rows (for profiler runs); prints those rows")
+    ap.add_argument("--dense-conv", action="store_true",
+                    help="also launch the 77-tap psp conv once per warm-up step on a dense input (the gradient tensor), "
+                         "whose tiles run on the matrix cores (for profiler runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain copy of known size (a zero-delay shift of half the tensor: "
                          "%d bytes read, as many written) to scale hardware counters by" % (4 * 6 * 16 * 34 * 34 * 300))
@@ -676,6 +690,9 @@ def main():
 
     for i in range(args.warmup):
         step(pool[i])
+        if args.dense_conv:
+            for _ in range(3):
+                slayerCuda.conv(grad, srm_t, 1.0)
     if args.copy_calibration:
         slayerCuda.shift(grad[:6], 0.0, 1.0)
     torch.cuda.synchronize()
@@ -719,7 +736,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": KERNEL_OF[dominant], "op": dominant, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "launch_ms": dominant_ms,
-                     "traffic": TRAFFIC_BYTES.get(dominant)},
+                     "traffic": measured_traffic(dominant)[0], "traffic_source": measured_traffic(dominant)[1]},
         # the whole step (six launches and the gaps between them) against the HBM peak
         "chain_hbm_frac": chain_gbs / HBM_PEAK_GBS,
     }
