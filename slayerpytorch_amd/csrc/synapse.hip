@@ -513,6 +513,248 @@ __global__ __launch_bounds__(256) void synapse_wgrad_mfma_kernel(WgradMfmaArgs g
     }
 }
 
+// ---- weight gradient on the matrix cores, input patch of a block of pixels in LDS -------------------
+// The kernel above fetches every input row once per tap that uses it (the working set of four
+// wavefronts does not stay in the 32 KB L1), 64 bytes at a time: it is bound by the number of cache
+// line requests a compute unit can have in flight.  Here a work-group takes kWgPix consecutive output
+// pixels of one output row at a time and, per step of 32 time samples, copies the input patch under
+// those pixels - the channels of its column group x KH filter rows x WX columns, one whole 128-byte
+// line each - into LDS once (out-of-image positions as zeros); the B operands of all pixels and taps
+// come from there with one 16-byte LDS read per tile and half step, the A operands (gradOut rows,
+// used once) straight from global memory, both halves of a line by consecutive instructions.  The
+// eight 16-byte units of a patch row are stored at (unit ^ row % 8), so that the 16 lanes of a read,
+// which address 16 different rows, spread over the banks.  Two patches are resident: while the matrix
+// instructions work on one, the loads of the next (pixel block, step) pair are in flight in registers
+// and are written to the other before the pair's single barrier.  A work-group owns a contiguous
+// range of the pairs of the whole batch, so all work-groups do the same amount of work whatever the
+// map's size; each wavefront takes one pixel, and the four add their tiles up in LDS at the end, in
+// wavefront order, into one workspace row per range.
+constexpr int kWgPix = 4;            // pixels per block (one per wavefront)
+constexpr int kWgRow = 128;          // bytes per patch row: 32 samples
+constexpr int kWgMaxRows = 288;      // patch rows per buffer (9 passes of 32); row kWgMaxRows of a buffer holds zeros
+constexpr int kWgBuf = (kWgMaxRows + 1) * kWgRow;
+
+struct WgradLdsArgs {
+    const float *gradOut, *in;
+    float *partial;
+    SynGeom s;
+    int Cg, Og, CK;
+    int oGroups, colGroups;
+    int WX, rows;              // patch width in input pixels, patch rows = channels * KH * WX
+    int blocksPerRow, steps;   // pixel blocks per output row, steps of 32 samples per row
+    int pairs, slices, pairsPerSlice, nW;
+    FastDiv byColGroups, byOGroups, byGroups, byKK, byKW, bySteps, byBlocks, byBlocksPerRow, byPatch, byWX;
+};
+
+template <int MT, int NT, int NS>
+__global__ __launch_bounds__(256, 2) void synapse_wgrad_lds_kernel(WgradLdsArgs g)
+{
+    extern __shared__ __align__(16) float lds[];
+    char *const ldsBytes = reinterpret_cast<char *>(lds);
+    const SynGeom &s = g.s;
+    uint32_t rest = xcd_contiguous(blockIdx.x, gridDim.x);
+    uint32_t qq = fastdiv(rest, g.byColGroups);
+    const int cg = static_cast<int>(rest - qq * g.byColGroups.d);
+    rest = qq; qq = fastdiv(rest, g.byOGroups);
+    const int og = static_cast<int>(rest - qq * g.byOGroups.d);
+    rest = qq; qq = fastdiv(rest, g.byGroups);
+    const int grp = static_cast<int>(rest - qq * g.byGroups.d);
+    const int slice = static_cast<int>(qq);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, h = lane >> 4;
+    const int c0 = static_cast<int>(fastdiv(static_cast<uint32_t>(cg * NT * 16), g.byKK));  // first channel of the column group
+    const int64_t goPlane = static_cast<int64_t>(s.OH) * s.OW * s.T, inPlane = static_cast<int64_t>(s.H) * s.W * s.T;
+    BufferRsrc goB = make_buffer(g.gradOut), inB = make_buffer(g.in);   // (of the batch item at hand: set by place())
+    const int rowBytes = s.W * s.T * 4, pixBytes = s.T * 4;
+
+    // This lane copies unit u (samples 4u..4u+3 of the step) of patch rows tid / 8 + 32 m, m < NS; a patch row is
+    // (channel, filter row, patch column).  (tid / 8 + 32 m) % 8 does not depend on m: one LDS address, immediate
+    // offsets for the passes.
+    const int u = tid & 7;
+    const int stageAddr = (tid >> 3) * kWgRow + ((u ^ ((tid >> 3) & 7)) << 4);
+
+    // rows of this lane: output channel of every A tile, patch row (this wavefront's pixel) of every B tile
+    int offA[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int o = ((og * MT + mt) << 4) + r;
+        offA[mt] = masked_offset(o < g.Og, o * static_cast<int>(goPlane) * 4 + h * 16);
+    }
+    int bAddr[2][NT];                      // (columns past the filter read the zero row)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int col = ((cg * NT + nt) << 4) + r;
+        const uint32_t cl = fastdiv(static_cast<uint32_t>(col), g.byKK);
+        const int ij = col - static_cast<int>(cl * g.byKK.d);
+        const int i = static_cast<int>(fastdiv(static_cast<uint32_t>(ij), g.byKW));
+        const int j = ij - i * s.KW;
+        const int row = col < g.CK ? ((static_cast<int>(cl) - c0) * s.KH + i) * g.WX + j * s.dW + wave * s.sW : kWgMaxRows;
+        bAddr[0][nt] = row * kWgRow + ((h ^ (row & 7)) << 4);
+        bAddr[1][nt] = row * kWgRow + (((4 + h) ^ (row & 7)) << 4);
+    }
+
+    floatx4 acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    if (tid < 2 * (kWgRow / 4)) {
+        const int b = tid / (kWgRow / 4), e = tid - b * (kWgRow / 4);
+        lds[(b * kWgBuf + kWgMaxRows * kWgRow) / 4 + e] = 0.f;
+    }
+
+    const int p0 = slice * g.pairsPerSlice, p1 = min(g.pairs, p0 + g.pairsPerSlice);
+    int sOff[NS], aOff[MT];
+    // offsets of a pixel block: patch positions outside the image, or right of what the block's valid
+    // pixels read, are loaded as zeros; so are the A rows of pixels past the end of the output row
+    auto place = [&](int blockOfAll) {
+        const int n = static_cast<int>(fastdiv(static_cast<uint32_t>(blockOfAll), g.byBlocks));
+        const int block = blockOfAll - n * static_cast<int>(g.byBlocks.d);
+        goB = make_buffer(g.gradOut + (static_cast<int64_t>(n) * s.O + grp * g.Og) * goPlane);
+        inB = make_buffer(g.in + (static_cast<int64_t>(n) * s.C + grp * g.Cg + c0) * inPlane);
+        const int a = static_cast<int>(fastdiv(static_cast<uint32_t>(block), g.byBlocksPerRow));
+        const int b0 = (block - a * g.blocksPerRow) * kWgPix;
+        const int nv = min(kWgPix, s.OW - b0);
+        const int xLimit = (nv - 1) * s.sW + (s.KW - 1) * s.dW + 1;
+        const int y0 = a * s.sH - s.pH, x0 = b0 * s.sW - s.pW;
+#pragma unroll
+        for (int m = 0; m < NS; ++m) {
+            const int row = (tid >> 3) + 32 * m;
+            const uint32_t cl = fastdiv(static_cast<uint32_t>(row), g.byPatch);
+            const int rem = row - static_cast<int>(cl * g.byPatch.d);
+            const int i = static_cast<int>(fastdiv(static_cast<uint32_t>(rem), g.byWX));
+            const int x = rem - i * g.WX;
+            const int y = y0 + i * s.dH, xx = x0 + x;
+            const bool ok = row < g.rows && c0 + static_cast<int>(cl) < g.Cg && x < xLimit &&
+                            static_cast<unsigned>(y) < static_cast<unsigned>(s.H) &&
+                            static_cast<unsigned>(xx) < static_cast<unsigned>(s.W);
+            sOff[m] = masked_offset(ok, static_cast<int>(cl) * static_cast<int>(inPlane) * 4 + y * rowBytes + xx * pixBytes + u * 16);
+        }
+        const int b = b0 + wave;
+        const int pix = (a * s.OW + b) * pixBytes;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) aOff[mt] = masked_offset(b < s.OW && offA[mt] != kOutOfRange, offA[mt] + pix);
+    };
+    // Always the same number of loads, masked when there is no next pair: the waits in the loop then leave
+    // exactly this batch in flight on every path.  `plain`: every sample of the step exists, so the block's
+    // offsets are used as they are.
+    auto issue = [&](float4 (&R)[NS], float4 (&A)[2][MT], int st, bool more) {
+        const int tBytes = st << 7;
+        if (more && (st << 5) + 32 <= s.T) {
+#pragma unroll
+            for (int m = 0; m < NS; ++m) R[m] = buffer_load4<0>(inB, sOff[m], tBytes);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                A[0][mt] = buffer_load4<0>(goB, aOff[mt], tBytes);
+                A[1][mt] = buffer_load4<0>(goB, aOff[mt], tBytes + 64);
+            }
+        } else {
+            const bool liveU = more && (st << 5) + (u << 2) < s.T;
+            const bool liveH0 = more && (st << 5) + (h << 2) < s.T, liveH1 = more && (st << 5) + 16 + (h << 2) < s.T;
+#pragma unroll
+            for (int m = 0; m < NS; ++m) R[m] = buffer_load4<0>(inB, liveU ? sOff[m] : kOutOfRange, tBytes);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                A[0][mt] = buffer_load4<0>(goB, liveH0 ? aOff[mt] : kOutOfRange, tBytes);
+                A[1][mt] = buffer_load4<0>(goB, liveH1 ? aOff[mt] : kOutOfRange, tBytes + 64);
+            }
+        }
+    };
+    auto stage = [&](const float4 (&R)[NS], int buf) {
+#pragma unroll
+        for (int m = 0; m < NS; ++m) *reinterpret_cast<float4 *>(ldsBytes + buf + stageAddr + m * 32 * kWgRow) = R[m];
+    };
+#define SLAYER_WGRAD_LDS_MFMA(HALF, E)                                                                    \
+    _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)     \
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[HALF][mt].E, B[nt].E, acc[mt][nt], 0, 0, 0);
+    // (the second half of a row's last step may lie past the end of the row: nothing to add then)
+    auto multiply = [&](const float4 (&A)[2][MT], int buf, bool second) {
+        {
+            float4 B[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) B[nt] = *reinterpret_cast<const float4 *>(ldsBytes + buf + bAddr[0][nt]);
+            SLAYER_WGRAD_LDS_MFMA(0, x)
+            SLAYER_WGRAD_LDS_MFMA(0, y)
+            SLAYER_WGRAD_LDS_MFMA(0, z)
+            SLAYER_WGRAD_LDS_MFMA(0, w)
+        }
+        if (second) {
+            float4 B[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) B[nt] = *reinterpret_cast<const float4 *>(ldsBytes + buf + bAddr[1][nt]);
+            SLAYER_WGRAD_LDS_MFMA(1, x)
+            SLAYER_WGRAD_LDS_MFMA(1, y)
+            SLAYER_WGRAD_LDS_MFMA(1, z)
+            SLAYER_WGRAD_LDS_MFMA(1, w)
+        }
+    };
+#undef SLAYER_WGRAD_LDS_MFMA
+
+    {
+        // Trip k of the loop loads pair p0 + k into registers, multiplies pair p0 + k - 1 from its LDS buffer
+        // ((k - 1) % 2) and then writes the registers to the other buffer: the loop's code exists once, its
+        // first trip only loads.
+        int block = static_cast<int>(fastdiv(static_cast<uint32_t>(p0), g.bySteps));
+        int st = p0 - block * g.steps;
+        float4 R[NS], A[2][MT];
+        int buf = kWgBuf;
+        bool first = true, second = false;
+#pragma nounroll
+        for (int p = p0 - 1;; ++p) {
+            const bool more = p + 1 < p1;
+            bool moved = first;
+            if (more && !first && ++st == g.steps) {
+                st = 0;
+                ++block;
+                moved = true;
+            }
+            if (more && moved) place(block);
+            float4 An[2][MT];
+            issue(R, An, st, more);
+            __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the pair's matrix work
+            if (!first) multiply(A, buf, second);
+            __builtin_amdgcn_sched_barrier(0);
+            if (!more) break;
+            second = (st << 5) + 16 < s.T;
+            buf = kWgBuf - buf;
+            stage(R, buf);
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) A[hf][mt] = An[hf][mt];
+            __syncthreads();
+            first = false;
+        }
+    }
+
+    // every wavefront puts its tiles into LDS (the patches are no longer needed); the work-group adds the four
+    // copies in wavefront order and writes one workspace row.  Element v of a lane's accumulator is row 4 * h + v,
+    // column r of the tile.
+    __syncthreads();
+    floatx4 *const red = reinterpret_cast<floatx4 *>(lds);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) red[(wave * MT * NT + mt * NT + nt) * 64 + lane] = acc[mt][nt];
+    __syncthreads();
+    float *row = g.partial + static_cast<int64_t>(slice) * g.nW;
+#pragma unroll 1
+    for (int e = tid; e < MT * NT * 64; e += 256) {
+        const int tile = e >> 6, l = e & 63;
+        const int mt = tile / NT, nt = tile - mt * NT;
+        const floatx4 sum = ((red[e] + red[MT * NT * 64 + e]) + red[2 * MT * NT * 64 + e]) + red[3 * MT * NT * 64 + e];
+        const int o = ((og * MT + mt) << 4) + ((l >> 4) << 2);
+        const int col = ((cg * NT + nt) << 4) + (l & 15);
+        if (col < g.CK) {
+            float *cell = row + static_cast<int64_t>(grp * g.Og + o) * g.CK + col;
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (o + v < g.Og) cell[static_cast<int64_t>(v) * g.CK] = sum[v];
+        }
+    }
+}
+
 // gradW[q] = sum of the workspace rows: lane (q, part) adds rows part, part+PARTS, ... in order, then
 // the PARTS sums of a weight are added in order (a fixed association for a given geometry).  A group
 // handles 256 / PARTS weights; few weights take more parts so that the launch still fills the GPU.
@@ -776,6 +1018,111 @@ static int launch_wgrad_mfma(const float *gradOut, const float *in, float *works
     return status == SLAYER_OK ? s.N * p.slices : -status;
 }
 
+// Tiling of the LDS-staged matrix-core weight gradient: the tiles of plan_wgrad_mfma, blocks of kWgPix
+// pixels, and ranges of (block, step) pairs so that one wave of work-groups (two per compute unit of the
+// 256) covers the tensor.
+struct LdsPlan {
+    bool use;
+    int NS, WX, rows, blocksPerRow, steps, pairs, slices, pairsPerSlice;
+};
+
+static LdsPlan plan_wgrad_lds(const SynGeom &s, const MfmaPlan &m)
+{
+    LdsPlan p{};
+    if (!m.use) return p;
+    const int Cg = s.C / s.groups, KK = s.KH * s.KW, CK = Cg * KK;
+    const int64_t WX = static_cast<int64_t>(kWgPix - 1) * s.sW + static_cast<int64_t>(s.KW - 1) * s.dW + 1;
+    int channels = 0;  // most channels that one column group's columns belong to
+    for (int cg = 0; cg < m.colGroups; ++cg) {
+        const int col0 = cg * m.NT * 16, col1 = (CK < col0 + m.NT * 16 ? CK : col0 + m.NT * 16) - 1;
+        if (col1 >= col0 && col1 / KK - col0 / KK + 1 > channels) channels = col1 / KK - col0 / KK + 1;
+    }
+    const int64_t rows = channels * s.KH * WX;
+    if (rows < 1 || rows > kWgMaxRows) return p;
+    p.use = true;
+    p.WX = static_cast<int>(WX);
+    p.rows = static_cast<int>(rows);
+    p.NS = rows <= 96 ? 3 : rows <= 192 ? 6 : 9;       // passes of 32 rows
+    p.blocksPerRow = static_cast<int>(ceil_div(s.OW, kWgPix));
+    p.steps = (s.T + 31) / 32;
+    const int64_t pairs = static_cast<int64_t>(s.N) * s.OH * p.blocksPerRow * p.steps;   // of the whole batch
+    if (pairs >= (1LL << 30)) {
+        p.use = false;
+        return p;
+    }
+    p.pairs = static_cast<int>(pairs);
+    const int64_t base = static_cast<int64_t>(s.groups) * m.oGroups * m.colGroups;
+    // two work-groups per compute unit; a few short of the 512 places, which measured faster than all of them
+    // (504: 110 us, 512: 123 us on the 2 -> 16 channel 5 x 5 layer)
+    int64_t slices = 504 / base;
+    if (slices < 1) slices = 1;
+    if (slices > pairs) slices = pairs;
+    p.pairsPerSlice = static_cast<int>(ceil_div(pairs, slices));
+    p.slices = static_cast<int>(ceil_div(pairs, p.pairsPerSlice));
+    return p;
+}
+
+template <int MT, int NT, int NS>
+static void launch_wgrad_lds_one(const WgradLdsArgs &g, unsigned blocks, hipStream_t st)
+{
+    // two patches of kWgBuf bytes: more than the 64 KB a kernel may use without asking
+    static const hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&synapse_wgrad_lds_kernel<MT, NT, NS>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kWgBuf);
+    if (raised != hipSuccess) {
+        note_hip_error(raised);
+        return;
+    }
+    hipLaunchKernelGGL((synapse_wgrad_lds_kernel<MT, NT, NS>), dim3(blocks), dim3(256), 2 * kWgBuf, st, g);
+}
+
+template <int MT, int NS>
+static void launch_wgrad_lds_nt(const WgradLdsArgs &g, int NT, unsigned blocks, hipStream_t st)
+{
+    switch (NT) {
+        case 9: launch_wgrad_lds_one<MT, 9, NS>(g, blocks, st); break;
+        case 6: launch_wgrad_lds_one<MT, 6, NS>(g, blocks, st); break;
+        case 4: launch_wgrad_lds_one<MT, 4, NS>(g, blocks, st); break;
+        case 2: launch_wgrad_lds_one<MT, 2, NS>(g, blocks, st); break;
+        default: launch_wgrad_lds_one<MT, 1, NS>(g, blocks, st); break;
+    }
+}
+
+// Returns the number of workspace rows written, or a negative status.
+static int launch_wgrad_lds(const float *gradOut, const float *in, float *workspace, const SynGeom &s,
+                            const MfmaPlan &m, const LdsPlan &p, int nW, hipStream_t st)
+{
+    WgradLdsArgs g{};
+    g.gradOut = gradOut; g.in = in; g.partial = workspace; g.s = s;
+    g.Cg = s.C / s.groups; g.Og = s.O / s.groups; g.CK = g.Cg * s.KH * s.KW;
+    g.oGroups = m.oGroups; g.colGroups = m.colGroups;
+    g.WX = p.WX; g.rows = p.rows; g.blocksPerRow = p.blocksPerRow; g.steps = p.steps;
+    g.pairs = p.pairs; g.slices = p.slices; g.pairsPerSlice = p.pairsPerSlice; g.nW = nW;
+    g.byColGroups = make_fastdiv(static_cast<uint32_t>(m.colGroups));
+    g.byOGroups = make_fastdiv(static_cast<uint32_t>(m.oGroups));
+    g.byGroups = make_fastdiv(static_cast<uint32_t>(s.groups));
+    g.byKK = make_fastdiv(static_cast<uint32_t>(s.KH * s.KW));
+    g.byKW = make_fastdiv(static_cast<uint32_t>(s.KW));
+    g.byBlocks = make_fastdiv(static_cast<uint32_t>(s.OH * p.blocksPerRow));
+    g.bySteps = make_fastdiv(static_cast<uint32_t>(p.steps));
+    g.byBlocksPerRow = make_fastdiv(static_cast<uint32_t>(p.blocksPerRow));
+    g.byPatch = make_fastdiv(static_cast<uint32_t>(s.KH * p.WX));
+    g.byWX = make_fastdiv(static_cast<uint32_t>(p.WX));
+    const int64_t blocks = static_cast<int64_t>(s.groups) * m.oGroups * m.colGroups * p.slices;
+    if (blocks >= (1LL << 31)) return -SLAYER_EUNSUPPORTED;
+    const unsigned nb = static_cast<unsigned>(blocks);
+    if (m.MT == 2) {
+        if (p.NS == 9) launch_wgrad_lds_nt<2, 9>(g, m.NT, nb, st);
+        else if (p.NS == 6) launch_wgrad_lds_nt<2, 6>(g, m.NT, nb, st);
+        else launch_wgrad_lds_nt<2, 3>(g, m.NT, nb, st);
+    } else {
+        if (p.NS == 9) launch_wgrad_lds_nt<1, 9>(g, m.NT, nb, st);
+        else if (p.NS == 6) launch_wgrad_lds_nt<1, 6>(g, m.NT, nb, st);
+        else launch_wgrad_lds_nt<1, 3>(g, m.NT, nb, st);
+    }
+    const int status = launch_status();
+    return status == SLAYER_OK ? p.slices : -status;
+}
+
 template <int OBW, int TAPS>
 static void launch_wgrad_vec(const WgradArgs &g, int VEC, unsigned blocks, hipStream_t st)
 {
@@ -844,7 +1191,11 @@ extern "C" int64_t slayer_synapse_conv_grad_weight_workspace_bytes(const slayer_
     if (nW == 0 || s.N == 0) return 0;
     const WgradPlan p = plan_wgrad(s, s.T % 4 == 0);
     const MfmaPlan m = plan_wgrad_mfma(s);
-    const int64_t rows = static_cast<int64_t>(s.N) * (m.use && m.slices > p.slicesPerItem ? m.slices : p.slicesPerItem);
+    const LdsPlan l = plan_wgrad_lds(s, m);
+    int64_t most = p.slicesPerItem;
+    if (m.use && m.slices > most) most = m.slices;
+    int64_t rows = static_cast<int64_t>(s.N) * most;
+    if (l.use && l.slices > rows) rows = l.slices;
     return rows * nW * static_cast<int64_t>(sizeof(float));
 }
 
@@ -872,7 +1223,9 @@ extern "C" int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gr
         const bool vec = vecT && aligned16(gradOut) && aligned16(in);
         const MfmaPlan m = plan_wgrad_mfma(s);
         if (m.use && vec && !generic_forced()) {
-            rows = launch_wgrad_mfma(gradOut, in, workspace, s, m, nW, st);
+            const LdsPlan l = plan_wgrad_lds(s, m);
+            rows = l.use ? launch_wgrad_lds(gradOut, in, workspace, s, m, l, nW, st)
+                         : launch_wgrad_mfma(gradOut, in, workspace, s, m, nW, st);
             if (rows < 0) return -rows;
             launch_wgrad_sum(gradW, workspace, rows, nW, st);
             return launch_status();

@@ -57,6 +57,11 @@ CASES = [
     (2, 32, 10, 11, 16, 48, (3, 2), (2, 1), (1, 0), (1, 2), 2),  # groups of 24 channels x 96 columns, stride, dilation
     (2, 15, 8, 9, 24, 9, (3, 3), 2, 1, 1, 1),         # stride 2, 9 output channels, 135 columns
     (1, 8, 6, 6, 64, 72, (3, 3), 1, 1, 1, 1),         # 72 output channels: two blocks of four tiles
+    # ... with the input patch of four pixels staged in LDS per step of 32 samples: ragged pixel blocks (13 columns),
+    # a last step of 12 samples, ranges of (block, step) pairs that cross batch items
+    (3, 16, 9, 13, 44, 32, (3, 3), 1, 1, 1, 1),
+    (2, 8, 6, 7, 100, 16, (5, 5), 1, 2, 1, 1),        # 200 columns: two column groups of 6 and 3 channels
+    (2, 16, 6, 6, 36, 16, (3, 3), 1, 0, 2, 1),        # dilation 2 without padding: 2 x 2 output pixels
 ]
 IDS = ["%dx%dx%dx%dx%d-o%d-k%s-s%s-p%s-d%s-g%d" % c for c in CASES]
 
