@@ -3,24 +3,30 @@
 //
 //   conv: out[n][t] = Ts * sum_i in[n][t-i] * filt[i]     corr: out[n][t] = Ts * sum_i in[n][t+i] * filt[i]
 //
-// Every output is one chain acc = fma(in, filt[i], acc) over i = 0,1,..,F-1 starting from 0,
-// then one multiply by Ts, exactly like the sequential loop; samples outside [0,T) enter as
-// zeros, which leaves the chain's value unchanged.
+// The reference's definition of an output is one chain acc = fma(in, filt[i], acc) over i = 0,1,..,F-1
+// starting from 0, then one multiply by Ts; samples outside [0,T) enter as zeros, which leaves the
+// chain's value unchanged.
 //
-// Three kernels share that definition (the plain correlation with 34 to 129 taps on rows of whole 16-byte
-// vectors goes to the matrix-core kernel of fir_mfma.hip instead, which agrees with it to rounding):
-//  * direct: rows of whole 16-byte vectors and filters of at most 33 taps (81 for the
-//    correlation): everything in registers, addressing of a plain copy;
+// Three kernels here (the plain correlation with 34 to 129 taps on rows of whole 16-byte vectors goes to
+// the matrix-core kernel of fir_mfma.hip first):
+//  * direct: rows of whole 16-byte vectors and filters of at most 33 taps: everything in registers,
+//    addressing of a plain copy, the chain bit for bit;
 //  * tiled: the convolution is the correlation on a reversed time axis, so both share one core
 //    Y[m] = sum_i X[m+i] * filt[i].  A work-group of 256 lanes owns R consecutive neuron rows
 //    and one time tile; it stages the rows' samples (plus the F-1 sample halo, zero padded) into
-//    LDS as X[R][LD] with 16-byte loads (reversed in time for the convolution).  Dense tiles are
-//    cut into chunks of U (8 or 16) consecutive outputs of one row; lanes take chunks in row-major
-//    order, keep a (U+4)-sample register window of X and slide it 4 samples per 4 taps with one
-//    16-byte LDS read, i.e. one LDS read feeds 4 U FMAs; filter taps are wave-uniform and come
-//    through scalar loads.  Tiles whose input is almost all zeros (spike trains) take an
-//    event-driven path instead.  An FIR with F = 77 taps needs 154 flop per 8 bytes moved, which
-//    is at the FP32 ridge of the machine: on dense input the kernel is FMA-issue bound;
+//    LDS as X[R][LD] with 16-byte loads (reversed in time for the convolution) and counts the non-zero
+//    vectors on the way.  Then one of three paths per tile:
+//      - almost all zeros (spike trains): event-driven, one update per non-zero sample, the bits of the
+//        chain with its zero terms left out;
+//      - dense, 34 to 129 taps, whole-vector rows (template DM > 0): the tile's outputs as products of
+//        a banded Toeplitz matrix of the filter with blocks of 16 samples on the matrix cores
+//        (v_mfma_f32_16x16x4_f32; fir_core.h has the formulation): agrees with the chain to rounding,
+//        a tile with a non-finite sample is recomputed as chains so that infinities and NaNs land
+//        where the reference puts them;
+//      - otherwise the chain on the vector ALUs: chunks of U (8 or 16) consecutive outputs of one row
+//        per lane, a (U+4)-sample register window slid 4 samples per 4 taps with one 16-byte LDS read,
+//        taps through scalar loads; bit-identical to the sequential loop.  An FIR with F = 77 taps
+//        needs 154 flop per 8 bytes moved, the FP32 ridge of the machine: this path is FMA-issue bound;
 //  * generic: one lane per output, any shape.
 #include "common.h"
 #include "fir_core.h"

@@ -171,7 +171,8 @@ constexpr int kTileScalar = 0, kTileVec = 1, kTileFlat = 2;
 // Optional time shift of the spike output (the delayShift that follows spike() in networks with
 // axonal delays, fused into the store of the spikes): s[t] = spike[t - k], k = (int)(delay / Ts),
 // with one delay for all rows or one per neuron of a batch item (row % lutSize).  The membrane
-// potential is not shifted.  Only tiles whose rows travel whole support it.
+// potential is not shifted.  Tiles whose rows travel whole read the shifted bits from the tile's masks; rows in
+// pieces keep the spike bits of the whole row in LDS (rows of whole vectors up to kSpikeRecordMaxT samples).
 struct SpikeDelay {
     const float *lut;   // per-neuron delays, or NULL
     int64_t lutSize;    // neurons per batch item when lut is given
