@@ -453,7 +453,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                 return m;
             };
             // the same from the record of the whole row (rows in pieces): the four bits from bit c2 on
-            const int nBits = T + LAG, nWords = (nBits + 31) >> 5;
+            const int nBits = T + LAG;
             auto bits_of_row = [&](int r, int c2) -> uint32_t {
                 // no branches: the LDS reads of all vectors of a step go out together.  Bits before LAG and from
                 // nBits on are never set, and the word behind a row's last is kept at zero.

@@ -210,6 +210,129 @@ __global__ __launch_bounds__(256) void synapse_gather_kernel(GatherArgs g)
 }
 
 
+// ---- gather with few destination channels: several pixels of a row per lane ---------------------------
+// With one or two destination channels (the input gradient of a network's first layer) the kernel above
+// issues one 16-byte load per 4 or 8 multiply-adds and is bound by its loads.  Here a lane owns PX adjacent
+// destination pixels of one row (unit stride and dilation along W: pixel p's tap j reads source column
+// p + j or p - j, so the PX pixels' KW taps fall on E = PX + KW - 1 distinct columns): per source channel and
+// filter row it loads those columns once, and each loaded vector feeds every (pixel, tap) pair that
+// lands on it - PX * KW * MB * 4 multiply-adds per E loads.  KW is a template parameter, so which pairs those
+// are is known at compile time and the filter row's weights sit in registers; the E loads of a filter row are
+// issued one row ahead of its multiply-adds (two rows per trip, so that the two sets of registers swap roles
+// without copies).  Weights come from LDS in chunks of whole filter rows, [row][j][m].
+constexpr int kGatherRowPx = 4;
+
+template <int MB, int KW, bool BACKWARD>
+__global__ __launch_bounds__(256) void synapse_gather_row_kernel(GatherArgs g)
+{
+    constexpr int PX = kGatherRowPx, E = PX + KW - 1;
+    constexpr int kRows = kTapChunk / KW;                 // filter rows per chunk of weights
+    __shared__ __attribute__((aligned(16))) float wl[kRows * KW * MB];
+
+    uint32_t rest = xcd_contiguous(blockIdx.x, gridDim.x);
+    const uint32_t nc = fastdiv(rest, g.byMBlocks);
+    const int mb0 = static_cast<int>(rest - nc * g.byMBlocks.d) * MB;
+    const uint32_t ng = fastdiv(nc, g.byChunks);
+    const int chunk = static_cast<int>(nc - ng * g.byChunks.d);
+    const uint32_t n = fastdiv(ng, g.byGroups);
+    const int grp = static_cast<int>(ng - n * g.byGroups.d);
+
+    // lane -> (row a, group of PX pixels, vector of time samples); g.P counts those, g.byDW divides by the
+    // pixel groups per row
+    const int p = chunk * 256 + static_cast<int>(threadIdx.x);
+    const bool live = p < g.P;
+    const uint32_t pg = fastdiv(static_cast<uint32_t>(live ? p : 0), g.byTV);
+    const int tv = (live ? p : 0) - static_cast<int>(pg * g.byTV.d);
+    const int a = static_cast<int>(fastdiv(pg, g.byDW));
+    const int b0 = (static_cast<int>(pg) - a * static_cast<int>(g.byDW.d)) * PX;
+
+    const int64_t srcPlane = static_cast<int64_t>(g.SH) * g.SW * g.T;
+    const BufferRsrc srcB = make_buffer(g.src + (static_cast<int64_t>(n) * g.SC + static_cast<int64_t>(grp) * g.Qg) * srcPlane);
+    const int rowBytes = g.SW * g.T * 4, pixBytes = g.T * 4, planeBytes = static_cast<int>(srcPlane) * 4;
+    const int yBase = a * g.mulH;
+    // source column of pixel p, tap j: b0 + p + offW + j * stepW with stepW = 1 (forward) or -1 (gradient), i.e.
+    // x0 + e with e = p + j or p - j + KW - 1, 0 <= e < E
+    const int x0 = b0 + g.offW - (BACKWARD ? KW - 1 : 0);
+    // the lane's columns: byte offsets within a source row, masked where the column is outside the image
+    int colOff[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+        colOff[e] = masked_offset(live && static_cast<unsigned>(x0 + e) < static_cast<unsigned>(g.SW), (x0 + e) * pixBytes + tv * 16);
+
+    TimeVec<4> acc[PX][MB];
+#pragma unroll
+    for (int px = 0; px < PX; ++px)
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[px][m].zero();
+
+    const int KK = g.KH * KW;
+    const int rows = g.Qg * g.KH;                      // (source channel, filter row) pairs
+    for (int r0 = 0; r0 < rows; r0 += kRows) {
+        const int rc = min(kRows, rows - r0);
+        __syncthreads();
+        for (int e = threadIdx.x; e < rc * KW * MB; e += 256) {
+            const int tap = r0 * KW + e / MB, m = mb0 + e % MB;   // tap in (q, i, j) order
+            const int q = tap / KK, ij = tap - q * KK;
+            float v = 0.f;
+            if (m < g.Mg) {
+                const int64_t idx = BACKWARD
+                    ? (static_cast<int64_t>(grp * g.Og + q) * g.Cg + m) * KK + ij
+                    : (static_cast<int64_t>(grp * g.Og + m) * g.Cg + q) * KK + ij;
+                v = g.w[idx];
+            }
+            wl[e] = v;
+        }
+        __syncthreads();
+
+        int q = r0 / g.KH, i = r0 - q * g.KH;          // the filter row to load next (wave-uniform)
+        auto fetch = [&](TimeVec<4> (&X)[E], bool more) {
+            const int y = yBase + g.offH + i * g.stepH;
+            const bool ok = more && static_cast<unsigned>(y) < static_cast<unsigned>(g.SH);
+            const int rowOff = q * planeBytes + y * rowBytes;
+#pragma unroll
+            for (int e = 0; e < E; ++e) X[e].load(srcB, ok && colOff[e] != kOutOfRange ? colOff[e] + rowOff : kOutOfRange);
+            if (++i == g.KH) { i = 0; ++q; }
+        };
+        auto madd = [&](const TimeVec<4> (&X)[E], int row) {
+            float w[KW][MB];
+            const float *wr = wl + row * KW * MB;
+#pragma unroll
+            for (int j = 0; j < KW; ++j)
+#pragma unroll
+                for (int m = 0; m < MB; ++m) w[j][m] = wr[j * MB + m];
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+#pragma unroll
+                for (int px = 0; px < PX; ++px) {
+                    const int j = BACKWARD ? px - e + KW - 1 : e - px;
+                    if (j >= 0 && j < KW) {
+#pragma unroll
+                        for (int m = 0; m < MB; ++m) acc[px][m].fma(w[j][m], X[e]);
+                    }
+                }
+        };
+        TimeVec<4> XA[E], XB[E];
+        fetch(XA, true);
+        for (int r = 0; r < rc; r += 2) {
+            fetch(XB, r + 1 < rc);
+            madd(XA, r);
+            fetch(XA, r + 2 < rc);
+            if (r + 1 < rc) madd(XB, r + 1);
+        }
+    }
+
+    const int64_t dstPlane = static_cast<int64_t>(g.DH) * g.DW * g.T;
+    const BufferRsrc dstB = make_buffer(g.dst + (static_cast<int64_t>(n) * g.DC + static_cast<int64_t>(grp) * g.Mg) * dstPlane);
+    const int dstPlaneBytes = static_cast<int>(dstPlane) * 4;
+#pragma unroll
+    for (int px = 0; px < PX; ++px)
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+            acc[px][m].store(dstB, masked_offset(live && b0 + px < g.DW && mb0 + m < g.Mg,
+                                                 (mb0 + m) * dstPlaneBytes + ((a * g.DW + b0 + px) * g.T) * 4 + tv * 16));
+}
+
+
 // Input gradient of a one-channel synapse whose windows do not overlap (stride = window, no padding,
 // no dilation: the pooling layers).  Every input pixel belongs to exactly one window, so a lane
 // reads one vector of gradOut, scales it by the weight of its position in the window and writes
@@ -874,10 +997,36 @@ static int launch_gather(float *dst, const float *src, const float *w, const Syn
         else hipLaunchKernelGGL(synapse_window_bwd_kernel<1>, dim3(static_cast<unsigned>(nBlocks)), dim3(256), 0, st, a);
         return launch_status();
     }
-    g.P = g.DH * g.DW * (g.T / VEC);
-    g.chunks = static_cast<int>(ceil_div(g.P, 256));
     // destination channels per lane: as many as the group has, up to 16
     const int MB = g.Mg >= 12 ? 16 : g.Mg >= 6 ? 8 : g.Mg >= 3 ? 4 : g.Mg == 2 ? 2 : 1;
+    // one or two of them, and a filter wide enough for neighbouring pixels to share source columns: PX pixels per lane
+    if (MB <= 2 && vec && !strided && g.mulW == 1 && g.stepW == (BACKWARD ? -1 : 1) && (g.KW == 3 || g.KW == 5 || g.KW == 7) &&
+        static_cast<int64_t>(g.Qg) * g.KH * g.KW >= 32 && !generic_forced()) {
+        const int pixelGroups = static_cast<int>(ceil_div(g.DW, kGatherRowPx));
+        g.P = g.DH * pixelGroups * (g.T / 4);
+        g.chunks = static_cast<int>(ceil_div(g.P, 256));
+        g.mBlocks = static_cast<int>(ceil_div(g.Mg, MB));
+        const int64_t blocks = static_cast<int64_t>(s.N) * s.groups * g.mBlocks * g.chunks;
+        if (blocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+        g.byChunks = make_fastdiv(static_cast<uint32_t>(g.chunks));
+        g.byMBlocks = make_fastdiv(static_cast<uint32_t>(g.mBlocks));
+        g.byGroups = make_fastdiv(static_cast<uint32_t>(s.groups));
+        g.byTV = make_fastdiv(static_cast<uint32_t>(g.T / 4));
+        g.byDW = make_fastdiv(static_cast<uint32_t>(pixelGroups));
+        const dim3 nb(static_cast<unsigned>(blocks));
+#define SLAYER_GATHER_ROW(MBV)                                                                                          \
+    do {                                                                                                                \
+        if (g.KW == 3) hipLaunchKernelGGL((synapse_gather_row_kernel<MBV, 3, BACKWARD>), nb, dim3(256), 0, st, g);       \
+        else if (g.KW == 5) hipLaunchKernelGGL((synapse_gather_row_kernel<MBV, 5, BACKWARD>), nb, dim3(256), 0, st, g);  \
+        else hipLaunchKernelGGL((synapse_gather_row_kernel<MBV, 7, BACKWARD>), nb, dim3(256), 0, st, g);                 \
+    } while (0)
+        if (MB == 2) SLAYER_GATHER_ROW(2);
+        else SLAYER_GATHER_ROW(1);
+#undef SLAYER_GATHER_ROW
+        return launch_status();
+    }
+    g.P = g.DH * g.DW * (g.T / VEC);
+    g.chunks = static_cast<int>(ceil_div(g.P, 256));
     g.mBlocks = static_cast<int>(ceil_div(g.Mg, MB));
     const int64_t blocks = static_cast<int64_t>(s.N) * s.groups * g.mBlocks * g.chunks;
     if (blocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;

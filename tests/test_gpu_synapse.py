@@ -62,6 +62,11 @@ CASES = [
     (3, 16, 9, 13, 44, 32, (3, 3), 1, 1, 1, 1),
     (2, 8, 6, 7, 100, 16, (5, 5), 1, 2, 1, 1),        # 200 columns: two column groups of 6 and 3 channels
     (2, 16, 6, 6, 36, 16, (3, 3), 1, 0, 2, 1),        # dilation 2 without padding: 2 x 2 output pixels
+    # one or two destination channels and a filter at least 3 wide: four pixels of a row per lane
+    (1, 8, 7, 9, 8, 2, (3, 3), 1, 1, 1, 1),           # forward with 2 output channels, 9 columns = 2 groups + 1 pixel
+    (2, 1, 9, 11, 16, 8, (3, 5), 1, (1, 2), 1, 1),    # input gradient with 1 channel, 3 x 5 filter
+    (1, 2, 10, 10, 8, 8, (3, 3), 1, (2, 1), (2, 1), 1),   # dilation along H only
+    (1, 2, 6, 40, 4, 12, (1, 7), 1, (0, 3), 1, 1),    # 1 x 7 filter: 84 taps, 10 columns per lane
 ]
 IDS = ["%dx%dx%dx%dx%d-o%d-k%s-s%s-p%s-d%s-g%d" % c for c in CASES]
 
