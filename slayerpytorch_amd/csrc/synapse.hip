@@ -10,6 +10,8 @@
 // as the reduction axis, runs on the matrix cores (with a vector kernel for small or unaligned
 // shapes); pooling has a streaming input gradient.  Work-groups that read the same rows are kept
 // on the same die (xcd_contiguous).
+#include <atomic>
+
 #include "common.h"
 
 namespace slayer {
@@ -1212,27 +1214,33 @@ static LdsPlan plan_wgrad_lds(const SynGeom &s, const MfmaPlan &m)
 }
 
 template <int MT, int NT, int NS>
-static void launch_wgrad_lds_one(const WgradLdsArgs &g, unsigned blocks, hipStream_t st)
+static int launch_wgrad_lds_one(const WgradLdsArgs &g, unsigned blocks, hipStream_t st)
 {
-    // two patches of kWgBuf bytes: more than the 64 KB a kernel may use without asking
-    static const hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&synapse_wgrad_lds_kernel<MT, NT, NS>),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kWgBuf);
-    if (raised != hipSuccess) {
-        note_hip_error(raised);
-        return;
+    // two patches of kWgBuf bytes: more than the 64 KB a kernel may use without asking; asked once per device
+    // (a host-side setting of the kernel, no allocation)
+    static std::atomic<bool> raised[64];
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err == hipSuccess && (device < 0 || device >= 64)) err = hipErrorInvalidDevice;
+    if (err == hipSuccess && !raised[device].load(std::memory_order_acquire)) {
+        err = hipFuncSetAttribute(reinterpret_cast<const void *>(&synapse_wgrad_lds_kernel<MT, NT, NS>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kWgBuf);
+        if (err == hipSuccess) raised[device].store(true, std::memory_order_release);
     }
+    if (err != hipSuccess) return note_hip_error(err);
     hipLaunchKernelGGL((synapse_wgrad_lds_kernel<MT, NT, NS>), dim3(blocks), dim3(256), 2 * kWgBuf, st, g);
+    return launch_status();
 }
 
 template <int MT, int NS>
-static void launch_wgrad_lds_nt(const WgradLdsArgs &g, int NT, unsigned blocks, hipStream_t st)
+static int launch_wgrad_lds_nt(const WgradLdsArgs &g, int NT, unsigned blocks, hipStream_t st)
 {
     switch (NT) {
-        case 9: launch_wgrad_lds_one<MT, 9, NS>(g, blocks, st); break;
-        case 6: launch_wgrad_lds_one<MT, 6, NS>(g, blocks, st); break;
-        case 4: launch_wgrad_lds_one<MT, 4, NS>(g, blocks, st); break;
-        case 2: launch_wgrad_lds_one<MT, 2, NS>(g, blocks, st); break;
-        default: launch_wgrad_lds_one<MT, 1, NS>(g, blocks, st); break;
+        case 9: return launch_wgrad_lds_one<MT, 9, NS>(g, blocks, st);
+        case 6: return launch_wgrad_lds_one<MT, 6, NS>(g, blocks, st);
+        case 4: return launch_wgrad_lds_one<MT, 4, NS>(g, blocks, st);
+        case 2: return launch_wgrad_lds_one<MT, 2, NS>(g, blocks, st);
+        default: return launch_wgrad_lds_one<MT, 1, NS>(g, blocks, st);
     }
 }
 
@@ -1259,16 +1267,14 @@ static int launch_wgrad_lds(const float *gradOut, const float *in, float *worksp
     const int64_t blocks = static_cast<int64_t>(s.groups) * m.oGroups * m.colGroups * p.slices;
     if (blocks >= (1LL << 31)) return -SLAYER_EUNSUPPORTED;
     const unsigned nb = static_cast<unsigned>(blocks);
+    int status;
     if (m.MT == 2) {
-        if (p.NS == 9) launch_wgrad_lds_nt<2, 9>(g, m.NT, nb, st);
-        else if (p.NS == 6) launch_wgrad_lds_nt<2, 6>(g, m.NT, nb, st);
-        else launch_wgrad_lds_nt<2, 3>(g, m.NT, nb, st);
+        status = p.NS == 9 ? launch_wgrad_lds_nt<2, 9>(g, m.NT, nb, st)
+               : p.NS == 6 ? launch_wgrad_lds_nt<2, 6>(g, m.NT, nb, st) : launch_wgrad_lds_nt<2, 3>(g, m.NT, nb, st);
     } else {
-        if (p.NS == 9) launch_wgrad_lds_nt<1, 9>(g, m.NT, nb, st);
-        else if (p.NS == 6) launch_wgrad_lds_nt<1, 6>(g, m.NT, nb, st);
-        else launch_wgrad_lds_nt<1, 3>(g, m.NT, nb, st);
+        status = p.NS == 9 ? launch_wgrad_lds_nt<1, 9>(g, m.NT, nb, st)
+               : p.NS == 6 ? launch_wgrad_lds_nt<1, 6>(g, m.NT, nb, st) : launch_wgrad_lds_nt<1, 3>(g, m.NT, nb, st);
     }
-    const int status = launch_status();
     return status == SLAYER_OK ? p.slices : -status;
 }
 
