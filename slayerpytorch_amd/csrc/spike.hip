@@ -213,6 +213,14 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     float tap[NU];
 #pragma unroll
     for (int j = 0; j < NU; ++j) tap[j] = (j < nuSize) ? nu[j] : -0.0f;
+    // this lane's taps in the candidate walk (lane p of a row: taps p, p + 64 / R, ...; -0.0f past the kernel, also
+    // past NU: those samples lie in the row's padding or belong to taps that do not exist)
+    float myTap[(NU + kWave / R - 1) / (kWave / R)];
+#pragma unroll
+    for (int j = 0; j < (NU + kWave / R - 1) / (kWave / R); ++j) {
+        const int tj = lane % (kWave / R) + j * (kWave / R);
+        myTap[j] = tj < nuSize ? nu[tj] : -0.0f;
+    }
     // The normal refractory kernel only lowers the potential (every tap <= 0; a NaN tap fails the test).  A sample
     // below the threshold as it arrives can then never fire, so the sequential part need only visit the samples
     // at or above it ("candidates", a few per cent): all 64 lanes mark them while the tile is staged, and the
@@ -345,41 +353,66 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         const int W = last ? n + LAG : n;
         // going from candidate to candidate costs a round trip through LDS each, and the wavefront stays as long as
         // its busiest row: it pays while no row of the tile has more than a candidate per 24 samples
+        // The walking wavefront shares its SIMD's issue slots with the wavefronts that move data, so what counts
+        // here is the number of instructions, not the active lanes: all 64 lanes take part, kParts = 64 / R per
+        // row.  They count the row's candidates and note its non-empty candidate words together; in the walk every
+        // lane of a row follows the same candidates, and on a spike each adds its own taps of the refractory
+        // response (lane p: taps p, p + kParts, ...).
+        constexpr int kParts = kWave / R, kRounds = (NU + kParts - 1) / kParts;
+        const int cr = lane / kParts, part = lane - cr * kParts;
         bool hop = monotone;
+        uint32_t nzw = 0u;   // bit w: word w of the row has candidates (at most 18 words: 512 + 32 samples)
         if (monotone) {
             int mine = 0;
-            if (lane < R)
-                for (int w = 0; w < ((W + 31) >> 5); ++w) mine += __builtin_popcount(cand[lane * MP + w]);
+            for (int w = part; w < ((W + 31) >> 5); w += kParts) {
+                const uint32_t c = cand[cr * MP + w];
+                mine += __builtin_popcount(c);
+                nzw |= (c != 0u ? 1u : 0u) << w;
+            }
+#pragma unroll
+            for (int off = kParts / 2; off > 0; off >>= 1) {
+                mine += __shfl_xor(mine, off, kWave);
+                nzw |= __shfl_xor(nzw, off, kWave);
+            }
+            // going from candidate to candidate pays while no row of the tile has more than a candidate per 24 samples
             hop = __builtin_amdgcn_ballot_w64(mine * 24 > W) == 0;
         }
         if (hop) {
-            // lane = row; every lane keeps its own place in its row's candidate words (lanes without a row have none)
-            const int words = lane < R ? (W + 31) >> 5 : 0;
-            const uint32_t *cw = cand + (lane < R ? lane : 0) * MP;
-            uint32_t *mw = record ? rowMasks + (lane < R ? lane : 0) * MPT + (tL >> 5) : masks + (lane < R ? lane : 0) * MP;
-            float *mine = tile + (lane < R ? lane : 0) * P;
+            const int words = (W + 31) >> 5;
+            const uint32_t *cw = cand + cr * MP;
+            uint32_t *mw = record ? rowMasks + cr * MPT + (tL >> 5) : masks + cr * MP;
+            float *mine = tile + cr * P;
+            for (int w = part; w < words; w += kParts) mw[w] = 0u;   // words without candidates have no spikes
             int w = 0;
-            uint32_t cm = words > 0 ? cw[0] : 0u, fired = 0u;
-            for (;;) {
-                while (cm == 0u && w + 1 < words) {
-                    mw[w] = fired;
+            uint32_t cm = 0u, fired = 0u;
+            while (__builtin_amdgcn_ballot_w64((cm | nzw) != 0u) != 0) {
+                if (cm == 0u && nzw != 0u) {   // on to the row's next word with candidates
+                    if (fired != 0u) mw[w] = fired;
                     fired = 0u;
-                    ++w;
+                    w = __builtin_ctz(nzw);
+                    nzw &= nzw - 1u;
                     cm = cw[w];
                 }
-                if (__builtin_amdgcn_ballot_w64(cm != 0u) == 0) break;
                 if (cm != 0u) {
                     const int k = __builtin_ctz(cm);
                     cm &= cm - 1u;
-                    float *q = mine + (w << 5) + k;
-                    if (q[0] >= theta) {
+                    float *q = mine + (w << 5) + k + part;
+                    // (no lane reaches past the NU samples of the response: what lies behind the row's padding
+                    // belongs to the next row)
+                    float val[kRounds];
+#pragma unroll
+                    for (int j = 0; j < kRounds; ++j)
+                        if ((j + 1) * kParts <= NU || part + j * kParts < NU) val[j] = q[j * kParts];
+                    const float x0 = __shfl(val[0], cr * kParts, kWave);   // the candidate itself: the value lane 0 of the row read
+                    if (x0 >= theta) {
                         fired |= 1u << k;
 #pragma unroll
-                        for (int j = 0; j < NU; ++j) q[j] += tap[j];
+                        for (int j = 0; j < kRounds; ++j)
+                            if ((j + 1) * kParts <= NU || part + j * kParts < NU) q[j * kParts] = val[j] + myTap[j];
                     }
                 }
             }
-            if (words > 0) mw[w] = fired;
+            if (fired != 0u) mw[w] = fired;
         } else if (lane < R) {
             // every sample in turn: 32 samples at a time are pulled into a register window v[0 .. 32+LAG), a spike
             // adds nu[0..NU) onto v[k .. k+NU), and the 32 oldest samples go back to LDS with their spike mask
@@ -488,7 +521,39 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
             rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
             const int dr = kWave / perRow, dc = kWave % perRow;
             if constexpr (VEC) {
-                // a fixed number of (masked) stores, see above
+              if (!dl.on) {
+                // a fixed number of (masked) stores, see above.  Half of a step's vectors at a time: their LDS reads
+                // go out together, the stores follow (one read-wait-store chain per vector cost a third of a step)
+                constexpr int HB = (NBR + 1) / 2;
+#pragma unroll
+                for (int b0 = 0; b0 < NBR; b0 += HB) {
+                    float4 uu[HB];
+                    uint32_t word[HB];
+                    int offs[HB], sh[HB];
+#pragma unroll
+                    for (int i = 0; i < HB; ++i) {
+                        if (b0 + i < NBR) {
+                            const bool on = lane + (b0 + i) * kWave < total;
+                            const int r = on ? rc.r : 0, col = on ? first + rc.c * V : first;
+                            uu[i] = *reinterpret_cast<const float4 *>(tile + r * P + col);
+                            word[i] = masks[r * MP + (col >> 5)];
+                            sh[i] = col & 31;
+                            offs[i] = masked_offset(on, (r * T + tW + col) * 4);
+                            rc.advance(dr, dc, perRow);
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < HB; ++i) {
+                        if (b0 + i < NBR) {
+                            const uint32_t m = word[i] >> sh[i];
+                            buffer_store4(bufU, offs[i], 0, uu[i]);
+                            buffer_store4(bufS, offs[i], 0,
+                                          make_float4((m & 1u) ? amplitude : 0.0f, (m & 2u) ? amplitude : 0.0f,
+                                                      (m & 4u) ? amplitude : 0.0f, (m & 8u) ? amplitude : 0.0f));
+                        }
+                    }
+                }
+              } else {
 #pragma unroll
                 for (int b = 0; b < NBR; ++b) {
                     const bool on = lane + b * kWave < total;
@@ -506,6 +571,7 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                                               (m & 4u) ? amplitude : 0.0f, (m & 8u) ? amplitude : 0.0f));
                     rc.advance(dr, dc, perRow);
                 }
+              }
             } else {
 #pragma unroll 4
                 for (int g0 = lane; g0 < total; g0 += kWave) {
