@@ -195,6 +195,13 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
     constexpr int NB = R * kPiece / (FLAT ? 4 : V) / kWave;  // accesses per lane per piece, at most
     // vectors per lane that leave in one step, at most: a row's last piece also retires the LAG columns behind it
     constexpr int NBR = (R * (kPiece + (LAG == 32 ? LAG : 0)) / 4 + kWave - 1) / kWave;
+    // Rows of whole vectors in pieces: a piece is kHalves runs of 64 vectors per row, so vector b of a lane can be
+    // vector lane + 64 * (b % kHalves) of row b / kHalves in every step - no index arithmetic per vector, the row and
+    // the piece's time travel in scalar offsets.  (Whole rows, 75 vectors at T = 300, would need twice the memory
+    // instructions that way, half of them nearly empty.)
+    constexpr bool STATIC = VEC && LAG == 32;
+    constexpr int kHalves = kPiece / 256;
+    static_assert(!STATIC || (NB == R * kHalves && NBR == NB + R / 8), "static mapping of vectors to lanes");
     extern __shared__ __align__(16) float lds[];
     float *tile = lds;                                                    // [R][P], P = 4 (mod 32)
     uint32_t *masks = reinterpret_cast<uint32_t *>(lds + R * P);  // [R][MP]
@@ -253,6 +260,19 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         }
         const int n = min(Tc, T - tL);
         const int perRow = n / V;
+        if constexpr (STATIC) {
+            const int nR = rows_of(t);
+            int mine[kHalves];
+#pragma unroll
+            for (int hf = 0; hf < kHalves; ++hf) mine[hf] = masked_offset(lane + hf * kWave < perRow, (lane + hf * kWave) * 16);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const int row = b / kHalves, hf = b % kHalves;
+                const float4 q = buffer_load4(bufU, row < nR ? mine[hf] : kOutOfRange, (row * T + tL) * 4);
+                x[4 * b] = q.x; x[4 * b + 1] = q.y; x[4 * b + 2] = q.z; x[4 * b + 3] = q.w;
+            }
+            return;
+        }
         const int total = rows_of(t) * perRow;
         RowCol rc;
         rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
@@ -291,6 +311,22 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         }
         const int n = min(Tc, T - tL);
         const int perRow = n / V;
+        if constexpr (STATIC) {
+            const int nR = rows_of(t);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const int row = b / kHalves, c = lane + (b % kHalves) * kWave;
+                if (row < nR && c < perRow) {
+                    *reinterpret_cast<float4 *>(tile + row * P + LAG + c * 4) = make_float4(x[4 * b], x[4 * b + 1], x[4 * b + 2], x[4 * b + 3]);
+                    if (monotone) {  // (LAG and the column are multiples of 4: the four bits lie in one word; adding no bits is harmless)
+                        const uint32_t bits = (x[4 * b] >= theta ? 1u : 0u) | (x[4 * b + 1] >= theta ? 2u : 0u) |
+                                              (x[4 * b + 2] >= theta ? 4u : 0u) | (x[4 * b + 3] >= theta ? 8u : 0u);
+                        atomicOr(cand + row * MP + ((LAG + c * 4) >> 5), bits << ((c * 4) & 31));
+                    }
+                }
+            }
+            return;
+        }
         const int total = rows_of(t) * perRow;
         RowCol rc;
         rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
@@ -374,8 +410,11 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                 mine += __shfl_xor(mine, off, kWave);
                 nzw |= __shfl_xor(nzw, off, kWave);
             }
-            // going from candidate to candidate pays while no row of the tile has more than a candidate per 24 samples
-            hop = __builtin_amdgcn_ballot_w64(mine * 24 > W) == 0;
+            // going from candidate to candidate pays while no row of the tile has more than a candidate per 12 samples:
+            // the wavefront stays as long as its busiest row (1 in 24: 102 us, 1 in 12: 92 us, 1 in 4: 91 us on
+            // (64,256,1,1,2000) with 2.3 % candidates, where a few rows per launch exceed 1 in 24; tensors whose
+            // busiest rows are above the threshold most of the time take the window walk at any of these settings)
+            hop = __builtin_amdgcn_ballot_w64(mine * 12 > W) == 0;
         }
         if (hop) {
             const int words = (W + 31) >> 5;
@@ -520,6 +559,34 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
             RowCol rc;
             rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
             const int dr = kWave / perRow, dc = kWave % perRow;
+            // vector b of this lane in the retire step: row, first column, and whether it exists
+            auto where = [&](int b, int &r, int &col) -> bool {
+                bool on;
+                if constexpr (STATIC) {
+                    // as in issue() and commit(); the vectors past 64 * kHalves per row (the LAG columns that a
+                    // row's last piece retires as well) follow, eight per row and lane group
+                    int c;
+                    if (b < NB) {
+                        r = b / kHalves;
+                        c = lane + (b % kHalves) * kWave;
+                    } else {
+                        r = (b - NB) * 8 + (lane >> 3);
+                        c = kHalves * kWave + (lane & 7);
+                    }
+                    on = r < nRows && c < perRow;
+                    col = first + c * 4;
+                } else {
+                    on = lane + b * kWave < total;
+                    r = rc.r;
+                    col = first + rc.c * V;
+                    rc.advance(dr, dc, perRow);
+                }
+                if (!on) {
+                    r = 0;
+                    col = first;
+                }
+                return on;
+            };
             if constexpr (VEC) {
               if (!dl.on) {
                 // a fixed number of (masked) stores, see above.  Half of a step's vectors at a time: their LDS reads
@@ -533,13 +600,12 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 #pragma unroll
                     for (int i = 0; i < HB; ++i) {
                         if (b0 + i < NBR) {
-                            const bool on = lane + (b0 + i) * kWave < total;
-                            const int r = on ? rc.r : 0, col = on ? first + rc.c * V : first;
+                            int r, col;
+                            const bool on = where(b0 + i, r, col);
                             uu[i] = *reinterpret_cast<const float4 *>(tile + r * P + col);
                             word[i] = masks[r * MP + (col >> 5)];
                             sh[i] = col & 31;
                             offs[i] = masked_offset(on, (r * T + tW + col) * 4);
-                            rc.advance(dr, dc, perRow);
                         }
                     }
 #pragma unroll
@@ -556,8 +622,8 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
               } else {
 #pragma unroll
                 for (int b = 0; b < NBR; ++b) {
-                    const bool on = lane + b * kWave < total;
-                    const int r = on ? rc.r : 0, col = on ? first + rc.c * V : first;
+                    int r, col;
+                    const bool on = where(b, r, col);
                     const float *src = tile + r * P + col;
                     // rows in pieces with a shifted output: a shift towards later times only needs spikes that are
                     // final by now; the rows with a negative shift wait for their last piece
@@ -569,7 +635,6 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                     buffer_store4(bufS, shift < 0 ? kOutOfRange : off, 0,
                                   make_float4((m & 1u) ? amplitude : 0.0f, (m & 2u) ? amplitude : 0.0f,
                                               (m & 4u) ? amplitude : 0.0f, (m & 8u) ? amplitude : 0.0f));
-                    rc.advance(dr, dc, perRow);
                 }
               }
             } else {
