@@ -11,6 +11,7 @@
 // shapes); pooling has a streaming input gradient.  Work-groups that read the same rows are kept
 // on the same die (xcd_contiguous).
 #include <atomic>
+#include <type_traits>
 
 #include "common.h"
 
@@ -638,6 +639,271 @@ __global__ __launch_bounds__(256) void synapse_wgrad_mfma_kernel(WgradMfmaArgs g
     }
 }
 
+// ---- gather on the matrix cores --------------------------------------------------------------------------
+// For 16 output channels and 16 time samples of one pixel, dst[t][o] = sum_k X[k][t] * W[k][o] over the taps
+// k = (source channel, filter row, filter column) is a matrix product with the taps as the reduction axis:
+// v_mfma_f32_16x16x4_f32 takes four taps at a time, lane (r, h) supplying X[k0 + h][t0 + r] and W[k0 + h][o0 + r],
+// and leaves four consecutive time samples of channel o0 + r in its accumulator - one 16-byte store.  A
+// work-group of eight wavefronts takes kGmPix = 8 consecutive destination pixels of one row (one per wavefront)
+// and a step of 32 time samples at a time and copies the source patch under those pixels into LDS once - up to
+// 16 source channels ("a pass") x KH filter rows x WX columns, one whole 128-byte line each, out-of-image
+// positions as zeros - so the X operands are one LDS dword per matrix instruction at an address that is the
+// same in every step (a table of 36 registers per lane; the half of the step and the buffer are immediates).  The weights of all passes sit in LDS as
+// [pass][channel tile][lane][tap step], a lane's steps contiguous: one 16-byte read per four steps.  Two
+// patches are resident; the loads of the next (pixel block, step, pass) are in flight in registers while the
+// matrix instructions work, and are written to the other patch before the single barrier.  Source channels
+// beyond a pass are accumulated by running the passes of a (block, step) one after the other; the accumulators
+// leave after the last.  Work is cut into equal ranges of (block, step) pairs of the whole batch, one
+// work-group per compute unit (its LDS).
+constexpr int kGmPix = 8;
+constexpr int kGmRow = 128;                    // bytes per patch row: 32 samples
+constexpr int kGmMaxRows = 480;                // patch rows; row kGmMaxRows of a buffer holds zeros
+constexpr int kGmBuf = (kGmMaxRows + 1) * kGmRow;
+constexpr int kGmSteps = 36;                   // tap steps per pass: 144 taps (16 channels x 3 x 3)
+constexpr int kGmMaxWeightBytes = 4 * 64 * kGmSteps * 4;   // passes x channel tiles <= 4
+
+struct GatherMfmaArgs {
+    const float *src;
+    float *dst;
+    const float *w;
+    int SC, SH, SW, DC, DH, DW, T;
+    int Qg, Mg, groups, KH, KW, Cg, Og;
+    int mulH, mulW, offH, offW, stepH, stepW;
+    int chansPerPass, passes, WX, xBias, rows;   // patch: chansPerPass x KH x WX rows; xBias: patch column of tap 0 of pixel 0
+    int oGroups;                                 // blocks of 16 * OT destination channels per group
+    int blocksPerRow, steps, pairs, slices, pairsPerSlice;
+    FastDiv byOGroups, byGroups, byKK, byKW, bySteps, byBlocks, byBlocksPerRow, byPatch, byWX;
+};
+
+template <int OT, bool BACKWARD>
+__global__ __launch_bounds__(512) void synapse_gather_mfma_kernel(GatherMfmaArgs g)
+{
+    extern __shared__ __align__(16) float lds[];
+    char *const ldsBytes = reinterpret_cast<char *>(lds);
+    constexpr int KS = kGmSteps;
+    // (LDS addresses as plain 32-bit numbers: the tables below then hold final addresses, nothing is added per read)
+    typedef const float __attribute__((address_space(3))) *LdsFloat;
+    typedef const floatx4 __attribute__((address_space(3))) *LdsFloat4;
+    const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char *)ldsBytes));
+    uint32_t rest = xcd_contiguous(blockIdx.x, gridDim.x);
+    uint32_t qq = fastdiv(rest, g.byOGroups);
+    const int og = static_cast<int>(rest - qq * g.byOGroups.d);
+    rest = qq; qq = fastdiv(rest, g.byGroups);
+    const int grp = static_cast<int>(rest - qq * g.byGroups.d);
+    const int slice = static_cast<int>(qq);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, h = lane >> 4;
+    const int KK = g.KH * g.KW;
+    const int64_t srcPlane = static_cast<int64_t>(g.SH) * g.SW * g.T, dstPlane = static_cast<int64_t>(g.DH) * g.DW * g.T;
+    const int rowBytes = g.SW * g.T * 4, pixBytes = g.T * 4, planeBytes = static_cast<int>(srcPlane) * 4;
+    BufferRsrc srcB = make_buffer(g.src), dstB = make_buffer(g.dst);   // (of the batch item at hand: set by place())
+
+    // weights: wl[((pass * OT + ot) * 64 + lane) * KS + s] = W[tap 4 s + h of the pass][channel 16 (og OT + ot) + r]
+    float *const wl = lds + 2 * kGmBuf / 4;   // (behind the two patches and their zero rows)
+    for (int e = tid; e < g.passes * OT * 64 * KS; e += 512) {
+        const int s = e % KS, l = (e / KS) & 63, po = e / (KS * 64);
+        const int ot = po % OT, pass = po / OT;
+        const int k = 4 * s + (l >> 4), m = (og * OT + ot) * 16 + (l & 15);
+        const int cl = static_cast<int>(fastdiv(static_cast<uint32_t>(k), g.byKK)), ij = k - cl * KK, q = pass * g.chansPerPass + cl;
+        float v = 0.f;
+        if (cl < g.chansPerPass && q < g.Qg && m < g.Mg) {
+            const int64_t idx = BACKWARD ? (static_cast<int64_t>(grp * g.Og + q) * g.Cg + m) * KK + ij
+                                         : (static_cast<int64_t>(grp * g.Og + m) * g.Cg + q) * KK + ij;
+            v = g.w[idx];
+        }
+        wl[e] = v;
+    }
+    if (tid < 2 * (kGmRow / 4)) lds[kGmMaxRows * 2 * kGmRow / 4 + tid] = 0.f;   // the zero rows of both patches
+
+    // X operand of tap step s: LDS address of this lane's sample in the first half of the step's 32 samples (the
+    // second half lies 64 bytes on, the other patch kGmBuf bytes on: immediates).  Patch rows are not swizzled
+    // here: a read takes 64 contiguous bytes of each of 4 rows, at worst two of them in the same banks.  The rows
+    // of the two patches alternate (row r of patch b at (2 r + b) * 128 bytes), so that the patch, too, is an
+    // immediate within reach of a two-address LDS read.
+    int aTab[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        const int k = 4 * s + h;
+        const uint32_t cl = fastdiv(static_cast<uint32_t>(k), g.byKK);
+        const int ij = k - static_cast<int>(cl * g.byKK.d);
+        const int i = static_cast<int>(fastdiv(static_cast<uint32_t>(ij), g.byKW));
+        const int j = ij - i * g.KW;
+        const int row = static_cast<int>(cl) < g.chansPerPass
+            ? (static_cast<int>(cl) * g.KH + i) * g.WX + wave * g.mulW + j * g.stepW + g.xBias : kGmMaxRows;
+        aTab[s] = static_cast<int>(ldsBase) + row * 2 * kGmRow + (r << 2);
+    }
+    const uint32_t wAddr = ldsBase + 2 * kGmBuf + lane * KS * 4;
+
+    // destination rows of this lane: channel 16 (og OT + ot) + r, samples 4 h .. 4 h + 3 of a half step
+    int oOff[OT];
+#pragma unroll
+    for (int ot = 0; ot < OT; ++ot) {
+        const int m = (og * OT + ot) * 16 + r;
+        oOff[ot] = masked_offset(m < g.Mg, m * static_cast<int>(dstPlane) * 4 + h * 16);
+    }
+
+    // This lane copies unit u (samples 4u..4u+3 of the step) of patch rows tid / 8 + 64 m
+    constexpr int NS = 8;
+    const int u = tid & 7;
+    const int stageAddr = (tid >> 3) * 2 * kGmRow + (u << 4);
+
+    const int p0 = slice * g.pairsPerSlice, p1 = min(g.pairs, p0 + g.pairsPerSlice);
+    int sOff[NS];
+    int pixNext = 0;          // byte offset of this wavefront's destination pixel in a channel plane, or -1
+    auto place = [&](int blockOfAll) {
+        const int n = static_cast<int>(fastdiv(static_cast<uint32_t>(blockOfAll), g.byBlocks));
+        const int block = blockOfAll - n * static_cast<int>(g.byBlocks.d);
+        srcB = make_buffer(g.src + (static_cast<int64_t>(n) * g.SC + static_cast<int64_t>(grp) * g.Qg) * srcPlane);
+        const int a = static_cast<int>(fastdiv(static_cast<uint32_t>(block), g.byBlocksPerRow));
+        const int b0 = (block - a * g.blocksPerRow) * kGmPix;
+        const int nv = min(kGmPix, g.DW - b0);
+        const int xLimit = (nv - 1) * g.mulW + (g.KW - 1) * (g.stepW < 0 ? -g.stepW : g.stepW) + 1;
+        const int y0 = a * g.mulH + g.offH, x0 = b0 * g.mulW + g.offW - g.xBias;
+#pragma unroll
+        for (int m = 0; m < NS; ++m) {
+            const int row = (tid >> 3) + 64 * m;
+            const uint32_t cl = fastdiv(static_cast<uint32_t>(row), g.byPatch);
+            const int rem = row - static_cast<int>(cl * g.byPatch.d);
+            const int i = static_cast<int>(fastdiv(static_cast<uint32_t>(rem), g.byWX));
+            const int x = rem - i * g.WX;
+            const int y = y0 + i * g.stepH, xx = x0 + x;
+            const bool ok = row < g.rows && x < xLimit && static_cast<unsigned>(y) < static_cast<unsigned>(g.SH) &&
+                            static_cast<unsigned>(xx) < static_cast<unsigned>(g.SW);
+            sOff[m] = masked_offset(ok, static_cast<int>(cl) * planeBytes + y * rowBytes + xx * pixBytes + u * 16);
+        }
+        const int b = b0 + wave;
+        pixNext = b < g.DW ? (a * g.DW + b) * pixBytes : -1;
+        return n;
+    };
+    auto issue = [&](float4 (&R)[NS], int st, int pass, bool more) {
+        const int uniform = (st << 7) + pass * g.chansPerPass * planeBytes;
+        const bool live = more && (st << 5) + (u << 2) < g.T;
+#pragma unroll
+        for (int m = 0; m < NS; ++m) R[m] = buffer_load4<0>(srcB, live ? sOff[m] : kOutOfRange, uniform);
+    };
+    auto stage = [&](const float4 (&R)[NS], int buf) {
+#pragma unroll
+        for (int m = 0; m < NS; ++m)
+            if ((tid >> 3) + 64 * m < kGmMaxRows) *reinterpret_cast<float4 *>(ldsBytes + buf + stageAddr + m * 64 * 2 * kGmRow) = R[m];
+    };
+
+    floatx4 acc[2][OT];
+    auto clear = [&]() {
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int ot = 0; ot < OT; ++ot) acc[hf][ot] = floatx4{0.f, 0.f, 0.f, 0.f};
+    };
+    // the matrix work of one pass on the patch in buffer BUF (an immediate in every LDS read); HALVES = 1 when the
+    // second half of the step lies past the end of the row.  Straight-line code: the LDS reads run ahead of the
+    // matrix instructions that use them.
+    auto multiply = [&](auto bufTag, auto halvesTag, int pass) {
+        constexpr int BUF = decltype(bufTag)::value, HALVES = decltype(halvesTag)::value;
+        const uint32_t wp = wAddr + pass * OT * 64 * KS * 4;
+        // operands of four tap steps at a time, fetched one group ahead of the matrix instructions that use them
+        floatx4 bq[2][OT];
+        float av[2][HALVES][4];
+        auto fetch = [&](int set, int s4) {
+#pragma unroll
+            for (int ot = 0; ot < OT; ++ot)
+                bq[set][ot] = *reinterpret_cast<LdsFloat4>(static_cast<size_t>(wp + (ot * 64 * KS + s4) * 4));
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int hf = 0; hf < HALVES; ++hf)
+                    av[set][hf][e] = *reinterpret_cast<LdsFloat>(static_cast<size_t>(static_cast<uint32_t>(aTab[s4 + e]) + BUF * kGmRow + hf * 64));
+        };
+        fetch(0, 0);
+#pragma unroll
+        for (int s4 = 0; s4 < KS; s4 += 4) {
+            const int set = (s4 >> 2) & 1;
+            if (s4 + 4 < KS) fetch(set ^ 1, s4 + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int hf = 0; hf < HALVES; ++hf)
+#pragma unroll
+                    for (int ot = 0; ot < OT; ++ot)
+                        acc[hf][ot] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[set][hf][e], bq[set][ot][e], acc[hf][ot], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // the accumulators of a (block, step) leave: four consecutive samples of one channel per lane and tile.  A store
+    // instruction writes 64 bytes of each of 16 channel rows, and a pixel's row is 4 T bytes long: cached stores, so
+    // that L2 puts the pieces of a line together (streaming stores of these pieces: 137 us instead of 114 us on
+    // the 16 -> 32 channel layer)
+    auto store = [&](int pix, int st) {
+        if (pix < 0) return;
+        const int uniform = pix + (st << 7);
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            const bool live = (st << 5) + hf * 16 + (h << 2) < g.T;
+#pragma unroll
+            for (int ot = 0; ot < OT; ++ot)
+                buffer_store4<0>(dstB, live ? oOff[ot] : kOutOfRange, uniform + hf * 64,
+                                       make_float4(acc[hf][ot][0], acc[hf][ot][1], acc[hf][ot][2], acc[hf][ot][3]));
+        }
+    };
+
+    {
+        // Trip k of the loop loads (pair, pass) number k of the range into registers, multiplies number k - 1 from
+        // its LDS buffer ((k - 1) % 2) and then writes the registers to the other buffer: the loop's code exists
+        // once, its first trip only loads.
+        int block = static_cast<int>(fastdiv(static_cast<uint32_t>(p0), g.bySteps));
+        int st = p0 - block * g.steps, pass = 0;          // what is loaded next
+        int stCur = 0, passCur = 0, pixCur = -1, nCur = -1, nNext = -1;   // what is multiplied next
+        float4 R[NS];
+        int buf = 1;
+        bool first = true;
+        const int trips = (p1 - p0) * g.passes;
+        clear();
+#pragma nounroll
+        for (int k = 0;; ++k) {
+            const bool more = k < trips;
+            bool moved = first;
+            if (more && !first) {
+                if (++pass == g.passes) {
+                    pass = 0;
+                    if (++st == g.steps) {
+                        st = 0;
+                        ++block;
+                        moved = true;
+                    }
+                }
+            }
+            if (more && moved) nNext = place(block);
+            issue(R, st, pass, more);
+            __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the matrix work
+            if (!first) {
+                using I0 = std::integral_constant<int, 0>;
+                using I1 = std::integral_constant<int, 1>;
+                using I2 = std::integral_constant<int, 2>;
+                if ((stCur << 5) + 16 < g.T) {
+                    if (buf == 0) multiply(I0{}, I2{}, passCur);
+                    else multiply(I1{}, I2{}, passCur);
+                } else {
+                    if (buf == 0) multiply(I0{}, I1{}, passCur);
+                    else multiply(I1{}, I1{}, passCur);
+                }
+                if (passCur == g.passes - 1) {
+                    if (nCur >= 0) {
+                        dstB = make_buffer(g.dst + (static_cast<int64_t>(nCur) * g.DC + static_cast<int64_t>(grp) * g.Mg) * dstPlane);
+                        store(pixCur, stCur);
+                    }
+                    clear();
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (!more) break;
+            buf ^= 1;
+            stage(R, buf * kGmRow);
+            stCur = st; passCur = pass; pixCur = pixNext; nCur = nNext;
+            __syncthreads();
+            first = false;
+        }
+    }
+}
+
 // ---- weight gradient on the matrix cores, input patch of a block of pixels in LDS -------------------
 // The kernel above fetches every input row once per tap that uses it (the working set of four
 // wavefronts does not stay in the 32 KB L1), 64 bytes at a time: it is bound by the number of cache
@@ -957,6 +1223,76 @@ static void launch_gather_mb(const GatherArgs &g, bool strided, unsigned blocks,
         hipLaunchKernelGGL((synapse_gather_kernel<MB, VEC, BACKWARD, false>), dim3(blocks), dim3(256), 0, st, g);
 }
 
+// The matrix-core gather: unit stride in the gradient (forward: any stride), rows of whole vectors, passes of
+// whole source channels that fill most of the 36 tap steps, at least 16 destination channels, patch and weights
+// within LDS.  Returns SLAYER_EUNSUPPORTED (nothing launched) when the geometry does not qualify.
+template <bool BACKWARD>
+static int launch_gather_mfma(const GatherArgs &a, const SynGeom &s, bool strided, hipStream_t st)
+{
+    if (strided || a.Mg < 16) return SLAYER_EUNSUPPORTED;
+    const int KK = a.KH * a.KW;
+    if (KK > 4 * kGmSteps) return SLAYER_EUNSUPPORTED;
+    int chans = 4 * kGmSteps / KK;
+    if (chans > a.Qg) chans = a.Qg;
+    if (chans < 1 || a.Qg % chans != 0 || chans * KK < 96) return SLAYER_EUNSUPPORTED;
+    const int passes = a.Qg / chans;
+    const int OT = (a.Mg >= 32 && passes * 2 <= 4) ? 2 : 1;
+    if (passes * OT > 4) return SLAYER_EUNSUPPORTED;
+    const int absStepW = a.stepW < 0 ? -a.stepW : a.stepW;
+    const int64_t WX = static_cast<int64_t>(kGmPix - 1) * a.mulW + static_cast<int64_t>(a.KW - 1) * absStepW + 1;
+    const int64_t rows = static_cast<int64_t>(chans) * a.KH * WX;
+    if (rows > kGmMaxRows) return SLAYER_EUNSUPPORTED;
+    GatherMfmaArgs g{};
+    g.src = a.src; g.dst = a.dst; g.w = a.w;
+    g.SC = a.SC; g.SH = a.SH; g.SW = a.SW; g.DC = a.DC; g.DH = a.DH; g.DW = a.DW; g.T = a.T;
+    g.Qg = a.Qg; g.Mg = a.Mg; g.groups = a.groups; g.KH = a.KH; g.KW = a.KW; g.Cg = a.Cg; g.Og = a.Og;
+    g.mulH = a.mulH; g.mulW = a.mulW; g.offH = a.offH; g.offW = a.offW; g.stepH = a.stepH; g.stepW = a.stepW;
+    g.chansPerPass = chans; g.passes = passes; g.WX = static_cast<int>(WX);
+    g.xBias = a.stepW < 0 ? (a.KW - 1) * absStepW : 0;
+    g.rows = static_cast<int>(rows);
+    g.oGroups = static_cast<int>(ceil_div(a.Mg, 16 * OT));
+    g.blocksPerRow = static_cast<int>(ceil_div(a.DW, kGmPix));
+    g.steps = (a.T + 31) / 32;
+    const int64_t pairs = static_cast<int64_t>(s.N) * a.DH * g.blocksPerRow * g.steps;
+    if (pairs < 1 || pairs >= (1LL << 30)) return SLAYER_EUNSUPPORTED;
+    g.pairs = static_cast<int>(pairs);
+    // one work-group per compute unit (its LDS); a few short of the 256 places
+    const int64_t base = static_cast<int64_t>(a.groups) * g.oGroups;
+    int64_t slices = 252 / base;
+    if (slices < 1) slices = 1;
+    if (slices > pairs) slices = pairs;
+    g.pairsPerSlice = static_cast<int>(ceil_div(pairs, slices));
+    g.slices = static_cast<int>(ceil_div(pairs, g.pairsPerSlice));
+    g.byOGroups = make_fastdiv(static_cast<uint32_t>(g.oGroups));
+    g.byGroups = make_fastdiv(static_cast<uint32_t>(a.groups));
+    g.byKK = make_fastdiv(static_cast<uint32_t>(KK));
+    g.byKW = make_fastdiv(static_cast<uint32_t>(a.KW));
+    g.bySteps = make_fastdiv(static_cast<uint32_t>(g.steps));
+    g.byBlocks = make_fastdiv(static_cast<uint32_t>(a.DH * g.blocksPerRow));
+    g.byBlocksPerRow = make_fastdiv(static_cast<uint32_t>(g.blocksPerRow));
+    g.byPatch = make_fastdiv(static_cast<uint32_t>(a.KH * g.WX));
+    g.byWX = make_fastdiv(static_cast<uint32_t>(g.WX));
+    const int64_t blocks = base * g.slices;
+    if (blocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+    const int ldsBytes = 2 * kGmBuf + passes * OT * 64 * kGmSteps * 4;
+    // more LDS than a kernel may use without asking; asked once per device (a host-side setting, no allocation)
+    static std::atomic<bool> raised[2][64];
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err == hipSuccess && (device < 0 || device >= 64)) err = hipErrorInvalidDevice;
+    if (err == hipSuccess && !raised[OT - 1][device].load(std::memory_order_acquire)) {
+        const void *fn = OT == 2 ? reinterpret_cast<const void *>(&synapse_gather_mfma_kernel<2, BACKWARD>)
+                                 : reinterpret_cast<const void *>(&synapse_gather_mfma_kernel<1, BACKWARD>);
+        err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kGmBuf + kGmMaxWeightBytes);
+        if (err == hipSuccess) raised[OT - 1][device].store(true, std::memory_order_release);
+    }
+    if (err != hipSuccess) return note_hip_error(err);
+    const dim3 grid(static_cast<unsigned>(blocks));
+    if (OT == 2) hipLaunchKernelGGL((synapse_gather_mfma_kernel<2, BACKWARD>), grid, dim3(512), ldsBytes, st, g);
+    else hipLaunchKernelGGL((synapse_gather_mfma_kernel<1, BACKWARD>), grid, dim3(512), ldsBytes, st, g);
+    return launch_status();
+}
+
 template <bool BACKWARD>
 static int launch_gather(float *dst, const float *src, const float *w, const SynGeom &s, hipStream_t st)
 {
@@ -1001,6 +1337,10 @@ static int launch_gather(float *dst, const float *src, const float *w, const Syn
     }
     // destination channels per lane: as many as the group has, up to 16
     const int MB = g.Mg >= 12 ? 16 : g.Mg >= 6 ? 8 : g.Mg >= 3 ? 4 : g.Mg == 2 ? 2 : 1;
+    if (vec && !generic_forced()) {
+        const int status = launch_gather_mfma<BACKWARD>(g, s, strided, st);
+        if (status != SLAYER_EUNSUPPORTED) return status;
+    }
     // one or two of them, and a filter wide enough for neighbouring pixels to share source columns: PX pixels per lane
     if (MB <= 2 && vec && !strided && g.mulW == 1 && g.stepW == (BACKWARD ? -1 : 1) && (g.KW == 3 || g.KW == 5 || g.KW == 7) &&
         static_cast<int64_t>(g.Qg) * g.KH * g.KW >= 32 && !generic_forced()) {
