@@ -6,10 +6,14 @@
 // With time innermost the filter does not depend on the fastest axis, so every lane owns a run of
 // consecutive time samples (one 16-byte vector) of one pixel: loads and stores are contiguous along
 // T for any stride, padding or dilation, and the weights are wave-uniform.  Forward and input
-// gradient are one gather kernel on the vector ALUs; the weight gradient, a matrix product with time
-// as the reduction axis, runs on the matrix cores (with a vector kernel for small or unaligned
-// shapes); pooling has a streaming input gradient.  Work-groups that read the same rows are kept
-// on the same die (xcd_contiguous).
+// gradient are one gather: on the matrix cores for layers with at least 16 destination channels
+// and source channels that fill passes of about 144 taps (a source patch in LDS, the taps as the
+// reduction axis), on the vector ALUs otherwise (a general kernel, and one that keeps the columns
+// of a filter row in registers for layers with one or two destination channels).  The weight
+// gradient, a matrix product with time as the reduction axis, runs on the matrix cores from a
+// source patch in LDS (from global memory for patches that do not fit, and a vector kernel for
+// small or unaligned shapes); pooling has a streaming input gradient.  Work-groups that read the
+// same rows are kept on the same die (xcd_contiguous).
 #include <atomic>
 #include <type_traits>
 

@@ -67,6 +67,14 @@ CASES = [
     (2, 1, 9, 11, 16, 8, (3, 5), 1, (1, 2), 1, 1),    # input gradient with 1 channel, 3 x 5 filter
     (1, 2, 10, 10, 8, 8, (3, 3), 1, (2, 1), (2, 1), 1),   # dilation along H only
     (1, 2, 6, 40, 4, 12, (1, 7), 1, (0, 3), 1, 1),    # 1 x 7 filter: 84 taps, 10 columns per lane
+    # forward / input gradient on the matrix cores (at least 16 destination channels, passes of about 144 taps)
+    (2, 32, 6, 9, 36, 64, (3, 3), 1, 1, 1, 1),        # two passes x two channel tiles; gradient: four passes
+    (2, 32, 7, 10, 36, 32, (3, 3), 1, 1, 1, 2),       # two groups of 16 -> 16 channels, ranges crossing batch items
+    (1, 4, 9, 9, 20, 16, (5, 5), 1, 2, 1, 1),         # 5 x 5: passes of 4 channels x 25 taps
+    (1, 48, 5, 9, 32, 16, (3, 3), 1, 1, 1, 1),        # three passes; gradient: 48 channels = one and a half tile pairs
+    (1, 12, 6, 8, 32, 16, (3, 4), 1, 1, 1, 1),        # 12 channels x 12 taps
+    (1, 16, 8, 10, 64, 16, (3, 3), 1, (2, 1), (2, 1), 1),  # dilation along H
+    (1, 16, 5, 8, 32, 20, (3, 3), 1, 1, 1, 1),        # 20 = 16 + 4 destination channels
 ]
 IDS = ["%dx%dx%dx%dx%d-o%d-k%s-s%s-p%s-d%s-g%d" % c for c in CASES]
 
