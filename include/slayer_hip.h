@@ -166,10 +166,13 @@ int slayer_spike_bwd_corr_f32(float *gradIn, const float *gradOut, const float *
  *
  * u = Ts * conv(a, srm), then s and the refractory update of u as in slayer_get_spikes_f32, without
  * the round trip of u through memory when rows are whole 16-byte vectors of at most 352 samples,
- * nuSize <= 24 and F <= 160: the filter then runs as the sequential fused-multiply-add loop for every
- * input (the reference's bits; slayer_conv_f32 on its own may sum a dense input on the matrix cores and
- * differ in the last bit).  Other shapes run the two kernels one after the other.  u and s must not
- * alias a.
+ * nuSize <= 24 and F <= 160.  Filters of 34 to 129 taps (on rows of at least 16 samples) are summed on the
+ * matrix cores, which add the terms in another order than the sequential fused-multiply-add loop: the
+ * potentials agree with the reference's to rounding (1e-5 of the sum of each output's terms' magnitudes), the
+ * spikes are the spike function of exactly these potentials, and a tile of 16 rows that holds a non-finite
+ * sample is filtered with the sequential loop (the reference's bits, infinities and NaNs where it puts them).
+ * All other filters run the sequential loop for every input (the reference's bits).  Other shapes run the
+ * two kernels one after the other.  u and s must not alias a.
  */
 int slayer_psp_spike_f32(float *s, float *u, const float *a, const float *srm, const float *nu,
                          int64_t nNeurons, int64_t T, int64_t F, int64_t nuSize, float theta,

@@ -15,7 +15,7 @@
 //    Y[m] = sum_i X[m+i] * filt[i].  A work-group of 256 lanes owns R consecutive neuron rows
 //    and one time tile; it stages the rows' samples (plus the F-1 sample halo, zero padded) into
 //    LDS as X[R][LD] with 16-byte loads (reversed in time for the convolution) and counts the non-zero
-//    vectors on the way.  Then one of three paths per tile:
+//    samples on the way.  Then one of three paths per tile:
 //      - almost all zeros (spike trains): event-driven, one update per non-zero sample, the bits of the
 //        chain with its zero terms left out;
 //      - dense, 34 to 129 taps, whole-vector rows (template DM > 0): the tile's outputs as products of
@@ -146,12 +146,16 @@ __global__ __launch_bounds__(256) void fir_direct_kernel(float *__restrict__ out
 
 // ---- tiled kernel ---------------------------------------------------------------------------------
 // (the register-window core, window_of .. TailBlocks, is in fir_core.h)
-// true when any of the four samples is not (plus or minus) zero
-__device__ __forceinline__ bool any_nonzero(const float4 &v)
+// Non-zero samples ("events", low 16 bits) and non-zero vectors (high 16 bits) among the wavefront's vectors;
+// non-zero is anything but +0 and -0, by class (denormals and NaNs count).  A tile stages at most 12288 samples,
+// so sums of these over a tile stay within their 16 bits.
+__device__ __forceinline__ uint32_t count_nonzero(const float4 &v)
 {
-    const uint32_t bits = __builtin_bit_cast(uint32_t, v.x) | __builtin_bit_cast(uint32_t, v.y) |
-                          __builtin_bit_cast(uint32_t, v.z) | __builtin_bit_cast(uint32_t, v.w);
-    return (bits << 1) != 0;
+    constexpr int kNotZero = 0x3ff & ~0x60;  // every class but the two zeros
+    const uint64_t mx = __ballot(__builtin_amdgcn_classf(v.x, kNotZero)), my = __ballot(__builtin_amdgcn_classf(v.y, kNotZero));
+    const uint64_t mz = __ballot(__builtin_amdgcn_classf(v.z, kNotZero)), mw = __ballot(__builtin_amdgcn_classf(v.w, kNotZero));
+    const uint32_t events = __builtin_popcountll(mx) + __builtin_popcountll(my) + __builtin_popcountll(mz) + __builtin_popcountll(mw);
+    return events + (static_cast<uint32_t>(__builtin_popcountll(mx | my | mz | mw)) << 16);
 }
 
 // ---- event-driven path for sparse input (spike trains) -------------------------------------------
@@ -234,7 +238,7 @@ __global__ __launch_bounds__(256, DM > 0 ? 2 : 1) void fir_tiled_kernel(float *_
     extern __shared__ __align__(16) float X[];
     // filter copy for the sparse path: taps -63 .. 191, zeros outside [0, F)
     float *fL = X + R * LD + (kWave - 1);
-    uint32_t *nzCount = reinterpret_cast<uint32_t *>(X + R * LD + 4 * kWave);  // non-zero input vectors, per wavefront
+    uint32_t *nzCount = reinterpret_cast<uint32_t *>(X + R * LD + 4 * kWave);  // non-zero input samples and vectors, per wavefront
     uint32_t nonZero = 0;                                          // wave-uniform
 
     const int tid = threadIdx.x;
@@ -277,7 +281,7 @@ __global__ __launch_bounds__(256, DM > 0 ? 2 : 1) void fir_tiled_kernel(float *_
                     const float4 g = buffer_load4(bufGate, src, 0);
                     v = make_float4(gated(v.x, g.x), gated(v.y, g.y), gated(v.z, g.z), gated(v.w, g.w));
                 }
-                nonZero += __builtin_popcountll(__ballot(any_nonzero(v)));
+                nonZero += count_nonzero(v);
                 // (convolution: descending time, the vector lands mirrored)
                 *reinterpret_cast<float4 *>(reinterpret_cast<char *>(X) + dst) = CAUSAL ? make_float4(v.w, v.z, v.y, v.x) : v;
                 col += dc;
@@ -324,7 +328,7 @@ __global__ __launch_bounds__(256, DM > 0 ? 2 : 1) void fir_tiled_kernel(float *_
                 if (tl + 3 < T) v.w = at(tl + 3);
             }
             *reinterpret_cast<float4 *>(X + r * LD + j) = v;
-            nonZero += __builtin_popcountll(__ballot(any_nonzero(v)));
+            nonZero += count_nonzero(v);
         }
     }
     {
@@ -337,9 +341,15 @@ __global__ __launch_bounds__(256, DM > 0 ? 2 : 1) void fir_tiled_kernel(float *_
     // ---- sparse input: event-driven path
     {
         const uint32_t nz = nzCount[0] + nzCount[1] + nzCount[2] + nzCount[3];
-        const uint32_t vectors = static_cast<uint32_t>(nRows) * static_cast<uint32_t>(LD >> 2);
-        // (dense tiles cost less on the matrix cores, so the event-driven path pays up to a lower density there)
-        if (F <= kSparseMaxTaps && LD <= kSparseBlocks * kWave && nz * (DM > 0 ? 5u : 8u) <= vectors) {
+        const uint32_t events = nz & 0xffffu, vectors = nz >> 16;
+        const uint32_t samples = static_cast<uint32_t>(nRows) * static_cast<uint32_t>(LD);
+        // The event-driven path pays per event: up to one event per 20 staged samples next to the matrix cores, one
+        // per 32 next to the chains.  Spike trains that come in bursts (pooled ones: more than 3 events per 2
+        // non-zero vectors) put most of a tile's events into a few rows, and the tile lasts as long as the wavefront
+        // with the busiest rows: half that density for them.
+        constexpr uint32_t kPer = DM > 0 ? 20u : 32u;
+        const uint32_t per = 2u * events > 3u * vectors ? 2u * kPer : kPer;
+        if (F <= kSparseMaxTaps && LD <= kSparseBlocks * kWave && events * per <= samples) {
             fir_sparse_tile<CAUSAL>(bufOut, X, fL, nRows, LD, ttp, t0, tt, tHi, T, F, Ts);
             return;
         }

@@ -4,9 +4,10 @@
 //   u[n][t] = Ts * sum_{i<F} a[n][t-i] * srm[i]        (the causal convolution of fir.hip)
 //   then the sequential threshold / refractory loop of spike.hip on u, in place.
 //
-// Same values, bit for bit, as slayer_conv_f32 followed by slayer_get_spikes_f32, without the
-// round trip of u through memory: 12 bytes per neuron-timestep (read a, write u', write s)
-// instead of 20.  A 64-lane work-group owns 8 whole rows.  It stages them into LDS reversed in
+// Without the round trip of u through memory: 12 bytes per neuron-timestep (read a, write u', write s)
+// instead of 20.  Two kernels: filters of 34 to 129 taps on the matrix cores (further down; potentials
+// to rounding), all others with the register-window chain - the same values, bit for bit, as
+// slayer_conv_f32's chain kernels followed by slayer_get_spikes_f32.  There a 64-lane work-group owns 8 whole rows.  It stages them into LDS reversed in
 // time and zero padded (X[r][j] = a[r][tHi - j]), runs the register-window FIR core over
 // (row, 8-output chunk) items - every lane keeps the results of its items in registers until
 // all lanes have finished reading X - then lays the membrane potential out in the same LDS as
@@ -195,6 +196,383 @@ __global__ __launch_bounds__(64) void psp_spike_kernel(float *__restrict__ s, fl
     }
 }
 
+
+// ---- the same on the matrix cores, for filters of 34 to 129 taps ---------------------------------------------------
+// Above about 33 taps the register-window chain is bound by FMA issue.  Here a wavefront owns 16 whole rows and
+// filters them as products of a banded Toeplitz matrix of the filter with blocks of 16 samples
+// (v_mfma_f32_16x16x4_f32; the formulation of fir_mfma.hip on the reversed time axis, where the convolution is
+// a correlation): with m = 16 nBlk - 1 - t, output block j (in m) is the product of the filter band with the D
+// input blocks j .. j + D - 1, i.e. with time blocks q = nBlk - 1 - j down to q - D + 1.  Lane (c = lane % 16,
+// h = lane / 16) supplies, for instruction v of a block, component 3 - v of vector 3 - h of row c's time block
+// and filt[16d + 4h + v - i] for i = lane % 16; its accumulator holds the four outputs of that same vector
+// in descending time.  So a lane only ever reads and writes its own vectors of LDS: the walk goes down in time,
+// writes every output block over the input block that has just left the window, and leaves the membrane
+// potential where the spike walk wants it, tile[r][LAG + t].  The candidate bits of the spike walk are set as
+// the outputs are written; the walk (all 64 lanes, four per row) and the stores are those of spike.hip's
+// row tiles.  The matrix instruction sums four products per step in its own order: the potentials agree with
+// the sequential chain to rounding, and the spikes are the spike function of exactly these potentials.  A tile
+// with a non-finite sample is filtered as sequential chains instead (a structural zero of the band times an
+// infinity would put NaNs where the reference has none).
+constexpr int kFusedMfmaRows = 16;
+
+template <int D, int NU>
+__global__ __launch_bounds__(64, 2) void psp_spike_mfma_kernel(float *__restrict__ s, float *__restrict__ u,
+                                                            const float *__restrict__ a, const float *__restrict__ srm,
+                                                            const float *__restrict__ nu, int64_t rows, int T, int F,
+                                                            int nuSize, int P, int MP, float theta, float Ts)
+{
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    constexpr int R = kFusedMfmaRows, G = 32, W = D + 1;
+    constexpr int LAG = (NU + 2) & ~3;
+    constexpr int NBV = (R * (kFusedMaxT / 4) + kWave - 1) / kWave;  // vectors per lane of a tile, at most
+    constexpr int kParts = kWave / R, kRounds = (NU + kParts - 1) / kParts;
+    extern __shared__ __align__(16) float lds[];
+    float *tile = lds;                                               // [R][P]
+    uint32_t *masks = reinterpret_cast<uint32_t *>(lds + R * P);     // [R][MP] spike bits, bit = tile column
+    uint32_t *cand = masks + R * MP;                                 // [R][MP] samples at or above the threshold
+    float *zeros = reinterpret_cast<float *>(cand + R * MP);         // 64 bytes
+    // the refractory kernel with 3 entries in front and room behind, -0.0f (whose addition changes nothing) outside
+    float *tapL = zeros + 16 + 3;                                    // [-3, 29)
+
+    const int lane = threadIdx.x;
+    const int c = lane & 15, h = lane >> 4;
+    const int perRow = T >> 2;
+    const float amplitude = 1.0f / Ts;
+    const float quiet = __builtin_nanf("");
+    const int64_t tiles = (rows + R - 1) / R;
+
+    // A tile is one contiguous run of vectors (rows behind the last one arrive as zeros).  A wavefront walks over
+    // tiles; the next tile's samples are on their way into registers while this one is filtered, walked and stored.
+    float4 x[NBV];
+    auto fetch = [&](int64_t t) {
+        const int64_t r0 = t * R;
+        const int n = static_cast<int>(min(static_cast<int64_t>(R), rows - r0)) * perRow;
+        const BufferRsrc bufA = make_buffer(a + r0 * static_cast<int64_t>(T), n * 16);
+        // (always NBV loads, those behind the tile masked by the range check: a fixed number of memory instructions
+        // lets the wait for these loads leave the stores that are issued behind them in flight)
+#pragma unroll
+        for (int b = 0; b < NBV; ++b) x[b] = buffer_load4(bufA, (lane + b * kWave) * 16, 0);
+    };
+    // the lane index behind a barrier for the optimiser: the (row, vector) sequences of the staging and storing
+    // loops do not depend on the tile, and kept across the filter and the walk they would cost 2 registers per vector
+    auto lane_again = [&]() {
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        return l;
+    };
+    int64_t tileIdx = blockIdx.x;
+    if (tileIdx >= tiles) return;
+    fetch(tileIdx);
+    // the lane's column of the Toeplitz factor; the range check of a buffer that ends with the filter turns every
+    // index that is not a tap into a zero
+    float fa[D][4];
+    {
+        const BufferRsrc bufF = make_buffer(srm, F * 4);
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int tap = 16 * d + 4 * h + v - c;
+                fa[d][v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                         bufF, masked_offset(tap >= 0 && tap < F, tap * 4), 0, 0));
+            }
+    }
+    float tap[NU];
+#pragma unroll
+    for (int j = 0; j < NU; ++j) tap[j] = (j < nuSize) ? nu[j] : -0.0f;
+    float myTap[kRounds];  // this lane's taps in the candidate walk (lane p of a row: taps p kRounds ... )
+#pragma unroll
+    for (int j = 0; j < kRounds; ++j) {
+        const int tj = (lane % kParts) * kRounds + j;
+        myTap[j] = tj < nuSize ? nu[tj] : -0.0f;
+    }
+    // a refractory kernel without positive taps only lowers the potential: samples below the threshold never fire
+    bool monotone = true;
+#pragma unroll
+    for (int j = 0; j < NU; ++j) monotone = monotone && tap[j] <= 0.0f;
+
+    if (lane < 4) *reinterpret_cast<float4 *>(zeros + 4 * lane) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (lane < 32) tapL[lane - 3] = (lane >= 3 && lane - 3 < nuSize) ? nu[lane - 3] : -0.0f;
+    for (;;) {
+    const int64_t row0 = tileIdx * R;
+    const int nRows = static_cast<int>(min(static_cast<int64_t>(R), rows - row0));
+    const int nVec = nRows * perRow;
+    for (int i = lane; i < R * MP; i += kWave) cand[i] = 0u;
+    bool bad = false;
+    {
+        RowCol rc;
+        rc.init(lane_again(), perRow, 1.0f / static_cast<float>(perRow));
+        const int dr = kWave / perRow, dc = kWave % perRow;
+#pragma unroll
+        for (int b = 0; b < NBV; ++b) {
+            if (lane + b * kWave < R * perRow) {
+                *reinterpret_cast<float4 *>(tile + rc.r * P + LAG + (rc.c << 2)) = x[b];
+                // infinite or NaN (or four samples that add up to more than fp32 holds, which only costs time)
+                bad |= ((x[b].x + x[b].y) + (x[b].z + x[b].w)) * 0.0f != 0.0f;
+            }
+            rc.advance(dr, dc, perRow);
+        }
+    }
+    const bool chains = __builtin_amdgcn_ballot_w64(bad) != 0;
+    wave_sync();
+    const int64_t tileNext = tileIdx + gridDim.x;
+    if (tileNext < tiles) fetch(tileNext);
+
+    auto mark4 = [&](int r, int col, const float4 &y) {  // col is a multiple of 4: the four bits lie in one word
+        const uint32_t bits = (y.x >= theta ? 1u : 0u) | (y.y >= theta ? 2u : 0u) | (y.z >= theta ? 4u : 0u) |
+                              (y.w >= theta ? 8u : 0u);
+        if (bits) atomicOr(cand + r * MP + (col >> 5), bits << (col & 31));
+    };
+    if (chains) {
+        // a non-finite sample: the tile's potentials as sequential chains over the valid taps, from memory
+        for (int e = lane; e < nVec; e += kWave) {
+            const int r = e / perRow, t0 = (e - r * perRow) << 2;
+            const float *xr = a + (row0 + r) * static_cast<int64_t>(T);
+            float y[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int t = t0 + k;
+                const int taps = min(t + 1, F);
+                float acc = 0.0f;
+                for (int i = 0; i < taps; ++i) acc = __builtin_fmaf(xr[t - i], srm[i], acc);
+                y[k] = acc * Ts;
+            }
+            const float4 q = make_float4(y[0], y[1], y[2], y[3]);
+            *reinterpret_cast<float4 *>(tile + r * P + LAG + t0) = q;
+            if (monotone) mark4(r, LAG + t0, q);
+        }
+    } else {
+        // walk down in time: step j makes time block q = nBlk - 1 - j from time blocks q .. q - D + 1
+        const int nBlk = (T + 15) >> 4;
+        const int vecT = 4 * (3 - h);  // this lane's vector of a block, as a time offset
+        float *col = tile + c * P + LAG + vecT;
+        const float *zr = zeros + 4 * h;
+        auto block = [&](int jm) {  // block jm of the reversed axis; zeros before the row's start and behind its end
+            const int q = nBlk - 1 - jm;
+            const bool keep = q >= 0 && 16 * q + vecT < T;
+            return *reinterpret_cast<const float4 *>(keep ? col + 16 * q : zr);
+        };
+        float4 w[W];
+#pragma unroll
+        for (int d = 0; d < D; ++d) w[d] = block(d);
+        for (int j0 = 0; j0 < nBlk; j0 += W) {
+#pragma unroll
+            for (int k = 0; k < W; ++k) {
+                const int j = j0 + k;
+                if (j < nBlk) {
+                    w[(k + D) % W] = block(j + D);       // the block the next step adds
+                    __builtin_amdgcn_sched_barrier(0);  // (issued here, not after the step's matrix work)
+                    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int d = 0; d < D; ++d) {
+                        const float4 &xv = w[(k + d) % W];
+                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[d][0], xv.w, acc, 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[d][1], xv.z, acc, 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[d][2], xv.y, acc, 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[d][3], xv.x, acc, 0, 0, 0);
+                    }
+                    const int q = nBlk - 1 - j;
+                    if (16 * q + vecT < T) {
+                        const float4 y = make_float4(acc.w * Ts, acc.z * Ts, acc.y * Ts, acc.x * Ts);
+                        *reinterpret_cast<float4 *>(col + 16 * q) = y;
+                        if (monotone) mark4(c, LAG + 16 * q + vecT, y);
+                    }
+                }
+            }
+        }
+    }
+    wave_sync();
+
+    // ---- walk: columns [0, T + LAG) of the tile become final
+    const int Wc = T + LAG;
+    const int words = (Wc + 31) >> 5;
+    const int cr = lane / kParts, part = lane - cr * kParts;
+    bool hop = monotone;
+    uint32_t nzw = 0u;  // bit w: word w of the row has candidates
+    if (monotone) {
+        int mine = 0;
+        for (int wd = part; wd < words; wd += kParts) {
+            const uint32_t cw = cand[cr * MP + wd];
+            mine += __builtin_popcount(cw);
+            nzw |= (cw != 0u ? 1u : 0u) << wd;
+        }
+#pragma unroll
+        for (int off = kParts / 2; off > 0; off >>= 1) {
+            mine += __shfl_xor(mine, off, kWave);
+            nzw |= __shfl_xor(nzw, off, kWave);
+        }
+        // from candidate to candidate while no row of the tile has more than one per 12 samples (the wavefront
+        // stays as long as its busiest row)
+        hop = __builtin_amdgcn_ballot_w64(mine * 12 > Wc) == 0;
+    }
+    if (hop) {
+        // every lane of a row follows the row's candidates; on a spike each adds its own taps of the response
+        const uint32_t *cw = cand + cr * MP;
+        uint32_t *mw = masks + cr * MP;
+        float *mine = tile + cr * P;
+        for (int wd = part; wd < words; wd += kParts) mw[wd] = 0u;  // words without candidates have no spikes
+        int wd = 0;
+        uint32_t cm = 0u, fired = 0u;
+        while (__builtin_amdgcn_ballot_w64((cm | nzw) != 0u) != 0) {
+            if (cm == 0u && nzw != 0u) {  // on to the row's next word with candidates
+                if (fired != 0u) mw[wd] = fired;
+                fired = 0u;
+                wd = __builtin_ctz(nzw);
+                nzw &= nzw - 1u;
+                cm = cw[wd];
+            }
+            if (cm != 0u) {
+                const int k = __builtin_ctz(cm);
+                cm &= cm - 1u;
+                // the candidate itself (the same address for the row's lanes) and this lane's samples of the response
+                // in one round of reads: a walk is as long as the chain of its LDS round trips
+                const float *q0 = mine + (wd << 5) + k;
+                float *q = mine + (wd << 5) + k + part * kRounds;
+                const float x0 = *q0;
+                float val[kRounds];
+#pragma unroll
+                for (int j = 0; j < kRounds; ++j)
+                    if (part * kRounds + j < NU) val[j] = q[j];   // (what lies behind the response belongs to the next row)
+                if (x0 >= theta) {
+                    fired |= 1u << k;
+#pragma unroll
+                    for (int j = 0; j < kRounds; ++j)
+                        if (part * kRounds + j < NU) q[j] = val[j] + myTap[j];
+                }
+            }
+        }
+        if (fired != 0u) mw[wd] = fired;
+    } else {
+        // Every sample in turn, 32 samples at a time through a register window of 32 + LAG samples, as in spike.hip -
+        // but the window of a row is spread over the row's four lanes, lane p keeping the samples whose window index
+        // is p (mod 4).  The sample under test is broadcast within the quad (a lane-permuting move, no LDS); on a
+        // spike every lane adds the taps that fall on its own samples, NA instead of NU additions.
+        constexpr int NW = (G + LAG) / kParts;          // window registers per lane
+        constexpr int NA = (NU + kParts - 1) / kParts + 1;  // additions per spike and lane
+        float wq[NW];    // wq[m] = window sample 4 m + part
+        float tq[kParts][NA];  // tq[res][i] = nu[4 i + part - res]: what a spike at window index k = res (mod 4) adds to wq[k / 4 + i]
+#pragma unroll
+        for (int res = 0; res < kParts; ++res)
+#pragma unroll
+            for (int i = 0; i < NA; ++i) tq[res][i] = tapL[4 * i + part - res];
+        float *mine = tile + cr * P;
+#pragma unroll
+        for (int m = 0; m < LAG / kParts; ++m) wq[m] = quiet;
+        const int groups = (Wc + G - 1) / G;
+        for (int g = 0; g < groups; ++g) {
+            const int c0 = g * G;
+            if (c0 + G <= T) {
+#pragma unroll
+                for (int m = 0; m < G / kParts; ++m) wq[LAG / kParts + m] = mine[LAG + c0 + 4 * m + part];
+            } else {
+#pragma unroll
+                for (int m = 0; m < G / kParts; ++m)
+                    wq[LAG / kParts + m] = (c0 + 4 * m + part < T) ? mine[LAG + c0 + 4 * m + part] : quiet;
+            }
+            uint32_t fired = 0;
+            auto sample = [&](int k) {  // window sample k, from the lane of the quad that keeps it
+                constexpr int kQuad[4] = {0x00, 0x55, 0xaa, 0xff};  // quad_perm: all four lanes read lane k % 4
+                const int bitsIn = __builtin_bit_cast(int, wq[k / kParts]);
+                int bitsOut = 0;
+                switch (k % kParts) {
+                    case 0: bitsOut = __builtin_amdgcn_update_dpp(0, bitsIn, kQuad[0], 0xf, 0xf, false); break;
+                    case 1: bitsOut = __builtin_amdgcn_update_dpp(0, bitsIn, kQuad[1], 0xf, 0xf, false); break;
+                    case 2: bitsOut = __builtin_amdgcn_update_dpp(0, bitsIn, kQuad[2], 0xf, 0xf, false); break;
+                    default: bitsOut = __builtin_amdgcn_update_dpp(0, bitsIn, kQuad[3], 0xf, 0xf, false); break;
+                }
+                return __builtin_bit_cast(float, bitsOut);
+            };
+#pragma unroll
+            for (int k = 0; k < G; k += 2) {
+                // one scalar branch per two samples (the second sample is tested again inside, after the first one's
+                // refractory response)
+                const float xa = sample(k), xb = sample(k + 1);
+                if (__builtin_amdgcn_ballot_w64((xa >= theta) | (xb >= theta)) != 0) {
+                    if (xa >= theta) {
+                        fired |= 1u << k;
+#pragma unroll
+                        for (int i = 0; i < NA; ++i) wq[k / kParts + i] += tq[k % kParts][i];
+                    }
+                    if (sample(k + 1) >= theta) {
+                        fired |= 2u << k;
+#pragma unroll
+                        for (int i = 0; i < NA; ++i) wq[(k + 1) / kParts + i] += tq[(k + 1) % kParts][i];
+                    }
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < G / kParts; ++m) mine[c0 + 4 * m + part] = wq[m];
+            masks[cr * MP + g] = fired;  // (the same word from the four lanes of a row)
+#pragma unroll
+            for (int m = 0; m < LAG / kParts; ++m) wq[m] = wq[G / kParts + m];
+        }
+    }
+    wave_sync();
+
+    // ---- retire: u' and s of the whole tile, one contiguous run (a fixed number of stores, masked by the buffers'
+    //      range check: the wait for the next tile's loads, which are older, can then leave exactly these in flight)
+    {
+        const BufferRsrc bufU = make_buffer(u + row0 * static_cast<int64_t>(T), nVec * 16);
+        const BufferRsrc bufS = make_buffer(s + row0 * static_cast<int64_t>(T), nVec * 16);
+        RowCol rc;
+        rc.init(lane_again(), perRow, 1.0f / static_cast<float>(perRow));
+        const int dr = kWave / perRow, dc = kWave % perRow;
+#pragma unroll
+        for (int b = 0; b < NBV; ++b) {
+            const int r = min(rc.r, R - 1);  // (lanes behind the tile: their stores are dropped)
+            const int cl = LAG + (rc.c << 2);
+            const uint32_t m = masks[r * MP + (cl >> 5)] >> (cl & 31);
+            buffer_store4(bufU, (lane + b * kWave) * 16, 0, *reinterpret_cast<const float4 *>(tile + r * P + cl));
+            buffer_store4(bufS, (lane + b * kWave) * 16, 0,
+                          make_float4((m & 1u) ? amplitude : 0.0f, (m & 2u) ? amplitude : 0.0f,
+                                      (m & 4u) ? amplitude : 0.0f, (m & 8u) ? amplitude : 0.0f));
+            rc.advance(dr, dc, perRow);
+            if (b % 4 == 3) __builtin_amdgcn_sched_barrier(0);  // a few vectors at a time: they occupy registers
+        }
+    }
+    if (tileNext >= tiles) break;
+    wave_sync();
+    tileIdx = tileNext;
+    }
+}
+
+template <int NU>
+static int launch_psp_spike_mfma(float *s, float *u, const float *a, const float *srm, const float *nu, int64_t rows,
+                                 int T, int F, int nuSize, float theta, float Ts, hipStream_t st)
+{
+    constexpr int LAG = (NU + 2) & ~3;
+    // a row of the tile: LAG columns in front, the samples, and room for the response of a spike in the last sample
+    // (hop walk) or for whole groups of 32 (window walk); a pitch of 4 (mod 32) spreads the 16 rows over the banks
+    int P = LAG + T + NU;
+    if (P < ((T + LAG + 31) & ~31)) P = (T + LAG + 31) & ~31;
+    P = ((P - 4 + 31) & ~31) + 4;
+    const int MP = (T + LAG + 31) / 32 + 1;
+    const size_t lds = (static_cast<size_t>(kFusedMfmaRows) * P + 2 * kFusedMfmaRows * MP + 16 + 32) * sizeof(float);
+    // wavefronts resident at once (what the tiles' LDS leaves room for); each walks over its share of the tiles
+    const int64_t tiles = ceil_div(rows, kFusedMfmaRows);
+    const int64_t perUnit = 160 * 1024 / static_cast<int64_t>(lds);
+    const int64_t resident = static_cast<int64_t>(compute_units()) * (perUnit < 8 ? perUnit : 8);
+    const int64_t trips = ceil_div(tiles, resident);
+    const dim3 grid(static_cast<unsigned>(ceil_div(tiles, trips)));
+    const int D = (F + 14) / 16 + 1;
+#define SLAYER_PSP_SPIKE_MFMA(DD)                                                                                     \
+    case DD:                                                                                                          \
+        hipLaunchKernelGGL((psp_spike_mfma_kernel<DD, NU>), grid, dim3(kWave), lds, st, s, u, a, srm, nu, rows, T, F, \
+                           nuSize, P, MP, theta, Ts);                                                                 \
+        break
+    switch (D) {
+        SLAYER_PSP_SPIKE_MFMA(4);
+        SLAYER_PSP_SPIKE_MFMA(5);
+        SLAYER_PSP_SPIKE_MFMA(6);
+        SLAYER_PSP_SPIKE_MFMA(7);
+        SLAYER_PSP_SPIKE_MFMA(8);
+        default:
+            SLAYER_PSP_SPIKE_MFMA(9);
+    }
+#undef SLAYER_PSP_SPIKE_MFMA
+    return launch_status();
+}
+
 }  // namespace slayer
 
 extern "C" int slayer_psp_spike_f32(float *s, float *u, const float *a, const float *srm, const float *nu,
@@ -214,6 +592,13 @@ extern "C" int slayer_psp_spike_f32(float *s, float *u, const float *a, const fl
         const int status = slayer_conv_f32(u, a, srm, nNeurons, T, F, Ts, stream);
         if (status != SLAYER_OK) return status;
         return slayer_get_spikes_f32(s, u, nu, nNeurons, T, nuSize, theta, Ts, stream);
+    }
+    if (F >= kFirMfmaMinTaps && F <= kFirMfmaMaxTaps && T >= 16) {  // filters that pay on the matrix cores
+        if (nuSize <= 12)
+            return launch_psp_spike_mfma<12>(s, u, a, srm, nu, nNeurons, static_cast<int>(T), static_cast<int>(F),
+                                             static_cast<int>(nuSize), theta, Ts, st);
+        return launch_psp_spike_mfma<24>(s, u, a, srm, nu, nNeurons, static_cast<int>(T), static_cast<int>(F),
+                                         static_cast<int>(nuSize), theta, Ts, st);
     }
     const int ttp = static_cast<int>((T + kFusedU - 1) & ~static_cast<int64_t>(kFusedU - 1));
     const int LD = static_cast<int>((ttp + F + 4 + 3) & ~static_cast<int64_t>(3));  // tile, halo, window over-read

@@ -144,12 +144,13 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
 //    ("candidates", a few per cent) while the piece is staged, one bit per sample, and the walking lanes go from
 //    candidate to candidate: test the sample's current value and, on a spike, add nu[0..NU) onto the NU samples
 //    from it on, in place - the same fp32 additions in the same order as the sequential loop;
-//  * any other kernel: every sample in turn, also in place.
+//  * any other kernel, and tiles with a row that is above the threshold more than one sample in 12: every
+//    sample in turn through a register window that is spread over the lanes of the row (further down).
 // The last LAG samples of a piece are not final until the next piece arrives: they (and their candidate bits)
 // are copied to the front of the tile and open the next piece.  Taps beyond nuSize are -0.0f, whose addition
 // changes no value; a response may reach past the row's end into padding that is never stored.
-// Leaving most lanes idle during the walk is deliberate: the kernel is bound by HBM traffic,
-// not by the vector ALU, and short tiles keep many wavefronts (and bytes) in flight per CU.
+// Short tiles keep many wavefronts (and bytes) in flight per CU; the walking wavefront shares its SIMD's issue
+// slots with those that move data, so both walks use all 64 lanes (64 / R per row) to need fewer instructions.
 constexpr int kTileMaxPiece = 352;  // longest row (samples) that travels whole
 // Rows in pieces: samples per piece and row.  With 8-row tiles - tensors of few, long rows - the bytes in flight
 // per compute unit are what the rows in LDS amount to, so those pieces are longer.
@@ -228,6 +229,16 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         const int tj = lane % (kWave / R) + j * (kWave / R);
         myTap[j] = tj < nuSize ? nu[tj] : -0.0f;
     }
+    // ... and for the walk over every sample, the kernel in LDS with -0.0f (whose addition changes
+    // nothing) in front and behind: tapL[j] = nu[j] for j in [-(kLanesPerRow - 1), 48 - kLanesPerRow)
+    constexpr int kLanesPerRow = kWave / R;
+    constexpr int kAdds = (NU + kLanesPerRow - 1) / kLanesPerRow + 1;  // additions per spike and lane in that walk
+    static_assert(kLanesPerRow * kAdds <= 48 - kLanesPerRow + 1, "the padded kernel in LDS");
+    float *tapL = reinterpret_cast<float *>(rowMasks + R * MPT) + (kLanesPerRow - 1);
+    if (lane < 48) {
+        const int tj = lane - (kLanesPerRow - 1);
+        tapL[tj] = (tj >= 0 && tj < nuSize) ? nu[tj] : -0.0f;
+    }
     // The normal refractory kernel only lowers the potential (every tap <= 0; a NaN tap fails the test).  A sample
     // below the threshold as it arrives can then never fire, so the sequential part need only visit the samples
     // at or above it ("candidates", a few per cent): all 64 lanes mark them while the tile is staged, and the
@@ -240,7 +251,6 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
         if (x >= theta) atomicOr(cand + r * MP + (col >> 5), 1u << (col & 31));
     };
     constexpr int G = 32;               // samples per group of the window walk = bits of a spike mask
-    float v[G + LAG];                   // its register window
 
     // A "step" is one piece of one tile.  The global loads of a step are issued one step ahead
     // into x[] and stay in flight while the previous step is walked and retired.
@@ -452,55 +462,84 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                 }
             }
             if (fired != 0u) mw[w] = fired;
-        } else if (lane < R) {
-            // every sample in turn: 32 samples at a time are pulled into a register window v[0 .. 32+LAG), a spike
-            // adds nu[0..NU) onto v[k .. k+NU), and the 32 oldest samples go back to LDS with their spike mask
-            float *mine = tile + lane * P;
-            uint32_t *mw = record ? rowMasks + lane * MPT + (tL >> 5) : masks + lane * MP;
+        } else {
+            // Every sample in turn: 32 samples at a time pass through a register window of 32 + LAG
+            // samples that is spread over the row's kParts lanes - lane p keeps the samples whose window index is
+            // p (mod kParts).  The sample under test is broadcast within the row's lanes by lane-permuting moves (no
+            // LDS); on a spike every lane adds the taps that fall on its own samples, kAdds instead of NU additions,
+            // the same fp32 additions in the same order per sample as the sequential loop.  What counts in this
+            // walk is the number of instructions (the wavefront shares its SIMD's issue slots), not the active lanes.
+            constexpr int NW = (G + LAG + kParts - 1) / kParts;  // window registers per lane
+            float wq[NW];                                       // wq[m] = window sample kParts m + part
+            // tq[res][i] = nu[kParts i + part - res]: what a spike at a window index k = res (mod kParts) adds to
+            // this lane's sample kParts (k / kParts + i) + part
+            float tq[kParts][kAdds];
 #pragma unroll
-            for (int k = 0; k < LAG; ++k) v[k] = (tL == 0) ? quiet : mine[k];
+            for (int res = 0; res < kParts; ++res)
+#pragma unroll
+                for (int i = 0; i < kAdds; ++i) tq[res][i] = tapL[kParts * i + part - res];
+            float *mine = tile + cr * P;
+            // (the first LAG window samples: nothing before a row's start, else what the last piece left behind)
+#pragma unroll
+            for (int m = 0; m < NW; ++m) wq[m] = (tL == 0 || kParts * m + part >= LAG) ? quiet : mine[kParts * m + part];
+            auto sample = [&](int k) {  // window sample k, from the lane of the row that keeps it
+                const int in = __builtin_bit_cast(int, wq[k / kParts]);
+                int q = 0;
+                switch (k % 4) {  // quad_perm: the four lanes of a quad read its lane k % 4
+                    case 0: q = __builtin_amdgcn_update_dpp(0, in, 0x00, 0xf, 0xf, false); break;
+                    case 1: q = __builtin_amdgcn_update_dpp(0, in, 0x55, 0xf, 0xf, false); break;
+                    case 2: q = __builtin_amdgcn_update_dpp(0, in, 0xaa, 0xf, 0xf, false); break;
+                    default: q = __builtin_amdgcn_update_dpp(0, in, 0xff, 0xf, 0xf, false); break;
+                }
+                if constexpr (kParts == 8) {
+                    // the quad that does not keep the sample takes it from the other one: lane i of each group of
+                    // 8 reads lane 7 - i (row_half_mirror), written only in the banks (quads) that need it
+                    if ((k % 8) < 4) q = __builtin_amdgcn_update_dpp(q, q, 0x141, 0xf, 0xa, false);
+                    else q = __builtin_amdgcn_update_dpp(q, q, 0x141, 0xf, 0x5, false);
+                }
+                return __builtin_bit_cast(float, q);
+            };
+            uint32_t *mw = record ? rowMasks + cr * MPT + (tL >> 5) : masks + cr * MP;
             const int groups = (W + G - 1) / G;
             for (int g = 0; g < groups; ++g) {
                 const int c0 = g * G;
-                if (c0 + G <= n) {
 #pragma unroll
-                    for (int k = 0; k < G; k += 4) {
-                        const float4 q = *reinterpret_cast<const float4 *>(mine + LAG + c0 + k);
-                        v[LAG + k] = q.x; v[LAG + k + 1] = q.y; v[LAG + k + 2] = q.z; v[LAG + k + 3] = q.w;
-                    }
-                } else {
-#pragma unroll
-                    for (int k = 0; k < G; ++k) v[LAG + k] = (c0 + k < n) ? mine[LAG + c0 + k] : quiet;
+                for (int m = LAG / kParts; m < NW; ++m) {
+                    const int i = kParts * m + part;  // window index; sample c0 + i - LAG of the piece
+                    if (i >= LAG && i < LAG + G) wq[m] = (c0 + i - LAG < n) ? mine[c0 + i] : quiet;
                 }
                 uint32_t fired = 0;
 #pragma unroll
                 for (int k = 0; k < G; k += 2) {
-                    // One scalar branch per two samples: in most pairs no row spikes.  (The second
-                    // sample is tested again inside, after the first one's refractory response.)
-                    if (__builtin_amdgcn_ballot_w64((v[k] >= theta) | (v[k + 1] >= theta)) != 0) {
-                        if (v[k] >= theta) {
+                    // one scalar branch per two samples (the second sample is tested again inside, after the first
+                    // one's refractory response)
+                    const float xa = sample(k), xb = sample(k + 1);
+                    if (__builtin_amdgcn_ballot_w64((xa >= theta) | (xb >= theta)) != 0) {
+                        if (xa >= theta) {
                             fired |= 1u << k;
 #pragma unroll
-                            for (int j = 0; j < NU; ++j) v[k + j] += tap[j];
+                            for (int i = 0; i < kAdds; ++i)
+                                if (k / kParts + i < NW) wq[k / kParts + i] += tq[k % kParts][i];
                         }
-                        if (v[k + 1] >= theta) {
+                        if (sample(k + 1) >= theta) {
                             fired |= 2u << k;
 #pragma unroll
-                            for (int j = 0; j < NU; ++j) v[k + 1 + j] += tap[j];
+                            for (int i = 0; i < kAdds; ++i)
+                                if ((k + 1) / kParts + i < NW) wq[(k + 1) / kParts + i] += tq[(k + 1) % kParts][i];
                         }
                     }
                 }
 #pragma unroll
-                for (int k = 0; k < G; k += 4)
-                    *reinterpret_cast<float4 *>(mine + c0 + k) = make_float4(v[k], v[k + 1], v[k + 2], v[k + 3]);
-                mw[g] = fired;
+                for (int m = 0; m < G / kParts; ++m) mine[c0 + kParts * m + part] = wq[m];
+                mw[g] = fired;  // (the same word from all lanes of the row)
 #pragma unroll
-                for (int k = 0; k < LAG; ++k) v[k] = v[G + k];
+                for (int m = 0; m < (LAG + kParts - 1) / kParts; ++m) wq[m] = wq[m + G / kParts];
             }
             // the LAG columns behind the final ones have taken part of the responses: back to LDS for the next piece
             if (!last) {
 #pragma unroll
-                for (int k = 0; k < LAG; ++k) mine[W + k] = v[k];
+                for (int m = 0; m < (LAG + kParts - 1) / kParts; ++m)
+                    if (kParts * m + part < LAG) mine[W + kParts * m + part] = wq[m];
             }
         }
         wave_sync();
@@ -830,8 +869,9 @@ static int launch_get_spikes(float *s, float *u, const float *nu, int64_t nNeuro
         /* shifted spikes of rows in pieces: the spike bits of whole rows stay in LDS */                \
         const int MPT = (dl.on && !whole) ? static_cast<int>((T + LAGV + 31) / 32 + 1) : 0;             \
         auto lds_bytes = [&]() {                                                                        \
+            /* tile, spike and candidate bits, row shifts, whole rows' spike bits, the padded kernel */  \
             return (static_cast<size_t>(rowsPerTile) * P + 2 * rowsPerTile * MP + rowsPerTile +         \
-                    static_cast<size_t>(rowsPerTile) * MPT) * sizeof(float);                            \
+                    static_cast<size_t>(rowsPerTile) * MPT + 48) * sizeof(float);                       \
         };                                                                                              \
         /* eight wavefronts per compute unit are what the 8-row tiles of a small tensor need to be      \
            resident all at once: shorter pieces if the tile does not fit an eighth of the LDS */        \

@@ -409,12 +409,41 @@ def test_spike_bwd_corr_is_the_two_ops_in_one(impl, shape, Fl):
         assert np.array_equal(bits(got), bits(two)), "fused kernel differs from spikeBackward followed by corr"
 
 
+def spikes_follow_filtered_input(s, u, a, srm, nu, theta, Ts):
+    """Checks (s, u) = getSpikes(psp) for SOME psp that agrees with Ts * conv(a, srm) to rounding, without knowing
+    that psp's bits (a filter summed on the matrix cores): exactly, every sample without a spike ended below the
+    threshold and every sample with one ended at or above fl(theta + nu[0]) - a sample is last changed when it is
+    visited, and fp32 addition is monotone; and u minus the refractory responses of s is the filtered input within
+    1e-5 of the sum of its terms' magnitudes (plus the rounding of the at most len(nu) additions of responses)."""
+    T = a.shape[-1]
+    s2, u2, a2 = (np.asarray(v).reshape(-1, T) for v in (s, u, a))
+    spk = s2 != 0
+    if not np.all(s2[spk] == np.float32(1.0 / Ts)):
+        return False
+    nu = np.asarray(nu, np.float32)
+    floor = np.float32(theta) + nu[0] if len(nu) else np.float32(theta)
+    if np.any(u2[~spk] >= np.float32(theta)) or np.any(u2[spk] < floor):
+        return False
+    f64, nu64 = np.asarray(srm, np.float64), nu.astype(np.float64)
+    for r in range(a2.shape[0]):
+        exact = np.convolve(a2[r].astype(np.float64), f64)[:T] * Ts
+        bound = np.convolve(np.abs(a2[r]).astype(np.float64), np.abs(f64))[:T] * Ts
+        refr = np.convolve(spk[r].astype(np.float64), nu64)[:T] if len(nu) else np.zeros(T)
+        refr_mag = np.convolve(spk[r].astype(np.float64), np.abs(nu64))[:T] if len(nu) else np.zeros(T)
+        err = np.abs(u2[r].astype(np.float64) - refr - exact)
+        if np.any(err > 1e-5 * bound + 3e-6 * (np.abs(exact) + refr_mag) + 1e-37):
+            return False
+    return True
+
+
 @pytest.mark.parametrize("shape,Fl,nuSize", [((2, 6, 5, 3, 300), 77, 11), ((1, 9, 1, 1, 352), 160, 24), ((3, 7, 1, 1, 64), 8, 4),
                                              ((1, 1, 1, 1, 4), 1, 1), ((2, 5, 1, 1, 100), 130, 16), ((1, 17, 1, 1, 8), 77, 0),
-                                             ((1, 3, 1, 1, 350), 77, 11), ((1, 2, 1, 1, 2000), 8, 11), ((1, 4, 1, 1, 300), 77, 30)])
+                                             ((1, 3, 1, 1, 350), 77, 11), ((1, 2, 1, 1, 2000), 8, 11), ((1, 4, 1, 1, 300), 77, 30),
+                                             ((3, 11, 1, 1, 352), 129, 24), ((1, 40, 1, 1, 16), 34, 3), ((2, 9, 2, 2, 64), 50, 0),
+                                             ((1, 33, 1, 1, 300), 100, 13), ((2, 16, 1, 1, 20), 40, 12)])
 def test_psp_spike_is_conv_then_getSpikes(impl, shape, Fl, nuSize):
-    # spike(psp(x)) in one call: bit for bit what the two kernels give, on shapes that take the fused
-    # kernel (whole-vector rows up to 352 samples) and on shapes that do not
+    # spike(psp(x)) in one call: what the two kernels give, on shapes that take a fused kernel (whole-vector rows up
+    # to 352 samples) and on shapes that do not
     rng = np.random.default_rng(shape[-1] + Fl + nuSize)
     a = (rng.standard_normal(shape) * 2).astype(np.float32)
     srm = rng.random(Fl).astype(np.float32)
@@ -427,11 +456,11 @@ def test_psp_spike_is_conv_then_getSpikes(impl, shape, Fl, nuSize):
     wu = O.conv(a, srm, Ts, fused=True)
     ws, wu = O.get_spikes(wu, nu, theta, Ts)
     T = shape[-1]
-    one_kernel = T % 4 == 0 and T <= 352 and nuSize <= 24 and Fl <= 160
-    if one_kernel or not on_matrix_cores("conv", T, Fl, impl):
-        # the fused kernel filters with the chain: the oracle's bits, whatever kernel `conv` uses on its own
+    one_kernel = not impl and T % 4 == 0 and T <= 352 and nuSize <= 24 and Fl <= 160
+    mfma = on_matrix_cores("conv", T, Fl, impl)
+    if not mfma:
+        # the filter runs as the chain, fused or not: the oracle's bits
         assert np.array_equal(bits(host(s)), bits(ws)) and np.array_equal(bits(host(u)), bits(wu))
-    if not on_matrix_cores("conv", T, Fl, impl):
         assert torch.equal(s, s2) and np.array_equal(bits(host(u)), bits(host(u2)))
     else:
         # a dense input filtered on the matrix cores agrees with the chain to rounding; the spike function of exactly
@@ -439,9 +468,62 @@ def test_psp_spike_is_conv_then_getSpikes(impl, shape, Fl, nuSize):
         assert rel_err(psp2, O.conv(a, srm, Ts, fused=True)) <= REL_TOL
         ws2, wu2 = O.get_spikes(psp2, nu, theta, Ts)
         assert np.array_equal(bits(host(s2)), bits(ws2)) and np.array_equal(bits(host(u2)), bits(wu2))
-        if not one_kernel:
+        if one_kernel:   # the fused kernel's own potentials are not stored anywhere
+            assert spikes_follow_filtered_input(host(s), host(u), a, srm, nu, theta, Ts)
+            assert not spikes_follow_filtered_input(host(s), host(u) + np.float32(1e-3), a, srm, nu, theta, Ts)
+            # the fused kernel and the convolution kernel feed the matrix instructions the same operands in the same
+            # order, so on a finite dense input even the bits agree
+            assert torch.equal(s, s2) and np.array_equal(bits(host(u)), bits(host(u2)))
+        else:
             assert torch.equal(s, s2) and np.array_equal(bits(host(u)), bits(host(u2)))
     assert ws.sum() > 0 or shape[-1] < 64
+
+
+@pytest.mark.parametrize("kind", ["positive_tap", "busy_rows", "infinity", "nan", "ragged_tile"])
+def test_psp_spike_on_matrix_cores_special_cases(kind):
+    # the fused kernel for 34..129 taps: refractory kernels with a positive tap and rows above the threshold most of
+    # the time (every sample in turn instead of candidate to candidate), non-finite samples (the tile is filtered as
+    # chains: the reference's bits, infinities and NaNs where the reference puts them), a last tile of 3 rows
+    rng = np.random.default_rng(len(kind))
+    shape = (2, 19, 1, 1, 300) if kind == "ragged_tile" else (2, 24, 1, 1, 300)
+    a = (rng.standard_normal(shape) * 2).astype(np.float32)
+    srm = (rng.random(77).astype(np.float32) - 0.3)
+    nu = -(rng.random(11) * 5).astype(np.float32)
+    theta, Ts = 3.0, 1.0
+    if kind == "positive_tap":
+        nu[4] = 1.5
+    if kind == "busy_rows":
+        theta = -2.0
+    if kind == "infinity":
+        a[0, 3, 0, 0, 100] = np.inf
+        a[1, 20, 0, 0, 299] = -np.inf
+    if kind == "nan":
+        a[1, 7, 0, 0, 0] = np.nan
+    s, u = slayerCuda.pspSpike(dev(a), dev(srm), dev(nu), theta, Ts)
+    s, u = host(s), host(u)
+    flat_a, flat_s, flat_u = a.reshape(-1, 300), s.reshape(-1, 300), u.reshape(-1, 300)
+    chain_u = O.conv(a, srm, Ts, fused=True)
+    chain_s, chain_u = O.get_spikes(chain_u, nu, theta, Ts)
+    chain_s, chain_u = chain_s.reshape(-1, 300), chain_u.reshape(-1, 300)
+    for tile in range(0, flat_a.shape[0], 16):
+        rows = slice(tile, tile + 16)
+        if not np.all(np.isfinite(flat_a[rows])):
+            assert np.array_equal(bits(flat_s[rows]), bits(chain_s[rows]))
+            assert np.array_equal(bits(flat_u[rows]), bits(chain_u[rows]))
+        elif kind == "positive_tap":
+            # rows whose spikes are the chain's (a potential within rounding of the threshold may flip one) end at the
+            # chain's potentials to rounding
+            same = [r for r in range(tile, min(tile + 16, flat_a.shape[0])) if np.array_equal(flat_s[r], chain_s[r])]
+            assert len(same) >= 12
+            for r in same:
+                assert np.max(np.abs(flat_u[r].astype(np.float64) - chain_u[r])) <= 1e-5 * np.max(np.abs(chain_u[r]))
+        else:
+            assert spikes_follow_filtered_input(flat_s[rows], flat_u[rows], flat_a[rows], srm, nu, theta, Ts)
+    u2 = slayerCuda.conv(dev(a), dev(srm), Ts)
+    s2 = slayerCuda.getSpikes(u2, dev(nu), theta, Ts)
+    if kind in ("positive_tap", "busy_rows", "ragged_tile"):
+        assert np.array_equal(bits(s), bits(host(s2))) and np.array_equal(bits(u), bits(host(u2)))
+    assert flat_s.sum() > 0
 
 
 def test_spikes_many_long_rows_use_16_row_tiles():
