@@ -217,20 +217,25 @@ def test_fir_sparse_input_edges(impl, T, Fl, op):
 
 @pytest.mark.parametrize("T,Fl", [(300, 77), (304, 40), (2000, 110), (64, 129)])
 def test_conv_density_switch_is_per_tile(T, Fl):
-    # tiles of 16 rows choose between the event-driven path (at most one 16-byte vector in five is not zero) and the
-    # matrix cores: row blocks on both sides of the switch and right at it, in one tensor
+    # tiles of 16 rows choose between the event-driven path (at most one staged sample in 20 is an event; one in 40
+    # when the events come in bursts) and the matrix cores: row blocks on both sides of the switch and right at it,
+    # in one tensor
     rng = np.random.default_rng(T + Fl)
     f = np.array(alphaKernel(Fl / 7.7, 1.0, 2000), dtype=np.float32)[:Fl]
     f = np.concatenate([f, rng.random(Fl - len(f)).astype(np.float32)])
     blocks = []
-    for pvec in (0.0, 0.05, 0.15, 0.19, 0.2, 0.21, 0.3, 1.0):       # share of non-zero vectors
+    for pvec in (0.0, 0.05, 0.15, 0.19, 0.2, 0.21, 0.3, 1.0):       # share of non-zero vectors, one event each
         xb = np.zeros((32, T // 4, 4), np.float32)
         mask = rng.random((32, T // 4)) < pvec
         xb[mask, rng.integers(0, 4, size=int(mask.sum()))] = 1.0
         if pvec == 1.0:
             xb = rng.standard_normal(xb.shape).astype(np.float32)
         blocks.append(xb.reshape(32, T))
-    x = np.stack(blocks)                                             # (8, 32, T)
+    for pvec in (0.004, 0.006, 0.0125, 0.05):                        # ... four events each (bursts)
+        xb = np.zeros((32, T // 4, 4), np.float32)
+        xb[rng.random((32, T // 4)) < pvec] = 1.0
+        blocks.append(xb.reshape(32, T))
+    x = np.stack(blocks)                                             # (12, 32, T)
     for op in ("conv", "corr"):
         got = host(getattr(slayerCuda, op)(dev(x), dev(f), 1.0))
         want = getattr(O, op)(x, f, 1.0, fused=True)
