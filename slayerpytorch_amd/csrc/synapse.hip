@@ -853,8 +853,15 @@ __global__ __launch_bounds__(512) void synapse_gather_mfma_kernel(GatherMfmaArgs
         // Trip k of the loop loads (pair, pass) number k of the range into registers, multiplies number k - 1 from
         // its LDS buffer ((k - 1) % 2) and then writes the registers to the other buffer: the loop's code exists
         // once, its first trip only loads.
-        int block = static_cast<int>(fastdiv(static_cast<uint32_t>(p0), g.bySteps));
-        int st = p0 - block * g.steps, pass = 0;          // what is loaded next
+        // Pairs are numbered with the pixel block fastest, then the step, then the batch item: consecutive pairs of
+        // a range are neighbouring patches of the same 32 samples, whose shared rows and columns come from L2
+        // instead of from memory (with the step fastest every pair fetched all of its patch from beyond L2: 4.7 x
+        // the source tensor on the 16 -> 32 channel layer, 6 x in its input gradient).
+        const int perItem = static_cast<int>(g.byBlocks.d);   // pixel blocks of a batch item
+        int image = static_cast<int>(fastdiv(static_cast<uint32_t>(p0), g.byBlocks));
+        int inItem = p0 - image * perItem;                // pixel block within the batch item ..
+        int item = static_cast<int>(fastdiv(static_cast<uint32_t>(image), g.bySteps));
+        int st = image - item * g.steps, pass = 0;        // .. step and pass that are loaded next
         int stCur = 0, passCur = 0, pixCur = -1, nCur = -1, nNext = -1;   // what is multiplied next
         float4 R[NS];
         int buf = 1;
@@ -868,14 +875,17 @@ __global__ __launch_bounds__(512) void synapse_gather_mfma_kernel(GatherMfmaArgs
             if (more && !first) {
                 if (++pass == g.passes) {
                     pass = 0;
-                    if (++st == g.steps) {
-                        st = 0;
-                        ++block;
-                        moved = true;
+                    moved = true;
+                    if (++inItem == perItem) {
+                        inItem = 0;
+                        if (++st == g.steps) {
+                            st = 0;
+                            ++item;
+                        }
                     }
                 }
             }
-            if (more && moved) nNext = place(block);
+            if (more && moved) nNext = place(item * perItem + inItem);
             issue(R, st, pass, more);
             __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the matrix work
             if (!first) {
