@@ -49,9 +49,11 @@ def measured_traffic(op):
                                                  "kernel": rec.get("kernels", {}).get(op)}
     except (OSError, ValueError, KeyError):
         return None, None
-KERNEL_OF = {"psp_conv": "slayer::fir_tiled_kernel<true, true, 16, false, 6> (conv; spike trains: event-driven path)", "spike": "slayer::spike_tile_kernel<12, 1, 12, 8>",
+KERNEL_OF = {"psp_conv": "slayer::alpha_psp_kernel<true, 4> (conv with the alpha kernel as a recursion over time)",
+             "spike": "slayer::spike_tile_kernel<12, 1, 12, 8>",
              "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
-             "spike_bwd": "slayer::spike_bwd_vec_kernel", "psp_corr": "slayer::fir_mfma_kernel<6, 20, true, false> (corr, matrix cores)"}
+             "spike_bwd": "slayer::spike_bwd_vec_kernel",
+             "psp_corr": "slayer::alpha_psp_kernel<false, 4> (corr with the alpha kernel as a recursion over time)"}
 
 
 def neuron_params():
@@ -182,7 +184,7 @@ def flip_rate(device, srm_t, ref_t, params):
     shape = (2, 16, 34, 34, 300)
     spikes = (rng.random(shape) < 0.02).astype(np.float32)
     gain = np.float32(9.0)           # puts about 2 % of the samples above threshold
-    a = slayerCuda.conv(torch.from_numpy(spikes).to(device), srm_t, 1.0) * float(gain)
+    a = slayerCuda.pspAlpha(torch.from_numpy(spikes).to(device), srm_t, params["tauSr"], 1.0, 1.0, True) * float(gain)
     s_gpu = slayerCuda.getSpikes(a.contiguous(), ref_t, params["theta"], 1.0).cpu().numpy()
     a_cpu = O.conv(spikes, srm_t.cpu().numpy(), 1.0, fused=False) * gain
     s_cpu, _ = O.get_spikes(a_cpu, ref_t.cpu().numpy(), params["theta"], 1.0)
@@ -191,14 +193,14 @@ def flip_rate(device, srm_t, ref_t, params):
 
 def layer_flip_rate(device, srm_t, ref_t, params):
     """Part of the CPU leg.  The same for a whole layer of the NMNIST CNN: spike(conv 2->16 5x5 (psp(x))) on
-    (4, 2, 34, 34, 300) input spikes, the GPU chain (event-driven psp, fp32 synapse kernel, spike kernel)
+    (4, 2, 34, 34, 300) input spikes, the GPU chain (psp as the layers run it, fp32 synapse kernel, spike kernel)
     against the CPU oracle chain (separately rounded psp, synapse accumulated in double, spike loop)."""
     from oracle import oracle as O
     from slayerpytorch_amd import slayerCuda, synapse
     rng = np.random.default_rng(1)
     x = (rng.random((4, 2, 34, 34, 300)) < 0.02).astype(np.float32)
     w = (rng.standard_normal((16, 2, 5, 5)) * 1.5).astype(np.float32)     # about 3 % of the output samples spike
-    a = slayerCuda.conv(torch.from_numpy(x).to(device), srm_t, 1.0)
+    a = slayerCuda.pspAlpha(torch.from_numpy(x).to(device), srm_t, params["tauSr"], 1.0, 1.0, True)
     u = synapse.conv(a, torch.from_numpy(w).to(device), 1, 1)
     s_gpu = slayerCuda.getSpikes(u, ref_t, params["theta"], 1.0).cpu().numpy()
     threads = O.lib().oracle_get_threads()
@@ -618,8 +620,12 @@ def main():
     ap.add_argument("--synapse-only", action="store_true",
                     help="only the per-layer synapse kernel rows (for profiler runs); prints those rows")
     ap.add_argument("--dense-conv", action="store_true",
-                    help="also launch the 77-tap psp conv once per warm-up step on a dense input (the gradient tensor), "
-                         "whose tiles run on the matrix cores (for profiler runs)")
+                    help="also launch, in every warm-up step, the kernels that sum over the 77 taps: conv on a dense input "
+                         "(the gradient tensor: matrix cores), conv on the spike tensor (event-driven) and corr on the "
+                         "gradient tensor (matrix cores) (for profiler runs)")
+    ap.add_argument("--tap-kernels-chain", action="store_true",
+                    help="psp and its gradient in the chain as sums over the 77 taps (slayerCuda.conv / corr) instead "
+                         "of the recursion that the layers use for their alpha kernel")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain copy of known size (a zero-delay shift of half the tensor: "
                          "%d bytes read, as many written) to scale hardware counters by" % (4 * 6 * 16 * 34 * 34 * 300))
@@ -663,6 +669,17 @@ def main():
 
     spikes, u0, grad = make_inputs(SHAPE, device)
     numel = spikes.numel()
+    # psp and its gradient as spikeLayer.psp runs them: the layer's SRM kernel is an alpha kernel, which it filters
+    # as a recursion over time (same results as the sum over the 77 taps to rounding); --tap-kernels-chain times
+    # the chain with the sums instead, and the full run reports both
+    if args.tap_kernels_chain:
+        psp_fwd = lambda x: slayerCuda.conv(x, srm_t, 1.0)
+        psp_bwd = lambda g: slayerCuda.corr(g, srm_t, 1.0)
+        KERNEL_OF["psp_conv"] = "slayer::fir_tiled_kernel<true, true, 16, false, 6> (conv as a sum over the taps; spike trains: event-driven path)"
+        KERNEL_OF["psp_corr"] = "slayer::fir_mfma_kernel<6, 20, true, false> (corr as a sum over the taps, matrix cores)"
+    else:
+        psp_fwd = lambda x: slayerCuda.pspAlpha(x, srm_t, params["tauSr"], 1.0, 1.0, True)
+        psp_bwd = lambda g: slayerCuda.pspAlpha(g, srm_t, params["tauSr"], 1.0, 1.0, False)
     names = list(AB)
     probe = 0 if args.chain_only else max(args.steps, 1)   # untimed steps with an event pair around every launch
     pool = [u0.clone() for _ in range(args.warmup + probe + args.steps)]   # spike() consumes one copy per step
@@ -681,18 +698,20 @@ def main():
                 ev[k][1].record()
             return out
 
-        run(0, lambda: slayerCuda.conv(spikes, srm_t, 1.0))
+        run(0, lambda: psp_fwd(spikes))
         s = run(1, lambda: slayerCuda.getSpikes(u, ref_t, theta, 1.0))
         run(2, lambda: slayerCuda.shift(s, 1.0, 1.0))
         gd = run(3, lambda: slayerCuda.shift(grad, 1.0, 1.0, sign=-1.0))
         gs = run(4, lambda: slayerCuda.spikeBackward(gd, u, theta, tau, scale))
-        run(5, lambda: slayerCuda.corr(gs, srm_t, 1.0))
+        run(5, lambda: psp_bwd(gs))
 
     for i in range(args.warmup):
         step(pool[i])
         if args.dense_conv:
             for _ in range(3):
                 slayerCuda.conv(grad, srm_t, 1.0)
+                slayerCuda.conv(spikes, srm_t, 1.0)
+                slayerCuda.corr(grad, srm_t, 1.0)
     if args.copy_calibration:
         slayerCuda.shift(grad[:6], 0.0, 1.0)
     torch.cuda.synchronize()
@@ -730,8 +749,8 @@ def main():
         "unit": "neuron-timesteps/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "NMNIST-CNN-shaped activation tensor (12,16,34,34,300): psp conv (77 taps) + spike "
-                               "(11-tap refractory) + shift fwd, shift + spike pdf + psp corr bwd",
+        "config": {"workload": "NMNIST-CNN-shaped activation tensor (12,16,34,34,300): psp conv (77-tap alpha kernel) + "
+                               "spike (11-tap refractory) + shift fwd, shift + spike pdf + psp corr bwd",
                    "elements": numel, "algorithmic_bytes_per_element": sum(AB.values())},
         "roofline": {"bound": "hbm", "kernel": KERNEL_OF[dominant], "op": dominant, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
@@ -740,9 +759,9 @@ def main():
         # the whole step (six launches and the gaps between them) against the HBM peak
         "chain_hbm_frac": chain_gbs / HBM_PEAK_GBS,
     }
-    # the 77-tap filters sit at the FP32 ridge: also as a fraction of the FP32 vector peak
+    # summed over their 77 taps the filters sit at the FP32 ridge: then also as a fraction of the FP32 peak
     result["roofline"]["fp32_frac_if_fir"] = (2.0 * SRM_TAPS * numel / (dominant_ms * 1e-3) / 1e12 / FP32_PEAK_TFLOPS
-                                              if dominant in ("psp_conv", "psp_corr") else None)
+                                              if args.tap_kernels_chain and dominant in ("psp_conv", "psp_corr") else None)
     if per_kernel_ms is not None:
         result["per_kernel_ms"] = per_kernel_ms
         result["per_kernel_hbm_frac"] = {n: AB[n] * numel / (per_kernel_ms[n] * 1e-3) / 1e9 / HBM_PEAK_GBS
@@ -755,10 +774,10 @@ def main():
         pool = [u0.clone() for _ in range(args.warmup + args.steps + 2)]
 
         def fused_step(u):
-            slayerCuda.conv(spikes, srm_t, 1.0)
+            psp_fwd(spikes)
             slayerCuda.getSpikesDelayed(u, ref_t, theta, 1.0, 1.0, 1.0)
             gs = slayerCuda.spikeBackwardDelayed(grad, u, theta, tau, scale, 1.0, 1.0)
-            slayerCuda.corr(gs, srm_t, 1.0)
+            psp_bwd(gs)
 
         for i in range(args.warmup):
             fused_step(pool[i])
@@ -779,6 +798,30 @@ def main():
             "value": numel / fused, "unit": "neuron-timesteps/s", "algorithmic_bytes_per_element": 40,
             "hbm_frac": 40 * numel / fused / 1e9 / HBM_PEAK_GBS, "identical_to_unfused_results": same}
         del pool
+        if not args.tap_kernels_chain:
+            # the chain's two filters as sums over the taps (what slayerCuda.conv / corr run for any filter)
+            K = max(args.steps, 5)
+            def timed_us(fn):
+                for _ in range(3):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(K):
+                    fn()
+                torch.cuda.synchronize()
+                return (time.perf_counter() - t0) / K * 1e6
+            gs = slayerCuda.spikeBackward(grad, u0, theta, tau, scale)
+            tc, tr = timed_us(lambda: slayerCuda.conv(spikes, srm_t, 1.0)), timed_us(lambda: slayerCuda.corr(gs, srm_t, 1.0))
+            ya, yt = psp_fwd(spikes), slayerCuda.conv(spikes, srm_t, 1.0)
+            za, zt = psp_bwd(gs), slayerCuda.corr(gs, srm_t, 1.0)
+            result["psp_as_sums_over_the_taps"] = {
+                "psp_conv_us": tc, "psp_corr_us": tr,
+                "psp_conv_hbm_frac": 8 * numel / (tc * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                "psp_corr_hbm_frac": 8 * numel / (tr * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                "ms_per_step_with_them": ms_per_step + (tc + tr) * 1e-3 - (per_kernel_ms["psp_conv"] + per_kernel_ms["psp_corr"]),
+                "recursion_vs_sums_max_rel_diff": {"conv": float((ya - yt).abs().max() / yt.abs().max()),
+                                                    "corr": float((za - zt).abs().max() / zt.abs().max())}}
+            del gs, ya, yt, za, zt
         result["measured_copy_ceiling"] = copy_ceiling(grad)
         result["other_rows"] = other_rows(device, cpu_leg=not args.no_cpu_baseline)
         if not args.no_cpu_baseline:

@@ -179,6 +179,22 @@ int slayer_psp_spike_f32(float *s, float *u, const float *a, const float *srm, c
                          float Ts, void *stream);
 
 /*
+ * PSP filtering with an alpha kernel, filt[k] = mult * (k Ts / tau) * exp(1 - k Ts / tau) for k < F - the SRM
+ * kernel that the reference's layers build (src/slayer.py:98-123) and hand to slayerCuda.conv / corr
+ * (src/slayer.py:878-899, src/cuda/slayerKernels.cu:41-75) - computed as a two-term recursion over time instead of
+ * an F-tap sum: about 10 operations per sample whatever F is.  causal != 0: the convolution of slayer_conv_f32;
+ * causal == 0: the correlation of slayer_corr_f32.  `filt` must hold exactly that kernel (it is what a tile with a
+ * non-finite sample, and every shape outside rows of whole 16-byte vectors of at most 512 samples, is filtered
+ * with, through the F-tap kernels); the caller states tau and mult.  The result agrees with the F-tap chain to
+ * rounding, relative to the sum of the magnitudes of the terms of the UNTRUNCATED response
+ * (sum_k |x[t -+ k]| |mult| (k Ts / tau) exp(1 - k Ts / tau) over all k): 1e-5 of that sum at most, about 1e-6
+ * measured.  Optional: a caller that does not know its filter to be an alpha kernel keeps calling
+ * slayer_conv_f32 / slayer_corr_f32.
+ */
+int slayer_psp_alpha_f32(float *out, const float *in, const float *filt, int64_t nNeurons, int64_t T, int64_t F,
+                         float tau, float mult, float Ts, int causal, void *stream);
+
+/*
  * Spike generation with the time shift that follows it fused into the store of the spikes.
  * Replaces the call pair slayerCuda.getSpikes (src/cuda/slayerKernels.cu:14-39) -> slayerCuda.shift
  * (src/cuda/slayerKernels.cu:77-134) that `delayShift(spike(u), d)` / `delay(spike(u))` make

@@ -1,0 +1,236 @@
+// PSP filtering with the alpha kernel that SLAYER's layers use, h[k] = mult * (k Ts / tau) * exp(1 - k Ts / tau)
+// for k < L (src/slayer.py:98-123), as a recursion instead of an L-tap sum:
+//
+//   conv: y[t] = Ts * sum_{k<L} h[k] x[t-k]          corr: y[t] = Ts * sum_{k<L} h[k] x[t+k]
+//
+// With a = exp(-Ts / tau) and g = mult * e * Ts / tau the kernel is h[k] = g k a^k.  The two running sums
+//
+//   p[t] = sum_{k>=0} a^k x[t-k]   = a p[t-1] + x[t]
+//   q[t] = sum_{k>=0} k a^k x[t-k] = a (q[t-1] + p[t-1])
+//
+// give the untruncated response g q[t]; the taps from L on amount to a^L (L p[t-L] + q[t-L]) = a^L r[t-L] with
+// r = L p + q, so
+//
+//   y[t] = Ts g (q[t] - a^L r[t-L]).
+//
+// About 10 floating-point operations per sample instead of 2 L: at 77 taps the L-tap sum sits on the FP32 ridge
+// of the machine (matrix-pipe bound at 0.47 of HBM peak); the recursion is a memory stream.
+//
+// A wavefront owns 4 consecutive rows of whole 16-byte vectors, in LDS as they lie in memory.  Sixteen lanes serve
+// a row, each a contiguous segment of its time axis: pass 1 runs the recursion over the segment from zero state,
+// the segments' end states are chained through the row's lanes (state after n more samples: p' = a^n p,
+// q' = a^n (q + n p), plus the segment's own sums), pass 2 runs the recursion again from the true state and
+// leaves q[t] (over x[t]) and r[t] in LDS; then all lanes combine q[t] and r[t -+ L] vector by vector on the way
+// out.  The correlation is the same on the reversed time axis.  Every output is a sum of the same products as
+// the L-tap chain (with a^k taken as a product of a's instead of one rounded tap), added in another order, and
+// the difference of the two running sums: it agrees with the chain to rounding relative to the sum of the
+// magnitudes of the UNTRUNCATED response's terms, sum_k |x[t-k]| g k a^k - a bound that also holds where the
+// truncated sum is small or zero (behind a large sample that has left the window).  A tile that holds a
+// non-finite sample is filtered with the L-tap chain from the given filter, so that infinities and NaNs reach
+// exactly the samples the reference lets them reach.
+#include "common.h"
+
+namespace slayer {
+
+// Rows per wavefront.  4 rows of T = 300 are 4800 bytes, whole 64-byte blocks; their two copies in LDS take 9.6 KB, so
+// 16 wavefronts fit a compute unit (8 rows per wavefront, 8 wavefronts: 131 us instead of 96 us on the benchmark tensor).
+constexpr int kAlphaRows = 4;
+constexpr int kAlphaMaxT = 512;   // two copies of 4 rows in LDS: 16 KiB at most
+
+struct AlphaArgs {
+    float *out;
+    const float *in, *filt;
+    int64_t rows;
+    int T, L, P;        // P: floats per row in LDS, P / 4 odd
+    float a;            // exp(-Ts / tau)
+    float aSeg[2];      // a^n for segments of perRow / parts and perRow / parts + 1 vectors (n = 4 times that)
+    float aL;           // a^L
+    float scale;        // Ts * mult * e * Ts / tau
+    float Ts;
+};
+
+template <bool CAUSAL, int R>
+__global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
+{
+    constexpr int kParts = kWave / R;
+    constexpr int NB = (R * (kAlphaMaxT / 4) + kWave - 1) / kWave;  // vectors per lane of a tile, at most
+    extern __shared__ __align__(16) float lds[];
+    const int T = p.T, P = p.P, L = p.L;
+    float *Q = lds;            // [R][P]: x, then q
+    float *Rr = lds + R * P;   // [R][P]: r
+
+    const int lane = threadIdx.x;
+    const int perRow = T >> 2;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
+    const int nRows = static_cast<int>(min(static_cast<int64_t>(R), p.rows - row0));
+    const int nVec = nRows * perRow;
+
+    // ---- the tile, one contiguous run of vectors (rows behind the last one arrive as zeros)
+    bool bad = false;
+    {
+        const BufferRsrc bufIn = make_buffer(p.in + row0 * static_cast<int64_t>(T), nVec * 16);
+        float4 x[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            if (b * kWave < R * perRow) x[b] = buffer_load4(bufIn, (lane + b * kWave) * 16, 0);
+        RowCol rc;
+        rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
+        const int dr = kWave / perRow, dc = kWave % perRow;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            if (b * kWave < R * perRow) {
+                if (lane + b * kWave < R * perRow) {
+                    *reinterpret_cast<float4 *>(Q + rc.r * P + (rc.c << 2)) = x[b];
+                    // infinite or NaN (or four samples that add up to more than fp32 holds, which only costs time)
+                    bad |= ((x[b].x + x[b].y) + (x[b].z + x[b].w)) * 0.0f != 0.0f;
+                }
+                rc.advance(dr, dc, perRow);
+            }
+        }
+    }
+    const bool chains = __builtin_amdgcn_ballot_w64(bad) != 0;
+    wave_sync();
+
+    if (chains) {
+        // a non-finite sample: the tile's outputs as the sequential chains over the valid taps, from memory
+        for (int e = lane; e < nRows * T; e += kWave) {
+            const int r = e / T, t = e - r * T;
+            const float *x = p.in + (row0 + r) * static_cast<int64_t>(T);
+            const int taps = CAUSAL ? min(t + 1, L) : min(T - t, L);
+            float acc = 0.0f;
+            for (int k = 0; k < taps; ++k) acc = __builtin_fmaf(CAUSAL ? x[t - k] : x[t + k], p.filt[k], acc);
+            p.out[(row0 + r) * static_cast<int64_t>(T) + t] = acc * p.Ts;
+        }
+        return;
+    }
+
+    // ---- lane (row r, part j): the logical vectors [v0, v1) of the row; logical time runs forward for the
+    //      convolution and backward for the correlation (logical vector V = memory vector perRow - 1 - V, mirrored)
+    const int r = lane / kParts, j = lane - r * kParts;
+    const int v0 = (j * perRow) / kParts, v1 = ((j + 1) * perRow) / kParts;
+    const float a = p.a;
+    float *q4 = Q + r * P, *r4 = Rr + r * P;
+    auto vector_at = [&](int V) { return (CAUSAL ? V : perRow - 1 - V) << 2; };
+    auto step = [&](float &pp, float &qq, float x) {
+        qq = a * (qq + pp);                 // q[t] = a (q[t-1] + p[t-1])
+        pp = __builtin_fmaf(a, pp, x);      // p[t] = a p[t-1] + x[t]
+    };
+    float sp = 0.0f, sq = 0.0f;   // the segment's own sums (its end state from a zero start)
+#pragma unroll 2
+    for (int V = v0; V < v1; ++V) {
+        const float4 x = *reinterpret_cast<const float4 *>(q4 + vector_at(V));
+        step(sp, sq, CAUSAL ? x.x : x.w);
+        step(sp, sq, CAUSAL ? x.y : x.z);
+        step(sp, sq, CAUSAL ? x.z : x.y);
+        step(sp, sq, CAUSAL ? x.w : x.x);
+    }
+    // the state in front of every segment: the end state of the one before it, handed down the row's lanes
+    const int n = (v1 - v0) << 2;
+    const float fn = static_cast<float>(n);
+    const float aN = p.aSeg[(v1 - v0) - perRow / kParts];
+    float cp = 0.0f, cq = 0.0f;
+#pragma unroll
+    for (int k = 0; k + 1 < kParts; ++k) {
+        const float ep = __builtin_fmaf(aN, cp, sp), eq = __builtin_fmaf(aN, __builtin_fmaf(fn, cp, cq), sq);
+        // row_shr:1 - every lane reads the lane below it (within the row's lanes for j >= 1)
+        const float np = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ep), 0x111, 0xf, 0xf, false));
+        const float nq = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, eq), 0x111, 0xf, 0xf, false));
+        if (j == k + 1) {
+            cp = np;
+            cq = nq;
+        }
+    }
+    // pass 2: q over x, r next to it
+    {
+        const float fL = static_cast<float>(L);
+        float pp = cp, qq = cq;
+#pragma unroll 2
+        for (int V = v0; V < v1; ++V) {
+            const int at = vector_at(V);
+            const float4 x = *reinterpret_cast<const float4 *>(q4 + at);
+            float qv[4], rv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float xe = CAUSAL ? (e == 0 ? x.x : e == 1 ? x.y : e == 2 ? x.z : x.w)
+                                        : (e == 0 ? x.w : e == 1 ? x.z : e == 2 ? x.y : x.x);
+                step(pp, qq, xe);
+                qv[e] = qq;
+                rv[e] = __builtin_fmaf(fL, pp, qq);
+            }
+            *reinterpret_cast<float4 *>(q4 + at) = CAUSAL ? make_float4(qv[0], qv[1], qv[2], qv[3]) : make_float4(qv[3], qv[2], qv[1], qv[0]);
+            *reinterpret_cast<float4 *>(r4 + at) = CAUSAL ? make_float4(rv[0], rv[1], rv[2], rv[3]) : make_float4(rv[3], rv[2], rv[1], rv[0]);
+        }
+    }
+    wave_sync();
+
+    // ---- out: y[t] = scale (q[t] - a^L r[t -+ L]); the four r of a vector lie in two aligned vectors, L & 3
+    //      samples off (the same for every lane)
+    {
+        const BufferRsrc bufOut = make_buffer(p.out + row0 * static_cast<int64_t>(T), nVec * 16);
+        const float aL = p.aL, scale = p.scale;
+        const int shift = CAUSAL ? -L : L;           // r[t + shift]
+        const int lo = shift >> 2, off = shift & 3;  // r[4 c + e + shift] = element (e + off) of vectors c + lo, c + lo + 1
+        RowCol rc;
+        rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
+        const int dr = kWave / perRow, dc = kWave % perRow;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            if (b * kWave < R * perRow) {
+                const int row = min(rc.r, R - 1);  // (lanes behind the tile: their stores are dropped)
+                const int ca = rc.c + lo, cb = ca + 1;
+                const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                const float4 qv = *reinterpret_cast<const float4 *>(Q + row * P + (rc.c << 2));
+                const float4 ra = (ca >= 0 && ca < perRow) ? *reinterpret_cast<const float4 *>(Rr + row * P + (ca << 2)) : zero;
+                const float4 rb = (off != 0 && cb >= 0 && cb < perRow) ? *reinterpret_cast<const float4 *>(Rr + row * P + (cb << 2)) : zero;
+                float4 rs;
+                if (off == 0) rs = ra;
+                else if (off == 1) rs = make_float4(ra.y, ra.z, ra.w, rb.x);
+                else if (off == 2) rs = make_float4(ra.z, ra.w, rb.x, rb.y);
+                else rs = make_float4(ra.w, rb.x, rb.y, rb.z);
+                const float4 y = make_float4(scale * __builtin_fmaf(-aL, rs.x, qv.x), scale * __builtin_fmaf(-aL, rs.y, qv.y),
+                                             scale * __builtin_fmaf(-aL, rs.z, qv.z), scale * __builtin_fmaf(-aL, rs.w, qv.w));
+                buffer_store4(bufOut, (lane + b * kWave) * 16, 0, y);
+                rc.advance(dr, dc, perRow);
+            }
+        }
+    }
+}
+
+}  // namespace slayer
+
+extern "C" int slayer_psp_alpha_f32(float *out, const float *in, const float *filt, int64_t nNeurons, int64_t T, int64_t F,
+                                    float tau, float mult, float Ts, int causal, void *stream)
+{
+    using namespace slayer;
+    if (nNeurons < 0 || T < 0 || F < 1 || !(tau > 0.0f) || !(Ts > 0.0f)) return SLAYER_EINVAL;
+    if (nNeurons == 0 || T == 0) return SLAYER_OK;
+    if (!out || !in || !filt) return SLAYER_EINVAL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    constexpr int R = kAlphaRows, parts = kWave / R;
+    const int64_t tiles = ceil_div(nNeurons, R);
+    const bool served = !generic_forced() && T % 4 == 0 && T <= kAlphaMaxT && aligned16(out) && aligned16(in) &&
+                        tiles < (1LL << 31) && F < (1 << 20);
+    if (!served)   // the L-tap sum with the given filter
+        return causal ? slayer_conv_f32(out, in, filt, nNeurons, T, F, Ts, stream)
+                      : slayer_corr_f32(out, in, filt, nNeurons, T, F, Ts, stream);
+    AlphaArgs a{};
+    a.out = out; a.in = in; a.filt = filt;
+    a.rows = nNeurons;
+    a.T = static_cast<int>(T);
+    a.L = static_cast<int>(F);
+    a.P = static_cast<int>(T) + (((T / 4) % 2 == 0) ? 4 : 0);   // P / 4 odd: the 8 rows start in different banks
+    const double ratio = static_cast<double>(Ts) / static_cast<double>(tau);
+    const double av = exp(-ratio);
+    a.a = static_cast<float>(av);
+    // (powers of the rounded a, which is what the recursion multiplies by)
+    a.aSeg[0] = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(4 * ((T / 4) / parts))));
+    a.aSeg[1] = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(4 * ((T / 4) / parts + 1))));
+    a.aL = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(F)));
+    a.scale = static_cast<float>(static_cast<double>(Ts) * static_cast<double>(mult) * exp(1.0) * ratio);
+    a.Ts = Ts;
+    const size_t lds = static_cast<size_t>(2) * R * a.P * sizeof(float);
+    const dim3 grid(static_cast<unsigned>(tiles));
+    if (causal) hipLaunchKernelGGL((alpha_psp_kernel<true, R>), grid, dim3(kWave), lds, st, a);
+    else hipLaunchKernelGGL((alpha_psp_kernel<false, R>), grid, dim3(kWave), lds, st, a);
+    return launch_status();
+}

@@ -29,6 +29,12 @@ from . import slayerCuda
 from . import synapse
 
 
+# spikeLayer.psp filters with the alpha kernel as a recursion over time when the kernel has more taps than this
+# (shorter kernels are memory streams as sums already); PSP_RECURSION = False keeps the sums everywhere.
+PSP_RECURSION = True
+PSP_RECURSION_MIN_TAPS = 16
+
+
 def alphaKernel(tau, Ts, tSample, mult=1.0, EPSILON=0.01):
     """Samples ``mult * t/tau * exp(1 - t/tau)`` at t = 0, Ts, 2Ts, ... < tSample and stops
     (exclusively) at the first sample past the peak whose magnitude is below ``EPSILON``
@@ -72,8 +78,32 @@ class spikeLayer(nn.Module):
         return alphaKernel(tau, self.simulation["Ts"], self.simulation["tSample"], mult, EPSILON)
 
     def psp(self, spike):
-        """PSP filtering of a spike tensor (same shape out)."""
-        return _pspFunction.apply(spike, self.srmKernel, self.simulation["Ts"])
+        """PSP filtering of a spike tensor (same shape out).  While ``srmKernel`` is the alpha kernel
+        that ``calculateSrmKernel`` built (checked once per kernel tensor, against the values
+        computed on the host) and has more than ``PSP_RECURSION_MIN_TAPS`` taps, filter and
+        gradient run as a recursion over time (``slayerCuda.pspAlpha``), which agrees with the
+        sum over the taps to rounding; a kernel that was replaced or edited takes the sums."""
+        alpha = self._srmKernelIsAlpha()
+        return _pspFunction.apply(spike, self.srmKernel, self.simulation["Ts"], alpha)
+
+    def _srmKernelIsAlpha(self):
+        """(tau, mult) when ``srmKernel`` still holds ``alphaKernel(tauSr, ...)`` and the recursion
+        is switched on, else None.  Comparing costs a copy to the host, so the verdict is kept per
+        tensor object and version."""
+        kernel = self.srmKernel
+        if not PSP_RECURSION or not kernel.is_cuda or kernel.numel() <= PSP_RECURSION_MIN_TAPS:
+            return None
+        stamp = (id(kernel), kernel.data_ptr(), kernel._version)
+        if getattr(self, "_srmAlphaStamp", None) != stamp:
+            tau = self.neuron.get("tauSr") if hasattr(self.neuron, "get") else None   # (the Loihi layer has none)
+            same = False
+            if tau is not None and float(tau) > 0:
+                expected = torch.FloatTensor(self._calculateAlphaKernel(tau))
+                same = kernel.shape == expected.shape and kernel.dtype == expected.dtype and \
+                    bool(torch.equal(kernel.detach().cpu(), expected))
+            self._srmAlphaStamp = stamp
+            self._srmAlpha = (float(tau), 1.0) if same else None
+        return self._srmAlpha
 
     def spike(self, membranePotential):
         """Spike function with refractory response.  A contiguous ``membranePotential`` is
@@ -379,20 +409,29 @@ class _pspSpikeFunction(torch.autograd.Function):
 
 class _pspFunction(torch.autograd.Function):
     """Forward: causal conv with the SRM kernel; backward: correlation with the same kernel;
-    the kernel itself gets no gradient (src/slayer.py:875-899)."""
+    the kernel itself gets no gradient (src/slayer.py:875-899).  ``alpha`` = (tau, mult) when the
+    kernel is known to be that alpha kernel: both then run as recursions over time."""
 
     @staticmethod
-    def forward(ctx, spike, filter, Ts):
-        psp = slayerCuda.conv(spike.contiguous(), filter, Ts)
+    def forward(ctx, spike, filter, Ts, alpha=None):
+        if alpha is None:
+            psp = slayerCuda.conv(spike.contiguous(), filter, Ts)
+        else:
+            psp = slayerCuda.pspAlpha(spike.contiguous(), filter, alpha[0], alpha[1], Ts, causal=True)
         ctx.save_for_backward(filter)
         ctx.Ts = float(Ts)
+        ctx.alpha = alpha
         return psp
 
     @staticmethod
     def backward(ctx, gradOutput):
         (filter,) = ctx.saved_tensors
-        gradInput = slayerCuda.corr(gradOutput.contiguous(), filter, ctx.Ts)
-        return gradInput, None, None
+        if ctx.alpha is None:
+            gradInput = slayerCuda.corr(gradOutput.contiguous(), filter, ctx.Ts)
+        else:
+            gradInput = slayerCuda.pspAlpha(gradOutput.contiguous(), filter, ctx.alpha[0], ctx.alpha[1], ctx.Ts,
+                                            causal=False)
+        return gradInput, None, None, None
 
 
 class _delayLayer(nn.Module):

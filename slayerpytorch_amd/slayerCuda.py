@@ -31,7 +31,7 @@ import torch
 from . import _lib
 
 __all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "spikeBackwardCorr", "pspSpike", "delayGrad",
-           "getSpikesDelayed", "spikeBackwardDelayed", "spikeLoss"]
+           "getSpikesDelayed", "spikeBackwardDelayed", "spikeLoss", "pspAlpha"]
 
 
 def _check_input(x, name):
@@ -148,6 +148,27 @@ def conv(input, filter, Ts):
 def corr(input, filter, Ts):
     """Anti-causal correlation in time (adjoint of :func:`conv`), times ``Ts``."""
     return _fir("slayer_corr_f32", "corr", input, filter, Ts)
+
+
+def pspAlpha(input, filter, tau, mult, Ts, causal=True):
+    """``conv(input, filter, Ts)`` (``causal``) or ``corr(input, filter, Ts)`` for a ``filter`` that holds the
+    alpha kernel ``mult * t/tau * exp(1 - t/tau)`` sampled at ``t = 0, Ts, 2 Ts, ...`` (what
+    ``spikeLayer.calculateSrmKernel`` builds), computed as a recursion over time instead of a sum over
+    the taps.  Agrees with ``conv`` / ``corr`` to rounding; see ``slayer_psp_alpha_f32`` in the header
+    for the bound.  The caller vouches for ``filter`` being that kernel."""
+    _check_input(input, "input")
+    _check_input(filter, "filter")
+    _check_device(input, filter, "input", "filter")
+    tau, mult, Ts = _scalar(tau, "tau"), _scalar(mult, "mult"), _scalar(Ts, "Ts")
+    if filter.numel() < 1:
+        raise RuntimeError("pspAlpha needs a filter of at least one tap")
+    lib = _lib.load()
+    output = torch.empty_like(input)
+    n, T = _rows(input)
+    with _on_device_of(input) as stream:
+        _lib.check(lib.slayer_psp_alpha_f32(_ptr(output), _ptr(input), _ptr(filter), n, T, filter.numel(), tau, mult,
+                                            Ts, 1 if causal else 0, stream), "slayer_psp_alpha_f32")
+    return output
 
 
 def shift(input, shiftLUT, Ts=1.0, sign=1.0):

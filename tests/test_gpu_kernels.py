@@ -246,6 +246,95 @@ def test_conv_density_switch_is_per_tile(T, Fl):
             assert np.array_equal(bits(got[:3]), bits(want[:3]))
 
 
+# ------------------------------------------------------------------------------------------ alpha kernel as a recursion
+def alpha_full(tau, mult, Ts, n):
+    k = np.arange(n, dtype=np.float64)
+    return mult * (k * Ts / tau) * np.exp(1 - k * Ts / tau)
+
+
+def close_to_alpha_sum(got, x, f, tau, mult, Ts, causal):
+    """|got - exact| <= 1e-5 * Ts * sum_k |x| |h_k| element by element, h the UNTRUNCATED alpha response (the bound the
+    recursion is held to; it exceeds the truncated sum's by the terms behind the window, under 1 % for gaussian or
+    spike input); exact = the sum over the taps of `f` in double precision."""
+    T = x.shape[-1]
+    flat, out = np.asarray(x, np.float64).reshape(-1, T), np.asarray(got, np.float64).reshape(-1, T)
+    h = np.abs(alpha_full(tau, mult, Ts, T + 1))
+    f64 = np.asarray(f, np.float64)
+    for r in range(flat.shape[0]):
+        xr = flat[r] if causal else flat[r][::-1]
+        yr = out[r] if causal else out[r][::-1]
+        exact = np.convolve(xr, f64)[:T] * Ts
+        bound = np.convolve(np.abs(xr), h)[:T] * Ts
+        if np.any(np.abs(yr - exact) > 1e-5 * bound + 1e-37):
+            return False
+    return True
+
+
+@pytest.mark.parametrize("shape,tau,mult,Ts", [((2, 6, 5, 3, 300), 10.0, 1.0, 1.0), ((1, 3, 1, 7, 64), 10.0, 1.0, 1.0),
+                                               ((1, 5, 1, 1, 16), 10.0, 2.0, 1.0), ((1, 2, 1, 1, 4), 1.0, -20.0, 1.0),
+                                               ((3, 9, 1, 1, 512), 20.0, 1.0, 0.5), ((1, 13, 1, 1, 352), 4.0, 1.0, 1.0),
+                                               ((1, 4, 1, 1, 28), 2.0, 1.0, 1.0), ((1, 1, 1, 1, 300), 10.0, -3.0, 2.0)])
+@pytest.mark.parametrize("kind", ["dense", "spikes"])
+def test_psp_alpha_is_the_sum_over_the_taps_to_rounding(shape, tau, mult, Ts, kind):
+    rng = np.random.default_rng(shape[-1] + int(tau))
+    f = np.array(alphaKernel(tau, Ts, 5000, mult), dtype=np.float32)
+    x = rng.standard_normal(shape).astype(np.float32) if kind == "dense" else (rng.random(shape) < 0.04).astype(np.float32)
+    for causal, op in ((True, "conv"), (False, "corr")):
+        got = host(slayerCuda.pspAlpha(dev(x), dev(f), tau, mult, Ts, causal))
+        want = getattr(O, op)(x, f, Ts, fused=True)
+        assert rel_err(got, want) <= REL_TOL, op
+        assert close_to_alpha_sum(got, x, f, tau, mult, Ts, causal), op
+        # ... and the adjoint identity between the two directions
+    a = rng.standard_normal(shape).astype(np.float32)
+    ya = host(slayerCuda.pspAlpha(dev(x), dev(f), tau, mult, Ts, True)).astype(np.float64)
+    za = host(slayerCuda.pspAlpha(dev(a), dev(f), tau, mult, Ts, False)).astype(np.float64)
+    lhs, rhs = float((ya * a).sum()), float((x.astype(np.float64) * za).sum())
+    assert abs(lhs - rhs) <= 1e-5 * float((np.abs(ya) * np.abs(a)).sum() + 1e-30)
+
+
+def test_psp_alpha_keeps_the_reach_of_a_large_sample():
+    # a sample of 1e6 leaves the window after F steps: the sum over the taps is exactly zero there, the recursion's
+    # difference of two running sums is zero to rounding of the untruncated terms
+    tau, Ts = 10.0, 1.0
+    f = np.array(alphaKernel(tau, Ts, 300), dtype=np.float32)
+    x = np.zeros((1, 4, 1, 1, 300), np.float32)
+    x[0, 1, 0, 0, 40] = 1e6
+    x[0, 2, 0, 0, 200] = -1e6
+    for causal, op in ((True, "conv"), (False, "corr")):
+        got = host(slayerCuda.pspAlpha(dev(x), dev(f), tau, 1.0, Ts, causal))
+        want = getattr(O, op)(x, f, Ts, fused=True)
+        assert close_to_alpha_sum(got, x, f, tau, 1.0, Ts, causal)
+        assert rel_err(got, want) <= 1e-6
+        assert np.all(got[0, 0] == 0) and np.all(got[0, 3] == 0)
+
+
+@pytest.mark.parametrize("kind", ["infinity", "nan"])
+def test_psp_alpha_filters_a_tile_with_a_non_finite_sample_with_the_taps(kind):
+    # (a recursion would carry an infinity to the end of the row; the reference lets it reach F samples)
+    rng = np.random.default_rng(9)
+    tau, Ts = 10.0, 1.0
+    f = np.array(alphaKernel(tau, Ts, 300), dtype=np.float32)
+    x = rng.standard_normal((1, 12, 1, 1, 300)).astype(np.float32)
+    x[0, 5, 0, 0, 100] = np.inf if kind == "infinity" else np.nan
+    for causal, op in ((True, "conv"), (False, "corr")):
+        got = host(slayerCuda.pspAlpha(dev(x), dev(f), tau, 1.0, Ts, causal)).reshape(12, 300)
+        want = getattr(O, op)(x, f, Ts, fused=True).reshape(12, 300)
+        assert np.array_equal(bits(got[4:8]), bits(want[4:8]))      # the tile of 4 rows with the sample: the chain
+        assert np.all(np.isfinite(got[:4])) and np.all(np.isfinite(got[8:]))
+        assert rel_err(np.delete(got, slice(4, 8), 0), np.delete(want, slice(4, 8), 0)) <= REL_TOL
+
+
+@pytest.mark.parametrize("shape", [(1, 3, 1, 1, 350), (1, 2, 1, 1, 1000), (2, 2, 1, 1, 7)])
+def test_psp_alpha_outside_its_shapes_is_conv_and_corr(impl, shape):
+    # rows that are not whole vectors, rows longer than 512 samples, and forced generic kernels: the taps
+    rng = np.random.default_rng(shape[-1])
+    tau, Ts = 10.0, 1.0
+    f = np.array(alphaKernel(tau, Ts, 300), dtype=np.float32)
+    x = (rng.random(shape) < 0.1).astype(np.float32)
+    assert torch.equal(slayerCuda.pspAlpha(dev(x), dev(f), tau, 1.0, Ts, True), slayerCuda.conv(dev(x), dev(f), Ts))
+    assert torch.equal(slayerCuda.pspAlpha(dev(x), dev(f), tau, 1.0, Ts, False), slayerCuda.corr(dev(x), dev(f), Ts))
+
+
 def test_gated_corr_on_the_matrix_cores_keeps_non_finite_samples_in_place():
     # an infinite gradient sample reaches exactly the outputs within Fl taps before it, as in the chain; so does an
     # infinite membrane potential (gate 0 times a finite sample is 0, times an infinite one NaN)

@@ -43,7 +43,10 @@ def host(t):
 
 
 # ------------------------------------------------------------------------------------------ psp
-def test_psp_forward_backward_matches_oracle():
+@pytest.mark.parametrize("recursion", [True, False])
+def test_psp_forward_backward_matches_oracle(recursion, monkeypatch):
+    import slayerpytorch_amd.slayer as slayer_module
+    monkeypatch.setattr(slayer_module, "PSP_RECURSION", recursion)
     layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 300}).to(DEV)
     rng = np.random.default_rng(0)
     x = (rng.random((3, 4, 5, 5, 300)) < 0.05).astype(np.float32)
@@ -52,10 +55,31 @@ def test_psp_forward_backward_matches_oracle():
     y = layer.psp(xt)
     y.backward(dev(g))
     srm = host(layer.srmKernel)
-    assert np.array_equal(host(y), O.conv(x, srm, 1.0))
+    if recursion:
+        # the alpha kernel as a recursion over time: the sum over the taps to rounding
+        assert layer._srmKernelIsAlpha() == (10.0, 1.0)
+        assert rel_err(host(y), O.conv(x, srm, 1.0)) <= REL_TOL
+    else:
+        assert layer._srmKernelIsAlpha() is None
+        assert np.array_equal(host(y), O.conv(x, srm, 1.0))
     # (the correlation of these rows runs on the matrix cores: another summation order than the chain)
     assert rel_err(host(xt.grad), O.corr(g, srm, 1.0)) <= REL_TOL
     assert layer.srmKernel.grad is None
+
+
+def test_psp_takes_the_sums_for_a_kernel_that_is_not_the_layers_alpha_kernel():
+    # an edited or replaced srmKernel is filtered as it is (the recursion only stands in for the kernel that
+    # calculateSrmKernel built): the chain's bits on spike trains
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 300}).to(DEV)
+    rng = np.random.default_rng(1)
+    x = (rng.random((2, 3, 1, 1, 300)) < 0.05).astype(np.float32)
+    assert layer._srmKernelIsAlpha() is not None
+    layer.srmKernel[3] *= 1.5                      # in place: the tensor's version changes
+    assert layer._srmKernelIsAlpha() is None
+    assert np.array_equal(host(layer.psp(dev(x))), O.conv(x, host(layer.srmKernel), 1.0))
+    layer.srmKernel = torch.ones(40, device=DEV)   # replaced
+    assert layer._srmKernelIsAlpha() is None
+    assert np.array_equal(host(layer.psp(dev(x))), O.conv(x, np.ones(40, np.float32), 1.0))
 
 
 def test_psp_equals_padded_conv3d_layer():
@@ -74,7 +98,7 @@ def test_psp_accepts_non_contiguous_input_and_tensor_Ts():
     x = torch.randn((2, 3, 4, 100, 5), device=DEV).permute(0, 1, 2, 4, 3)       # time last, not contiguous
     assert not x.is_contiguous()
     want = O.conv(host(x.contiguous()), host(layer.srmKernel), 0.5)
-    assert np.array_equal(host(layer.psp(x)), want)
+    assert rel_err(host(layer.psp(x)), want) <= REL_TOL      # (the layer filters its alpha kernel as a recursion)
     # the extension accepts a 0-dim tensor wherever the reference passed one for Ts
     got = slayerCuda.conv(x.contiguous(), layer.srmKernel, torch.tensor(0.5, device=DEV))
     assert np.array_equal(host(got), want)
