@@ -569,6 +569,10 @@ def other_rows(device, cpu_leg=False):
                    shape, moved=12))
     out.append(row("psp77_then_spike_two_kernels", 20, a.numel(),
                    timed(lambda: slayerCuda.getSpikes(slayerCuda.conv(a, srm77, 1.0), ref11, 10.0, 1.0), K), shape))
+    # ... as the layers run it for their alpha kernel: the recursion over time, then the spike kernel
+    out.append(row("psp77_as_recursion_then_spike_two_kernels", 20, a.numel(),
+                   timed(lambda: slayerCuda.getSpikes(slayerCuda.pspAlpha(a, srm77, 10.0, 1.0, 1.0, True), ref11, 10.0, 1.0), K), shape))
+    out.append(row("psp77_as_recursion_dense_input", 8, a.numel(), timed(lambda: slayerCuda.pspAlpha(a, srm77, 10.0, 1.0, 1.0, True), K), shape))
     gs = torch.randn(shape, generator=g).to(device)
     out.append(row("spike_pdf_then_corr77_fused", 20, a.numel(),
                    timed(lambda: slayerCuda.spikeBackwardCorr(gs, a, srm77, 10.0, 10.0, 1.0, 1.0), K), shape, moved=12))

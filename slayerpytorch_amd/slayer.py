@@ -128,9 +128,10 @@ class spikeLayer(nn.Module):
 
     def pspSpike(self, input):
         """``spike(psp(input))`` - the layer ordering of the reference's MLP example
-        (example/02_NMNIST_MLP/nmnistMLP.py:59-60) - as one forward and one backward kernel
+        (example/02_NMNIST_MLP/nmnistMLP.py:59-60) - as one Function with one backward kernel
         (extension; same values as the two calls)."""
-        return _pspSpikeFunction.apply(input, self.srmKernel, self.refKernel, self.neuron, self.simulation["Ts"])
+        return _pspSpikeFunction.apply(input, self.srmKernel, self.refKernel, self.neuron, self.simulation["Ts"],
+                                       self._srmKernelIsAlpha())
 
     def delayShift(self, input, delay, Ts=1):
         """Delays ``input`` in time by ``delay`` (number, one-element tensor, or one value per
@@ -389,9 +390,15 @@ class _pspSpikeFunction(torch.autograd.Function):
     followed by the correlation with the SRM kernel, also in one kernel."""
 
     @staticmethod
-    def forward(ctx, input, srmKernel, refractoryResponse, neuron, Ts):
-        spikes, membranePotential = slayerCuda.pspSpike(input.contiguous(), srmKernel, refractoryResponse,
-                                                        neuron["theta"], Ts)
+    def forward(ctx, input, srmKernel, refractoryResponse, neuron, Ts, alpha=None):
+        if alpha is None:
+            spikes, membranePotential = slayerCuda.pspSpike(input.contiguous(), srmKernel, refractoryResponse,
+                                                            neuron["theta"], Ts)
+        else:
+            # the alpha kernel as a recursion over time, then the spike kernel: two memory streams, which together
+            # take less time than the one kernel that sums over the taps (and the very values of psp() + spike())
+            membranePotential = slayerCuda.pspAlpha(input.contiguous(), srmKernel, alpha[0], alpha[1], Ts, causal=True)
+            spikes = slayerCuda.getSpikes(membranePotential, refractoryResponse, neuron["theta"], Ts)
         ctx.save_for_backward(membranePotential, srmKernel)
         ctx.theta = float(neuron["theta"])
         ctx.pdfTimeConstant = float(neuron["tauRho"] * neuron["theta"])
@@ -404,7 +411,7 @@ class _pspSpikeFunction(torch.autograd.Function):
         membranePotential, srmKernel = ctx.saved_tensors
         gradInput = slayerCuda.spikeBackwardCorr(gradOutput.contiguous(), membranePotential, srmKernel, ctx.theta,
                                                  ctx.pdfTimeConstant, ctx.pdfScale, ctx.Ts)
-        return gradInput, None, None, None, None
+        return gradInput, None, None, None, None, None
 
 
 class _pspFunction(torch.autograd.Function):
