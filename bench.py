@@ -723,7 +723,7 @@ def main():
     # Per-kernel pass (untimed): every launch bracketed.  The event records themselves cost a few
     # microseconds per launch, so the timed region below brackets the dominant kernel only.
     per_kernel_ms = None
-    dominant = "psp_corr"
+    dominant = "spike"
     if probe:
         evs = [{k: event_pair() for k in range(len(names))} for _ in range(probe)]
         for i in range(probe):

@@ -18,8 +18,8 @@
 //
 // A wavefront owns 4 consecutive rows of whole 16-byte vectors, in LDS as they lie in memory.  Sixteen lanes serve
 // a row, each a contiguous segment of its time axis: pass 1 runs the recursion over the segment from zero state,
-// the segments' end states are chained through the row's lanes (state after n more samples: p' = a^n p,
-// q' = a^n (q + n p), plus the segment's own sums), pass 2 runs the recursion again from the true state and
+// a scan over the row's lanes composes the segments (state after n more samples: p' = a^n p,
+// q' = a^n (q + n p), plus the run's own sums) into the state in front of each, pass 2 runs the recursion again from the true state and
 // leaves q[t] (over x[t]) and r[t] in LDS; then all lanes combine q[t] and r[t -+ L] vector by vector on the way
 // out.  The correlation is the same on the reversed time axis.  Every output is a sum of the same products as
 // the L-tap chain (with a^k taken as a product of a's instead of one rounded tap), added in another order, and
@@ -29,6 +29,7 @@
 // non-finite sample is filtered with the L-tap chain from the given filter, so that infinities and NaNs reach
 // exactly the samples the reference lets them reach.
 #include "common.h"
+#include <type_traits>
 
 namespace slayer {
 
@@ -41,7 +42,7 @@ struct AlphaArgs {
     float *out;
     const float *in, *filt;
     int64_t rows;
-    int T, L, P;        // P: floats per row in LDS, P / 4 odd
+    int T, L;
     float a;            // exp(-Ts / tau)
     float aSeg[2];      // a^n for segments of perRow / parts and perRow / parts + 1 vectors (n = 4 times that)
     float aL;           // a^L
@@ -55,9 +56,9 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
     constexpr int kParts = kWave / R;
     constexpr int NB = (R * (kAlphaMaxT / 4) + kWave - 1) / kWave;  // vectors per lane of a tile, at most
     extern __shared__ __align__(16) float lds[];
-    const int T = p.T, P = p.P, L = p.L;
-    float *Q = lds;            // [R][P]: x, then q
-    float *Rr = lds + R * P;   // [R][P]: r
+    const int T = p.T, P = p.T, L = p.L;   // rows follow each other in LDS as in memory
+    float *Q = lds;            // [R][T]: x, then q
+    float *Rr = lds + R * P;   // [R][T]: r
 
     const int lane = threadIdx.x;
     const int perRow = T >> 2;
@@ -65,7 +66,8 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
     const int nRows = static_cast<int>(min(static_cast<int64_t>(R), p.rows - row0));
     const int nVec = nRows * perRow;
 
-    // ---- the tile, one contiguous run of vectors (rows behind the last one arrive as zeros)
+    // ---- the tile, one contiguous run of vectors, in LDS exactly as it lies in memory (rows behind the last one
+    //      arrive as zeros): vector e of the tile is vector e of LDS, no index arithmetic
     bool bad = false;
     {
         const BufferRsrc bufIn = make_buffer(p.in + row0 * static_cast<int64_t>(T), nVec * 16);
@@ -73,18 +75,14 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
 #pragma unroll
         for (int b = 0; b < NB; ++b)
             if (b * kWave < R * perRow) x[b] = buffer_load4(bufIn, (lane + b * kWave) * 16, 0);
-        RowCol rc;
-        rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
-        const int dr = kWave / perRow, dc = kWave % perRow;
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             if (b * kWave < R * perRow) {
                 if (lane + b * kWave < R * perRow) {
-                    *reinterpret_cast<float4 *>(Q + rc.r * P + (rc.c << 2)) = x[b];
+                    *reinterpret_cast<float4 *>(Q + 4 * (lane + b * kWave)) = x[b];
                     // infinite or NaN (or four samples that add up to more than fp32 holds, which only costs time)
                     bad |= ((x[b].x + x[b].y) + (x[b].z + x[b].w)) * 0.0f != 0.0f;
                 }
-                rc.advance(dr, dc, perRow);
             }
         }
     }
@@ -124,21 +122,33 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
         step(sp, sq, CAUSAL ? x.z : x.y);
         step(sp, sq, CAUSAL ? x.w : x.x);
     }
-    // the state in front of every segment: the end state of the one before it, handed down the row's lanes
-    const int n = (v1 - v0) << 2;
-    const float fn = static_cast<float>(n);
-    const float aN = p.aSeg[(v1 - v0) - perRow / kParts];
-    float cp = 0.0f, cq = 0.0f;
-#pragma unroll
-    for (int k = 0; k + 1 < kParts; ++k) {
-        const float ep = __builtin_fmaf(aN, cp, sp), eq = __builtin_fmaf(aN, __builtin_fmaf(fn, cp, cq), sq);
-        // row_shr:1 - every lane reads the lane below it (within the row's lanes for j >= 1)
-        const float np = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ep), 0x111, 0xf, 0xf, false));
-        const float nq = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, eq), 0x111, 0xf, 0xf, false));
-        if (j == k + 1) {
-            cp = np;
-            cq = nq;
-        }
+    // The state in front of every segment.  A run of n samples takes a state (p, q) to (a^n p, a^n (q + n p)) plus
+    // its own sums; runs compose, so an inclusive scan over the row's lanes (4 steps of lane-shifting moves, each
+    // lane taking in the run that ends d lanes below it) leaves the state behind every segment, and the lane
+    // below hands it up.  Lanes without a lane d below take in the empty run (1, 0, 0, 0).
+    float cp, cq;
+    {
+        float rA = p.aSeg[(v1 - v0) - perRow / kParts], rN = static_cast<float>((v1 - v0) << 2), rP = sp, rQ = sq;
+        auto below = [&](float own, float identity, auto ctrlTag) {   // row_shr:d as a compile-time constant
+            return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity),
+                                                                         __builtin_bit_cast(int, own), decltype(ctrlTag)::value,
+                                                                         0xf, 0xf, false));
+        };
+        auto take_in = [&](auto ctrlTag) {
+            const float lA = below(rA, 1.0f, ctrlTag), lN = below(rN, 0.0f, ctrlTag), lP = below(rP, 0.0f, ctrlTag),
+                        lQ = below(rQ, 0.0f, ctrlTag);
+            rQ = __builtin_fmaf(rA, __builtin_fmaf(rN, lP, lQ), rQ);
+            rP = __builtin_fmaf(rA, lP, rP);
+            rA *= lA;
+            rN += lN;
+        };
+        static_assert(kParts == 16, "a row's lanes are one row of the lane-shifting moves");
+        take_in(std::integral_constant<int, 0x111>{});
+        take_in(std::integral_constant<int, 0x112>{});
+        take_in(std::integral_constant<int, 0x114>{});
+        take_in(std::integral_constant<int, 0x118>{});
+        cp = below(rP, 0.0f, std::integral_constant<int, 0x111>{});
+        cq = below(rQ, 0.0f, std::integral_constant<int, 0x111>{});
     }
     // pass 2: q over x, r next to it
     {
@@ -170,18 +180,18 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
         const float aL = p.aL, scale = p.scale;
         const int shift = CAUSAL ? -L : L;           // r[t + shift]
         const int lo = shift >> 2, off = shift & 3;  // r[4 c + e + shift] = element (e + off) of vectors c + lo, c + lo + 1
-        RowCol rc;
-        rc.init(lane, perRow, 1.0f / static_cast<float>(perRow));
-        const int dr = kWave / perRow, dc = kWave % perRow;
+        static_assert(R == 4, "the row of a vector from three comparisons");
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             if (b * kWave < R * perRow) {
-                const int row = min(rc.r, R - 1);  // (lanes behind the tile: their stores are dropped)
-                const int ca = rc.c + lo, cb = ca + 1;
+                const int e = min(lane + b * kWave, R * perRow - 1);  // (lanes behind the tile: their stores are dropped)
+                const int row = (e >= perRow ? 1 : 0) + (e >= 2 * perRow ? 1 : 0) + (e >= 3 * perRow ? 1 : 0);
+                const int c = e - row * perRow;
+                const int ca = c + lo, cb = ca + 1;
                 const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                const float4 qv = *reinterpret_cast<const float4 *>(Q + row * P + (rc.c << 2));
-                const float4 ra = (ca >= 0 && ca < perRow) ? *reinterpret_cast<const float4 *>(Rr + row * P + (ca << 2)) : zero;
-                const float4 rb = (off != 0 && cb >= 0 && cb < perRow) ? *reinterpret_cast<const float4 *>(Rr + row * P + (cb << 2)) : zero;
+                const float4 qv = *reinterpret_cast<const float4 *>(Q + 4 * e);
+                const float4 ra = (ca >= 0 && ca < perRow) ? *reinterpret_cast<const float4 *>(Rr + 4 * (e + lo)) : zero;
+                const float4 rb = (off != 0 && cb >= 0 && cb < perRow) ? *reinterpret_cast<const float4 *>(Rr + 4 * (e + lo + 1)) : zero;
                 float4 rs;
                 if (off == 0) rs = ra;
                 else if (off == 1) rs = make_float4(ra.y, ra.z, ra.w, rb.x);
@@ -190,7 +200,6 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
                 const float4 y = make_float4(scale * __builtin_fmaf(-aL, rs.x, qv.x), scale * __builtin_fmaf(-aL, rs.y, qv.y),
                                              scale * __builtin_fmaf(-aL, rs.z, qv.z), scale * __builtin_fmaf(-aL, rs.w, qv.w));
                 buffer_store4(bufOut, (lane + b * kWave) * 16, 0, y);
-                rc.advance(dr, dc, perRow);
             }
         }
     }
@@ -218,7 +227,6 @@ extern "C" int slayer_psp_alpha_f32(float *out, const float *in, const float *fi
     a.rows = nNeurons;
     a.T = static_cast<int>(T);
     a.L = static_cast<int>(F);
-    a.P = static_cast<int>(T) + (((T / 4) % 2 == 0) ? 4 : 0);   // P / 4 odd: the 8 rows start in different banks
     const double ratio = static_cast<double>(Ts) / static_cast<double>(tau);
     const double av = exp(-ratio);
     a.a = static_cast<float>(av);
@@ -228,7 +236,7 @@ extern "C" int slayer_psp_alpha_f32(float *out, const float *in, const float *fi
     a.aL = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(F)));
     a.scale = static_cast<float>(static_cast<double>(Ts) * static_cast<double>(mult) * exp(1.0) * ratio);
     a.Ts = Ts;
-    const size_t lds = static_cast<size_t>(2) * R * a.P * sizeof(float);
+    const size_t lds = static_cast<size_t>(2) * R * T * sizeof(float);
     const dim3 grid(static_cast<unsigned>(tiles));
     if (causal) hipLaunchKernelGGL((alpha_psp_kernel<true, R>), grid, dim3(kWave), lds, st, a);
     else hipLaunchKernelGGL((alpha_psp_kernel<false, R>), grid, dim3(kWave), lds, st, a);

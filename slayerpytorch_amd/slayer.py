@@ -384,6 +384,11 @@ class _spikeDelayedFunction(torch.autograd.Function):
         return gradInput, None, None, None, gradDelay, None
 
 
+def _recursion_serves(x):
+    """Row lengths that ``slayerCuda.pspAlpha`` runs as a recursion (others it would hand to conv / corr itself)."""
+    return x.shape[-1] % 4 == 0 and x.shape[-1] <= 512
+
+
 class _pspSpikeFunction(torch.autograd.Function):
     """``_pspFunction`` followed by ``_spikeFunction`` (src/slayer.py:817-899) as one Function:
     forward is ``slayerCuda.pspSpike``; backward is the spike function's surrogate gradient
@@ -391,7 +396,7 @@ class _pspSpikeFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, srmKernel, refractoryResponse, neuron, Ts, alpha=None):
-        if alpha is None:
+        if alpha is None or not _recursion_serves(input):
             spikes, membranePotential = slayerCuda.pspSpike(input.contiguous(), srmKernel, refractoryResponse,
                                                             neuron["theta"], Ts)
         else:
@@ -421,6 +426,8 @@ class _pspFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, spike, filter, Ts, alpha=None):
+        if alpha is not None and not _recursion_serves(spike):
+            alpha = None
         if alpha is None:
             psp = slayerCuda.conv(spike.contiguous(), filter, Ts)
         else:
