@@ -576,6 +576,9 @@ def other_rows(device, cpu_leg=False):
     gs = torch.randn(shape, generator=g).to(device)
     out.append(row("spike_pdf_then_corr77_fused", 20, a.numel(),
                    timed(lambda: slayerCuda.spikeBackwardCorr(gs, a, srm77, 10.0, 10.0, 1.0, 1.0), K), shape, moved=12))
+    # ... for the layers' alpha kernel: the surrogate gradient on the way in, the correlation as a recursion
+    out.append(row("spike_pdf_then_corr77_as_recursion_fused", 20, a.numel(),
+                   timed(lambda: slayerCuda.spikeBackwardPspAlpha(gs, a, srm77, 10.0, 1.0, 10.0, 10.0, 1.0, 1.0), K), shape, moved=12))
     del a, gs
     # NMNIST-shaped MLP end to end (dense layers are library GEMMs): forward, spike-time loss, backward
     out.append(mlp_row(device, timed))

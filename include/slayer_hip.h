@@ -195,6 +195,18 @@ int slayer_psp_alpha_f32(float *out, const float *in, const float *filt, int64_t
                          float tau, float mult, float Ts, int causal, void *stream);
 
 /*
+ * slayer_spike_bwd_corr_f32 for such an alpha kernel: the surrogate gradient of the spike function, applied to the
+ * samples on their way in, then the correlation as that recursion - the backward pass of spike(psp(x)) (the
+ * reference's MLP ordering, example/02_NMNIST_MLP/nmnistMLP.py:59-60; src/slayer.py:857-865 followed by :887-899)
+ * in one kernel, 12 bytes per neuron-timestep.  Same bound as slayer_psp_alpha_f32 with
+ * x = gradOut * (scale / tauRho) * exp(-|u - theta| / tauRho); tauRho here is the scaled time constant (the `tau`
+ * of slayer_spike_bwd_f32).  Shapes outside the recursion's reach run slayer_spike_bwd_corr_f32.
+ */
+int slayer_spike_bwd_psp_alpha_f32(float *gradIn, const float *gradOut, const float *u, const float *filt,
+                                   int64_t nNeurons, int64_t T, int64_t F, float tau, float mult, float theta,
+                                   float tauRho, float scale, float Ts, void *stream);
+
+/*
  * Spike generation with the time shift that follows it fused into the store of the spikes.
  * Replaces the call pair slayerCuda.getSpikes (src/cuda/slayerKernels.cu:14-39) -> slayerCuda.shift
  * (src/cuda/slayerKernels.cu:77-134) that `delayShift(spike(u), d)` / `delay(spike(u))` make

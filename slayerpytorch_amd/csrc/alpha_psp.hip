@@ -48,9 +48,13 @@ struct AlphaArgs {
     float aL;           // a^L
     float scale;        // Ts * mult * e * Ts / tau
     float Ts;
+    // GATED: the samples are in * gain * exp(-|u - theta| / tauRho) (the spike function's surrogate gradient),
+    // applied on the way into LDS
+    const float *u;
+    float theta, tauRho, gain;
 };
 
-template <bool CAUSAL, int R>
+template <bool CAUSAL, int R, bool GATED>
 __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
 {
     constexpr int kParts = kWave / R;
@@ -71,14 +75,24 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
     bool bad = false;
     {
         const BufferRsrc bufIn = make_buffer(p.in + row0 * static_cast<int64_t>(T), nVec * 16);
-        float4 x[NB];
+        const BufferRsrc bufU = make_buffer((GATED ? p.u : p.in) + row0 * static_cast<int64_t>(T), nVec * 16);
+        float4 x[NB], gu[GATED ? NB : 1];
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
-            if (b * kWave < R * perRow) x[b] = buffer_load4(bufIn, (lane + b * kWave) * 16, 0);
+        for (int b = 0; b < NB; ++b) {
+            if (b * kWave < R * perRow) {
+                x[b] = buffer_load4(bufIn, (lane + b * kWave) * 16, 0);
+                if (GATED) gu[b] = buffer_load4(bufU, (lane + b * kWave) * 16, 0);
+            }
+        }
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             if (b * kWave < R * perRow) {
                 if (lane + b * kWave < R * perRow) {
+                    if (GATED)
+                        x[b] = make_float4(x[b].x * spike_pdf(gu[b].x, p.theta, p.tauRho, p.gain),
+                                           x[b].y * spike_pdf(gu[b].y, p.theta, p.tauRho, p.gain),
+                                           x[b].z * spike_pdf(gu[b].z, p.theta, p.tauRho, p.gain),
+                                           x[b].w * spike_pdf(gu[b].w, p.theta, p.tauRho, p.gain));
                     *reinterpret_cast<float4 *>(Q + 4 * (lane + b * kWave)) = x[b];
                     // infinite or NaN (or four samples that add up to more than fp32 holds, which only costs time)
                     bad |= ((x[b].x + x[b].y) + (x[b].z + x[b].w)) * 0.0f != 0.0f;
@@ -95,8 +109,10 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
             const int r = e / T, t = e - r * T;
             const float *x = p.in + (row0 + r) * static_cast<int64_t>(T);
             const int taps = CAUSAL ? min(t + 1, L) : min(T - t, L);
+            const float *gu = GATED ? p.u + (row0 + r) * static_cast<int64_t>(T) : nullptr;
+            auto sample = [&](int i) { return GATED ? x[i] * spike_pdf(gu[i], p.theta, p.tauRho, p.gain) : x[i]; };
             float acc = 0.0f;
-            for (int k = 0; k < taps; ++k) acc = __builtin_fmaf(CAUSAL ? x[t - k] : x[t + k], p.filt[k], acc);
+            for (int k = 0; k < taps; ++k) acc = __builtin_fmaf(sample(CAUSAL ? t - k : t + k), p.filt[k], acc);
             p.out[(row0 + r) * static_cast<int64_t>(T) + t] = acc * p.Ts;
         }
         return;
@@ -207,6 +223,42 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
 
 }  // namespace slayer
 
+namespace slayer {
+
+// Launches the recursion, or returns false (nothing launched) for shapes it does not serve.
+static bool launch_alpha(float *out, const float *in, const float *filt, int64_t nNeurons, int64_t T, int64_t F, float tau,
+                         float mult, float Ts, bool causal, const float *u, float theta, float tauRho, float gain,
+                         hipStream_t st)
+{
+    constexpr int R = kAlphaRows, parts = kWave / R;
+    const int64_t tiles = ceil_div(nNeurons, R);
+    if (generic_forced() || T % 4 != 0 || T > kAlphaMaxT || !aligned16(out) || !aligned16(in) || (u && !aligned16(u)) ||
+        tiles >= (1LL << 31) || F >= (1 << 20))
+        return false;
+    AlphaArgs a{};
+    a.out = out; a.in = in; a.filt = filt;
+    a.rows = nNeurons;
+    a.T = static_cast<int>(T);
+    a.L = static_cast<int>(F);
+    const double ratio = static_cast<double>(Ts) / static_cast<double>(tau);
+    a.a = static_cast<float>(exp(-ratio));
+    // (powers of the rounded a, which is what the recursion multiplies by)
+    a.aSeg[0] = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(4 * ((T / 4) / parts))));
+    a.aSeg[1] = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(4 * ((T / 4) / parts + 1))));
+    a.aL = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(F)));
+    a.scale = static_cast<float>(static_cast<double>(Ts) * static_cast<double>(mult) * exp(1.0) * ratio);
+    a.Ts = Ts;
+    a.u = u; a.theta = theta; a.tauRho = tauRho; a.gain = gain;
+    const size_t lds = static_cast<size_t>(2) * R * T * sizeof(float);
+    const dim3 grid(static_cast<unsigned>(tiles));
+    if (u) hipLaunchKernelGGL((alpha_psp_kernel<false, R, true>), grid, dim3(kWave), lds, st, a);
+    else if (causal) hipLaunchKernelGGL((alpha_psp_kernel<true, R, false>), grid, dim3(kWave), lds, st, a);
+    else hipLaunchKernelGGL((alpha_psp_kernel<false, R, false>), grid, dim3(kWave), lds, st, a);
+    return true;
+}
+
+}  // namespace slayer
+
 extern "C" int slayer_psp_alpha_f32(float *out, const float *in, const float *filt, int64_t nNeurons, int64_t T, int64_t F,
                                     float tau, float mult, float Ts, int causal, void *stream)
 {
@@ -214,31 +266,24 @@ extern "C" int slayer_psp_alpha_f32(float *out, const float *in, const float *fi
     if (nNeurons < 0 || T < 0 || F < 1 || !(tau > 0.0f) || !(Ts > 0.0f)) return SLAYER_EINVAL;
     if (nNeurons == 0 || T == 0) return SLAYER_OK;
     if (!out || !in || !filt) return SLAYER_EINVAL;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    constexpr int R = kAlphaRows, parts = kWave / R;
-    const int64_t tiles = ceil_div(nNeurons, R);
-    const bool served = !generic_forced() && T % 4 == 0 && T <= kAlphaMaxT && aligned16(out) && aligned16(in) &&
-                        tiles < (1LL << 31) && F < (1 << 20);
-    if (!served)   // the L-tap sum with the given filter
-        return causal ? slayer_conv_f32(out, in, filt, nNeurons, T, F, Ts, stream)
-                      : slayer_corr_f32(out, in, filt, nNeurons, T, F, Ts, stream);
-    AlphaArgs a{};
-    a.out = out; a.in = in; a.filt = filt;
-    a.rows = nNeurons;
-    a.T = static_cast<int>(T);
-    a.L = static_cast<int>(F);
-    const double ratio = static_cast<double>(Ts) / static_cast<double>(tau);
-    const double av = exp(-ratio);
-    a.a = static_cast<float>(av);
-    // (powers of the rounded a, which is what the recursion multiplies by)
-    a.aSeg[0] = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(4 * ((T / 4) / parts))));
-    a.aSeg[1] = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(4 * ((T / 4) / parts + 1))));
-    a.aL = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(F)));
-    a.scale = static_cast<float>(static_cast<double>(Ts) * static_cast<double>(mult) * exp(1.0) * ratio);
-    a.Ts = Ts;
-    const size_t lds = static_cast<size_t>(2) * R * T * sizeof(float);
-    const dim3 grid(static_cast<unsigned>(tiles));
-    if (causal) hipLaunchKernelGGL((alpha_psp_kernel<true, R>), grid, dim3(kWave), lds, st, a);
-    else hipLaunchKernelGGL((alpha_psp_kernel<false, R>), grid, dim3(kWave), lds, st, a);
-    return launch_status();
+    if (launch_alpha(out, in, filt, nNeurons, T, F, tau, mult, Ts, causal != 0, nullptr, 0.0f, 1.0f, 0.0f,
+                     static_cast<hipStream_t>(stream)))
+        return launch_status();
+    // the sum over the taps of the given filter
+    return causal ? slayer_conv_f32(out, in, filt, nNeurons, T, F, Ts, stream)
+                  : slayer_corr_f32(out, in, filt, nNeurons, T, F, Ts, stream);
+}
+
+extern "C" int slayer_spike_bwd_psp_alpha_f32(float *gradIn, const float *gradOut, const float *u, const float *filt,
+                                              int64_t nNeurons, int64_t T, int64_t F, float tau, float mult, float theta,
+                                              float tauRho, float scale, float Ts, void *stream)
+{
+    using namespace slayer;
+    if (nNeurons < 0 || T < 0 || F < 1 || !(tau > 0.0f) || !(Ts > 0.0f) || tauRho == 0.0f) return SLAYER_EINVAL;
+    if (nNeurons == 0 || T == 0) return SLAYER_OK;
+    if (!gradIn || !gradOut || !u || !filt) return SLAYER_EINVAL;
+    if (launch_alpha(gradIn, gradOut, filt, nNeurons, T, F, tau, mult, Ts, false, u, theta, tauRho, scale / tauRho,
+                     static_cast<hipStream_t>(stream)))
+        return launch_status();
+    return slayer_spike_bwd_corr_f32(gradIn, gradOut, u, filt, nNeurons, T, F, theta, tauRho, scale, Ts, stream);
 }

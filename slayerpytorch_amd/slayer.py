@@ -405,6 +405,7 @@ class _pspSpikeFunction(torch.autograd.Function):
             membranePotential = slayerCuda.pspAlpha(input.contiguous(), srmKernel, alpha[0], alpha[1], Ts, causal=True)
             spikes = slayerCuda.getSpikes(membranePotential, refractoryResponse, neuron["theta"], Ts)
         ctx.save_for_backward(membranePotential, srmKernel)
+        ctx.alpha = alpha if alpha is not None and _recursion_serves(input) else None
         ctx.theta = float(neuron["theta"])
         ctx.pdfTimeConstant = float(neuron["tauRho"] * neuron["theta"])
         ctx.pdfScale = float(neuron["scaleRho"])
@@ -414,8 +415,13 @@ class _pspSpikeFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gradOutput):
         membranePotential, srmKernel = ctx.saved_tensors
-        gradInput = slayerCuda.spikeBackwardCorr(gradOutput.contiguous(), membranePotential, srmKernel, ctx.theta,
-                                                 ctx.pdfTimeConstant, ctx.pdfScale, ctx.Ts)
+        if ctx.alpha is None:
+            gradInput = slayerCuda.spikeBackwardCorr(gradOutput.contiguous(), membranePotential, srmKernel, ctx.theta,
+                                                     ctx.pdfTimeConstant, ctx.pdfScale, ctx.Ts)
+        else:
+            gradInput = slayerCuda.spikeBackwardPspAlpha(gradOutput.contiguous(), membranePotential, srmKernel,
+                                                         ctx.alpha[0], ctx.alpha[1], ctx.theta, ctx.pdfTimeConstant,
+                                                         ctx.pdfScale, ctx.Ts)
         return gradInput, None, None, None, None, None
 
 

@@ -31,7 +31,7 @@ import torch
 from . import _lib
 
 __all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "spikeBackwardCorr", "pspSpike", "delayGrad",
-           "getSpikesDelayed", "spikeBackwardDelayed", "spikeLoss", "pspAlpha"]
+           "getSpikesDelayed", "spikeBackwardDelayed", "spikeLoss", "pspAlpha", "spikeBackwardPspAlpha"]
 
 
 def _check_input(x, name):
@@ -169,6 +169,31 @@ def pspAlpha(input, filter, tau, mult, Ts, causal=True):
         _lib.check(lib.slayer_psp_alpha_f32(_ptr(output), _ptr(input), _ptr(filter), n, T, filter.numel(), tau, mult,
                                             Ts, 1 if causal else 0, stream), "slayer_psp_alpha_f32")
     return output
+
+
+def spikeBackwardPspAlpha(gradOutput, membranePotential, filter, tauSr, mult, theta, tau, scale, Ts):
+    """:func:`spikeBackwardCorr` for a ``filter`` that holds the alpha kernel of :func:`pspAlpha`
+    (``tauSr``, ``mult``): the surrogate gradient (``theta``, ``tau``, ``scale`` as in
+    :func:`spikeBackward`) and the correlation as a recursion over time, in one kernel."""
+    _check_input(gradOutput, "gradOutput")
+    _check_input(membranePotential, "membranePotential")
+    _check_input(filter, "filter")
+    _check_device(gradOutput, membranePotential, "gradOutput", "membranePotential")
+    _check_device(gradOutput, filter, "gradOutput", "filter")
+    if gradOutput.shape != membranePotential.shape:
+        raise RuntimeError("gradOutput and membranePotential must have the same shape")
+    if filter.numel() < 1:
+        raise RuntimeError("spikeBackwardPspAlpha needs a filter of at least one tap")
+    tauSr, mult, theta, tau = _scalar(tauSr, "tauSr"), _scalar(mult, "mult"), _scalar(theta, "theta"), _scalar(tau, "tau")
+    scale, Ts = _scalar(scale, "scale"), _scalar(Ts, "Ts")
+    lib = _lib.load()
+    gradInput = torch.empty_like(gradOutput)
+    n, T = _rows(gradOutput)
+    with _on_device_of(gradOutput) as stream:
+        _lib.check(lib.slayer_spike_bwd_psp_alpha_f32(_ptr(gradInput), _ptr(gradOutput), _ptr(membranePotential), _ptr(filter),
+                                                      n, T, filter.numel(), tauSr, mult, theta, tau, scale, Ts, stream),
+                   "slayer_spike_bwd_psp_alpha_f32")
+    return gradInput
 
 
 def shift(input, shiftLUT, Ts=1.0, sign=1.0):

@@ -335,6 +335,50 @@ def test_psp_alpha_outside_its_shapes_is_conv_and_corr(impl, shape):
     assert torch.equal(slayerCuda.pspAlpha(dev(x), dev(f), tau, 1.0, Ts, False), slayerCuda.corr(dev(x), dev(f), Ts))
 
 
+@pytest.mark.parametrize("shape,tau", [((2, 6, 5, 3, 300), 10.0), ((1, 9, 1, 1, 352), 4.0), ((3, 7, 1, 1, 64), 10.0),
+                                       ((1, 1, 1, 1, 4), 1.0), ((2, 5, 1, 1, 512), 20.0), ((1, 3, 1, 1, 350), 10.0),
+                                       ((1, 2, 1, 1, 1000), 10.0)])
+def test_spike_backward_psp_alpha_is_spikeBackward_then_corr(impl, shape, tau):
+    # the surrogate gradient on the way in, then the correlation with the alpha kernel as a recursion: the values of
+    # spikeBackward followed by pspAlpha bit for bit (the same products enter the same recursion), which is the sum over
+    # the taps to rounding; shapes outside the recursion's reach run spikeBackwardCorr
+    rng = np.random.default_rng(shape[-1])
+    Ts, theta, tauRho, scale = 1.0, 10.0, 10.0, 1.0
+    f = np.array(alphaKernel(tau, Ts, 5000), dtype=np.float32)
+    g = rng.standard_normal(shape).astype(np.float32)
+    v = (rng.standard_normal(shape) * 4 + 8).astype(np.float32)
+    got = slayerCuda.spikeBackwardPspAlpha(dev(g), dev(v), dev(f), tau, 1.0, theta, tauRho, scale, Ts)
+    T = shape[-1]
+    if not impl and T % 4 == 0 and T <= 512:
+        two = slayerCuda.pspAlpha(slayerCuda.spikeBackward(dev(g), dev(v), theta, tauRho, scale), dev(f), tau, 1.0, Ts, False)
+        assert np.array_equal(bits(host(got)), bits(host(two)))
+    else:
+        assert torch.equal(got, slayerCuda.spikeBackwardCorr(dev(g), dev(v), dev(f), theta, tauRho, scale, Ts))
+    gs = O.spike_bwd(g, v, theta, tauRho, scale)
+    assert rel_err(host(got), O.corr(gs, f, Ts, fused=True)) <= REL_TOL
+    assert close_to_alpha_sum(host(got), gs, f, tau, 1.0, Ts, False)
+
+
+def test_spike_backward_psp_alpha_keeps_non_finite_samples_in_place():
+    rng = np.random.default_rng(21)
+    tau, Ts = 10.0, 1.0
+    f = np.array(alphaKernel(tau, Ts, 300), dtype=np.float32)
+    g = rng.standard_normal((12, 300)).astype(np.float32).reshape(1, 12, 1, 1, 300)
+    v = (rng.standard_normal((12, 300)) * 3 + 8).astype(np.float32).reshape(g.shape)
+    g[0, 1, 0, 0, 150] = np.inf
+    v[0, 9, 0, 0, 7] = np.inf          # (gate 0 times a finite sample is 0)
+    g[0, 10, 0, 0, 40] = np.nan
+    got = host(slayerCuda.spikeBackwardPspAlpha(dev(g), dev(v), dev(f), tau, 1.0, 10.0, 5.0, 1.0, Ts)).reshape(12, 300)
+    want = O.corr(O.spike_bwd(g, v, 10.0, 5.0, 1.0), f, Ts, fused=True).reshape(12, 300)
+    fin = np.isfinite(want)
+    assert not fin.all()
+    assert np.array_equal(np.isfinite(got), fin) and np.array_equal(got[~fin], want[~fin], equal_nan=True)
+    assert rel_err(np.where(fin, got, 0), np.where(fin, want, 0)) <= REL_TOL
+    # (the tiles with these samples are sums over the taps: what the kernel that sums them gives, bit for bit)
+    taps = host(slayerCuda.spikeBackwardCorr(dev(g), dev(v), dev(f), 10.0, 5.0, 1.0, Ts)).reshape(12, 300)
+    assert np.array_equal(bits(got[8:12]), bits(taps[8:12]))
+
+
 def test_gated_corr_on_the_matrix_cores_keeps_non_finite_samples_in_place():
     # an infinite gradient sample reaches exactly the outputs within Fl taps before it, as in the chain; so does an
     # infinite membrane potential (gate 0 times a finite sample is 0, times an infinite one NaN)
