@@ -16,7 +16,7 @@
 // About 10 floating-point operations per sample instead of 2 L: at 77 taps the L-tap sum sits on the FP32 ridge
 // of the machine (matrix-pipe bound at 0.47 of HBM peak); the recursion is a memory stream.
 //
-// A wavefront owns 4 consecutive rows of whole 16-byte vectors, in LDS as they lie in memory.  Sixteen lanes serve
+// A wavefront owns 4 consecutive rows - always a run of whole 16-byte vectors - in LDS as they lie in memory.  Sixteen lanes serve
 // a row, each a contiguous segment of its time axis: pass 1 runs the recursion over the segment from zero state,
 // a scan over the row's lanes composes the segments (state after n more samples: p' = a^n p,
 // q' = a^n (q + n p), plus the run's own sums) into the state in front of each, pass 2 runs the recursion again from the true state and
@@ -54,7 +54,10 @@ struct AlphaArgs {
     float theta, tauRho, gain;
 };
 
-template <bool CAUSAL, int R, bool GATED>
+// VEC: rows are whole 16-byte vectors (T % 4 == 0).  Otherwise a tile of 4 rows is still a contiguous, 16-byte aligned
+// run of whole vectors (4 T floats) and travels the same way, but a vector may hold the end of one row and the start of
+// the next: the passes then read and write LDS sample by sample, and the way out places every sample in its row.
+template <bool CAUSAL, int R, bool GATED, bool VEC>
 __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
 {
     constexpr int kParts = kWave / R;
@@ -65,10 +68,11 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
     float *Rr = lds + R * P;   // [R][T]: r
 
     const int lane = threadIdx.x;
-    const int perRow = T >> 2;
+    const int perRow = T >> 2;                 // (VEC: vectors per row)
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
     const int nRows = static_cast<int>(min(static_cast<int64_t>(R), p.rows - row0));
-    const int nVec = nRows * perRow;
+    const int nVec = (nRows * T) >> 2;         // the tile is whole vectors: the host checked (rows * T) % 4 == 0
+    const int tileVec = (R * T) >> 2;
 
     // ---- the tile, one contiguous run of vectors, in LDS exactly as it lies in memory (rows behind the last one
     //      arrive as zeros): vector e of the tile is vector e of LDS, no index arithmetic
@@ -79,15 +83,15 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
         float4 x[NB], gu[GATED ? NB : 1];
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            if (b * kWave < R * perRow) {
+            if (b * kWave < tileVec) {
                 x[b] = buffer_load4(bufIn, (lane + b * kWave) * 16, 0);
                 if (GATED) gu[b] = buffer_load4(bufU, (lane + b * kWave) * 16, 0);
             }
         }
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            if (b * kWave < R * perRow) {
-                if (lane + b * kWave < R * perRow) {
+            if (b * kWave < tileVec) {
+                if (lane + b * kWave < tileVec) {
                     if (GATED)
                         x[b] = make_float4(x[b].x * spike_pdf(gu[b].x, p.theta, p.tauRho, p.gain),
                                            x[b].y * spike_pdf(gu[b].y, p.theta, p.tauRho, p.gain),
@@ -118,25 +122,33 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
         return;
     }
 
-    // ---- lane (row r, part j): the logical vectors [v0, v1) of the row; logical time runs forward for the
-    //      convolution and backward for the correlation (logical vector V = memory vector perRow - 1 - V, mirrored)
+    // ---- lane (row r, part j): a segment of the row's logical time axis - vectors [v0, v1) (VEC) or samples
+    //      [v0, v1) - where logical time runs forward for the convolution and backward for the correlation (logical
+    //      vector V = memory vector perRow - 1 - V, mirrored; logical sample i = memory sample T - 1 - i)
     const int r = lane / kParts, j = lane - r * kParts;
-    const int v0 = (j * perRow) / kParts, v1 = ((j + 1) * perRow) / kParts;
+    const int units = VEC ? perRow : T;
+    const int v0 = (j * units) / kParts, v1 = ((j + 1) * units) / kParts;
     const float a = p.a;
     float *q4 = Q + r * P, *r4 = Rr + r * P;
     auto vector_at = [&](int V) { return (CAUSAL ? V : perRow - 1 - V) << 2; };
+    auto sample_at = [&](int i) { return CAUSAL ? i : T - 1 - i; };
     auto step = [&](float &pp, float &qq, float x) {
         qq = a * (qq + pp);                 // q[t] = a (q[t-1] + p[t-1])
         pp = __builtin_fmaf(a, pp, x);      // p[t] = a p[t-1] + x[t]
     };
     float sp = 0.0f, sq = 0.0f;   // the segment's own sums (its end state from a zero start)
+    if constexpr (VEC) {
 #pragma unroll 2
-    for (int V = v0; V < v1; ++V) {
-        const float4 x = *reinterpret_cast<const float4 *>(q4 + vector_at(V));
-        step(sp, sq, CAUSAL ? x.x : x.w);
-        step(sp, sq, CAUSAL ? x.y : x.z);
-        step(sp, sq, CAUSAL ? x.z : x.y);
-        step(sp, sq, CAUSAL ? x.w : x.x);
+        for (int V = v0; V < v1; ++V) {
+            const float4 x = *reinterpret_cast<const float4 *>(q4 + vector_at(V));
+            step(sp, sq, CAUSAL ? x.x : x.w);
+            step(sp, sq, CAUSAL ? x.y : x.z);
+            step(sp, sq, CAUSAL ? x.z : x.y);
+            step(sp, sq, CAUSAL ? x.w : x.x);
+        }
+    } else {
+#pragma unroll 4
+        for (int i = v0; i < v1; ++i) step(sp, sq, q4[sample_at(i)]);
     }
     // The state in front of every segment.  A run of n samples takes a state (p, q) to (a^n p, a^n (q + n p)) plus
     // its own sums; runs compose, so an inclusive scan over the row's lanes (4 steps of lane-shifting moves, each
@@ -144,7 +156,7 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
     // below hands it up.  Lanes without a lane d below take in the empty run (1, 0, 0, 0).
     float cp, cq;
     {
-        float rA = p.aSeg[(v1 - v0) - perRow / kParts], rN = static_cast<float>((v1 - v0) << 2), rP = sp, rQ = sq;
+        float rA = p.aSeg[(v1 - v0) - units / kParts], rN = static_cast<float>(VEC ? (v1 - v0) << 2 : v1 - v0), rP = sp, rQ = sq;
         auto below = [&](float own, float identity, auto ctrlTag) {   // row_shr:d as a compile-time constant
             return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity),
                                                                          __builtin_bit_cast(int, own), decltype(ctrlTag)::value,
@@ -170,21 +182,31 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
     {
         const float fL = static_cast<float>(L);
         float pp = cp, qq = cq;
+        if constexpr (VEC) {
 #pragma unroll 2
-        for (int V = v0; V < v1; ++V) {
-            const int at = vector_at(V);
-            const float4 x = *reinterpret_cast<const float4 *>(q4 + at);
-            float qv[4], rv[4];
+            for (int V = v0; V < v1; ++V) {
+                const int at = vector_at(V);
+                const float4 x = *reinterpret_cast<const float4 *>(q4 + at);
+                float qv[4], rv[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float xe = CAUSAL ? (e == 0 ? x.x : e == 1 ? x.y : e == 2 ? x.z : x.w)
-                                        : (e == 0 ? x.w : e == 1 ? x.z : e == 2 ? x.y : x.x);
-                step(pp, qq, xe);
-                qv[e] = qq;
-                rv[e] = __builtin_fmaf(fL, pp, qq);
+                for (int e = 0; e < 4; ++e) {
+                    const float xe = CAUSAL ? (e == 0 ? x.x : e == 1 ? x.y : e == 2 ? x.z : x.w)
+                                            : (e == 0 ? x.w : e == 1 ? x.z : e == 2 ? x.y : x.x);
+                    step(pp, qq, xe);
+                    qv[e] = qq;
+                    rv[e] = __builtin_fmaf(fL, pp, qq);
+                }
+                *reinterpret_cast<float4 *>(q4 + at) = CAUSAL ? make_float4(qv[0], qv[1], qv[2], qv[3]) : make_float4(qv[3], qv[2], qv[1], qv[0]);
+                *reinterpret_cast<float4 *>(r4 + at) = CAUSAL ? make_float4(rv[0], rv[1], rv[2], rv[3]) : make_float4(rv[3], rv[2], rv[1], rv[0]);
             }
-            *reinterpret_cast<float4 *>(q4 + at) = CAUSAL ? make_float4(qv[0], qv[1], qv[2], qv[3]) : make_float4(qv[3], qv[2], qv[1], qv[0]);
-            *reinterpret_cast<float4 *>(r4 + at) = CAUSAL ? make_float4(rv[0], rv[1], rv[2], rv[3]) : make_float4(rv[3], rv[2], rv[1], rv[0]);
+        } else {
+#pragma unroll 4
+            for (int i = v0; i < v1; ++i) {
+                const int at = sample_at(i);
+                step(pp, qq, q4[at]);
+                q4[at] = qq;
+                r4[at] = __builtin_fmaf(fL, pp, qq);
+            }
         }
     }
     wave_sync();
@@ -196,23 +218,35 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
         const float aL = p.aL, scale = p.scale;
         const int shift = CAUSAL ? -L : L;           // r[t + shift]
         const int lo = shift >> 2, off = shift & 3;  // r[4 c + e + shift] = element (e + off) of vectors c + lo, c + lo + 1
-        static_assert(R == 4, "the row of a vector from three comparisons");
+        static_assert(R == 4, "the row of a vector or sample from three comparisons");
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            if (b * kWave < R * perRow) {
-                const int e = min(lane + b * kWave, R * perRow - 1);  // (lanes behind the tile: their stores are dropped)
-                const int row = (e >= perRow ? 1 : 0) + (e >= 2 * perRow ? 1 : 0) + (e >= 3 * perRow ? 1 : 0);
-                const int c = e - row * perRow;
-                const int ca = c + lo, cb = ca + 1;
-                const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (b * kWave < tileVec) {
+                const int e = min(lane + b * kWave, tileVec - 1);  // (lanes behind the tile: their stores are dropped)
                 const float4 qv = *reinterpret_cast<const float4 *>(Q + 4 * e);
-                const float4 ra = (ca >= 0 && ca < perRow) ? *reinterpret_cast<const float4 *>(Rr + 4 * (e + lo)) : zero;
-                const float4 rb = (off != 0 && cb >= 0 && cb < perRow) ? *reinterpret_cast<const float4 *>(Rr + 4 * (e + lo + 1)) : zero;
                 float4 rs;
-                if (off == 0) rs = ra;
-                else if (off == 1) rs = make_float4(ra.y, ra.z, ra.w, rb.x);
-                else if (off == 2) rs = make_float4(ra.z, ra.w, rb.x, rb.y);
-                else rs = make_float4(ra.w, rb.x, rb.y, rb.z);
+                if constexpr (VEC) {
+                    const int row = (e >= perRow ? 1 : 0) + (e >= 2 * perRow ? 1 : 0) + (e >= 3 * perRow ? 1 : 0);
+                    const int c = e - row * perRow;
+                    const int ca = c + lo, cb = ca + 1;
+                    const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    const float4 ra = (ca >= 0 && ca < perRow) ? *reinterpret_cast<const float4 *>(Rr + 4 * (e + lo)) : zero;
+                    const float4 rb = (off != 0 && cb >= 0 && cb < perRow) ? *reinterpret_cast<const float4 *>(Rr + 4 * (e + lo + 1)) : zero;
+                    if (off == 0) rs = ra;
+                    else if (off == 1) rs = make_float4(ra.y, ra.z, ra.w, rb.x);
+                    else if (off == 2) rs = make_float4(ra.z, ra.w, rb.x, rb.y);
+                    else rs = make_float4(ra.w, rb.x, rb.y, rb.z);
+                } else {
+                    float rk[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {   // sample g of the tile lies in row g / T; its partner r must lie in the same row
+                        const int g = 4 * e + k;
+                        const int row = (g >= T ? 1 : 0) + (g >= 2 * T ? 1 : 0) + (g >= 3 * T ? 1 : 0);
+                        const int t = g - row * T + shift;
+                        rk[k] = (t >= 0 && t < T) ? Rr[g + shift] : 0.0f;
+                    }
+                    rs = make_float4(rk[0], rk[1], rk[2], rk[3]);
+                }
                 const float4 y = make_float4(scale * __builtin_fmaf(-aL, rs.x, qv.x), scale * __builtin_fmaf(-aL, rs.y, qv.y),
                                              scale * __builtin_fmaf(-aL, rs.z, qv.z), scale * __builtin_fmaf(-aL, rs.w, qv.w));
                 buffer_store4(bufOut, (lane + b * kWave) * 16, 0, y);
@@ -232,8 +266,10 @@ static bool launch_alpha(float *out, const float *in, const float *filt, int64_t
 {
     constexpr int R = kAlphaRows, parts = kWave / R;
     const int64_t tiles = ceil_div(nNeurons, R);
-    if (generic_forced() || T % 4 != 0 || T > kAlphaMaxT || !aligned16(out) || !aligned16(in) || (u && !aligned16(u)) ||
-        tiles >= (1LL << 31) || F >= (1 << 20))
+    // rows of whole vectors, or at least a tensor of whole vectors (then every tile of 4 rows is one, too)
+    const bool vec = T % 4 == 0;
+    if (generic_forced() || (!vec && (nNeurons * T) % 4 != 0) || T > kAlphaMaxT || !aligned16(out) || !aligned16(in) ||
+        (u && !aligned16(u)) || tiles >= (1LL << 31) || F >= (1 << 20))
         return false;
     AlphaArgs a{};
     a.out = out; a.in = in; a.filt = filt;
@@ -242,18 +278,26 @@ static bool launch_alpha(float *out, const float *in, const float *filt, int64_t
     a.L = static_cast<int>(F);
     const double ratio = static_cast<double>(Ts) / static_cast<double>(tau);
     a.a = static_cast<float>(exp(-ratio));
-    // (powers of the rounded a, which is what the recursion multiplies by)
-    a.aSeg[0] = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(4 * ((T / 4) / parts))));
-    a.aSeg[1] = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(4 * ((T / 4) / parts + 1))));
+    // (powers of the rounded a, which is what the recursion multiplies by; a lane's segment is units / 16 or one more
+    // units long, a unit being a vector or a sample)
+    const int64_t perUnit = vec ? 4 : 1, shortest = (vec ? T / 4 : T) / parts;
+    a.aSeg[0] = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(perUnit * shortest)));
+    a.aSeg[1] = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(perUnit * (shortest + 1))));
     a.aL = static_cast<float>(pow(static_cast<double>(a.a), static_cast<double>(F)));
     a.scale = static_cast<float>(static_cast<double>(Ts) * static_cast<double>(mult) * exp(1.0) * ratio);
     a.Ts = Ts;
     a.u = u; a.theta = theta; a.tauRho = tauRho; a.gain = gain;
     const size_t lds = static_cast<size_t>(2) * R * T * sizeof(float);
     const dim3 grid(static_cast<unsigned>(tiles));
-    if (u) hipLaunchKernelGGL((alpha_psp_kernel<false, R, true>), grid, dim3(kWave), lds, st, a);
-    else if (causal) hipLaunchKernelGGL((alpha_psp_kernel<true, R, false>), grid, dim3(kWave), lds, st, a);
-    else hipLaunchKernelGGL((alpha_psp_kernel<false, R, false>), grid, dim3(kWave), lds, st, a);
+#define SLAYER_ALPHA_LAUNCH(VEC)                                                                                       \
+    do {                                                                                                              \
+        if (u) hipLaunchKernelGGL((alpha_psp_kernel<false, R, true, VEC>), grid, dim3(kWave), lds, st, a);             \
+        else if (causal) hipLaunchKernelGGL((alpha_psp_kernel<true, R, false, VEC>), grid, dim3(kWave), lds, st, a);   \
+        else hipLaunchKernelGGL((alpha_psp_kernel<false, R, false, VEC>), grid, dim3(kWave), lds, st, a);              \
+    } while (0)
+    if (vec) SLAYER_ALPHA_LAUNCH(true);
+    else SLAYER_ALPHA_LAUNCH(false);
+#undef SLAYER_ALPHA_LAUNCH
     return true;
 }
 

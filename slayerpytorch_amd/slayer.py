@@ -385,8 +385,9 @@ class _spikeDelayedFunction(torch.autograd.Function):
 
 
 def _recursion_serves(x):
-    """Row lengths that ``slayerCuda.pspAlpha`` runs as a recursion (others it would hand to conv / corr itself)."""
-    return x.shape[-1] % 4 == 0 and x.shape[-1] <= 512
+    """Shapes that ``slayerCuda.pspAlpha`` runs as a recursion (others it would hand to conv / corr itself): rows of at
+    most 512 samples in a tensor of whole 16-byte vectors."""
+    return x.shape[-1] <= 512 and x.numel() % 4 == 0
 
 
 class _pspSpikeFunction(torch.autograd.Function):
