@@ -49,11 +49,11 @@ def measured_traffic(op):
                                                  "kernel": rec.get("kernels", {}).get(op)}
     except (OSError, ValueError, KeyError):
         return None, None
-KERNEL_OF = {"psp_conv": "slayer::alpha_psp_kernel<true, 4, false> (conv with the alpha kernel as a recursion over time)",
+KERNEL_OF = {"psp_conv": "slayer::alpha_psp_kernel<true, 4, false, true> (conv with the alpha kernel as a recursion over time)",
              "spike": "slayer::spike_tile_kernel<12, 1, 12, 8>",
              "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
              "spike_bwd": "slayer::spike_bwd_vec_kernel",
-             "psp_corr": "slayer::alpha_psp_kernel<false, 4, false> (corr with the alpha kernel as a recursion over time)"}
+             "psp_corr": "slayer::alpha_psp_kernel<false, 4, false, true> (corr with the alpha kernel as a recursion over time)"}
 
 
 def neuron_params():
