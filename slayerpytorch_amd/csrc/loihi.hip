@@ -85,6 +85,45 @@ __device__ __forceinline__ uint32_t loihi_step(LoihiState &st, const LoihiParams
     return spike ? 1u : 0u;
 }
 
+// The same step for states of small magnitude, at about two thirds of the cost (a 32-bit integer
+// multiplication takes four times as long as the other instructions here, a 24-bit one does not).
+// For |x| * keep < 2^31 nothing wraps around and sign * ((|x| * keep) >> 12) is x * keep / 4096
+// rounded toward zero = (x * keep + (x < 0 ? 4095 : 0)) >> 12 with an arithmetic shift.  Valid while
+// keep <= 4096 and both states stay inside (-kLoihiSmall, kLoihiSmall); lo / hi collect the extremes
+// of the new current and voltage so that the caller can check that afterwards: a value is
+// computed correctly whenever the previous state was in range, so the first value that leaves the
+// range is itself correct and is seen.
+constexpr int kLoihiSmall = 1 << 19;
+
+__device__ __forceinline__ int loihi_decay_small(int x, int keep)
+{
+    int scaled;  // x * keep + bias from the low 24 bits of x and keep (the compiler's own choice for
+                 // __mul24 plus an addition is a 64-bit multiply-add, as slow as the 32-bit multiplication)
+    asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(scaled) : "v"(x), "v"(keep), "v"((x >> 31) & 4095));
+    return scaled >> 12;
+}
+
+__device__ __forceinline__ uint32_t loihi_step_small(LoihiState &st, const LoihiParams &p, float w,
+                                                     float &cOut, float &vOut, int &lo, int &hi)
+{
+    const uint32_t wi = static_cast<uint32_t>(cvt_trunc_sat(w));
+    const int cNew = static_cast<int>(static_cast<uint32_t>(loihi_decay_small(st.current, static_cast<int>(p.keepI))) +
+                                      (wi << p.weightShift));
+    const int vNew = static_cast<int>(static_cast<uint32_t>(loihi_decay_small(st.voltage, static_cast<int>(p.keepV))) +
+                                      static_cast<uint32_t>(cNew));
+    lo = min(min(lo, cNew), vNew);
+    hi = max(max(hi, cNew), vNew);
+    const int cd = max(st.countdown - 1, 0);
+    const bool quiet = cd == 0;
+    const bool spike = quiet & (vNew > p.theta);
+    st.voltage = (quiet & !spike) ? vNew : 0;
+    st.countdown = spike ? p.refDelay : cd;
+    st.current = cNew;
+    cOut = static_cast<float>(cNew);
+    vOut = spike ? static_cast<float>(static_cast<int>(p.vDecay)) : static_cast<float>(st.voltage);
+    return spike ? 1u : 0u;
+}
+
 // ---- generic kernel: one lane per neuron, straight from global memory ---------------------------
 __global__ __launch_bounds__(256) void loihi_generic_kernel(float *__restrict__ s, float *__restrict__ v,
                                                             float *__restrict__ u,
@@ -279,9 +318,13 @@ __global__ __launch_bounds__(64) void loihi_tile_kernel(float *__restrict__ s, f
 // all accesses stay aligned; what changes is that the vector in which a row ends can also hold
 // the first samples of the next row.  Loads simply fetch such a vector for both rows, and the
 // hand-over of a row's first line to the row above works sample by sample.  R * T * 4 is a
-// multiple of 128 for R = 32, so a tile still begins and ends on a line boundary.
-template <int R, int LPP, bool MERGE, bool ELEM = false>
-__global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, float *__restrict__ v,
+// multiple of 128 for R = 32 or 64, so a tile still begins and ends on a line boundary.
+//
+// OUTS: 0 = the pointers say which outputs are wanted; 2 = spikes and voltage (u is null), 1 = spikes
+// alone (v and u are null), known at compile time so that the unwanted results cost neither
+// instructions nor registers, nor (the voltage tile of OUTS = 1) shared memory.
+template <int R, int LPP, bool MERGE, bool ELEM = false, int OUTS = 0>
+__global__ __launch_bounds__(64, 2) void loihi_lines_kernel(float *__restrict__ s, float *__restrict__ v,
                                                          float *__restrict__ u, const float *__restrict__ w,
                                                          int64_t rows, int T, int64_t tiles, LoihiParams p)
 {
@@ -291,9 +334,12 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
     constexpr int RPI = kWave / QP;    // rows covered by one wave-wide access
     constexpr int NB = R / RPI;        // accesses per lane per piece
     constexpr int P = TC + 4;          // LDS pitch = 4 (mod 32): 16-byte aligned rows in different banks
+    constexpr bool kCur = OUTS == 0, kVol = OUTS != 1;  // results that may be wanted at all
     __shared__ __align__(16) float tileC[R * P];  // input, then current
-    __shared__ __align__(16) float tileV[R * P];  // voltage
+    __shared__ __align__(16) float tileV[kVol ? R * P : 4];  // voltage
     __shared__ uint32_t masks[R * LPP];
+    if (OUTS != 0) u = nullptr;
+    if (OUTS == 1) v = nullptr;
 
     const int lane = threadIdx.x;
     const int subRow = lane / QP;         // row within an access
@@ -304,7 +350,7 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
     static_assert(!ELEM || (MERGE && (R * 4) % 128 == 0), "rows that are not whole vectors need merged lines and line-aligned tiles");
     LoihiState st = {0, 0, 0};
     float4 x[NB];
-    float headC[MERGE ? G : 1], headV[MERGE ? G : 1];  // results of this row's first line (MERGE)
+    float headC[MERGE && kCur ? G : 1], headV[MERGE && kVol ? G : 1];  // results of this row's first line (MERGE)
     uint32_t headFired = 0;
     uint32_t prevFired = 0;  // undelayed spike bits of this row's previous group
 
@@ -332,12 +378,12 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
     issue(t, j);
     {
         // The loop below keeps one piece of loads and one piece of stores in flight and waits only
-        // for the loads ("all but the 3*NB most recent memory instructions").  Entering it with the
+        // for the loads ("all but the most recent memory instructions", 3*NB of them with all outputs).  Entering it with the
         // same number of stores behind the first loads - dropped by the range check - lets the
         // compiler use that count on every trip instead of waiting for everything.
         const BufferRsrc none = make_buffer(w);
 #pragma unroll
-        for (int b = 0; b < 3 * NB; ++b)  // distinct (all out-of-range) addresses, so none is folded away
+        for (int b = 0; b < (OUTS == 0 ? 3 : OUTS) * NB; ++b)  // distinct (all out-of-range) addresses, so none is folded away
             buffer_store4(none, kOutOfRange + 16 * b, 0, make_float4(static_cast<float>(b), 0.0f, 0.0f, 0.0f));
     }
     while (t < tiles) {
@@ -357,7 +403,7 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
         if (R == kWave || lane < R) {
             if (j == 0) { st = {0, 0, 0}; prevFired = 0; }
             float *mineC = tileC + lane * P;
-            float *mineV = tileV + lane * P;
+            float *mineV = tileV + (kVol ? lane * P : 0);
             const int tRow = TC * j - ((o0 + lane * T) & 31);
             // pieces that lie inside every row need no per-sample checks
             const bool inside = j >= 1 && TC * (j + 1) <= T;
@@ -371,7 +417,18 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
                     in[k] = q.x; in[k + 1] = q.y; in[k + 2] = q.z; in[k + 3] = q.w;
                 }
                 uint32_t fired = 0;
-                if (inside) {
+                bool small = inside && p.keepI <= 4096u && p.keepV <= 4096u;
+                if (small) {
+                    // on the assumption that both states stay small; checked afterwards
+                    const LoihiState before = st;
+                    int lo = min(st.current, st.voltage), hi = max(st.current, st.voltage);
+#pragma unroll
+                    for (int k = 0; k < G; ++k) fired |= loihi_step_small(st, p, in[k], cur[k], vol[k], lo, hi) << k;
+                    small = __builtin_amdgcn_ballot_w64(lo <= -kLoihiSmall || hi >= kLoihiSmall) == 0;
+                    if (!small) { st = before; fired = 0; }
+                }
+                if (small) {
+                } else if (inside) {
 #pragma unroll
                     for (int k = 0; k < G; ++k) fired |= loihi_step(st, p, in[k], cur[k], vol[k]) << k;
                 } else {
@@ -394,8 +451,8 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
                 }
 #pragma unroll
                 for (int k = 0; k < G; k += 4) {
-                    *reinterpret_cast<float4 *>(mineC + c0 + k) = make_float4(cur[k], cur[k + 1], cur[k + 2], cur[k + 3]);
-                    *reinterpret_cast<float4 *>(mineV + c0 + k) = make_float4(vol[k], vol[k + 1], vol[k + 2], vol[k + 3]);
+                    if (kCur) *reinterpret_cast<float4 *>(mineC + c0 + k) = make_float4(cur[k], cur[k + 1], cur[k + 2], cur[k + 3]);
+                    if (kVol) *reinterpret_cast<float4 *>(mineV + c0 + k) = make_float4(vol[k], vol[k + 1], vol[k + 2], vol[k + 3]);
                 }
                 // the delayed bits; those that would land beyond the end of the row are dropped
                 // (the end of this row's last line belongs to the next row)
@@ -408,7 +465,10 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
                 masks[lane * LPP + g] = out;
                 if (MERGE && j == 0) {
 #pragma unroll
-                    for (int k = 0; k < G; ++k) { headC[k] = cur[k]; headV[k] = vol[k]; }
+                    for (int k = 0; k < G; ++k) {
+                        if (kCur) headC[k] = cur[k];
+                        if (kVol) headV[k] = vol[k];
+                    }
                     headFired = out;
                 }
             }
@@ -419,18 +479,21 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
                 const int lastAbove = (T - 1 + skewAbove) >> 5;    // piece in which the row above ends
                 if (lane > 0 && lane < nRows && skew > 0 && j == lastAbove) {
                     float *aboveC = tileC + (lane - 1) * P;
-                    float *aboveV = tileV + (lane - 1) * P;
+                    float *aboveV = tileV + (kVol ? (lane - 1) * P : 0);
                     if (ELEM) {
 #pragma unroll
                         for (int k = 0; k < G; ++k) {
-                            if (k >= skew) { aboveC[k] = headC[k]; aboveV[k] = headV[k]; }
+                            if (k >= skew) {
+                                if (kCur) aboveC[k] = headC[k];
+                                if (kVol) aboveV[k] = headV[k];
+                            }
                         }
                     } else {
 #pragma unroll
                         for (int k = 0; k < G; k += 4) {
                             if (k >= skew) {
-                                *reinterpret_cast<float4 *>(aboveC + k) = make_float4(headC[k], headC[k + 1], headC[k + 2], headC[k + 3]);
-                                *reinterpret_cast<float4 *>(aboveV + k) = make_float4(headV[k], headV[k + 1], headV[k + 2], headV[k + 3]);
+                                if (kCur) *reinterpret_cast<float4 *>(aboveC + k) = make_float4(headC[k], headC[k + 1], headC[k + 2], headC[k + 3]);
+                                if (kVol) *reinterpret_cast<float4 *>(aboveV + k) = make_float4(headV[k], headV[k + 1], headV[k + 2], headV[k + 3]);
                             }
                         }
                     }
@@ -460,8 +523,9 @@ __global__ __launch_bounds__(64) void loihi_lines_kernel(float *__restrict__ s, 
                 }
                 const int off = masked_offset(ok, (r * T + time) * 4);
                 const uint32_t m = masks[r * LPP + (col >> 5)] >> (col & 31);
-                if (u) buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + r * P + col));
-                if (v) buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + r * P + col));
+                if (OUTS == 0 && u) buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + r * P + col));
+                if (OUTS == 2 || (OUTS == 0 && v))
+                    buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + (kVol ? r * P + col : 0)));
                 buffer_store4(bufS, off, 0,
                               make_float4((m & 1u) ? 1.0f : 0.0f, (m & 2u) ? 1.0f : 0.0f,
                                           (m & 4u) ? 1.0f : 0.0f, (m & 8u) ? 1.0f : 0.0f));
@@ -517,30 +581,39 @@ static int launch_loihi(float *s, float *v, float *u, const float *w, int64_t nN
                                (!u || (reinterpret_cast<uintptr_t>(u) & 127) == phase);
         const bool elem = (T % 4 != 0) && T >= 64 && (nNeurons * T) % 4 == 0 && aligned16(s) && aligned16(v) &&
                           aligned16(u) && aligned16(w) && samePhase && LOIHI_LPP == 1 && LOIHI_ROWS == 32;
-        if (elem) {
-            constexpr int kR = 32;
-            const int64_t lineTiles = ceil_div(nNeurons, kR);
-            const int64_t ldsBytes = (2LL * kR * (32 + 4) + kR) * 4;
+        // Without the current among the outputs the sequential update, not the stores, sets the pace:
+        // 64 rows per wavefront then use every lane in it (measured on (8,16,32,32,300): spikes alone
+        // 80 us against 112 us, spikes and voltage 112 us against 120 us; all three outputs 145-249 us
+        // against 147-237 us, so those keep 32 rows).
+        const bool wide = !u && LOIHI_ROWS == 32;
+        auto lines_grid = [&](int rowsPerTile, int lpp, int tilesInLds, int64_t &lineTiles) {
+            lineTiles = ceil_div(nNeurons, rowsPerTile);
+            const int64_t ldsBytes = (static_cast<int64_t>(tilesInLds) * rowsPerTile * (32 * lpp + 4) + rowsPerTile * lpp) * 4 + 16;
             const int64_t fit = static_cast<int64_t>(compute_units()) * (160 * 1024 / ldsBytes);
-            const dim3 grid(static_cast<unsigned>(lineTiles < fit ? lineTiles : fit));
-            hipLaunchKernelGGL((loihi_lines_kernel<kR, 1, true, true>), grid, dim3(kWave), 0, st, s, v, u, w, nNeurons,
-                               static_cast<int>(T), lineTiles, p);
+            return dim3(static_cast<unsigned>(lineTiles < fit ? lineTiles : fit));
+        };
+#define SLAYER_LOIHI_LINES(R_, LPP_, MERGE_, ELEM_, OUTS_)                                                           \
+    do {                                                                                                             \
+        int64_t lineTiles;                                                                                           \
+        const dim3 grid = lines_grid(R_, LPP_, (OUTS_) == 1 ? 1 : 2, lineTiles);                                     \
+        hipLaunchKernelGGL((loihi_lines_kernel<R_, LPP_, MERGE_, ELEM_, OUTS_>), grid, dim3(kWave), 0, st, s, v, u, \
+                           w, nNeurons, static_cast<int>(T), lineTiles, p);                                          \
+    } while (0)
+        if (elem) {
+            if (wide && !v) SLAYER_LOIHI_LINES(64, 1, true, true, 1);
+            else if (wide) SLAYER_LOIHI_LINES(64, 1, true, true, 2);
+            else SLAYER_LOIHI_LINES(32, 1, true, true, 0);
             return launch_status();
         }
         if (vec && samePhase) {
             constexpr int kR = LOIHI_ROWS, kLpp = LOIHI_LPP;
-            const int64_t lineTiles = ceil_div(nNeurons, kR);
-            const int64_t ldsBytes = (2LL * kR * (32 * kLpp + 4) + kR * kLpp) * 4;
-            const int64_t fit = static_cast<int64_t>(compute_units()) * (160 * 1024 / ldsBytes);
-            const dim3 grid(static_cast<unsigned>(lineTiles < fit ? lineTiles : fit));
-            if (kLpp == 1 && T >= 64)
-                hipLaunchKernelGGL((loihi_lines_kernel<kR, kLpp, kLpp == 1>), grid, dim3(kWave), 0, st, s, v,
-                                   u, w, nNeurons, static_cast<int>(T), lineTiles, p);
-            else
-                hipLaunchKernelGGL((loihi_lines_kernel<kR, kLpp, false>), grid, dim3(kWave), 0, st, s, v, u, w, nNeurons,
-                                   static_cast<int>(T), lineTiles, p);
+            if (kLpp == 1 && T >= 64 && wide && !v) SLAYER_LOIHI_LINES(64, 1, true, false, 1);
+            else if (kLpp == 1 && T >= 64 && wide) SLAYER_LOIHI_LINES(64, 1, true, false, 2);
+            else if (kLpp == 1 && T >= 64) SLAYER_LOIHI_LINES(kR, kLpp, kLpp == 1, false, 0);
+            else SLAYER_LOIHI_LINES(kR, kLpp, false, false, 0);
             return launch_status();
         }
+#undef SLAYER_LOIHI_LINES
         if (vec)
             hipLaunchKernelGGL((loihi_tile_kernel<true, kRows, kPiece>), dim3(grid), dim3(kWave), lds, st, s, v, u,
                                w, nNeurons, static_cast<int>(T), Tc, P, MP, tiles, p);

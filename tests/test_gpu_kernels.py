@@ -767,6 +767,28 @@ def test_loihi_parameters_wraparound_and_truncation(impl, params):
         assert np.array_equal(bits(host(a)), bits(b)), name
 
 
+@pytest.mark.parametrize("scale", [1, 6, 30, 200])
+@pytest.mark.parametrize("params", [(0, 80 * 64, 1024, 128, 2), (2, 3000 * 64, 64, 16, 1), (3, 100000 * 64, 0, 0, 3),
+                                    (1, 5000, 4096, 4096, 1), (0, 5000, 5000, 4097, 1)])
+def test_loihi_states_around_the_range_of_the_short_multiplication(impl, scale, params):
+    # the kernel multiplies with 24-bit operands while current and voltage stay below 2^19 in magnitude and
+    # falls back to the 32-bit wrap-around arithmetic for the 32 samples in which either leaves that range:
+    # inputs scaled so that rows stay inside, cross the limit in both directions, or live far outside it
+    rng = np.random.default_rng(scale + params[0])
+    w = (loihi_input(rng, (3, 50, 300), p=0.3) * scale).astype(np.float32)
+    w[1] = np.abs(w[1])                                  # monotonic rows reach the limit soonest
+    w[2, :25] = -np.abs(w[2, :25])
+    want = O.loihi_get_spikes(w, *params)
+    assert max(np.abs(want[1]).max(), np.abs(want[2]).max()) > 2 ** 19 or scale <= 6
+    got = slayerLoihiCuda.getSpikes(dev(w), *params)
+    for a, b, name in zip(got, want, ("spike", "voltage", "current")):
+        assert np.array_equal(bits(host(a)), bits(b)), name
+    s2, v2, _ = slayerLoihiCuda.getSpikesDelayed(dev(w), *params, 0, voltage=True, current=False)
+    assert np.array_equal(bits(host(s2)), bits(want[0])) and np.array_equal(bits(host(v2)), bits(want[1]))
+    s3, _, _ = slayerLoihiCuda.getSpikesDelayed(dev(w), *params, 1, voltage=False, current=False)
+    assert np.array_equal(bits(host(s3)), bits(O.shift(want[0], 1.0, 1.0)))
+
+
 @pytest.mark.parametrize("T", [64, 68, 72, 100, 124, 128, 132, 196, 300, 332])
 @pytest.mark.parametrize("rows", [(1, 1), (3, 67), (2, 64), (5, 13)])
 def test_loihi_rows_sharing_memory_lines(impl, T, rows):
@@ -779,14 +801,19 @@ def test_loihi_rows_sharing_memory_lines(impl, T, rows):
     for a, b, name in zip(got, want, ("spike", "voltage", "current")):
         assert np.array_equal(bits(host(a)), bits(b)), name
     assert want[0].sum() > 0
+    # without the current among the outputs a tile is 64 rows
+    s2, v2, _ = slayerLoihiCuda.getSpikesDelayed(dev(w), 0, 20 * 64, 1024, 128, 2, 0, voltage=True, current=False)
+    assert np.array_equal(bits(host(s2)), bits(want[0])) and np.array_equal(bits(host(v2)), bits(want[1]))
+    s3, _, _ = slayerLoihiCuda.getSpikesDelayed(dev(w), 0, 20 * 64, 1024, 128, 2, 2, voltage=False, current=False)
+    assert np.array_equal(bits(host(s3)), bits(O.shift(want[0], 2.0, 1.0)))
 
 
 @pytest.mark.parametrize("T", [65, 66, 67, 95, 97, 101, 127, 129, 350, 351, 2001])
-@pytest.mark.parametrize("rows", [(4, 1), (4, 33), (8, 8), (2, 2, 3, 5), (12, 3)])
+@pytest.mark.parametrize("rows", [(4, 1), (4, 33), (8, 8), (2, 2, 3, 5), (12, 3), (4, 67)])
 @pytest.mark.parametrize("delay", [0, 3])
 def test_loihi_rows_that_are_not_whole_vectors(impl, T, rows, delay):
     # T % 4 != 0 in a tensor of whole vectors: the 16-byte vector in which a row ends also holds the
-    # first samples of the next row; tiles of 32 rows still begin and end on memory lines
+    # first samples of the next row; tiles of 32 or 64 rows still begin and end on memory lines
     rng = np.random.default_rng(T + len(rows))
     w = loihi_input(rng, rows + (T,), p=0.3)
     ws, wv, wu = O.loihi_get_spikes(w, 0, 20 * 64, 1024, 128, 2)
@@ -795,6 +822,11 @@ def test_loihi_rows_that_are_not_whole_vectors(impl, T, rows, delay):
     assert np.array_equal(bits(host(v)), bits(wv)), "voltage"
     assert np.array_equal(bits(host(u)), bits(wu)), "current"
     assert ws.sum() > 0
+    # without the current among the outputs a tile is 64 rows
+    s2, v2, _ = slayerLoihiCuda.getSpikesDelayed(dev(w), 0, 20 * 64, 1024, 128, 2, delay, voltage=True, current=False)
+    assert np.array_equal(bits(host(s2)), bits(host(s))) and np.array_equal(bits(host(v2)), bits(wv))
+    s3, _, _ = slayerLoihiCuda.getSpikesDelayed(dev(w), 0, 20 * 64, 1024, 128, 2, delay, voltage=False, current=False)
+    assert np.array_equal(bits(host(s3)), bits(host(s)))
 
 
 def test_loihi_unaligned_tensors_take_the_general_kernel():
