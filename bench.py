@@ -552,14 +552,19 @@ def other_rows(device, cpu_leg=False):
     out.append(row("spike_T2000_then_per_neuron_delay_fused", 20, n,
                    timed(lambda u: slayerCuda.getSpikesDelayed(u, ref, 10.0, 1.0, lut, 1.0), K, (pool, restore)), shape, moved=12))
     del x, grad, u0, ub, y, pool
-    # the 77-tap PSP filter over the density of its input: spike trains take the event-driven path tile by tile,
-    # denser tiles the matrix cores
+    # the 77-tap PSP filter over the density of its input, as the sum over the taps (slayerCuda.conv: spike trains
+    # take the event-driven path tile by tile, denser tiles the matrix cores) and as the recursion that the layers
+    # run for their own alpha kernel
     shape = SHAPE
     srm77 = torch.tensor(alphaKernel(10.0, 1.0, 300), dtype=torch.float32, device=device)
     for p in (0.02, 0.05, 0.10, 0.40, None):
         xin = (torch.randn(shape, generator=g) if p is None else (torch.rand(shape, generator=g) < p).float()).to(device)
-        out.append(row("psp_conv77_input_density_%s" % ("dense" if p is None else "%.2f" % p), 8, xin.numel(),
-                       timed(lambda: slayerCuda.conv(xin, srm77, 1.0), K), shape))
+        r = row("psp_conv77_input_density_%s" % ("dense" if p is None else "%.2f" % p), 8, xin.numel(),
+                timed(lambda: slayerCuda.conv(xin, srm77, 1.0), K), shape)
+        rec = timed(lambda: slayerCuda.pspAlpha(xin, srm77, 10.0, 1.0, 1.0, True), K)
+        r["us_as_recursion"] = rec * 1e6
+        r["hbm_frac_as_recursion"] = 8 * xin.numel() / rec / 1e9 / HBM_PEAK_GBS
+        out.append(r)
         del xin
     # MLP ordering spike(psp(fc(x))): dense input to the 77-tap PSP filter, then the spike function
     shape = SHAPE
