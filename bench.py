@@ -625,6 +625,8 @@ def main():
                          "other rows or CPU baseline")
     ap.add_argument("--cnn-only", action="store_true",
                     help="only the NMNIST CNN training step of the other rows (for profiler runs); prints that row")
+    ap.add_argument("--mlp-only", action="store_true",
+                    help="only the NMNIST MLP training step of the other rows (for profiler runs); prints that row")
     ap.add_argument("--delay-only", action="store_true",
                     help="only the long-sequence delay network's training step (for profiler runs); prints that row")
     ap.add_argument("--loihi-only", action="store_true",
@@ -653,7 +655,7 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    if args.cnn_only or args.synapse_only or args.delay_only or args.loihi_only:
+    if args.cnn_only or args.mlp_only or args.synapse_only or args.delay_only or args.loihi_only:
         def wall(fn):
             ts = []
             for _ in range(args.warmup + args.steps):
@@ -665,6 +667,8 @@ def main():
             return float(np.median(ts[args.warmup:]))
         if args.cnn_only:
             print(json.dumps(cnn_row(device, wall)))
+        elif args.mlp_only:
+            print(json.dumps(mlp_row(device, wall)))
         elif args.delay_only:
             print(json.dumps(delay_mlp_row(device, wall)))
         elif args.loihi_only:

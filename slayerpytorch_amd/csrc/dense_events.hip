@@ -1,0 +1,158 @@
+// Weight gradient of the fully connected synapse on sparse input, event by event.
+//
+// The dense layer of the reference (slayer._denseLayer, src/slayer.py:393-440) is a 3-D convolution whose
+// kernel spans the whole (C, H, W) extent of its input: per batch item one matrix product
+// out[O x T] = W[O x K] * x[K x T], K = C*H*W, and its weight gradient is
+//
+//   gradW[o][k] = sum over n, t of gradOut[n][o][t] * x[n][k][t].
+//
+// The input is a spike tensor: a few per cent of x is non-zero, and a sum that skips the zeros does a
+// few per cent of the work.  The rows of x are contiguous in t, so a wavefront that owns an input
+// channel reads them as they are; the output channels o are on the lanes, so what an event fetches is
+// one contiguous row of O floats of the transposed gradient gT[n][t][O] (the caller transposes it; it is
+// small next to x).  The sum runs over the events in ascending (n, t), so the result does not depend on
+// scheduling.  It is the dense product up to the order of the additions (and up to the 0 * inf = NaN
+// terms that a dense product has for non-finite gradients).  The work is proportional to the number
+// of events: for inputs that are not sparse the matrix product of a library is the better choice, and
+// the caller decides.  (The forward product of the same layer was tried the same way - the events of
+// every column (n, t) listed, then summed with the lanes on o: its columns are strided in memory, and
+// listing them alone took as long as half the library's product.)
+#include "common.h"
+
+namespace slayer {
+
+__device__ __forceinline__ float cached_load(BufferRsrc b, int laneBytes, int uniformBytes)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(b, laneBytes, uniformBytes, 0));
+}
+
+struct DenseEventWgradArgs {
+    float *part;  // [slices][K][O]
+    const float *x, *gT;
+    int N, K, O, T;
+    int blocksPerItem;   // ceil(T / 64)
+    int blocksPerSlice;  // blocks of 64 samples per slice
+};
+
+// One wavefront per (input channel k, slice of the batch's samples): it reads the channel's samples 64
+// at a time, and for every non-zero one adds value * gT[n][t][o] to its accumulators (lane l the output
+// channels l + 64 r), four events at a time; part[slice][k][:] takes the sums.  Slices exist so that
+// layers with few input channels still fill the GPU; the caller adds them up.
+template <int OR>
+__global__ __launch_bounds__(64) void dense_events_wgrad_kernel(DenseEventWgradArgs p)
+{
+    const int lane = threadIdx.x;
+    const int k = blockIdx.x % p.K, slice = blockIdx.x / p.K;  // channels of one slice run together: they share gT rows
+    const int blocks = p.N * p.blocksPerItem;
+    const int b0 = slice * p.blocksPerSlice;
+    const int b1 = min(b0 + p.blocksPerSlice, blocks);
+
+    float acc[OR];
+    int oBytes[OR];
+#pragma unroll
+    for (int r = 0; r < OR; ++r) {
+        acc[r] = 0.0f;
+        oBytes[r] = masked_offset(lane + 64 * r < p.O, (lane + 64 * r) * 4);
+    }
+
+    // four blocks of 64 samples at a time, so that their loads travel together
+    for (int b = b0; b < b1; b += 4) {
+        float v[4];
+        int n4[4], t4[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int bj = min(b + j, b1 - 1);
+            n4[j] = bj / p.blocksPerItem;
+            t4[j] = (bj - n4[j] * p.blocksPerItem) * 64;
+            // one row of x: accesses past its end read zeros (and so does a block past the slice's last)
+            const BufferRsrc bx = make_buffer(p.x + (static_cast<int64_t>(n4[j]) * p.K + k) * p.T, p.T * 4);
+            v[j] = buffer_load(bx, masked_offset(b + j < b1, (t4[j] + lane) * 4), 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const BufferRsrc bg = make_buffer(p.gT + static_cast<int64_t>(n4[j]) * p.T * p.O, p.T * p.O * 4);
+            uint64_t todo = __builtin_amdgcn_ballot_w64(v[j] != 0.0f);
+            while (todo != 0) {
+                int tt[4];
+                float val[4], g[4][OR];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool live = todo != 0;
+                    const int pos = live ? __builtin_ctzll(todo) : 0;
+                    todo &= todo - 1;  // (0 stays 0)
+                    tt[i] = t4[j] + pos;
+                    val[i] = live ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v[j]), pos)) : 0.0f;
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int r = 0; r < OR; ++r) g[i][r] = cached_load(bg, oBytes[r], tt[i] * p.O * 4);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int r = 0; r < OR; ++r) acc[r] = fmaf(val[i], g[i][r], acc[r]);
+            }
+        }
+    }
+
+    float *dst = p.part + (static_cast<int64_t>(slice) * p.K + k) * p.O;
+#pragma unroll
+    for (int r = 0; r < OR; ++r)
+        if (lane + 64 * r < p.O) dst[lane + 64 * r] = acc[r];
+}
+
+}  // namespace slayer
+
+namespace {
+
+// Everything the kernel addresses with 32-bit byte offsets: one batch item of gT, one row of x.
+bool dense_events_fits(int64_t N, int64_t K, int64_t O, int64_t T)
+{
+    const int64_t lim = (1LL << 31) - 64;
+    return N < (1LL << 24) && O * T * 4 < lim && T * 4 < lim;
+}
+
+}  // namespace
+
+extern "C" int64_t slayer_dense_events_grad_weight_slices(int64_t N, int64_t K, int64_t O, int64_t T)
+{
+    using namespace slayer;
+    if (N <= 0 || K <= 0 || O <= 0 || T <= 0) return 0;
+    const int64_t blocks = N * ceil_div(T, 64);
+    // about eight wavefronts per SIMD of the whole GPU, each with at least 16 blocks of 64 samples
+    const int64_t want = ceil_div(static_cast<int64_t>(compute_units()) * 32, K);
+    const int64_t most = ceil_div(blocks, 16);
+    int64_t slices = want < most ? want : most;
+    if (slices < 1) slices = 1;
+    const int64_t per = ceil_div(blocks, slices);
+    return ceil_div(blocks, per);
+}
+
+extern "C" int slayer_dense_events_grad_weight_f32(float *part, const float *gT, const float *x, int64_t N,
+                                                   int64_t K, int64_t O, int64_t T, void *stream)
+{
+    using namespace slayer;
+    if (N < 0 || K < 0 || O < 0 || T < 0) return SLAYER_EINVAL;
+    if (K == 0 || O == 0) return SLAYER_OK;
+    if (!part) return SLAYER_EINVAL;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    if (N == 0 || T == 0) return SLAYER_OK;  // no samples, no slices: nothing to write
+    if (!gT || !x) return SLAYER_EINVAL;
+    if (!dense_events_fits(N, K, O, T) || O > 64 * 16) return SLAYER_EUNSUPPORTED;
+    const int64_t slices = slayer_dense_events_grad_weight_slices(N, K, O, T);
+    DenseEventWgradArgs p;
+    p.part = part; p.x = x; p.gT = gT;
+    p.N = static_cast<int>(N); p.K = static_cast<int>(K); p.O = static_cast<int>(O); p.T = static_cast<int>(T);
+    p.blocksPerItem = static_cast<int>(ceil_div(T, 64));
+    const int64_t blocks = N * p.blocksPerItem;
+    if (blocks >= (1LL << 31) || slices * K >= (1LL << 26)) return SLAYER_EUNSUPPORTED;
+    p.blocksPerSlice = static_cast<int>(ceil_div(blocks, slices));
+    const dim3 grid(static_cast<unsigned>(slices * K));
+    const int perLane = static_cast<int>(ceil_div(O, 64));
+    if (perLane <= 1) hipLaunchKernelGGL((dense_events_wgrad_kernel<1>), grid, dim3(64), 0, st, p);
+    else if (perLane <= 2) hipLaunchKernelGGL((dense_events_wgrad_kernel<2>), grid, dim3(64), 0, st, p);
+    else if (perLane <= 4) hipLaunchKernelGGL((dense_events_wgrad_kernel<4>), grid, dim3(64), 0, st, p);
+    else if (perLane <= 8) hipLaunchKernelGGL((dense_events_wgrad_kernel<8>), grid, dim3(64), 0, st, p);
+    else hipLaunchKernelGGL((dense_events_wgrad_kernel<16>), grid, dim3(64), 0, st, p);
+    return launch_status();
+}

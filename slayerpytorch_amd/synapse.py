@@ -14,7 +14,8 @@ import torch
 from . import _lib
 from .slayerCuda import _check_device, _check_input, _on_device_of, _ptr
 
-__all__ = ["conv", "convGradInput", "convGradWeight", "outShape", "supported", "synapseConv", "synapseConvTranspose"]
+__all__ = ["conv", "convGradInput", "convGradWeight", "outShape", "supported", "synapseConv", "synapseConvTranspose",
+           "denseEventsGradWeight", "denseEventsSupported", "synapseDenseEvents"]
 
 
 def _pair(v, name):
@@ -208,3 +209,61 @@ def synapseConvTranspose(input, weight, stride=1, padding=0, dilation=1, groups=
         return torch.nn.functional.conv_transpose3d(input, w5, None, _triple(stride, 1), _triple(padding, 0), 0, groups,
                                                     _triple(dilation, 1))
     return _synapseConvTransposeFunction.apply(input, weight, stride, padding, dilation, groups)
+
+
+def denseEventsSupported(N, K, O, T):
+    """Whether ``denseEventsGradWeight`` takes these extents (the limits the header states)."""
+    lim = (1 << 31) - 64
+    return N < (1 << 24) and O * T * 4 < lim and O <= 1024
+
+
+def denseEventsGradWeight(gradOutput, input):
+    """Weight gradient of the dense layer's product ``out[n] = weight @ input[n]``, ``input`` (N, K, T),
+    ``gradOutput`` (N, O, T): ``sum_n gradOutput[n] @ input[n].T`` as (O, K), summed over the non-zero
+    inputs only, in a fixed order.  The work grows with the number of non-zero inputs."""
+    _check_input(gradOutput, "gradOutput")
+    _check_input(input, "input")
+    _check_device(gradOutput, input, "gradOutput", "input")
+    if input.dim() != 3 or gradOutput.dim() != 3 or gradOutput.shape[0] != input.shape[0] \
+            or gradOutput.shape[2] != input.shape[2]:
+        raise RuntimeError("denseEventsGradWeight takes gradOutput (N, O, T) and input (N, K, T); got %r and %r"
+                           % (tuple(gradOutput.shape), tuple(input.shape)))
+    N, K, T = (int(v) for v in input.shape)
+    O = int(gradOutput.shape[1])
+    lib = _lib.load()
+    slices = int(lib.slayer_dense_events_grad_weight_slices(N, K, O, T))
+    if slices == 0:
+        return torch.zeros((O, K), dtype=input.dtype, device=input.device)
+    gT = gradOutput.transpose(1, 2).contiguous()
+    part = torch.empty((slices, K, O), dtype=input.dtype, device=input.device)
+    with _on_device_of(input) as stream:
+        _lib.check(lib.slayer_dense_events_grad_weight_f32(_ptr(part), _ptr(gT), _ptr(input), N, K, O, T, stream),
+                   "slayer_dense_events_grad_weight_f32")
+    return (part[0] if slices == 1 else part.sum(0)).t()
+
+
+class _synapseDenseEventsFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, weight):
+        ctx.save_for_backward(input, weight)
+        N, K, O = input.shape[0], input.shape[1], weight.shape[0]
+        return torch.bmm(weight.unsqueeze(0).expand(N, O, K), input)
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        input, weight = ctx.saved_tensors
+        gradOutput = gradOutput.contiguous()
+        gradInput = gradWeight = None
+        if ctx.needs_input_grad[0]:
+            N, K, O = input.shape[0], input.shape[1], weight.shape[0]
+            gradInput = torch.bmm(weight.t().unsqueeze(0).expand(N, K, O), gradOutput)
+        if ctx.needs_input_grad[1]:
+            gradWeight = denseEventsGradWeight(gradOutput, input)
+        return gradInput, gradWeight
+
+
+def synapseDenseEvents(input, weight):
+    """``weight @ input[n]`` for every batch item (``input`` (N, K, T), ``weight`` (O, K)) as library matrix
+    products, with the weight gradient summed over the non-zero inputs only (``denseEventsGradWeight``):
+    for inputs that are spike tensors."""
+    return _synapseDenseEventsFunction.apply(input.contiguous(), weight)

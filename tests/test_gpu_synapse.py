@@ -290,3 +290,112 @@ def test_layer_gradients_match_torch_cpu(kind):
     for got, ref in ((yg, yc), (xg.grad, xc.grad), (mod.weight.grad, wc.grad)):
         assert got.shape == ref.shape
         assert float((got.detach().cpu().double() - ref.detach()).abs().max()) <= 1e-5 * float(ref.abs().max())
+
+
+# ------------------------------------------------------- dense layer: weight gradient event by event
+def dense_input(rng, shape, density, binary):
+    x = (rng.random(shape) < density).astype(np.float32)
+    if not binary:
+        x *= rng.standard_normal(shape).astype(np.float32)
+    return x
+
+
+# (N, K, O, T, density, binary input)
+DENSE_EVENT_CASES = [
+    (2, 300, 37, 50, 0.05, True),          # ragged everything
+    (1, 2312, 512, 64, 0.015, True),       # the NMNIST MLP's first layer: eight output channels per lane
+    (3, 200, 256, 130, 0.04, False),       # T % 4 != 0, real-valued events
+    (2, 600, 10, 33, 1.0, False),          # nothing to skip
+    (2, 64, 700, 48, 0.1, True),           # 11 output channels per lane
+    (5, 40, 1024, 70, 0.2, True),          # the most output channels; five blocks: one group of four and one more
+    (4, 7, 3, 5, 0.5, False),              # tiny
+    (2, 513, 65, 16, 0.0, True),           # no events at all
+]
+
+
+@pytest.mark.parametrize("case", DENSE_EVENT_CASES)
+def test_dense_events_weight_gradient(case):
+    N, K, O, T, density, binary = case
+    rng = np.random.default_rng(N + K + O + T)
+    x = dense_input(rng, (N, K, T), density, binary)
+    x[0, 0, : min(T, 3)] = -0.0                               # a negative zero is no event
+    g = rng.standard_normal((N, O, T)).astype(np.float32)
+    refW = np.einsum("not,nkt->ok", g.astype(np.float64), x.astype(np.float64))
+    scaleW = np.einsum("not,nkt->ok", np.abs(g).astype(np.float64), np.abs(x).astype(np.float64))
+    gotW = synapse.denseEventsGradWeight(dev(g), dev(x))
+    close(host(gotW), refW, scaleW)
+    assert torch.equal(gotW, synapse.denseEventsGradWeight(dev(g), dev(x)))      # fixed order of the additions
+    if density == 0.0:
+        assert not host(gotW).any()
+
+
+def test_dense_events_weight_gradient_in_slices():
+    # few input channels and many samples: the batch's samples are cut into slices that the caller adds
+    lib = _lib.load()
+    N, K, O, T = 16, 12, 20, 2000
+    assert lib.slayer_dense_events_grad_weight_slices(N, K, O, T) > 1
+    assert lib.slayer_dense_events_grad_weight_slices(0, K, O, T) == 0
+    rng = np.random.default_rng(5)
+    x = dense_input(rng, (N, K, T), 0.03, True)
+    g = rng.standard_normal((N, O, T)).astype(np.float32)
+    refW = np.einsum("not,nkt->ok", g.astype(np.float64), x.astype(np.float64))
+    scaleW = np.einsum("not,nkt->ok", np.abs(g).astype(np.float64), np.abs(x).astype(np.float64))
+    close(host(synapse.denseEventsGradWeight(dev(g), dev(x))), refW, scaleW)
+
+
+def test_dense_events_status_codes():
+    lib = _lib.load()
+    t = torch.zeros(64, device="cuda")
+    p = t.data_ptr()
+    assert lib.slayer_dense_events_grad_weight_f32(None, None, None, 1, 0, 5, 8, None) == 0     # no weights: nothing to do
+    assert lib.slayer_dense_events_grad_weight_f32(p, None, None, 0, 5, 5, 8, None) == 0        # no samples: no slices
+    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, 1, 5, 1025, 8, None) == 2
+    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, 1, 5, 1024, 1 << 20, None) == 2      # an item of gT over 2 GiB
+    assert lib.slayer_dense_events_grad_weight_f32(None, p, p, 1, 5, 5, 8, None) == 1
+    assert lib.slayer_dense_events_grad_weight_f32(p, None, p, 1, 5, 5, 8, None) == 1
+    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, -1, 5, 5, 8, None) == 1
+    with pytest.raises(_lib.SlayerHipError, match="not supported"):
+        synapse.denseEventsGradWeight(torch.zeros((1, 1025, 8), device="cuda"), torch.zeros((1, 5, 8), device="cuda"))
+
+
+@pytest.mark.parametrize("shape", [((34, 34, 2), 40, 12), (50, 10, 33)])
+def test_dense_layer_sums_its_weight_gradient_over_the_events_of_sparse_input(shape, monkeypatch):
+    """_denseLayer with the event-driven weight gradient against the library product: same output (the forward
+    pass is the same product) and gradients to rounding; left to itself the layer measures its input and
+    picks the events for spike tensors with many channels only."""
+    from slayerpytorch_amd import slayer as slayer_module
+    inFeatures, O, T = shape
+    params = {"type": "SRMALPHA", "theta": 10, "tauSr": 10.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
+    layer = snn.layer(params, {"Ts": 1.0, "tSample": T}).cuda()
+    torch.manual_seed(3)
+    fc = layer.dense(inFeatures, O).cuda()
+    C, H, W = fc.weight.shape[1:4]
+    rng = np.random.default_rng(9)
+    x = dense_input(rng, (3, C, H, W, T), 0.02, True)
+    g = dev(rng.standard_normal((3, O, 1, 1, T)).astype(np.float32))
+    results = []
+    for mode in (True, False):
+        monkeypatch.setattr(slayer_module, "DENSE_EVENTS", mode)
+        xt = dev(x).requires_grad_(True)
+        fc.weight.grad = None
+        y = fc(xt)
+        y.backward(g)
+        results.append((y.detach(), xt.grad.clone(), fc.weight.grad.clone()))
+    assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+    K = C * H * W
+    w2 = host(fc.weight).reshape(O, K).astype(np.float64)
+    x3 = x.reshape(3, K, T).astype(np.float64)
+    g3 = host(g).reshape(3, O, T).astype(np.float64)
+    for y, gx, gw in results:
+        close(host(y).reshape(3, O, T), np.einsum("ok,nkt->not", w2, x3), np.einsum("ok,nkt->not", np.abs(w2), np.abs(x3)))
+        close(host(gx).reshape(3, K, T), np.einsum("ok,not->nkt", w2, g3), np.einsum("ok,not->nkt", np.abs(w2), np.abs(g3)))
+        close(host(gw).reshape(O, K), np.einsum("not,nkt->ok", g3, x3), np.einsum("not,nkt->ok", np.abs(g3), np.abs(x3)))
+    monkeypatch.setattr(slayer_module, "DENSE_EVENTS", "auto")
+    fc(dev(x))
+    many = K >= slayer_module.DENSE_EVENTS_MIN_CHANNELS
+    assert fc._eventsOn is (True if many else None)
+    other = layer.dense(inFeatures, O).cuda()
+    other(dev(rng.standard_normal((3, C, H, W, T)).astype(np.float32)))
+    assert other._eventsOn is (False if many else None)
+    with torch.no_grad():
+        assert not fc._inputIsSparse(dev(x).reshape(3, K, T))      # no gradient, no choice to make
