@@ -18,7 +18,8 @@
  *     calls - with two exceptions, both stated where they are declared: the process-wide test knob
  *     slayer_force_generic_kernels, and the fixed device array of slayer_delay_grad_static_f32.
  *   - The library never allocates device memory.  Outputs (and the workspaces of
- *     slayer_delay_grad_f32, slayer_synapse_conv_grad_weight_f32 and slayer_spike_loss_f32) are allocated by
+ *     slayer_delay_grad_f32, slayer_synapse_conv_grad_weight_f32, slayer_dense_events_grad_weight_f32 and
+ *     slayer_spike_loss_f32) are allocated by
  *     the caller.
  *   - Return value: SLAYER_OK (0) or one of the SLAYER_E* codes; nothing has been launched
  *     when a SLAYER_EINVAL / SLAYER_EUNSUPPORTED code is returned.  Empty tensors
@@ -363,23 +364,23 @@ int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gradOut, cons
 
 /*
  * ---- Fully connected synapse on sparse input: the weight gradient -------------------------------
- * sum over s of part[s][k][o] = sum_{n,t} gT[n][t][o] * x[n][k][t], summed over the non-zero x only, in
- * ascending (n, t): the transposed weight gradient of _denseLayer (src/slayer.py:393-440: an F.conv3d
- * whose kernel spans the whole (C, H, W) extent of the input, i.e. per batch item the matrix product
- * W[O x K] * x[K x T] with K = C*H*W; replaces the weight gradient autograd derives for that call) for
- * inputs that are spike tensors.  x is [N][K][T]; gT is the gradient of the layer's output transposed to
- * [N][T][O]; part is [slices][K][O] with slices = slayer_dense_events_grad_weight_slices(N, K, O, T) (at
- * least 1 when no extent is 0; layers with few input channels are cut along the batch's samples so that
- * they still fill the GPU), every element of which is written; the caller adds the slices.  The result
+ * gradW[o][k] = sum_{n,t} gradOut[n][o][t] * x[n][k][t], summed over the non-zero x only, in ascending
+ * (n, t): the weight gradient of _denseLayer (src/slayer.py:393-440: an F.conv3d whose kernel spans the
+ * whole (C, H, W) extent of the input, i.e. per batch item the matrix product W[O x K] * x[K x T] with
+ * K = C*H*W; replaces the weight gradient autograd derives for that call) for inputs that are spike
+ * tensors.  x is [N][K][T], gradOut [N][O][T], gradW [O][K] (every element is written).  Three launches:
+ * gradOut is transposed to [N][T][O], so that an event fetches one contiguous row; one wavefront per
+ * input channel and slice of the batch's samples sums its events; the slices are added in a fixed
+ * order.  `workspace` holds slayer_dense_events_grad_weight_workspace_bytes(N, K, O, T) bytes.  The result
  * is the dense product up to the order of the additions, and without the 0 * inf = NaN terms a dense
  * product has when gradients are not finite.  The work grows with the number of non-zero inputs: above a
  * few per cent, or with few input channels, a library matrix product is faster, and the caller chooses.
- * O <= 1024, and one batch item of gT must stay below 2 GiB, else SLAYER_EUNSUPPORTED.  With N == 0 or
- * T == 0 there are no slices and nothing is written.
+ * O <= 1024, N <= 65535, and one batch item of gradOut must stay below 2 GiB, else SLAYER_EUNSUPPORTED.
  */
-int64_t slayer_dense_events_grad_weight_slices(int64_t N, int64_t K, int64_t O, int64_t T);
-int slayer_dense_events_grad_weight_f32(float *part, const float *gT, const float *x, int64_t N,
-                                        int64_t K, int64_t O, int64_t T, void *stream);
+int64_t slayer_dense_events_grad_weight_workspace_bytes(int64_t N, int64_t K, int64_t O, int64_t T);
+int slayer_dense_events_grad_weight_f32(float *gradW, const float *gradOut, const float *x,
+                                        float *workspace, int64_t N, int64_t K, int64_t O, int64_t T,
+                                        void *stream);
 
 /*
  * ---- Spike event files to spike tensors -------------------------------------------------------

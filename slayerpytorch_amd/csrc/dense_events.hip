@@ -9,7 +9,7 @@
 // The input is a spike tensor: a few per cent of x is non-zero, and a sum that skips the zeros does a
 // few per cent of the work.  The rows of x are contiguous in t, so a wavefront that owns an input
 // channel reads them as they are; the output channels o are on the lanes, so what an event fetches is
-// one contiguous row of O floats of the transposed gradient gT[n][t][O] (the caller transposes it; it is
+// one contiguous row of O floats of the transposed gradient gT[n][t][O] (transposed here first; it is
 // small next to x).  The sum runs over the events in ascending (n, t), so the result does not depend on
 // scheduling.  It is the dense product up to the order of the additions (and up to the 0 * inf = NaN
 // terms that a dense product has for non-finite gradients).  The work is proportional to the number
@@ -37,7 +37,7 @@ struct DenseEventWgradArgs {
 // One wavefront per (input channel k, slice of the batch's samples): it reads the channel's samples 64
 // at a time, and for every non-zero one adds value * gT[n][t][o] to its accumulators (lane l the output
 // channels l + 64 r), four events at a time; part[slice][k][:] takes the sums.  Slices exist so that
-// layers with few input channels still fill the GPU; the caller adds them up.
+// layers with few input channels still fill the GPU; transpose_sum_kernel adds them up.
 template <int OR>
 __global__ __launch_bounds__(64) void dense_events_wgrad_kernel(DenseEventWgradArgs p)
 {
@@ -101,6 +101,34 @@ __global__ __launch_bounds__(64) void dense_events_wgrad_kernel(DenseEventWgradA
         if (lane + 64 * r < p.O) dst[lane + 64 * r] = acc[r];
 }
 
+// dst[b][c][r] = sum over s of src[b * S + s][r][c]: tiles of 32 x 32 through LDS, so that both sides are
+// read and written along their rows.  Transposes the gradient (S = 1, one matrix per batch item) and adds
+// and transposes the slices of the weight gradient (one batch of S matrices).
+__global__ __launch_bounds__(256) void transpose_sum_kernel(float *__restrict__ dst, const float *__restrict__ src,
+                                                            int S, int R, int C)
+{
+    __shared__ float tile[32][33];
+    const int x = threadIdx.x & 31, y = threadIdx.x >> 5;  // 32 x 8 threads
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    const int64_t matrix = static_cast<int64_t>(R) * C;
+    const float *from = src + static_cast<int64_t>(blockIdx.z) * S * matrix;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int r = r0 + y + 8 * j, c = c0 + x;
+        float sum = 0.0f;
+        if (r < R && c < C)
+            for (int s = 0; s < S; ++s) sum += from[s * matrix + static_cast<int64_t>(r) * C + c];
+        tile[y + 8 * j][x] = sum;
+    }
+    __syncthreads();
+    float *to = dst + static_cast<int64_t>(blockIdx.z) * matrix;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int c = c0 + y + 8 * j, r = r0 + x;
+        if (r < R && c < C) to[static_cast<int64_t>(c) * R + r] = tile[x][y + 8 * j];
+    }
+}
+
 }  // namespace slayer
 
 namespace {
@@ -112,9 +140,7 @@ bool dense_events_fits(int64_t N, int64_t K, int64_t O, int64_t T)
     return N < (1LL << 24) && O * T * 4 < lim && T * 4 < lim;
 }
 
-}  // namespace
-
-extern "C" int64_t slayer_dense_events_grad_weight_slices(int64_t N, int64_t K, int64_t O, int64_t T)
+int64_t dense_events_slices(int64_t N, int64_t K, int64_t O, int64_t T)
 {
     using namespace slayer;
     if (N <= 0 || K <= 0 || O <= 0 || T <= 0) return 0;
@@ -128,25 +154,44 @@ extern "C" int64_t slayer_dense_events_grad_weight_slices(int64_t N, int64_t K, 
     return ceil_div(blocks, per);
 }
 
-extern "C" int slayer_dense_events_grad_weight_f32(float *part, const float *gT, const float *x, int64_t N,
-                                                   int64_t K, int64_t O, int64_t T, void *stream)
+}  // namespace
+
+extern "C" int64_t slayer_dense_events_grad_weight_workspace_bytes(int64_t N, int64_t K, int64_t O, int64_t T)
+{
+    if (N <= 0 || K <= 0 || O <= 0 || T <= 0) return 0;
+    // the transposed gradient [N][T][O], then the slices [slices][K][O]
+    return (N * T * O + dense_events_slices(N, K, O, T) * K * O) * 4;
+}
+
+extern "C" int slayer_dense_events_grad_weight_f32(float *gradW, const float *gradOut, const float *x,
+                                                   float *workspace, int64_t N, int64_t K, int64_t O, int64_t T,
+                                                   void *stream)
 {
     using namespace slayer;
     if (N < 0 || K < 0 || O < 0 || T < 0) return SLAYER_EINVAL;
     if (K == 0 || O == 0) return SLAYER_OK;
-    if (!part) return SLAYER_EINVAL;
+    if (!gradW) return SLAYER_EINVAL;
+    if (N > 0 && T > 0 && (!gradOut || !x || !workspace)) return SLAYER_EINVAL;
+    if (!dense_events_fits(N, K, O, T) || O > 64 * 16 || K * O >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
     const hipStream_t st = static_cast<hipStream_t>(stream);
-    if (N == 0 || T == 0) return SLAYER_OK;  // no samples, no slices: nothing to write
-    if (!gT || !x) return SLAYER_EINVAL;
-    if (!dense_events_fits(N, K, O, T) || O > 64 * 16) return SLAYER_EUNSUPPORTED;
-    const int64_t slices = slayer_dense_events_grad_weight_slices(N, K, O, T);
+    if (N == 0 || T == 0) {  // no samples: the gradient is zero (one slice that is all zeros would do the same)
+        hipLaunchKernelGGL(transpose_sum_kernel, dim3(static_cast<unsigned>(ceil_div(O, 32)), static_cast<unsigned>(ceil_div(K, 32)), 1),
+                           dim3(256), 0, st, gradW, gradW, 0, static_cast<int>(K), static_cast<int>(O));
+        return launch_status();
+    }
+    const int64_t slices = dense_events_slices(N, K, O, T);
+    float *gT = workspace, *part = workspace + N * T * O;
     DenseEventWgradArgs p;
     p.part = part; p.x = x; p.gT = gT;
     p.N = static_cast<int>(N); p.K = static_cast<int>(K); p.O = static_cast<int>(O); p.T = static_cast<int>(T);
     p.blocksPerItem = static_cast<int>(ceil_div(T, 64));
     const int64_t blocks = N * p.blocksPerItem;
-    if (blocks >= (1LL << 31) || slices * K >= (1LL << 26)) return SLAYER_EUNSUPPORTED;
+    if (blocks >= (1LL << 31) || slices * K >= (1LL << 26) || N > 65535 || ceil_div(K, 32) > 65535 || ceil_div(O, 32) > 65535)
+        return SLAYER_EUNSUPPORTED;
     p.blocksPerSlice = static_cast<int>(ceil_div(blocks, slices));
+    // gT[n][t][o] = gradOut[n][o][t]
+    hipLaunchKernelGGL(transpose_sum_kernel, dim3(static_cast<unsigned>(ceil_div(T, 32)), static_cast<unsigned>(ceil_div(O, 32)), static_cast<unsigned>(N)),
+                       dim3(256), 0, st, gT, gradOut, 1, static_cast<int>(O), static_cast<int>(T));
     const dim3 grid(static_cast<unsigned>(slices * K));
     const int perLane = static_cast<int>(ceil_div(O, 64));
     if (perLane <= 1) hipLaunchKernelGGL((dense_events_wgrad_kernel<1>), grid, dim3(64), 0, st, p);
@@ -154,5 +199,8 @@ extern "C" int slayer_dense_events_grad_weight_f32(float *part, const float *gT,
     else if (perLane <= 4) hipLaunchKernelGGL((dense_events_wgrad_kernel<4>), grid, dim3(64), 0, st, p);
     else if (perLane <= 8) hipLaunchKernelGGL((dense_events_wgrad_kernel<8>), grid, dim3(64), 0, st, p);
     else hipLaunchKernelGGL((dense_events_wgrad_kernel<16>), grid, dim3(64), 0, st, p);
+    // gradW[o][k] = sum over the slices of part[s][k][o]
+    hipLaunchKernelGGL(transpose_sum_kernel, dim3(static_cast<unsigned>(ceil_div(O, 32)), static_cast<unsigned>(ceil_div(K, 32)), 1),
+                       dim3(256), 0, st, gradW, part, static_cast<int>(slices), static_cast<int>(K), static_cast<int>(O));
     return launch_status();
 }

@@ -214,7 +214,7 @@ def synapseConvTranspose(input, weight, stride=1, padding=0, dilation=1, groups=
 def denseEventsSupported(N, K, O, T):
     """Whether ``denseEventsGradWeight`` takes these extents (the limits the header states)."""
     lim = (1 << 31) - 64
-    return N < (1 << 24) and O * T * 4 < lim and O <= 1024
+    return N <= 65535 and O * T * 4 < lim and O <= 1024 and K * O < (1 << 31)
 
 
 def denseEventsGradWeight(gradOutput, input):
@@ -231,15 +231,14 @@ def denseEventsGradWeight(gradOutput, input):
     N, K, T = (int(v) for v in input.shape)
     O = int(gradOutput.shape[1])
     lib = _lib.load()
-    slices = int(lib.slayer_dense_events_grad_weight_slices(N, K, O, T))
-    if slices == 0:
-        return torch.zeros((O, K), dtype=input.dtype, device=input.device)
-    gT = gradOutput.transpose(1, 2).contiguous()
-    part = torch.empty((slices, K, O), dtype=input.dtype, device=input.device)
+    gradW = torch.empty((O, K), dtype=input.dtype, device=input.device)
+    nbytes = lib.slayer_dense_events_grad_weight_workspace_bytes(N, K, O, T)
+    workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=input.device)
     with _on_device_of(input) as stream:
-        _lib.check(lib.slayer_dense_events_grad_weight_f32(_ptr(part), _ptr(gT), _ptr(input), N, K, O, T, stream),
+        _lib.check(lib.slayer_dense_events_grad_weight_f32(_ptr(gradW), _ptr(gradOutput), _ptr(input), _ptr(workspace),
+                                                           N, K, O, T, stream),
                    "slayer_dense_events_grad_weight_f32")
-    return (part[0] if slices == 1 else part.sum(0)).t()
+    return gradW
 
 
 class _synapseDenseEventsFunction(torch.autograd.Function):

@@ -330,11 +330,11 @@ def test_dense_events_weight_gradient(case):
 
 
 def test_dense_events_weight_gradient_in_slices():
-    # few input channels and many samples: the batch's samples are cut into slices that the caller adds
+    # few input channels and many samples: the batch's samples are cut into slices that are added up afterwards
     lib = _lib.load()
     N, K, O, T = 16, 12, 20, 2000
-    assert lib.slayer_dense_events_grad_weight_slices(N, K, O, T) > 1
-    assert lib.slayer_dense_events_grad_weight_slices(0, K, O, T) == 0
+    assert lib.slayer_dense_events_grad_weight_workspace_bytes(N, K, O, T) > (N * T * O + K * O) * 4   # more than one slice
+    assert lib.slayer_dense_events_grad_weight_workspace_bytes(0, K, O, T) == 0
     rng = np.random.default_rng(5)
     x = dense_input(rng, (N, K, T), 0.03, True)
     g = rng.standard_normal((N, O, T)).astype(np.float32)
@@ -345,15 +345,19 @@ def test_dense_events_weight_gradient_in_slices():
 
 def test_dense_events_status_codes():
     lib = _lib.load()
-    t = torch.zeros(64, device="cuda")
+    t = torch.full((64,), 7.0, device="cuda")
     p = t.data_ptr()
-    assert lib.slayer_dense_events_grad_weight_f32(None, None, None, 1, 0, 5, 8, None) == 0     # no weights: nothing to do
-    assert lib.slayer_dense_events_grad_weight_f32(p, None, None, 0, 5, 5, 8, None) == 0        # no samples: no slices
-    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, 1, 5, 1025, 8, None) == 2
-    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, 1, 5, 1024, 1 << 20, None) == 2      # an item of gT over 2 GiB
-    assert lib.slayer_dense_events_grad_weight_f32(None, p, p, 1, 5, 5, 8, None) == 1
-    assert lib.slayer_dense_events_grad_weight_f32(p, None, p, 1, 5, 5, 8, None) == 1
-    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, -1, 5, 5, 8, None) == 1
+    assert lib.slayer_dense_events_grad_weight_f32(None, None, None, None, 1, 0, 5, 8, None) == 0     # no weights: nothing to do
+    assert lib.slayer_dense_events_grad_weight_f32(p, None, None, None, 0, 5, 5, 8, None) == 0        # no samples: zeros
+    torch.cuda.synchronize()
+    assert not t[:25].any() and bool((t[25:] == 7.0).all())
+    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, p, 1, 5, 1025, 8, None) == 2
+    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, p, 1, 5, 1024, 1 << 20, None) == 2         # an item of gradOut over 2 GiB
+    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, p, 65536, 5, 5, 8, None) == 2
+    assert lib.slayer_dense_events_grad_weight_f32(None, p, p, p, 1, 5, 5, 8, None) == 1
+    assert lib.slayer_dense_events_grad_weight_f32(p, None, p, p, 1, 5, 5, 8, None) == 1
+    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, None, 1, 5, 5, 8, None) == 1
+    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, p, -1, 5, 5, 8, None) == 1
     with pytest.raises(_lib.SlayerHipError, match="not supported"):
         synapse.denseEventsGradWeight(torch.zeros((1, 1025, 8), device="cuda"), torch.zeros((1, 5, 8), device="cuda"))
 
