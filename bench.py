@@ -49,11 +49,11 @@ def measured_traffic(op):
                                                  "kernel": rec.get("kernels", {}).get(op)}
     except (OSError, ValueError, KeyError):
         return None, None
-KERNEL_OF = {"psp_conv": "slayer::alpha_psp_kernel<true, 4, false, true> (conv with the alpha kernel as a recursion over time)",
+KERNEL_OF = {"psp_conv": "slayer::alpha_psp_kernel<true, 4, 0, true> (conv with the alpha kernel as a recursion over time)",
              "spike": "slayer::spike_tile_kernel<12, 1, 12, 8>",
              "shift": "slayer::shift_vec_kernel<0>", "shift_bwd": "slayer::shift_vec_kernel<0>",
              "spike_bwd": "slayer::spike_bwd_vec_kernel",
-             "psp_corr": "slayer::alpha_psp_kernel<false, 4, false, true> (corr with the alpha kernel as a recursion over time)"}
+             "psp_corr": "slayer::alpha_psp_kernel<false, 4, 0, true> (corr with the alpha kernel as a recursion over time)"}
 
 
 def neuron_params():
@@ -358,9 +358,24 @@ def cnn_row(device, timed):
         for m in mods:
             m.weight.grad = None
 
+    def step_paired():
+        # the same network with every hidden layer's spike function and the next layer's PSP filter as one call
+        # (spikeLayer.spikePsp: same values, one backward kernel for the pair)
+        a = layer.psp(x)
+        for syn in (conv1, pool1, conv2, pool2, conv3):
+            s, a = layer.spikePsp(syn(a))
+        s = layer.spike(fc1(a))
+        error.spikeTime(s, target).backward()
+        for m in mods:
+            m.weight.grad = None
+
     t = timed(step)
-    return {"op": "nmnist_cnn_fwd_loss_bwd", "shape": [12, 2, 34, 34, 300], "us": t * 1e6, "samples_per_s": 12 / t,
-            "spike_rate_per_layer": [round(float(r.detach().mean()), 4) for r in rates]}
+    row = {"op": "nmnist_cnn_fwd_loss_bwd", "shape": [12, 2, 34, 34, 300], "us": t * 1e6, "samples_per_s": 12 / t,
+           "spike_rate_per_layer": [round(float(r.detach().mean()), 4) for r in rates]}
+    tp = timed(step_paired)
+    row["us_with_spike_and_next_psp_as_one_call"] = tp * 1e6
+    row["samples_per_s"] = 12 / min(t, tp)
+    return row
 
 
 SYNAPSE_LAYERS = (

@@ -208,6 +208,21 @@ int slayer_spike_bwd_psp_alpha_f32(float *gradIn, const float *gradOut, const fl
                                    float tauRho, float scale, float Ts, void *stream);
 
 /*
+ * The other order of the same two operations, the backward pass of psp(spike(u)) - what every layer of the
+ * reference's convolutional networks does with its spikes (example/03_NMNIST_CNN/nmnistCNN.py:55-60:
+ * spike(conv(psp(spike(...))))): gradIn = pdf(u) * (corr(gradPsp) + gradSpike), i.e.
+ * _pspFunction.backward (src/slayer.py:888-893) followed by _spikeFunction.backward (src/slayer.py:858-865)
+ * in one kernel, without the intermediate tensor.  gradPsp is the gradient with respect to the PSP signal,
+ * gradSpike (may be NULL) the gradient that reaches the spikes directly; filt, tau, mult as in
+ * slayer_psp_alpha_f32, theta, tauRho, scale as in slayer_spike_bwd_f32.  Only as the recursion: shapes it
+ * does not serve (see slayer_psp_alpha_f32) return SLAYER_EUNSUPPORTED, and the caller runs
+ * slayer_corr_f32, adds, and runs slayer_spike_bwd_f32.
+ */
+int slayer_psp_spike_bwd_alpha_f32(float *gradIn, const float *gradPsp, const float *gradSpike, const float *u,
+                                   const float *filt, int64_t nNeurons, int64_t T, int64_t F, float tau, float mult,
+                                   float theta, float tauRho, float scale, float Ts, void *stream);
+
+/*
  * Spike generation with the time shift that follows it fused into the store of the spikes.
  * Replaces the call pair slayerCuda.getSpikes (src/cuda/slayerKernels.cu:14-39) -> slayerCuda.shift
  * (src/cuda/slayerKernels.cu:77-134) that `delayShift(spike(u), d)` / `delay(spike(u))` make

@@ -44,6 +44,8 @@ SIGNATURES = {
                                             _stream]),
     "slayer_spike_bwd_psp_alpha_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _i64, _i64, _i64, _f32, _f32, _f32,
                                                       _f32, _f32, _f32, _stream]),
+    "slayer_psp_spike_bwd_alpha_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _f32p, _i64, _i64, _i64, _f32, _f32,
+                                                      _f32, _f32, _f32, _f32, _stream]),
     "slayer_spike_bwd_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32, _f32, _f32, _i64, _stream]),
     "slayer_spike_bwd_corr_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _i64, _i64, _i64, _f32, _f32, _f32, _f32,
                                                  _stream]),

@@ -48,18 +48,21 @@ struct AlphaArgs {
     float aL;           // a^L
     float scale;        // Ts * mult * e * Ts / tau
     float Ts;
-    // GATED: the samples are in * gain * exp(-|u - theta| / tauRho) (the spike function's surrogate gradient),
-    // applied on the way into LDS
+    // GATE = 1: the samples are in * gain * exp(-|u - theta| / tauRho) (the spike function's surrogate gradient),
+    // applied on the way into LDS.  GATE = 2: the same factor, of the same positions, multiplies the results on the
+    // way out instead, after `add` (same shape, may be null) has been added to them.
     const float *u;
     float theta, tauRho, gain;
+    const float *add;
 };
 
 // VEC: rows are whole 16-byte vectors (T % 4 == 0).  Otherwise a tile of 4 rows is still a contiguous, 16-byte aligned
 // run of whole vectors (4 T floats) and travels the same way, but a vector may hold the end of one row and the start of
 // the next: the passes then read and write LDS sample by sample, and the way out places every sample in its row.
-template <bool CAUSAL, int R, bool GATED, bool VEC>
+template <bool CAUSAL, int R, int GATE, bool VEC>
 __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
 {
+    constexpr bool GATED = GATE == 1, GATED_OUT = GATE == 2;
     constexpr int kParts = kWave / R;
     constexpr int NB = (R * (kAlphaMaxT / 4) + kWave - 1) / kWave;  // vectors per lane of a tile, at most
     extern __shared__ __align__(16) float lds[];
@@ -77,15 +80,16 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
     // ---- the tile, one contiguous run of vectors, in LDS exactly as it lies in memory (rows behind the last one
     //      arrive as zeros): vector e of the tile is vector e of LDS, no index arithmetic
     bool bad = false;
+    float4 gu[GATE != 0 ? NB : 1];  // the membrane potentials of this lane's vectors (GATE = 2: kept for the way out)
     {
         const BufferRsrc bufIn = make_buffer(p.in + row0 * static_cast<int64_t>(T), nVec * 16);
-        const BufferRsrc bufU = make_buffer((GATED ? p.u : p.in) + row0 * static_cast<int64_t>(T), nVec * 16);
-        float4 x[NB], gu[GATED ? NB : 1];
+        const BufferRsrc bufU = make_buffer((GATE != 0 ? p.u : p.in) + row0 * static_cast<int64_t>(T), nVec * 16);
+        float4 x[NB];
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             if (b * kWave < tileVec) {
                 x[b] = buffer_load4(bufIn, (lane + b * kWave) * 16, 0);
-                if (GATED) gu[b] = buffer_load4(bufU, (lane + b * kWave) * 16, 0);
+                if (GATE != 0) gu[b] = buffer_load4(bufU, (lane + b * kWave) * 16, 0);
             }
         }
 #pragma unroll
@@ -117,7 +121,13 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
             auto sample = [&](int i) { return GATED ? x[i] * spike_pdf(gu[i], p.theta, p.tauRho, p.gain) : x[i]; };
             float acc = 0.0f;
             for (int k = 0; k < taps; ++k) acc = __builtin_fmaf(sample(CAUSAL ? t - k : t + k), p.filt[k], acc);
-            p.out[(row0 + r) * static_cast<int64_t>(T) + t] = acc * p.Ts;
+            acc *= p.Ts;
+            if (GATED_OUT) {
+                const int64_t at = (row0 + r) * static_cast<int64_t>(T) + t;
+                if (p.add) acc += p.add[at];
+                acc *= spike_pdf(p.u[at], p.theta, p.tauRho, p.gain);
+            }
+            p.out[(row0 + r) * static_cast<int64_t>(T) + t] = acc;
         }
         return;
     }
@@ -247,8 +257,17 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
                     }
                     rs = make_float4(rk[0], rk[1], rk[2], rk[3]);
                 }
-                const float4 y = make_float4(scale * __builtin_fmaf(-aL, rs.x, qv.x), scale * __builtin_fmaf(-aL, rs.y, qv.y),
-                                             scale * __builtin_fmaf(-aL, rs.z, qv.z), scale * __builtin_fmaf(-aL, rs.w, qv.w));
+                float4 y = make_float4(scale * __builtin_fmaf(-aL, rs.x, qv.x), scale * __builtin_fmaf(-aL, rs.y, qv.y),
+                                       scale * __builtin_fmaf(-aL, rs.z, qv.z), scale * __builtin_fmaf(-aL, rs.w, qv.w));
+                if (GATED_OUT) {
+                    if (p.add) {
+                        const BufferRsrc bufAdd = make_buffer(p.add + row0 * static_cast<int64_t>(T), nVec * 16);
+                        const float4 more = buffer_load4(bufAdd, (lane + b * kWave) * 16, 0);
+                        y = make_float4(y.x + more.x, y.y + more.y, y.z + more.z, y.w + more.w);
+                    }
+                    y = make_float4(y.x * spike_pdf(gu[b].x, p.theta, p.tauRho, p.gain), y.y * spike_pdf(gu[b].y, p.theta, p.tauRho, p.gain),
+                                    y.z * spike_pdf(gu[b].z, p.theta, p.tauRho, p.gain), y.w * spike_pdf(gu[b].w, p.theta, p.tauRho, p.gain));
+                }
                 buffer_store4(bufOut, (lane + b * kWave) * 16, 0, y);
             }
         }
@@ -262,14 +281,14 @@ namespace slayer {
 // Launches the recursion, or returns false (nothing launched) for shapes it does not serve.
 static bool launch_alpha(float *out, const float *in, const float *filt, int64_t nNeurons, int64_t T, int64_t F, float tau,
                          float mult, float Ts, bool causal, const float *u, float theta, float tauRho, float gain,
-                         hipStream_t st)
+                         hipStream_t st, bool gateOut = false, const float *add = nullptr)
 {
     constexpr int R = kAlphaRows, parts = kWave / R;
     const int64_t tiles = ceil_div(nNeurons, R);
     // rows of whole vectors, or at least a tensor of whole vectors (then every tile of 4 rows is one, too)
     const bool vec = T % 4 == 0;
     if (generic_forced() || (!vec && (nNeurons * T) % 4 != 0) || T > kAlphaMaxT || !aligned16(out) || !aligned16(in) ||
-        (u && !aligned16(u)) || tiles >= (1LL << 31) || F >= (1 << 20))
+        (u && !aligned16(u)) || (add && !aligned16(add)) || tiles >= (1LL << 31) || F >= (1 << 20))
         return false;
     AlphaArgs a{};
     a.out = out; a.in = in; a.filt = filt;
@@ -287,13 +306,15 @@ static bool launch_alpha(float *out, const float *in, const float *filt, int64_t
     a.scale = static_cast<float>(static_cast<double>(Ts) * static_cast<double>(mult) * exp(1.0) * ratio);
     a.Ts = Ts;
     a.u = u; a.theta = theta; a.tauRho = tauRho; a.gain = gain;
+    a.add = add;
     const size_t lds = static_cast<size_t>(2) * R * T * sizeof(float);
     const dim3 grid(static_cast<unsigned>(tiles));
 #define SLAYER_ALPHA_LAUNCH(VEC)                                                                                       \
     do {                                                                                                              \
-        if (u) hipLaunchKernelGGL((alpha_psp_kernel<false, R, true, VEC>), grid, dim3(kWave), lds, st, a);             \
-        else if (causal) hipLaunchKernelGGL((alpha_psp_kernel<true, R, false, VEC>), grid, dim3(kWave), lds, st, a);   \
-        else hipLaunchKernelGGL((alpha_psp_kernel<false, R, false, VEC>), grid, dim3(kWave), lds, st, a);              \
+        if (u && gateOut) hipLaunchKernelGGL((alpha_psp_kernel<false, R, 2, VEC>), grid, dim3(kWave), lds, st, a);    \
+        else if (u) hipLaunchKernelGGL((alpha_psp_kernel<false, R, 1, VEC>), grid, dim3(kWave), lds, st, a);          \
+        else if (causal) hipLaunchKernelGGL((alpha_psp_kernel<true, R, 0, VEC>), grid, dim3(kWave), lds, st, a);      \
+        else hipLaunchKernelGGL((alpha_psp_kernel<false, R, 0, VEC>), grid, dim3(kWave), lds, st, a);                 \
     } while (0)
     if (vec) SLAYER_ALPHA_LAUNCH(true);
     else SLAYER_ALPHA_LAUNCH(false);
@@ -330,4 +351,18 @@ extern "C" int slayer_spike_bwd_psp_alpha_f32(float *gradIn, const float *gradOu
                      static_cast<hipStream_t>(stream)))
         return launch_status();
     return slayer_spike_bwd_corr_f32(gradIn, gradOut, u, filt, nNeurons, T, F, theta, tauRho, scale, Ts, stream);
+}
+
+extern "C" int slayer_psp_spike_bwd_alpha_f32(float *gradIn, const float *gradPsp, const float *gradSpike, const float *u,
+                                              const float *filt, int64_t nNeurons, int64_t T, int64_t F, float tau, float mult,
+                                              float theta, float tauRho, float scale, float Ts, void *stream)
+{
+    using namespace slayer;
+    if (nNeurons < 0 || T < 0 || F < 1 || !(tau > 0.0f) || !(Ts > 0.0f) || tauRho == 0.0f) return SLAYER_EINVAL;
+    if (nNeurons == 0 || T == 0) return SLAYER_OK;
+    if (!gradIn || !gradPsp || !u || !filt) return SLAYER_EINVAL;
+    if (launch_alpha(gradIn, gradPsp, filt, nNeurons, T, F, tau, mult, Ts, false, u, theta, tauRho, scale / tauRho,
+                     static_cast<hipStream_t>(stream), true, gradSpike))
+        return launch_status();
+    return SLAYER_EUNSUPPORTED;  // the caller runs slayer_corr_f32, adds and calls slayer_spike_bwd_f32
 }

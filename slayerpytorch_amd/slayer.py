@@ -133,6 +133,14 @@ class spikeLayer(nn.Module):
         return _pspSpikeFunction.apply(input, self.srmKernel, self.refKernel, self.neuron, self.simulation["Ts"],
                                        self._srmKernelIsAlpha())
 
+    def spikePsp(self, membranePotential):
+        """``s = spike(membranePotential)`` and ``psp(s)``, returned as the pair ``(s, psp(s))`` - what every layer
+        of the reference's convolutional example does with its spikes, ``spike(conv(psp(spike(...))))``
+        (example/03_NMNIST_CNN/nmnistCNN.py:55-60) - as one Function whose backward pass is one kernel
+        (extension; same values as the two calls, gradients to rounding)."""
+        return _spikePspFunction.apply(membranePotential, self.refKernel, self.srmKernel, self.neuron,
+                                       self.simulation["Ts"], self._srmKernelIsAlpha())
+
     def delayShift(self, input, delay, Ts=1):
         """Delays ``input`` in time by ``delay`` (number, one-element tensor, or one value per
         neuron); the gradient flows to ``input`` only."""
@@ -487,6 +495,51 @@ class _pspFunction(torch.autograd.Function):
             gradInput = slayerCuda.pspAlpha(gradOutput.contiguous(), filter, ctx.alpha[0], ctx.alpha[1], ctx.Ts,
                                             causal=False)
         return gradInput, None, None, None
+
+
+class _spikePspFunction(torch.autograd.Function):
+    """``_spikeFunction`` followed by ``_pspFunction`` (src/slayer.py:817-899) with both results as outputs.
+    Forward: ``slayerCuda.getSpikes``, then the PSP filter; backward: correlation of the PSP gradient, plus the
+    gradient that reaches the spikes directly, times the surrogate gradient - one kernel when the PSP kernel
+    is the layer's alpha kernel and the recursion serves the shape, else the three calls."""
+
+    @staticmethod
+    def forward(ctx, membranePotential, refractoryResponse, filter, neuron, Ts, alpha=None):
+        theta = neuron["theta"]
+        ctx.set_materialize_grads(False)   # an output that was not used brings None, not a tensor of zeros
+        spikes = slayerCuda.getSpikes(membranePotential.contiguous(), refractoryResponse, theta, Ts)
+        if alpha is not None and not _recursion_serves(spikes):
+            alpha = None
+        if alpha is None:
+            psp = slayerCuda.conv(spikes, filter, Ts)
+        else:
+            psp = slayerCuda.pspAlpha(spikes, filter, alpha[0], alpha[1], Ts, causal=True)
+        ctx.save_for_backward(membranePotential, filter)
+        ctx.theta = float(theta)
+        ctx.pdfTimeConstant = float(neuron["tauRho"] * neuron["theta"])
+        ctx.pdfScale = float(neuron["scaleRho"])
+        ctx.Ts = float(Ts)
+        ctx.alpha = alpha
+        return spikes, psp
+
+    @staticmethod
+    def backward(ctx, gradSpikes, gradPsp):
+        membranePotential, filter = ctx.saved_tensors
+        u = membranePotential.contiguous()
+        if gradPsp is None and gradSpikes is None:
+            return None, None, None, None, None, None
+        if gradPsp is None:      # only the spikes were used
+            grad = slayerCuda.spikeBackward(gradSpikes.contiguous(), u, ctx.theta, ctx.pdfTimeConstant, ctx.pdfScale)
+        elif ctx.alpha is not None:
+            grad = slayerCuda.pspSpikeBackwardAlpha(gradPsp.contiguous(), None if gradSpikes is None else gradSpikes.contiguous(),
+                                                    u, filter, ctx.alpha[0], ctx.alpha[1], ctx.theta, ctx.pdfTimeConstant,
+                                                    ctx.pdfScale, ctx.Ts)
+        else:
+            grad = slayerCuda.corr(gradPsp.contiguous(), filter, ctx.Ts)
+            if gradSpikes is not None:
+                grad = grad + gradSpikes
+            grad = slayerCuda.spikeBackward(grad, u, ctx.theta, ctx.pdfTimeConstant, ctx.pdfScale)
+        return grad, None, None, None, None, None
 
 
 class _delayLayer(nn.Module):

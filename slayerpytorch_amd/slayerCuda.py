@@ -31,7 +31,8 @@ import torch
 from . import _lib
 
 __all__ = ["getSpikes", "conv", "corr", "shift", "spikeBackward", "spikeBackwardCorr", "pspSpike", "delayGrad",
-           "getSpikesDelayed", "spikeBackwardDelayed", "spikeLoss", "pspAlpha", "spikeBackwardPspAlpha"]
+           "getSpikesDelayed", "spikeBackwardDelayed", "spikeLoss", "pspAlpha", "spikeBackwardPspAlpha",
+           "pspSpikeBackwardAlpha"]
 
 
 def _check_input(x, name):
@@ -193,6 +194,44 @@ def spikeBackwardPspAlpha(gradOutput, membranePotential, filter, tauSr, mult, th
         _lib.check(lib.slayer_spike_bwd_psp_alpha_f32(_ptr(gradInput), _ptr(gradOutput), _ptr(membranePotential), _ptr(filter),
                                                       n, T, filter.numel(), tauSr, mult, theta, tau, scale, Ts, stream),
                    "slayer_spike_bwd_psp_alpha_f32")
+    return gradInput
+
+
+def pspSpikeBackwardAlpha(gradPsp, gradSpike, membranePotential, filter, tauSr, mult, theta, tau, scale, Ts):
+    """Backward pass of ``psp(spike(u))`` for a ``filter`` that holds the alpha kernel of :func:`pspAlpha`
+    (``tauSr``, ``mult``): ``spikeBackward(corr(gradPsp, filter, Ts) + gradSpike, u, theta, tau, scale)`` in one
+    kernel; ``gradSpike`` (the gradient that reaches the spikes directly) may be ``None``.  Shapes the
+    recursion does not serve take those three calls."""
+    _check_input(gradPsp, "gradPsp")
+    _check_input(membranePotential, "membranePotential")
+    _check_input(filter, "filter")
+    _check_device(gradPsp, membranePotential, "gradPsp", "membranePotential")
+    _check_device(gradPsp, filter, "gradPsp", "filter")
+    if gradPsp.shape != membranePotential.shape:
+        raise RuntimeError("gradPsp and membranePotential must have the same shape")
+    if gradSpike is not None:
+        _check_input(gradSpike, "gradSpike")
+        _check_device(gradPsp, gradSpike, "gradPsp", "gradSpike")
+        if gradSpike.shape != gradPsp.shape:
+            raise RuntimeError("gradSpike and gradPsp must have the same shape")
+    if filter.numel() < 1:
+        raise RuntimeError("pspSpikeBackwardAlpha needs a filter of at least one tap")
+    tauSr, mult, theta, tau = _scalar(tauSr, "tauSr"), _scalar(mult, "mult"), _scalar(theta, "theta"), _scalar(tau, "tau")
+    scale, Ts = _scalar(scale, "scale"), _scalar(Ts, "Ts")
+    lib = _lib.load()
+    gradInput = torch.empty_like(gradPsp)
+    n, T = _rows(gradPsp)
+    with _on_device_of(gradPsp) as stream:
+        status = lib.slayer_psp_spike_bwd_alpha_f32(_ptr(gradInput), _ptr(gradPsp),
+                                                    _ptr(gradSpike) if gradSpike is not None else None,
+                                                    _ptr(membranePotential), _ptr(filter), n, T, filter.numel(), tauSr, mult,
+                                                    theta, tau, scale, Ts, stream)
+    if status == 2:  # not a shape for the recursion
+        grad = corr(gradPsp, filter, Ts)
+        if gradSpike is not None:
+            grad = grad + gradSpike
+        return spikeBackward(grad, membranePotential, theta, tau, scale)
+    _lib.check(status, "slayer_psp_spike_bwd_alpha_f32")
     return gradInput
 
 

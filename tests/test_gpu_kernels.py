@@ -363,6 +363,61 @@ def test_spike_backward_psp_alpha_is_spikeBackward_then_corr(impl, shape, tau):
     assert close_to_alpha_sum(host(got), gs, f, tau, 1.0, Ts, False)
 
 
+@pytest.mark.parametrize("shape,tau", [((2, 6, 5, 3, 300), 10.0), ((1, 9, 1, 1, 352), 4.0), ((3, 7, 1, 1, 64), 10.0),
+                                       ((1, 1, 1, 1, 4), 1.0), ((2, 5, 1, 1, 512), 20.0), ((1, 3, 1, 1, 350), 10.0),
+                                       ((1, 2, 1, 1, 1000), 10.0), ((2, 6, 1, 1, 350), 10.0)])
+@pytest.mark.parametrize("direct", [False, True])
+def test_psp_spike_backward_alpha_is_corr_then_spikeBackward(impl, shape, tau, direct):
+    # the other order: the correlation with the alpha kernel as a recursion, plus the gradient that reaches the spikes
+    # directly, times the surrogate gradient on the way out: the values of pspAlpha (+ add) followed by spikeBackward
+    # (the same recursion; the product with the gate rounds once in both), which is the sum over the taps to rounding;
+    # shapes outside the recursion's reach run corr, the addition and spikeBackward
+    rng = np.random.default_rng(shape[-1] + direct)
+    Ts, theta, tauRho, scale = 1.0, 10.0, 10.0, 1.0
+    f = np.array(alphaKernel(tau, Ts, 5000), dtype=np.float32)
+    g = rng.standard_normal(shape).astype(np.float32)
+    gs = rng.standard_normal(shape).astype(np.float32) if direct else None
+    v = (rng.standard_normal(shape) * 4 + 8).astype(np.float32)
+    got = slayerCuda.pspSpikeBackwardAlpha(dev(g), dev(gs) if direct else None, dev(v), dev(f), tau, 1.0, theta, tauRho, scale, Ts)
+    T = shape[-1]
+    recursion = not impl and g.size % 4 == 0 and T <= 512
+    inner = slayerCuda.pspAlpha(dev(g), dev(f), tau, 1.0, Ts, False) if recursion else slayerCuda.corr(dev(g), dev(f), Ts)
+    if direct:
+        inner = inner + dev(gs)
+    two = slayerCuda.spikeBackward(inner, dev(v), theta, tauRho, scale)
+    assert np.array_equal(bits(host(got)), bits(host(two)))
+    pdf = O.spike_bwd(np.ones(shape, np.float32), v, theta, tauRho, scale).astype(np.float64)
+    want = (O.corr(g, f, Ts, fused=True).astype(np.float64) + (gs if direct else 0.0)) * pdf
+    assert rel_err(host(got), want.astype(np.float32)) <= REL_TOL
+    # element by element: the gate scales value and bound alike; the direct term adds one rounding of its own size
+    T_ = shape[-1]
+    h = np.abs(alpha_full(tau, 1.0, Ts, T_ + 1))
+    flat_g = np.abs(g.astype(np.float64)).reshape(-1, T_)
+    bound = np.stack([np.convolve(r[::-1], h)[:T_][::-1] for r in flat_g]).reshape(shape) * Ts
+    if direct:
+        bound = bound + np.abs(gs)
+    assert np.all(np.abs(host(got) - want) <= (1e-5 * bound + 1e-37) * pdf * (1 + 1e-5) + 1e-37)
+
+
+def test_psp_spike_backward_alpha_keeps_non_finite_samples_in_place():
+    rng = np.random.default_rng(22)
+    tau, Ts = 10.0, 1.0
+    f = np.array(alphaKernel(tau, Ts, 300), dtype=np.float32)
+    g = rng.standard_normal((12, 300)).astype(np.float32).reshape(1, 12, 1, 1, 300)
+    v = (rng.standard_normal((12, 300)) * 3 + 8).astype(np.float32).reshape(g.shape)
+    g[0, 1, 0, 0, 150] = np.inf
+    g[0, 10, 0, 0, 40] = np.nan
+    got = slayerCuda.pspSpikeBackwardAlpha(dev(g), None, dev(v), dev(f), tau, 1.0, 10.0, 5.0, 1.0, Ts)
+    # (the tiles with these samples are sums over the taps: corr, then the gate, bit for bit)
+    two = slayerCuda.spikeBackward(slayerCuda.corr(dev(g), dev(f), Ts), dev(v), 10.0, 5.0, 1.0)
+    gotn, twon = host(got).reshape(12, 300), host(two).reshape(12, 300)
+    fin = np.isfinite(twon)
+    assert not fin.all()
+    assert np.array_equal(np.isfinite(gotn), fin) and np.array_equal(gotn[~fin], twon[~fin], equal_nan=True)
+    assert np.array_equal(bits(gotn[0:4]), bits(twon[0:4])) and np.array_equal(bits(gotn[8:12]), bits(twon[8:12]))
+    assert rel_err(np.where(fin, gotn, 0), np.where(fin, twon, 0)) <= REL_TOL
+
+
 def test_spike_backward_psp_alpha_keeps_non_finite_samples_in_place():
     rng = np.random.default_rng(21)
     tau, Ts = 10.0, 1.0

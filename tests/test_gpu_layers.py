@@ -159,6 +159,38 @@ def test_pspSpike_layer_call_matches_spike_of_psp(T):
         assert torch.equal(x1.grad, x2.grad)
 
 
+@pytest.mark.parametrize("T", [300, 350, 600])
+@pytest.mark.parametrize("use", ["psp", "both", "spikes"])
+def test_spikePsp_layer_call_matches_psp_of_spike(T, use):
+    # the CNN ordering psp(spike(u)) of the reference's example: same spikes and PSP signal as the two calls, and one
+    # backward kernel for whichever of the two results were used (T = 600: rows beyond the recursion take the sums over the taps)
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": T}).to(DEV)
+    rng = np.random.default_rng(T)
+    shape = (2, 24, 1, 1, T)
+    u = (rng.standard_normal(shape) * 6 + 3).astype(np.float32)
+    ga, gs = dev(rng.standard_normal(shape).astype(np.float32)), dev(rng.standard_normal(shape).astype(np.float32))
+
+    def loss(s, a):
+        return ((a * ga).sum() if use != "spikes" else 0) + ((s * gs).sum() if use != "psp" else 0)
+
+    u1 = dev(u).requires_grad_(True)
+    w1 = u1 * 1.0                       # (the spike function updates its input in place)
+    s1, a1 = layer.spikePsp(w1)
+    loss(s1, a1).backward()
+    u2 = dev(u).requires_grad_(True)
+    w2 = u2 * 1.0
+    s2 = layer.spike(w2)
+    a2 = layer.psp(s2)
+    loss(s2, a2).backward()
+    assert torch.equal(s1, s2) and torch.equal(a1, a2) and torch.equal(w1, w2) and float(s1.detach().sum()) > 0
+    if use == "spikes" or T % 4 != 0 or T > 512:
+        # (rows of whole vectors beyond the recursion: the separate correlation runs on the matrix cores)
+        assert torch.equal(u1.grad, u2.grad) or (T > 512 and rel_err(host(u1.grad), host(u2.grad)) <= REL_TOL)
+    else:
+        assert torch.equal(u1.grad, u2.grad)
+    assert float(u1.grad.abs().sum()) > 0
+
+
 def test_get_spikes_requires_five_dimensions():
     f = torch.ones(3, device=DEV)
     with pytest.raises(IndexError):
