@@ -18,8 +18,8 @@
  *     calls - with two exceptions, both stated where they are declared: the process-wide test knob
  *     slayer_force_generic_kernels, and the fixed device array of slayer_delay_grad_static_f32.
  *   - The library never allocates device memory.  Outputs (and the workspaces of
- *     slayer_delay_grad_f32, slayer_synapse_conv_grad_weight_f32, slayer_dense_events_grad_weight_f32 and
- *     slayer_spike_loss_f32) are allocated by
+ *     slayer_delay_grad_f32, slayer_synapse_conv_grad_weight_f32, slayer_dense_events_f32,
+ *     slayer_dense_events_grad_weight_f32 and slayer_spike_loss_f32) are allocated by
  *     the caller.
  *   - Return value: SLAYER_OK (0) or one of the SLAYER_E* codes; nothing has been launched
  *     when a SLAYER_EINVAL / SLAYER_EUNSUPPORTED code is returned.  Empty tensors
@@ -378,7 +378,25 @@ int slayer_synapse_conv_grad_weight_f32(float *gradW, const float *gradOut, cons
                                         void *stream);
 
 /*
- * ---- Fully connected synapse on sparse input: the weight gradient -------------------------------
+ * ---- Fully connected synapse on sparse input ---------------------------------------------------
+ * out[n][o][t] = sum_k weight[o][k] * x[n][k][t], summed over the non-zero x only, in ascending k: the
+ * product of _denseLayer.forward (src/slayer.py:435-440: an F.conv3d whose kernel spans the whole
+ * (C, H, W) extent of the input, i.e. per batch item the matrix product W[O x K] * x[K x T] with
+ * K = C*H*W) for inputs that are spike tensors.  x is [N][K][T], weight [O][K], out [N][O][T] (every
+ * element is written).  Four launches: x is transposed to [N][T][K] and weight to [K][O], so that a
+ * column (n, t) of x is a contiguous row whose events fetch contiguous rows of the weights; one wavefront
+ * per column (and slice of the input channels) sums its events; the slices are added and the result goes
+ * back to [N][O][T].  `workspace` holds slayer_dense_events_workspace_bytes(N, K, O, T) bytes.  The result
+ * is the dense product up to the order of the additions, and without the 0 * inf = NaN terms a dense
+ * product has when weights are not finite.  The work grows with the number of non-zero inputs: above a
+ * few per cent, or with few input channels, a library matrix product is faster, and the caller chooses.
+ * O <= 1024, N <= 65535, weight below 2 GiB, else SLAYER_EUNSUPPORTED.
+ */
+int64_t slayer_dense_events_workspace_bytes(int64_t N, int64_t K, int64_t O, int64_t T);
+int slayer_dense_events_f32(float *out, const float *x, const float *weight, float *workspace, int64_t N,
+                            int64_t K, int64_t O, int64_t T, void *stream);
+
+/*
  * gradW[o][k] = sum_{n,t} gradOut[n][o][t] * x[n][k][t], summed over the non-zero x only, in ascending
  * (n, t): the weight gradient of _denseLayer (src/slayer.py:393-440: an F.conv3d whose kernel spans the
  * whole (C, H, W) extent of the input, i.e. per batch item the matrix product W[O x K] * x[K x T] with

@@ -1,22 +1,22 @@
-// Weight gradient of the fully connected synapse on sparse input, event by event.
+// Fully connected synapse on sparse input, event by event.
 //
 // The dense layer of the reference (slayer._denseLayer, src/slayer.py:393-440) is a 3-D convolution whose
 // kernel spans the whole (C, H, W) extent of its input: per batch item one matrix product
-// out[O x T] = W[O x K] * x[K x T], K = C*H*W, and its weight gradient is
+// out[O x T] = W[O x K] * x[K x T], K = C*H*W, with the weight gradient
 //
 //   gradW[o][k] = sum over n, t of gradOut[n][o][t] * x[n][k][t].
 //
 // The input is a spike tensor: a few per cent of x is non-zero, and a sum that skips the zeros does a
-// few per cent of the work.  The rows of x are contiguous in t, so a wavefront that owns an input
-// channel reads them as they are; the output channels o are on the lanes, so what an event fetches is
-// one contiguous row of O floats of the transposed gradient gT[n][t][O] (transposed here first; it is
-// small next to x).  The sum runs over the events in ascending (n, t), so the result does not depend on
-// scheduling.  It is the dense product up to the order of the additions (and up to the 0 * inf = NaN
-// terms that a dense product has for non-finite gradients).  The work is proportional to the number
-// of events: for inputs that are not sparse the matrix product of a library is the better choice, and
-// the caller decides.  (The forward product of the same layer was tried the same way - the events of
-// every column (n, t) listed, then summed with the lanes on o: its columns are strided in memory, and
-// listing them alone took as long as half the library's product.)
+// few per cent of the work.  For the weight gradient the rows of x are contiguous in t, so a wavefront
+// that owns an input channel reads them as they are; the output channels o are on the lanes, so what an
+// event fetches is one contiguous row of O floats of the transposed gradient gT[n][t][O] (transposed here
+// first; it is small next to x).  The sum runs over the events in ascending (n, t), so the result does
+// not depend on scheduling.  The product is the same sum with the roles changed: x transposed to
+// [N][T][K] makes a column (n, t) a contiguous row, whose events fetch rows of the transposed weights
+// wT[K][O]; the result [N][T][O] is transposed back.  Both are the dense products up to the order of the
+// additions (and up to the 0 * inf = NaN terms that a dense product has for non-finite factors).  The work
+// is proportional to the number of events: for inputs that are not sparse the matrix product of a
+// library is the better choice, and the caller decides.
 #include "common.h"
 
 namespace slayer {
@@ -101,23 +101,23 @@ __global__ __launch_bounds__(64) void dense_events_wgrad_kernel(DenseEventWgradA
         if (lane + 64 * r < p.O) dst[lane + 64 * r] = acc[r];
 }
 
-// dst[b][c][r] = sum over s of src[b * S + s][r][c]: tiles of 32 x 32 through LDS, so that both sides are
-// read and written along their rows.  Transposes the gradient (S = 1, one matrix per batch item) and adds
-// and transposes the slices of the weight gradient (one batch of S matrices).
+// dst[b][c][r] = sum over s of src[b][s][r][c], matrix (b, s) of src starting b * batchStride + s * sliceStride
+// floats in: tiles of 32 x 32 through LDS, so that both sides are read and written along their rows.
+// Transposes gradients, inputs and weights (S = 1) and adds and transposes the slices of a result.
 __global__ __launch_bounds__(256) void transpose_sum_kernel(float *__restrict__ dst, const float *__restrict__ src,
-                                                            int S, int R, int C)
+                                                            int S, int R, int C, int64_t batchStride, int64_t sliceStride)
 {
     __shared__ float tile[32][33];
     const int x = threadIdx.x & 31, y = threadIdx.x >> 5;  // 32 x 8 threads
     const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
     const int64_t matrix = static_cast<int64_t>(R) * C;
-    const float *from = src + static_cast<int64_t>(blockIdx.z) * S * matrix;
+    const float *from = src + static_cast<int64_t>(blockIdx.z) * batchStride;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int r = r0 + y + 8 * j, c = c0 + x;
         float sum = 0.0f;
         if (r < R && c < C)
-            for (int s = 0; s < S; ++s) sum += from[s * matrix + static_cast<int64_t>(r) * C + c];
+            for (int s = 0; s < S; ++s) sum += from[s * sliceStride + static_cast<int64_t>(r) * C + c];
         tile[y + 8 * j][x] = sum;
     }
     __syncthreads();
@@ -154,6 +154,41 @@ int64_t dense_events_slices(int64_t N, int64_t K, int64_t O, int64_t T)
     return ceil_div(blocks, per);
 }
 
+// dst[b][c][r] = sum_s src[...][r][c] (see transpose_sum_kernel); false when an extent does not fit a grid
+bool launch_transpose_sum(float *dst, const float *src, int64_t B, int64_t S, int64_t R, int64_t C, int64_t batchStride,
+                          int64_t sliceStride, hipStream_t st)
+{
+    using namespace slayer;
+    if (B > 65535 || ceil_div(R, 32) > 65535 || ceil_div(C, 32) >= (1LL << 31) || R >= (1LL << 31) || C >= (1LL << 31)) return false;
+    hipLaunchKernelGGL(transpose_sum_kernel,
+                       dim3(static_cast<unsigned>(ceil_div(C, 32)), static_cast<unsigned>(ceil_div(R, 32)), static_cast<unsigned>(B)),
+                       dim3(256), 0, st, dst, src, static_cast<int>(S), static_cast<int>(R), static_cast<int>(C), batchStride, sliceStride);
+    return true;
+}
+
+// part[s][k][o] = sum over the non-zero x[n][k][t] of slice s of x[n][k][t] * rows[n][t][o]; returns the number of slices
+// (0: the extents do not fit)
+int64_t launch_events(float *part, const float *rows, const float *x, int64_t N, int64_t K, int64_t O, int64_t T, hipStream_t st)
+{
+    using namespace slayer;
+    const int64_t slices = dense_events_slices(N, K, O, T);
+    DenseEventWgradArgs p;
+    p.part = part; p.x = x; p.gT = rows;
+    p.N = static_cast<int>(N); p.K = static_cast<int>(K); p.O = static_cast<int>(O); p.T = static_cast<int>(T);
+    p.blocksPerItem = static_cast<int>(ceil_div(T, 64));
+    const int64_t blocks = N * p.blocksPerItem;
+    if (blocks >= (1LL << 31) || slices * K >= (1LL << 26) || K >= (1LL << 31)) return 0;
+    p.blocksPerSlice = static_cast<int>(ceil_div(blocks, slices));
+    const dim3 grid(static_cast<unsigned>(slices * K));
+    const int perLane = static_cast<int>(ceil_div(O, 64));
+    if (perLane <= 1) hipLaunchKernelGGL((dense_events_wgrad_kernel<1>), grid, dim3(64), 0, st, p);
+    else if (perLane <= 2) hipLaunchKernelGGL((dense_events_wgrad_kernel<2>), grid, dim3(64), 0, st, p);
+    else if (perLane <= 4) hipLaunchKernelGGL((dense_events_wgrad_kernel<4>), grid, dim3(64), 0, st, p);
+    else if (perLane <= 8) hipLaunchKernelGGL((dense_events_wgrad_kernel<8>), grid, dim3(64), 0, st, p);
+    else hipLaunchKernelGGL((dense_events_wgrad_kernel<16>), grid, dim3(64), 0, st, p);
+    return slices;
+}
+
 }  // namespace
 
 extern "C" int64_t slayer_dense_events_grad_weight_workspace_bytes(int64_t N, int64_t K, int64_t O, int64_t T)
@@ -172,35 +207,58 @@ extern "C" int slayer_dense_events_grad_weight_f32(float *gradW, const float *gr
     if (K == 0 || O == 0) return SLAYER_OK;
     if (!gradW) return SLAYER_EINVAL;
     if (N > 0 && T > 0 && (!gradOut || !x || !workspace)) return SLAYER_EINVAL;
-    if (!dense_events_fits(N, K, O, T) || O > 64 * 16 || K * O >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
+    if (!dense_events_fits(N, K, O, T) || O > 64 * 16 || K * O >= (1LL << 31) || N > 65535 || ceil_div(K, 32) > 65535)
+        return SLAYER_EUNSUPPORTED;
     const hipStream_t st = static_cast<hipStream_t>(stream);
-    if (N == 0 || T == 0) {  // no samples: the gradient is zero (one slice that is all zeros would do the same)
-        hipLaunchKernelGGL(transpose_sum_kernel, dim3(static_cast<unsigned>(ceil_div(O, 32)), static_cast<unsigned>(ceil_div(K, 32)), 1),
-                           dim3(256), 0, st, gradW, gradW, 0, static_cast<int>(K), static_cast<int>(O));
+    if (N == 0 || T == 0) {  // no samples: the gradient is zero (the sum over no slices)
+        launch_transpose_sum(gradW, gradW, 1, 0, K, O, 0, 0, st);
         return launch_status();
     }
     const int64_t slices = dense_events_slices(N, K, O, T);
+    if (slices * K >= (1LL << 26) || N * ceil_div(T, 64) >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
     float *gT = workspace, *part = workspace + N * T * O;
-    DenseEventWgradArgs p;
-    p.part = part; p.x = x; p.gT = gT;
-    p.N = static_cast<int>(N); p.K = static_cast<int>(K); p.O = static_cast<int>(O); p.T = static_cast<int>(T);
-    p.blocksPerItem = static_cast<int>(ceil_div(T, 64));
-    const int64_t blocks = N * p.blocksPerItem;
-    if (blocks >= (1LL << 31) || slices * K >= (1LL << 26) || N > 65535 || ceil_div(K, 32) > 65535 || ceil_div(O, 32) > 65535)
-        return SLAYER_EUNSUPPORTED;
-    p.blocksPerSlice = static_cast<int>(ceil_div(blocks, slices));
     // gT[n][t][o] = gradOut[n][o][t]
-    hipLaunchKernelGGL(transpose_sum_kernel, dim3(static_cast<unsigned>(ceil_div(T, 32)), static_cast<unsigned>(ceil_div(O, 32)), static_cast<unsigned>(N)),
-                       dim3(256), 0, st, gT, gradOut, 1, static_cast<int>(O), static_cast<int>(T));
-    const dim3 grid(static_cast<unsigned>(slices * K));
-    const int perLane = static_cast<int>(ceil_div(O, 64));
-    if (perLane <= 1) hipLaunchKernelGGL((dense_events_wgrad_kernel<1>), grid, dim3(64), 0, st, p);
-    else if (perLane <= 2) hipLaunchKernelGGL((dense_events_wgrad_kernel<2>), grid, dim3(64), 0, st, p);
-    else if (perLane <= 4) hipLaunchKernelGGL((dense_events_wgrad_kernel<4>), grid, dim3(64), 0, st, p);
-    else if (perLane <= 8) hipLaunchKernelGGL((dense_events_wgrad_kernel<8>), grid, dim3(64), 0, st, p);
-    else hipLaunchKernelGGL((dense_events_wgrad_kernel<16>), grid, dim3(64), 0, st, p);
+    launch_transpose_sum(gT, gradOut, N, 1, O, T, O * T, 0, st);
+    launch_events(part, gT, x, N, K, O, T, st);
     // gradW[o][k] = sum over the slices of part[s][k][o]
-    hipLaunchKernelGGL(transpose_sum_kernel, dim3(static_cast<unsigned>(ceil_div(O, 32)), static_cast<unsigned>(ceil_div(K, 32)), 1),
-                       dim3(256), 0, st, gradW, part, static_cast<int>(slices), static_cast<int>(K), static_cast<int>(O));
+    launch_transpose_sum(gradW, part, 1, slices, K, O, 0, K * O, st);
+    return launch_status();
+}
+
+/* The forward product of the same layer on the same kernel: with the input transposed to xT[n][t][k], a column
+ * (n, t) of x is a row whose events fetch rows of the transposed weight matrix wT[k][o]. */
+extern "C" int64_t slayer_dense_events_workspace_bytes(int64_t N, int64_t K, int64_t O, int64_t T)
+{
+    if (N <= 0 || K <= 0 || O <= 0 || T <= 0) return 0;
+    // xT [N][T][K], wT [K][O], the slices [slices][N * T][O]
+    return (N * T * K + K * O + dense_events_slices(1, N * T, O, K) * N * T * O) * 4;
+}
+
+extern "C" int slayer_dense_events_f32(float *out, const float *x, const float *weight, float *workspace, int64_t N,
+                                       int64_t K, int64_t O, int64_t T, void *stream)
+{
+    using namespace slayer;
+    if (N < 0 || K < 0 || O < 0 || T < 0) return SLAYER_EINVAL;
+    if (N == 0 || O == 0 || T == 0) return SLAYER_OK;
+    if (!out) return SLAYER_EINVAL;
+    if (K > 0 && (!x || !weight || !workspace)) return SLAYER_EINVAL;
+    const int64_t lim = (1LL << 31) - 64;
+    if (O > 64 * 16 || O * K * 4 >= lim || K * 4 >= lim || N > 65535 || N * T >= (1LL << 31) || ceil_div(K, 32) > 65535 ||
+        ceil_div(T, 32) > 65535 || ceil_div(O, 32) > 65535)
+        return SLAYER_EUNSUPPORTED;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    if (K == 0) {  // no inputs: zeros (the sum over no slices)
+        launch_transpose_sum(out, out, N, 0, T, O, O * T, 0, st);
+        return launch_status();
+    }
+    const int64_t slices = dense_events_slices(1, N * T, O, K);
+    if (slices * N * T >= (1LL << 26)) return SLAYER_EUNSUPPORTED;
+    float *xT = workspace, *wT = xT + N * T * K, *part = wT + K * O;
+    launch_transpose_sum(xT, x, N, 1, K, T, K * T, 0, st);        // xT[n][t][k] = x[n][k][t]
+    launch_transpose_sum(wT, weight, 1, 1, O, K, 0, 0, st);       // wT[k][o] = weight[o][k]
+    // part[s][(n, t)][o] = sum over the non-zero xT[(n, t)][k] of slice s of xT * wT[k][o]: one batch item of N * T rows
+    launch_events(part, wT, xT, 1, N * T, O, K, st);
+    // out[n][o][t] = sum over the slices of part[s][n * T + t][o]
+    launch_transpose_sum(out, part, N, slices, T, O, T * O, N * T * O, st);
     return launch_status();
 }

@@ -190,13 +190,14 @@ class spikeLayer(nn.Module):
         return F.interpolate(input.reshape(N, C, H, W, 1), size=(H, W, Ns), mode="nearest")
 
 
-# The dense layer's weight gradient event by event (synapse.denseEventsGradWeight) when its input is sparse
-# enough and has enough channels for that to pay: True / False force the choice, "auto" measures the
-# fraction of non-zero inputs of a layer at its first call and at every DENSE_EVENTS_CHECK_EVERY-th one
-# after that (a device-to-host read, so not at every call, and never while a HIP graph is being captured:
-# the last measurement decides then).
+# The dense layer's product and weight gradient event by event (synapse.denseEvents, denseEventsGradWeight)
+# when its input is sparse enough and has enough channels for that to pay: True / False force the choice,
+# "auto" measures the fraction of non-zero inputs of a layer at its first call and at every
+# DENSE_EVENTS_CHECK_EVERY-th one after that (a device-to-host read, so not at every call, and never while a
+# HIP graph is being captured: the last measurement decides then).
 DENSE_EVENTS = "auto"
-DENSE_EVENTS_MAX_DENSITY = 0.03
+DENSE_EVENTS_MAX_DENSITY = 0.03           # weight gradient
+DENSE_EVENTS_MAX_DENSITY_FORWARD = 0.02   # product (its input has to be transposed first)
 DENSE_EVENTS_MIN_CHANNELS = 1024
 DENSE_EVENTS_CHECK_EVERY = 64
 
@@ -221,37 +222,39 @@ class _denseLayer(nn.Conv3d):
             self.weight = nn.Parameter(weightScale * self.weight)
         self.preHookFx = preHookFx
         self._eventCalls = 0
-        self._eventsOn = None
+        self._eventDensity = None
 
     def _inputIsSparse(self, x):
-        """Whether this call's weight gradient is summed over the events (see DENSE_EVENTS)."""
+        """(product, weight gradient): which of the two are summed over the events in this call (see DENSE_EVENTS)."""
         N, K, T = x.shape
         if DENSE_EVENTS is False or not x.is_cuda or x.dtype != torch.float32 or x.numel() == 0 \
-                or not self.weight.requires_grad or not torch.is_grad_enabled() \
                 or not synapse.denseEventsSupported(N, K, self.weight.shape[0], T):
-            return False
+            return False, False
         if DENSE_EVENTS is True:
-            return True
+            return True, True
         if K < DENSE_EVENTS_MIN_CHANNELS:
-            return False
-        if torch.cuda.is_current_stream_capturing():
-            return bool(self._eventsOn)
-        if self._eventsOn is None or self._eventCalls % DENSE_EVENTS_CHECK_EVERY == 0:
-            self._eventsOn = int(torch.count_nonzero(x)) <= DENSE_EVENTS_MAX_DENSITY * x.numel()
-        self._eventCalls += 1
-        return self._eventsOn
+            return False, False
+        if not torch.cuda.is_current_stream_capturing():
+            if self._eventDensity is None or self._eventCalls % DENSE_EVENTS_CHECK_EVERY == 0:
+                self._eventDensity = int(torch.count_nonzero(x)) / x.numel()
+            self._eventCalls += 1
+        if self._eventDensity is None:
+            return False, False
+        return self._eventDensity <= DENSE_EVENTS_MAX_DENSITY_FORWARD, self._eventDensity <= DENSE_EVENTS_MAX_DENSITY
 
     def forward(self, input):
         weight = self.weight if self.preHookFx is None else self.preHookFx(self.weight)
         # The kernel spans the whole (H, W) extent of the input, so the layer is one matrix product
         # per batch item, W[O, C*H*W] x X[C*H*W, T], with time innermost as the tensor already is:
         # a plain library GEMM instead of a 3-D convolution with a degenerate kernel; for the spike
-        # tensors these layers usually see, the weight gradient is a sum over the events instead.
+        # tensors these layers usually see, product and weight gradient are sums over the events instead.
         if input.dim() == 5 and tuple(input.shape[1:4]) == tuple(weight.shape[1:4]) and self.bias is None:
             N, T = input.shape[0], input.shape[4]
             O, K = weight.shape[0], weight.shape[1] * weight.shape[2] * weight.shape[3]
-            if self._inputIsSparse(input.reshape(N, K, T)):
-                return synapse.synapseDenseEvents(input.reshape(N, K, T), weight.reshape(O, K)).reshape(N, O, 1, 1, T)
+            product, gradient = self._inputIsSparse(input.reshape(N, K, T))
+            if product or gradient:
+                return synapse.synapseDenseEvents(input.reshape(N, K, T), weight.reshape(O, K), product,
+                                                  gradient).reshape(N, O, 1, 1, T)
             # batched product with the weight matrix repeated by a zero stride: torch.matmul of a
             # 2-D by a 3-D tensor would first copy the input into a (K, N*T) layout
             return torch.bmm(weight.reshape(1, O, K).expand(N, O, K), input.reshape(N, K, T)).reshape(N, O, 1, 1, T)

@@ -15,7 +15,7 @@ from . import _lib
 from .slayerCuda import _check_device, _check_input, _on_device_of, _ptr
 
 __all__ = ["conv", "convGradInput", "convGradWeight", "outShape", "supported", "synapseConv", "synapseConvTranspose",
-           "denseEventsGradWeight", "denseEventsSupported", "synapseDenseEvents"]
+           "denseEvents", "denseEventsGradWeight", "denseEventsSupported", "synapseDenseEvents"]
 
 
 def _pair(v, name):
@@ -212,9 +212,32 @@ def synapseConvTranspose(input, weight, stride=1, padding=0, dilation=1, groups=
 
 
 def denseEventsSupported(N, K, O, T):
-    """Whether ``denseEventsGradWeight`` takes these extents (the limits the header states)."""
+    """Whether ``denseEvents`` and ``denseEventsGradWeight`` take these extents (the limits the header states)."""
     lim = (1 << 31) - 64
-    return N <= 65535 and O * T * 4 < lim and O <= 1024 and K * O < (1 << 31)
+    return N <= 65535 and O * T * 4 < lim and O <= 1024 and K * O * 4 < lim and 0 < K and N * T < (1 << 22) \
+        and T < (1 << 21)
+
+
+def denseEvents(input, weight):
+    """``weight @ input[n]`` for every batch item, ``input`` (N, K, T), ``weight`` (O, K), summed over the
+    non-zero inputs only (ascending k): the dense layer's product for spike tensors.  The work grows with
+    the number of non-zero inputs."""
+    _check_input(input, "input")
+    _check_input(weight, "weight")
+    _check_device(input, weight, "input", "weight")
+    if input.dim() != 3 or weight.dim() != 2 or weight.shape[1] != input.shape[1]:
+        raise RuntimeError("denseEvents takes input (N, K, T) and weight (O, K); got %r and %r"
+                           % (tuple(input.shape), tuple(weight.shape)))
+    N, K, T = (int(v) for v in input.shape)
+    O = int(weight.shape[0])
+    lib = _lib.load()
+    out = torch.empty((N, O, T), dtype=input.dtype, device=input.device)
+    nbytes = lib.slayer_dense_events_workspace_bytes(N, K, O, T)
+    workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=input.device)
+    with _on_device_of(input) as stream:
+        _lib.check(lib.slayer_dense_events_f32(_ptr(out), _ptr(input), _ptr(weight), _ptr(workspace), N, K, O, T, stream),
+                   "slayer_dense_events_f32")
+    return out
 
 
 def denseEventsGradWeight(gradOutput, input):
@@ -243,8 +266,11 @@ def denseEventsGradWeight(gradOutput, input):
 
 class _synapseDenseEventsFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, input, weight):
+    def forward(ctx, input, weight, product, gradient):
         ctx.save_for_backward(input, weight)
+        ctx.gradient = gradient
+        if product:
+            return denseEvents(input, weight.contiguous())
         N, K, O = input.shape[0], input.shape[1], weight.shape[0]
         return torch.bmm(weight.unsqueeze(0).expand(N, O, K), input)
 
@@ -253,16 +279,20 @@ class _synapseDenseEventsFunction(torch.autograd.Function):
         input, weight = ctx.saved_tensors
         gradOutput = gradOutput.contiguous()
         gradInput = gradWeight = None
-        if ctx.needs_input_grad[0]:
+        if ctx.needs_input_grad[0]:   # the gradient is not sparse: a library product
             N, K, O = input.shape[0], input.shape[1], weight.shape[0]
             gradInput = torch.bmm(weight.t().unsqueeze(0).expand(N, K, O), gradOutput)
         if ctx.needs_input_grad[1]:
-            gradWeight = denseEventsGradWeight(gradOutput, input)
-        return gradInput, gradWeight
+            if ctx.gradient:
+                gradWeight = denseEventsGradWeight(gradOutput, input)
+            else:
+                gradWeight = torch.bmm(gradOutput, input.transpose(1, 2)).sum(0)
+        return gradInput, gradWeight, None, None
 
 
-def synapseDenseEvents(input, weight):
-    """``weight @ input[n]`` for every batch item (``input`` (N, K, T), ``weight`` (O, K)) as library matrix
-    products, with the weight gradient summed over the non-zero inputs only (``denseEventsGradWeight``):
-    for inputs that are spike tensors."""
-    return _synapseDenseEventsFunction.apply(input.contiguous(), weight)
+def synapseDenseEvents(input, weight, product=True, gradient=True):
+    """``weight @ input[n]`` for every batch item (``input`` (N, K, T), ``weight`` (O, K)) with its gradients,
+    for inputs that are spike tensors: the product (``product``) and the weight gradient (``gradient``) summed
+    over the non-zero inputs (``denseEvents``, ``denseEventsGradWeight``) or as library matrix products; the
+    input gradient - a product with the dense output gradient - always from the library."""
+    return _synapseDenseEventsFunction.apply(input.contiguous(), weight, product, gradient)

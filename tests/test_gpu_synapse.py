@@ -292,7 +292,7 @@ def test_layer_gradients_match_torch_cpu(kind):
         assert float((got.detach().cpu().double() - ref.detach()).abs().max()) <= 1e-5 * float(ref.abs().max())
 
 
-# ------------------------------------------------------- dense layer: weight gradient event by event
+# ------------------------------------------------------------------- dense layer, event by event
 def dense_input(rng, shape, density, binary):
     x = (rng.random(shape) < density).astype(np.float32)
     if not binary:
@@ -314,11 +314,19 @@ DENSE_EVENT_CASES = [
 
 
 @pytest.mark.parametrize("case", DENSE_EVENT_CASES)
-def test_dense_events_weight_gradient(case):
+def test_dense_events_product_and_weight_gradient(case):
     N, K, O, T, density, binary = case
     rng = np.random.default_rng(N + K + O + T)
     x = dense_input(rng, (N, K, T), density, binary)
     x[0, 0, : min(T, 3)] = -0.0                               # a negative zero is no event
+    w = rng.standard_normal((O, K)).astype(np.float32)
+    ref = np.einsum("ok,nkt->not", w.astype(np.float64), x.astype(np.float64))
+    scale = np.einsum("ok,nkt->not", np.abs(w).astype(np.float64), np.abs(x).astype(np.float64))
+    got = synapse.denseEvents(dev(x), dev(w))
+    close(host(got), ref, scale)
+    assert torch.equal(got, synapse.denseEvents(dev(x), dev(w)))                 # fixed order of the additions
+    if density == 0.0:
+        assert not host(got).any()
     g = rng.standard_normal((N, O, T)).astype(np.float32)
     refW = np.einsum("not,nkt->ok", g.astype(np.float64), x.astype(np.float64))
     scaleW = np.einsum("not,nkt->ok", np.abs(g).astype(np.float64), np.abs(x).astype(np.float64))
@@ -347,6 +355,17 @@ def test_dense_events_status_codes():
     lib = _lib.load()
     t = torch.full((64,), 7.0, device="cuda")
     p = t.data_ptr()
+    assert lib.slayer_dense_events_f32(None, None, None, None, 0, 5, 5, 8, None) == 0                 # empty: nothing to do
+    u = torch.full((64,), 7.0, device="cuda")
+    assert lib.slayer_dense_events_f32(u.data_ptr(), None, None, None, 2, 0, 3, 5, None) == 0         # no inputs: zeros
+    torch.cuda.synchronize()
+    assert not u[:30].any() and bool((u[30:] == 7.0).all())
+    assert lib.slayer_dense_events_f32(None, p, p, p, 1, 5, 5, 8, None) == 1
+    assert lib.slayer_dense_events_f32(p, p, p, None, 1, 5, 5, 8, None) == 1
+    assert lib.slayer_dense_events_f32(p, p, p, p, 1, 5, 1025, 8, None) == 2
+    assert lib.slayer_dense_events_f32(p, p, p, p, 65536, 5, 5, 8, None) == 2
+    assert lib.slayer_dense_events_f32(p, p, p, p, 1, 1 << 20, 1024, 8, None) == 2                    # weights over 2 GiB
+    assert lib.slayer_dense_events_workspace_bytes(0, 5, 5, 8) == 0
     assert lib.slayer_dense_events_grad_weight_f32(None, None, None, None, 1, 0, 5, 8, None) == 0     # no weights: nothing to do
     assert lib.slayer_dense_events_grad_weight_f32(p, None, None, None, 0, 5, 5, 8, None) == 0        # no samples: zeros
     torch.cuda.synchronize()
@@ -363,10 +382,10 @@ def test_dense_events_status_codes():
 
 
 @pytest.mark.parametrize("shape", [((34, 34, 2), 40, 12), (50, 10, 33)])
-def test_dense_layer_sums_its_weight_gradient_over_the_events_of_sparse_input(shape, monkeypatch):
-    """_denseLayer with the event-driven weight gradient against the library product: same output (the forward
-    pass is the same product) and gradients to rounding; left to itself the layer measures its input and
-    picks the events for spike tensors with many channels only."""
+def test_dense_layer_sums_over_the_events_of_sparse_input(shape, monkeypatch):
+    """_denseLayer with the event-driven product and weight gradient against the library products: same output and
+    gradients to rounding (the input gradient is the library's either way); left to itself the layer measures
+    its input and picks the events for spike tensors with many channels only."""
     from slayerpytorch_amd import slayer as slayer_module
     inFeatures, O, T = shape
     params = {"type": "SRMALPHA", "theta": 10, "tauSr": 10.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
@@ -385,7 +404,7 @@ def test_dense_layer_sums_its_weight_gradient_over_the_events_of_sparse_input(sh
         y = fc(xt)
         y.backward(g)
         results.append((y.detach(), xt.grad.clone(), fc.weight.grad.clone()))
-    assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+    assert torch.equal(results[0][1], results[1][1])
     K = C * H * W
     w2 = host(fc.weight).reshape(O, K).astype(np.float64)
     x3 = x.reshape(3, K, T).astype(np.float64)
@@ -397,9 +416,15 @@ def test_dense_layer_sums_its_weight_gradient_over_the_events_of_sparse_input(sh
     monkeypatch.setattr(slayer_module, "DENSE_EVENTS", "auto")
     fc(dev(x))
     many = K >= slayer_module.DENSE_EVENTS_MIN_CHANNELS
-    assert fc._eventsOn is (True if many else None)
+    assert fc._inputIsSparse(dev(x).reshape(3, K, T)) == ((True, True) if many else (False, False))
+    assert (abs(fc._eventDensity - float((x != 0).mean())) < 1e-6) if many else fc._eventDensity is None
     other = layer.dense(inFeatures, O).cuda()
     other(dev(rng.standard_normal((3, C, H, W, T)).astype(np.float32)))
-    assert other._eventsOn is (False if many else None)
-    with torch.no_grad():
-        assert not fc._inputIsSparse(dev(x).reshape(3, K, T))      # no gradient, no choice to make
+    assert other._inputIsSparse(dev(x).reshape(3, K, T)) == (False, False)      # (the measurement of the last call decides)
+    # in between: the weight gradient alone
+    third = layer.dense(inFeatures, O).cuda()
+    mid = dense_input(rng, (3, C, H, W, T), 0.025, True)
+    third(dev(mid))
+    assert third._inputIsSparse(dev(mid).reshape(3, K, T)) == ((False, True) if many else (False, False))
+    with torch.no_grad():                                          # inference takes the events as well
+        close(host(fc(dev(x))).reshape(3, O, T), np.einsum("ok,nkt->not", w2, x3), np.einsum("ok,nkt->not", np.abs(w2), np.abs(x3)))
