@@ -416,6 +416,16 @@ int slayer_dense_events_grad_weight_f32(float *gradW, const float *gradOut, cons
                                         void *stream);
 
 /*
+ * ---- Weight quantisation of the Loihi layers ---------------------------------------------------
+ * out[i] = round(in[i] / step) * step the way torch evaluates the expression on the GPU for a Python number
+ * `step`: in[i] times the fp32 rounding of the double-precision reciprocal of step, to the nearest integer with
+ * ties to even, times the fp32 rounding of step: quantizeWeights.forward
+ * (src/quantizeParams.py:17-23), which the Loihi layers apply to their weights in every forward pass
+ * (src/slayerLoihi.py:124-139), in one launch.  n <= 2^32 elements; out may be in.
+ */
+int slayer_quantize_f32(float *out, const float *in, int64_t n, double step, void *stream);
+
+/*
  * ---- Spike event files to spike tensors -------------------------------------------------------
  * Decodes packed spike events and bins them into spike tensors, one launch for a batch of samples.
  * Replaces spikeFileIO.read1Dspikes / read2Dspikes / read3Dspikes (src/spikeFileIO.py:162-184,

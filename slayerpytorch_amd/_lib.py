@@ -73,6 +73,7 @@ SIGNATURES = {
     "slayer_synapse_conv_grad_input_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _geomp, _stream]),
     "slayer_synapse_conv_grad_weight_workspace_bytes": (_i64, [_geomp]),
     "slayer_synapse_conv_grad_weight_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _geomp, _stream]),
+    "slayer_quantize_f32": (ctypes.c_int, [_f32p, _f32p, _i64, ctypes.c_double, _stream]),
     "slayer_dense_events_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "slayer_dense_events_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _i64, _i64, _i64, _i64, _stream]),
     "slayer_dense_events_grad_weight_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),

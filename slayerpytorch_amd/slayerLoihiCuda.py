@@ -12,7 +12,7 @@ import torch
 from . import _lib
 from .slayerCuda import _check_input, _on_device_of, _ptr, _rows
 
-__all__ = ["getSpikes", "getSpikesDelayed", "MAX_FUSED_DELAY"]
+__all__ = ["getSpikes", "getSpikesDelayed", "quantize", "MAX_FUSED_DELAY"]
 
 MAX_FUSED_DELAY = 31   # longest spike delay (samples) that getSpikesDelayed fuses into the neuron kernel
 
@@ -88,3 +88,17 @@ def getSpikesDelayed(weightedSpikes, wgtExp, theta, iDecay, vDecay, refDelay, de
             _ptr(weightedSpikes), n, T, wgtExp, theta, iDecay, vDecay, refDelay, delaySteps, stream),
             "slayer_loihi_get_spikes_delayed_f32")
     return [spike, volt, curr]
+
+
+def quantize(weights, step):
+    """``torch.round(weights / step) * step`` (src/quantizeParams.py:17-23) from one kernel, the same values
+    bit for bit.  Has no counterpart in the reference extension."""
+    _check_input(weights, "weights")
+    step = float(step)
+    if step == 0.0 or step != step:
+        raise ValueError("step must be a non-zero number")
+    lib = _lib.load()
+    out = torch.empty_like(weights)
+    with _on_device_of(weights) as stream:
+        _lib.check(lib.slayer_quantize_f32(_ptr(out), _ptr(weights), weights.numel(), step, stream), "slayer_quantize_f32")
+    return out

@@ -797,6 +797,27 @@ def test_loihi_delayed_spikes_and_optional_outputs(impl, shape, delay):
     assert torch.equal(s, two)
 
 
+@pytest.mark.parametrize("step", [2, 1, 0.5, 0.3, 3.0, -2.0, 1e-3])
+def test_loihi_weight_quantiser_is_the_tensor_expression(step):
+    # round(w / step) * step as one kernel: bit for bit what torch makes of the expression on the GPU, ties included
+    rng = np.random.default_rng(3)
+    w = (rng.standard_normal((7, 5, 3, 3, 1)) * 9).astype(np.float32)
+    w.reshape(-1)[:12] = np.array([0.5, 1.5, 2.5, -0.5, -1.5, 3.0, -3.0, 0.0, -0.0, 1.0, 1e9, -1e-9], np.float32) * step
+    wt = dev(w)
+    got = slayerLoihiCuda.quantize(wt, step)
+    want = torch.round(wt / step) * step
+    assert np.array_equal(bits(host(got)), bits(host(want)))
+    from slayerpytorch_amd import slayerLoihi
+    x = dev(w).requires_grad_(True)
+    y = slayerLoihi.quantize(x, step)
+    assert np.array_equal(bits(host(y)), bits(host(want)))
+    y.backward(torch.ones_like(y))
+    assert torch.equal(x.grad, torch.ones_like(x))           # straight-through gradient
+    assert slayerLoihiCuda.quantize(torch.zeros((0,), device="cuda"), 2).numel() == 0
+    with pytest.raises(ValueError):
+        slayerLoihiCuda.quantize(wt, 0)
+
+
 def test_loihi_delay_limits():
     w = dev(np.zeros((2, 3, 40), np.float32))
     with pytest.raises(ValueError):
