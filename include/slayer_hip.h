@@ -408,7 +408,7 @@ int slayer_dense_events_f32(float *out, const float *x, const float *weight, flo
  * is the dense product up to the order of the additions, and without the 0 * inf = NaN terms a dense
  * product has when gradients are not finite.  The work grows with the number of non-zero inputs: above a
  * few per cent, or with few input channels, a library matrix product is faster, and the caller chooses.
- * O <= 1024, N <= 65535, and one batch item of gradOut must stay below 2 GiB, else SLAYER_EUNSUPPORTED.
+ * O <= 1024, N <= 65535, and gradOut must stay below 2 GiB, else SLAYER_EUNSUPPORTED.
  */
 int64_t slayer_dense_events_grad_weight_workspace_bytes(int64_t N, int64_t K, int64_t O, int64_t T);
 int slayer_dense_events_grad_weight_f32(float *gradW, const float *gradOut, const float *x,

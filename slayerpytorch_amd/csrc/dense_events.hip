@@ -34,18 +34,27 @@ struct DenseEventWgradArgs {
     int blocksPerSlice;  // blocks of 64 samples per slice
 };
 
-// One wavefront per (input channel k, slice of the batch's samples): it reads the channel's samples 64
-// at a time, and for every non-zero one adds value * gT[n][t][o] to its accumulators (lane l the output
-// channels l + 64 r), four events at a time; part[slice][k][:] takes the sums.  Slices exist so that
-// layers with few input channels still fill the GPU; transpose_sum_kernel adds them up.
+constexpr int kDeBlocks = 8;  // blocks of 64 samples whose events are listed together
+constexpr int kDeBatch = 8;   // events whose rows are in flight together
+
+// One wavefront per (input channel k, slice of the batch's samples).  It reads the channel's samples 512 at a
+// time (8 loads in flight), lists the non-zero ones - value and byte offset of the row gT[n][t][:] - in
+// LDS in ascending (n, t), and adds value * row to its accumulators (lane l the output channels l + 64 r)
+// eight events at a time, whatever block they came from: at 1-2 % non-zero inputs a block of 64 samples
+// holds about one event, and taking the blocks one by one left every event's fetch a round trip of its
+// own.  part[slice][k][:] takes the sums.  Slices exist so that layers with few input channels still fill
+// the GPU; transpose_sum_kernel adds them up.
 template <int OR>
 __global__ __launch_bounds__(64) void dense_events_wgrad_kernel(DenseEventWgradArgs p)
 {
+    __shared__ float value[kDeBlocks * 64];
+    __shared__ int rowBytes[kDeBlocks * 64];
     const int lane = threadIdx.x;
     const int k = blockIdx.x % p.K, slice = blockIdx.x / p.K;  // channels of one slice run together: they share gT rows
     const int blocks = p.N * p.blocksPerItem;
     const int b0 = slice * p.blocksPerSlice;
     const int b1 = min(b0 + p.blocksPerSlice, blocks);
+    const BufferRsrc bg = make_buffer(p.gT, p.N * p.T * p.O * 4);
 
     float acc[OR];
     int oBytes[OR];
@@ -55,44 +64,50 @@ __global__ __launch_bounds__(64) void dense_events_wgrad_kernel(DenseEventWgradA
         oBytes[r] = masked_offset(lane + 64 * r < p.O, (lane + 64 * r) * 4);
     }
 
-    // four blocks of 64 samples at a time, so that their loads travel together
-    for (int b = b0; b < b1; b += 4) {
-        float v[4];
-        int n4[4], t4[4];
+    for (int b = b0; b < b1; b += kDeBlocks) {
+        float v[kDeBlocks];
+        int sample[kDeBlocks];  // n * T + t of this lane's sample of block j
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kDeBlocks; ++j) {
             const int bj = min(b + j, b1 - 1);
-            n4[j] = bj / p.blocksPerItem;
-            t4[j] = (bj - n4[j] * p.blocksPerItem) * 64;
+            const int n = bj / p.blocksPerItem;
+            const int t0 = (bj - n * p.blocksPerItem) * 64;
             // one row of x: accesses past its end read zeros (and so does a block past the slice's last)
-            const BufferRsrc bx = make_buffer(p.x + (static_cast<int64_t>(n4[j]) * p.K + k) * p.T, p.T * 4);
-            v[j] = buffer_load(bx, masked_offset(b + j < b1, (t4[j] + lane) * 4), 0);
+            const BufferRsrc bx = make_buffer(p.x + (static_cast<int64_t>(n) * p.K + k) * p.T, p.T * 4);
+            v[j] = buffer_load(bx, masked_offset(b + j < b1, (t0 + lane) * 4), 0);
+            sample[j] = n * p.T + t0 + lane;
         }
+        int m = 0;  // events of these blocks
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const BufferRsrc bg = make_buffer(p.gT + static_cast<int64_t>(n4[j]) * p.T * p.O, p.T * p.O * 4);
-            uint64_t todo = __builtin_amdgcn_ballot_w64(v[j] != 0.0f);
-            while (todo != 0) {
-                int tt[4];
-                float val[4], g[4][OR];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const bool live = todo != 0;
-                    const int pos = live ? __builtin_ctzll(todo) : 0;
-                    todo &= todo - 1;  // (0 stays 0)
-                    tt[i] = t4[j] + pos;
-                    val[i] = live ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v[j]), pos)) : 0.0f;
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int r = 0; r < OR; ++r) g[i][r] = cached_load(bg, oBytes[r], tt[i] * p.O * 4);
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int r = 0; r < OR; ++r) acc[r] = fmaf(val[i], g[i][r], acc[r]);
+        for (int j = 0; j < kDeBlocks; ++j) {
+            const bool nz = v[j] != 0.0f;
+            const uint64_t mask = __builtin_amdgcn_ballot_w64(nz);
+            const int at = m + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0));
+            if (nz) {
+                value[at] = v[j];
+                rowBytes[at] = sample[j] * p.O * 4;
             }
+            m += __builtin_popcountll(mask);
         }
+        wave_sync();
+        for (int e = 0; e < m; e += kDeBatch) {
+            float val[kDeBatch], g[kDeBatch][OR];
+#pragma unroll
+            for (int i = 0; i < kDeBatch; ++i) {
+                // entries past the end of the list are stale: row 0 with value 0 instead
+                const bool live = e + i < m;
+                const int at = (e + i) & (kDeBlocks * 64 - 1);
+                val[i] = live ? value[at] : 0.0f;
+                const int row = __builtin_amdgcn_readfirstlane(live ? rowBytes[at] : 0);
+#pragma unroll
+                for (int r = 0; r < OR; ++r) g[i][r] = cached_load(bg, oBytes[r], row);
+            }
+#pragma unroll
+            for (int i = 0; i < kDeBatch; ++i)
+#pragma unroll
+                for (int r = 0; r < OR; ++r) acc[r] = fmaf(val[i], g[i][r], acc[r]);
+        }
+        wave_sync();  // the lists are rewritten by the next round
     }
 
     float *dst = p.part + (static_cast<int64_t>(slice) * p.K + k) * p.O;
@@ -102,30 +117,37 @@ __global__ __launch_bounds__(64) void dense_events_wgrad_kernel(DenseEventWgradA
 }
 
 // dst[b][c][r] = sum over s of src[b][s][r][c], matrix (b, s) of src starting b * batchStride + s * sliceStride
-// floats in: tiles of 32 x 32 through LDS, so that both sides are read and written along their rows.
+// floats in: tiles of 32 x 32 (64 x 64 for large single matrices: 256 bytes of a row at a time) through LDS, so
+// that both sides are read and written along their rows.
 // Transposes gradients, inputs and weights (S = 1) and adds and transposes the slices of a result.
+template <int TILE>
 __global__ __launch_bounds__(256) void transpose_sum_kernel(float *__restrict__ dst, const float *__restrict__ src,
                                                             int S, int R, int C, int64_t batchStride, int64_t sliceStride)
 {
-    __shared__ float tile[32][33];
-    const int x = threadIdx.x & 31, y = threadIdx.x >> 5;  // 32 x 8 threads
-    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    __shared__ float tile[TILE][TILE + 1];
+    constexpr int ROWS = 256 / TILE;  // rows of the tile that the 256 threads cover at a time
+    const int x = threadIdx.x % TILE, y = threadIdx.x / TILE;
+    const int c0 = blockIdx.x * TILE, r0 = blockIdx.y * TILE;
     const int64_t matrix = static_cast<int64_t>(R) * C;
     const float *from = src + static_cast<int64_t>(blockIdx.z) * batchStride;
+    float v[TILE / ROWS];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int r = r0 + y + 8 * j, c = c0 + x;
-        float sum = 0.0f;
-        if (r < R && c < C)
-            for (int s = 0; s < S; ++s) sum += from[s * sliceStride + static_cast<int64_t>(r) * C + c];
-        tile[y + 8 * j][x] = sum;
+    for (int j = 0; j < TILE / ROWS; ++j) v[j] = 0.0f;
+    for (int s = 0; s < S; ++s) {  // (the loads of a slice in flight together)
+#pragma unroll
+        for (int j = 0; j < TILE / ROWS; ++j) {
+            const int r = r0 + y + ROWS * j, c = c0 + x;
+            v[j] += (r < R && c < C) ? from[s * sliceStride + static_cast<int64_t>(r) * C + c] : 0.0f;
+        }
     }
+#pragma unroll
+    for (int j = 0; j < TILE / ROWS; ++j) tile[y + ROWS * j][x] = v[j];
     __syncthreads();
     float *to = dst + static_cast<int64_t>(blockIdx.z) * matrix;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int c = c0 + y + 8 * j, r = r0 + x;
-        if (r < R && c < C) to[static_cast<int64_t>(c) * R + r] = tile[x][y + 8 * j];
+#pragma unroll 4
+    for (int j = 0; j < TILE / ROWS; ++j) {
+        const int c = c0 + y + ROWS * j, r = r0 + x;
+        if (r < R && c < C) to[static_cast<int64_t>(c) * R + r] = tile[x][y + ROWS * j];
     }
 }
 
@@ -133,11 +155,11 @@ __global__ __launch_bounds__(256) void transpose_sum_kernel(float *__restrict__ 
 
 namespace {
 
-// Everything the kernel addresses with 32-bit byte offsets: one batch item of gT, one row of x.
+// Everything the kernel addresses with 32-bit byte offsets: gT, one row of x.
 bool dense_events_fits(int64_t N, int64_t K, int64_t O, int64_t T)
 {
     const int64_t lim = (1LL << 31) - 64;
-    return N < (1LL << 24) && O * T * 4 < lim && T * 4 < lim;
+    return N < (1LL << 24) && N * O * T * 4 < lim && T * 4 < lim;
 }
 
 int64_t dense_events_slices(int64_t N, int64_t K, int64_t O, int64_t T)
@@ -160,9 +182,14 @@ bool launch_transpose_sum(float *dst, const float *src, int64_t B, int64_t S, in
 {
     using namespace slayer;
     if (B > 65535 || ceil_div(R, 32) > 65535 || ceil_div(C, 32) >= (1LL << 31) || R >= (1LL << 31) || C >= (1LL << 31)) return false;
-    hipLaunchKernelGGL(transpose_sum_kernel,
-                       dim3(static_cast<unsigned>(ceil_div(C, 32)), static_cast<unsigned>(ceil_div(R, 32)), static_cast<unsigned>(B)),
-                       dim3(256), 0, st, dst, src, static_cast<int>(S), static_cast<int>(R), static_cast<int>(C), batchStride, sliceStride);
+    if (S == 1 && R * C >= (1LL << 19))
+        hipLaunchKernelGGL(transpose_sum_kernel<64>,
+                           dim3(static_cast<unsigned>(ceil_div(C, 64)), static_cast<unsigned>(ceil_div(R, 64)), static_cast<unsigned>(B)),
+                           dim3(256), 0, st, dst, src, static_cast<int>(S), static_cast<int>(R), static_cast<int>(C), batchStride, sliceStride);
+    else
+        hipLaunchKernelGGL(transpose_sum_kernel<32>,
+                           dim3(static_cast<unsigned>(ceil_div(C, 32)), static_cast<unsigned>(ceil_div(R, 32)), static_cast<unsigned>(B)),
+                           dim3(256), 0, st, dst, src, static_cast<int>(S), static_cast<int>(R), static_cast<int>(C), batchStride, sliceStride);
     return true;
 }
 

@@ -196,8 +196,8 @@ class spikeLayer(nn.Module):
 # DENSE_EVENTS_CHECK_EVERY-th one after that (a device-to-host read, so not at every call, and never while a
 # HIP graph is being captured: the last measurement decides then).
 DENSE_EVENTS = "auto"
-DENSE_EVENTS_MAX_DENSITY = 0.03           # weight gradient
-DENSE_EVENTS_MAX_DENSITY_FORWARD = 0.02   # product (its input has to be transposed first)
+DENSE_EVENTS_MAX_DENSITY = 0.05           # weight gradient
+DENSE_EVENTS_MAX_DENSITY_FORWARD = 0.03   # product (its input has to be transposed first)
 DENSE_EVENTS_MIN_CHANNELS = 1024
 DENSE_EVENTS_CHECK_EVERY = 64
 

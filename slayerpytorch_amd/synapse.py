@@ -214,7 +214,7 @@ def synapseConvTranspose(input, weight, stride=1, padding=0, dilation=1, groups=
 def denseEventsSupported(N, K, O, T):
     """Whether ``denseEvents`` and ``denseEventsGradWeight`` take these extents (the limits the header states)."""
     lim = (1 << 31) - 64
-    return N <= 65535 and O * T * 4 < lim and O <= 1024 and K * O * 4 < lim and 0 < K and N * T < (1 << 22) \
+    return N <= 65535 and N * O * T * 4 < lim and O <= 1024 and K * O * 4 < lim and 0 < K and N * T < (1 << 22) \
         and T < (1 << 21)
 
 

@@ -371,7 +371,7 @@ def test_dense_events_status_codes():
     torch.cuda.synchronize()
     assert not t[:25].any() and bool((t[25:] == 7.0).all())
     assert lib.slayer_dense_events_grad_weight_f32(p, p, p, p, 1, 5, 1025, 8, None) == 2
-    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, p, 1, 5, 1024, 1 << 20, None) == 2         # an item of gradOut over 2 GiB
+    assert lib.slayer_dense_events_grad_weight_f32(p, p, p, p, 2, 5, 1024, 1 << 18, None) == 2         # gradOut of 2 GiB
     assert lib.slayer_dense_events_grad_weight_f32(p, p, p, p, 65536, 5, 5, 8, None) == 2
     assert lib.slayer_dense_events_grad_weight_f32(None, p, p, p, 1, 5, 5, 8, None) == 1
     assert lib.slayer_dense_events_grad_weight_f32(p, None, p, p, 1, 5, 5, 8, None) == 1
@@ -423,7 +423,7 @@ def test_dense_layer_sums_over_the_events_of_sparse_input(shape, monkeypatch):
     assert other._inputIsSparse(dev(x).reshape(3, K, T)) == (False, False)      # (the measurement of the last call decides)
     # in between: the weight gradient alone
     third = layer.dense(inFeatures, O).cuda()
-    mid = dense_input(rng, (3, C, H, W, T), 0.025, True)
+    mid = dense_input(rng, (3, C, H, W, T), 0.04, True)
     third(dev(mid))
     assert third._inputIsSparse(dev(mid).reshape(3, K, T)) == ((False, True) if many else (False, False))
     with torch.no_grad():                                          # inference takes the events as well
