@@ -84,7 +84,18 @@ class spikeLayer(nn.Module):
         gradient run as a recursion over time (``slayerCuda.pspAlpha``), which agrees with the
         sum over the taps to rounding; a kernel that was replaced or edited takes the sums."""
         alpha = self._srmKernelIsAlpha()
-        return _pspFunction.apply(spike, self.srmKernel, self.simulation["Ts"], alpha)
+        origin = getattr(spike, "_slayerSpikeOf", None) if PAIR_SPIKE_PSP and alpha is not None else None
+        if origin is not None and torch.is_grad_enabled() and spike.requires_grad and _recursion_serves(spike) \
+                and spike._version == origin[4] and type(spike.grad_fn).__name__ == "_spikeFunctionBackward":
+            membranePotential, theta, pdfTimeConstant, pdfScale, _ = origin
+            if membranePotential.shape == spike.shape and membranePotential.is_contiguous():
+                return _pspOfSpikeFunction.apply(spike, membranePotential, self.srmKernel, self.simulation["Ts"], alpha,
+                                                 theta, pdfTimeConstant, pdfScale)
+        psp = _pspFunction.apply(spike, self.srmKernel, self.simulation["Ts"], alpha)
+        if PAIR_SPIKE_PSP and alpha is not None and psp.requires_grad and _recursion_serves(spike):
+            # for spike(): what this signal was filtered from, and that it has not been touched since
+            psp._slayerPspOf = (spike, self.srmKernel, alpha, psp._version)
+        return psp
 
     def _srmKernelIsAlpha(self):
         """(tau, mult) when ``srmKernel`` still holds ``alphaKernel(tauSr, ...)`` and the recursion
@@ -108,7 +119,22 @@ class spikeLayer(nn.Module):
     def spike(self, membranePotential):
         """Spike function with refractory response.  A contiguous ``membranePotential`` is
         updated in place with the refractory response, as in the reference."""
-        return _spikeFunction.apply(membranePotential, self.refKernel, self.neuron, self.simulation["Ts"])
+        origin = getattr(membranePotential, "_slayerPspOf", None) if PAIR_SPIKE_PSP else None
+        if origin is not None and torch.is_grad_enabled() and membranePotential.requires_grad \
+                and membranePotential.is_contiguous() and membranePotential._version == origin[3] \
+                and type(membranePotential.grad_fn).__name__ == "_pspFunctionBackward" \
+                and origin[0].shape == membranePotential.shape:
+            # spike(psp(x)), the ordering of the reference's MLP example: the spikes' gradient goes past the PSP
+            # filter straight to x, surrogate gradient and correlation in one kernel
+            return _spikeOfPspFunction.apply(membranePotential, origin[0], self.refKernel, origin[1], self.neuron,
+                                             self.simulation["Ts"], origin[2])
+        spikes = _spikeFunction.apply(membranePotential, self.refKernel, self.neuron, self.simulation["Ts"])
+        if PAIR_SPIKE_PSP and spikes.requires_grad:
+            # for psp(): which potential these spikes came from, and that they have not been touched since
+            spikes._slayerSpikeOf = (membranePotential, float(self.neuron["theta"]),
+                                     float(self.neuron["tauRho"] * self.neuron["theta"]), float(self.neuron["scaleRho"]),
+                                     spikes._version)
+        return spikes
 
     def spikeDelayed(self, membranePotential, delay, Ts=None):
         """``delayShift(spike(membranePotential), delay, Ts)`` or, with a ``_delayLayer`` as ``delay``,
@@ -188,6 +214,16 @@ class spikeLayer(nn.Module):
         if mode != "nearest":
             raise Exception("Unsupported mode. It was {}".format(mode))
         return F.interpolate(input.reshape(N, C, H, W, 1), size=(H, W, Ns), mode="nearest")
+
+
+# psp(s) of a tensor s that spike() has just returned - what the layers of the reference's convolutional example
+# do, spike(conv(psp(spike(...)))) - sends its gradient past the spike function straight to the membrane
+# potential: correlation and surrogate gradient in one kernel (slayerCuda.pspSpikeBackwardAlpha) instead of
+# two with a tensor in between.  Gradients that reach s from elsewhere still pass through the spike function's
+# own backward pass; the sum at the membrane potential is the same.  Likewise spike(u) of a signal u that psp() has
+# just returned - the ordering of the reference's MLP example, spike(psp(fc(x))) - sends the spikes' gradient past
+# the PSP filter (slayerCuda.spikeBackwardPspAlpha).  False keeps the two Functions apart.
+PAIR_SPIKE_PSP = True
 
 
 # The dense layer's product and weight gradient event by event (synapse.denseEvents, denseEventsGradWeight)
@@ -381,6 +417,7 @@ class _spikeFunction(torch.autograd.Function):
         # caller's, exactly as in the reference.
         spikes = slayerCuda.getSpikes(membranePotential.contiguous(), refractoryResponse, theta, Ts)
         ctx.save_for_backward(membranePotential)
+        ctx.set_materialize_grads(False)   # no gradient for the spikes: no kernel, not a tensor of zeros through it
         ctx.theta = float(theta)
         ctx.pdfTimeConstant = float(neuron["tauRho"] * neuron["theta"])
         ctx.pdfScale = float(neuron["scaleRho"])
@@ -388,6 +425,8 @@ class _spikeFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gradOutput):
+        if gradOutput is None:
+            return None, None, None, None
         (membranePotential,) = ctx.saved_tensors
         gradInput = slayerCuda.spikeBackward(gradOutput.contiguous(), membranePotential.contiguous(),
                                              ctx.theta, ctx.pdfTimeConstant, ctx.pdfScale)
@@ -485,12 +524,15 @@ class _pspFunction(torch.autograd.Function):
         else:
             psp = slayerCuda.pspAlpha(spike.contiguous(), filter, alpha[0], alpha[1], Ts, causal=True)
         ctx.save_for_backward(filter)
+        ctx.set_materialize_grads(False)   # no gradient for the signal: no kernel, not a tensor of zeros through it
         ctx.Ts = float(Ts)
         ctx.alpha = alpha
         return psp
 
     @staticmethod
     def backward(ctx, gradOutput):
+        if gradOutput is None:
+            return None, None, None, None
         (filter,) = ctx.saved_tensors
         if ctx.alpha is None:
             gradInput = slayerCuda.corr(gradOutput.contiguous(), filter, ctx.Ts)
@@ -498,6 +540,59 @@ class _pspFunction(torch.autograd.Function):
             gradInput = slayerCuda.pspAlpha(gradOutput.contiguous(), filter, ctx.alpha[0], ctx.alpha[1], ctx.Ts,
                                             causal=False)
         return gradInput, None, None, None
+
+
+class _spikeOfPspFunction(torch.autograd.Function):
+    """``_spikeFunction`` (src/slayer.py:817-865) for a membrane potential that ``_pspFunction`` has just produced
+    from ``pspInput`` with the alpha kernel as a recursion.  Forward: the spike function.  Backward: the gradient
+    goes to ``pspInput`` directly - surrogate gradient, then the correlation of ``_pspFunction.backward``
+    (src/slayer.py:888-893), in one kernel - and nothing to ``membranePotential``, whose producer then only
+    carries what reaches the potential from elsewhere."""
+
+    @staticmethod
+    def forward(ctx, membranePotential, pspInput, refractoryResponse, filter, neuron, Ts, alpha):
+        spikes = slayerCuda.getSpikes(membranePotential, refractoryResponse, neuron["theta"], Ts)
+        ctx.save_for_backward(membranePotential, filter)
+        ctx.set_materialize_grads(False)
+        ctx.alpha, ctx.Ts = alpha, float(Ts)
+        ctx.theta = float(neuron["theta"])
+        ctx.pdfTimeConstant = float(neuron["tauRho"] * neuron["theta"])
+        ctx.pdfScale = float(neuron["scaleRho"])
+        return spikes
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        grad = None
+        if gradOutput is not None and ctx.needs_input_grad[1]:
+            membranePotential, filter = ctx.saved_tensors
+            grad = slayerCuda.spikeBackwardPspAlpha(gradOutput.contiguous(), membranePotential, filter, ctx.alpha[0],
+                                                    ctx.alpha[1], ctx.theta, ctx.pdfTimeConstant, ctx.pdfScale, ctx.Ts)
+        return None, grad, None, None, None, None, None
+
+
+class _pspOfSpikeFunction(torch.autograd.Function):
+    """``_pspFunction`` (src/slayer.py:875-899) for a spike tensor that ``_spikeFunction`` has just produced from
+    ``membranePotential``, with the alpha kernel as a recursion.  Forward: the PSP filter.  Backward: the
+    gradient goes to ``membranePotential`` directly - correlation, then the spike function's surrogate
+    gradient (src/slayer.py:858-865), in one kernel - and nothing to ``spike``, whose own backward pass then
+    only carries what reaches the spikes from elsewhere."""
+
+    @staticmethod
+    def forward(ctx, spike, membranePotential, filter, Ts, alpha, theta, pdfTimeConstant, pdfScale):
+        psp = slayerCuda.pspAlpha(spike.contiguous(), filter, alpha[0], alpha[1], Ts, causal=True)
+        ctx.save_for_backward(membranePotential, filter)
+        ctx.Ts, ctx.alpha = float(Ts), alpha
+        ctx.theta, ctx.pdfTimeConstant, ctx.pdfScale = theta, pdfTimeConstant, pdfScale
+        return psp
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        membranePotential, filter = ctx.saved_tensors
+        grad = None
+        if ctx.needs_input_grad[1]:
+            grad = slayerCuda.pspSpikeBackwardAlpha(gradOutput.contiguous(), None, membranePotential, filter, ctx.alpha[0],
+                                                    ctx.alpha[1], ctx.theta, ctx.pdfTimeConstant, ctx.pdfScale, ctx.Ts)
+        return None, grad, None, None, None, None, None, None
 
 
 class _spikePspFunction(torch.autograd.Function):

@@ -139,8 +139,10 @@ def test_spike_non_contiguous_input_is_left_untouched():
 
 
 @pytest.mark.parametrize("T", [300, 350])
-def test_pspSpike_layer_call_matches_spike_of_psp(T):
+def test_pspSpike_layer_call_matches_spike_of_psp(T, monkeypatch):
     # the MLP ordering spike(psp(fc(x))) of the reference's example as one forward and one backward kernel
+    from slayerpytorch_amd import slayer as slayer_module
+    monkeypatch.setattr(slayer_module, "PAIR_SPIKE_PSP", False)      # the two Functions as they are
     layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": T}).to(DEV)
     rng = np.random.default_rng(T)
     shape = (2, 24, 1, 1, T)
@@ -161,7 +163,7 @@ def test_pspSpike_layer_call_matches_spike_of_psp(T):
 
 @pytest.mark.parametrize("T", [300, 350, 600])
 @pytest.mark.parametrize("use", ["psp", "both", "spikes"])
-def test_spikePsp_layer_call_matches_psp_of_spike(T, use):
+def test_spikePsp_layer_call_matches_psp_of_spike(T, use, monkeypatch):
     # the CNN ordering psp(spike(u)) of the reference's example: same spikes and PSP signal as the two calls, and one
     # backward kernel for whichever of the two results were used (T = 600: rows beyond the recursion take the sums over the taps)
     layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": T}).to(DEV)
@@ -177,6 +179,8 @@ def test_spikePsp_layer_call_matches_psp_of_spike(T, use):
     w1 = u1 * 1.0                       # (the spike function updates its input in place)
     s1, a1 = layer.spikePsp(w1)
     loss(s1, a1).backward()
+    from slayerpytorch_amd import slayer as slayer_module
+    monkeypatch.setattr(slayer_module, "PAIR_SPIKE_PSP", False)      # the two Functions as they are
     u2 = dev(u).requires_grad_(True)
     w2 = u2 * 1.0
     s2 = layer.spike(w2)
@@ -189,6 +193,87 @@ def test_spikePsp_layer_call_matches_psp_of_spike(T, use):
     else:
         assert torch.equal(u1.grad, u2.grad)
     assert float(u1.grad.abs().sum()) > 0
+
+
+def test_psp_of_fresh_spikes_sends_its_gradient_past_the_spike_function(monkeypatch):
+    """Reference-style code, spike(conv(psp(spike(conv(psp(x)))))): psp() recognises a tensor that spike() has just
+    returned and runs correlation + surrogate gradient as one kernel; same values and the same gradients as with the two
+    Functions apart - bit for bit while the spikes have no other user, to rounding when they have."""
+    from slayerpytorch_amd import slayer as slayer_module
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 300}).to(DEV)
+    torch.manual_seed(5)
+    conv1, conv2 = layer.conv(2, 6, 3, padding=1, weightScale=60).to(DEV), layer.conv(6, 4, 3, padding=1, weightScale=60).to(DEV)
+    rng = np.random.default_rng(31)
+    x = dev((rng.random((2, 2, 8, 8, 300)) < 0.05).astype(np.float32))
+    g = dev(rng.standard_normal((2, 4, 8, 8, 300)).astype(np.float32))
+    gs = dev(rng.standard_normal((2, 6, 8, 8, 300)).astype(np.float32))
+
+    def run(pair, extra, touch=None):
+        monkeypatch.setattr(slayer_module, "PAIR_SPIKE_PSP", pair)
+        for m in (conv1, conv2):
+            m.weight.grad = None
+        s1 = layer.spike(conv1(layer.psp(x)))
+        if touch == "inplace":
+            s1 = s1.mul_(1.0)                        # no longer what the spike function returned
+        elif touch == "detach":
+            s1 = s1.detach()
+        a2 = layer.psp(s1)
+        s2 = layer.spike(conv2(a2))
+        out = (layer.psp(s2) * g).sum()
+        if extra:
+            out = out + (s1 * gs).sum()              # the hidden spikes have a second user
+        out.backward()
+        return s2.detach().clone(), conv1.weight.grad.clone() if conv1.weight.grad is not None else None, conv2.weight.grad.clone()
+
+    apart = run(False, False)
+    paired = run(True, False)
+    assert float(apart[0].sum()) > 0 and float(apart[1].abs().sum()) > 0
+    assert all(torch.equal(a, b) for a, b in zip(apart, paired))
+    apart2, paired2 = run(False, True), run(True, True)
+    assert torch.equal(apart2[0], paired2[0]) and torch.equal(apart2[2], paired2[2])
+    assert rel_err(host(paired2[1]), host(apart2[1])) <= REL_TOL and not torch.equal(apart2[1], apart[1])
+    # spikes that were modified, or detached, are not paired
+    assert all(torch.equal(a, b) for a, b in zip(run(False, False, "inplace"), run(True, False, "inplace")))
+    detached = run(True, False, "detach")
+    assert detached[1] is None and torch.equal(detached[2], apart[2])
+    # the pairing really happened: the node behind the PSP signal
+    monkeypatch.setattr(slayer_module, "PAIR_SPIKE_PSP", True)
+    s1 = layer.spike(conv1(layer.psp(x)))
+    assert type(layer.psp(s1).grad_fn).__name__ == "_pspOfSpikeFunctionBackward"
+    assert type(layer.psp(s1 * 1.0).grad_fn).__name__ == "_pspFunctionBackward"
+    with torch.no_grad():
+        assert layer.psp(s1).grad_fn is None
+
+
+def test_spike_of_a_fresh_psp_signal_sends_its_gradient_past_the_filter(monkeypatch):
+    """Reference-style MLP code, spike(psp(fc(spike(psp(fc(x)))))): spike() recognises a signal that psp() has just
+    returned and runs surrogate gradient + correlation as one kernel; same spikes, and the same gradients bit for bit
+    as with the two Functions apart; a signal that was touched in between is not paired."""
+    from slayerpytorch_amd import slayer as slayer_module
+    layer = snn.layer(neuron(), {"Ts": 1.0, "tSample": 300}).to(DEV)
+    torch.manual_seed(6)
+    fc1, fc2 = layer.dense(40, 30, weightScale=80).to(DEV), layer.dense(30, 7, weightScale=80).to(DEV)
+    rng = np.random.default_rng(32)
+    x = dev((rng.random((3, 40, 1, 1, 300)) < 0.05).astype(np.float32))
+    g = dev(rng.standard_normal((3, 7, 1, 1, 300)).astype(np.float32))
+
+    def run(pair, touch=False):
+        monkeypatch.setattr(slayer_module, "PAIR_SPIKE_PSP", pair)
+        for m in (fc1, fc2):
+            m.weight.grad = None
+        a1 = layer.psp(fc1(x))
+        if touch:
+            a1 = a1 * 1.0
+        s1 = layer.spike(a1)
+        s2 = layer.spike(layer.psp(fc2(s1)))
+        (layer.psp(s2) * g).sum().backward()
+        return s2.detach().clone(), fc1.weight.grad.clone(), fc2.weight.grad.clone(), type(s1.grad_fn).__name__
+
+    apart, paired, touched = run(False), run(True), run(True, True)
+    assert float(apart[0].sum()) > 0 and float(apart[1].abs().sum()) > 0
+    assert apart[3] == "_spikeFunctionBackward" and paired[3] == "_spikeOfPspFunctionBackward" and touched[3] == "_spikeFunctionBackward"
+    for other in (paired, touched):
+        assert all(torch.equal(a, b) for a, b in zip(apart[:3], other[:3]))
 
 
 def test_get_spikes_requires_five_dimensions():
