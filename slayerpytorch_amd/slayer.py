@@ -19,6 +19,7 @@ elementwise torch ops, and scalars saved for backward stay Python floats (no 0-d
 tensors, hence no device-to-host synchronisation in backward).
 """
 import math
+import weakref
 
 import numpy as np
 import torch
@@ -87,8 +88,8 @@ class spikeLayer(nn.Module):
         origin = getattr(spike, "_slayerSpikeOf", None) if PAIR_SPIKE_PSP and alpha is not None else None
         if origin is not None and torch.is_grad_enabled() and spike.requires_grad and _recursion_serves(spike) \
                 and spike._version == origin[4] and type(spike.grad_fn).__name__ == "_spikeFunctionBackward":
-            membranePotential, theta, pdfTimeConstant, pdfScale, _ = origin
-            if membranePotential.shape == spike.shape and membranePotential.is_contiguous():
+            membranePotential, theta, pdfTimeConstant, pdfScale = origin[0](), origin[1], origin[2], origin[3]
+            if membranePotential is not None and membranePotential.shape == spike.shape and membranePotential.is_contiguous():
                 return _pspOfSpikeFunction.apply(spike, membranePotential, self.srmKernel, self.simulation["Ts"], alpha,
                                                  theta, pdfTimeConstant, pdfScale)
         psp = _pspFunction.apply(spike, self.srmKernel, self.simulation["Ts"], alpha)
@@ -126,12 +127,14 @@ class spikeLayer(nn.Module):
                 and origin[0].shape == membranePotential.shape:
             # spike(psp(x)), the ordering of the reference's MLP example: the spikes' gradient goes past the PSP
             # filter straight to x, surrogate gradient and correlation in one kernel
+            del membranePotential._slayerPspOf     # (the note is what keeps x alive; the Function only needs its place in the graph)
             return _spikeOfPspFunction.apply(membranePotential, origin[0], self.refKernel, origin[1], self.neuron,
                                              self.simulation["Ts"], origin[2])
         spikes = _spikeFunction.apply(membranePotential, self.refKernel, self.neuron, self.simulation["Ts"])
         if PAIR_SPIKE_PSP and spikes.requires_grad:
-            # for psp(): which potential these spikes came from, and that they have not been touched since
-            spikes._slayerSpikeOf = (membranePotential, float(self.neuron["theta"]),
+            # for psp(): which potential these spikes came from (kept alive by the spike function's own record for the
+            # backward pass, not by this note), and that they have not been touched since
+            spikes._slayerSpikeOf = (weakref.ref(membranePotential), float(self.neuron["theta"]),
                                      float(self.neuron["tauRho"] * self.neuron["theta"]), float(self.neuron["scaleRho"]),
                                      spikes._version)
         return spikes
