@@ -85,13 +85,9 @@ class spikeLayer(nn.Module):
         gradient run as a recursion over time (``slayerCuda.pspAlpha``), which agrees with the
         sum over the taps to rounding; a kernel that was replaced or edited takes the sums."""
         alpha = self._srmKernelIsAlpha()
-        origin = getattr(spike, "_slayerSpikeOf", None) if PAIR_SPIKE_PSP and alpha is not None else None
-        if origin is not None and torch.is_grad_enabled() and spike.requires_grad and _recursion_serves(spike) \
-                and spike._version == origin[4] and type(spike.grad_fn).__name__ == "_spikeFunctionBackward":
-            membranePotential, theta, pdfTimeConstant, pdfScale = origin[0](), origin[1], origin[2], origin[3]
-            if membranePotential is not None and membranePotential.shape == spike.shape and membranePotential.is_contiguous():
-                return _pspOfSpikeFunction.apply(spike, membranePotential, self.srmKernel, self.simulation["Ts"], alpha,
-                                                 theta, pdfTimeConstant, pdfScale)
+        origin = _fresh_spikes(spike) if alpha is not None and _recursion_serves(spike) else None
+        if origin is not None:
+            return _pspOfSpikeFunction.apply(spike, origin[0], self.srmKernel, self.simulation["Ts"], alpha, *origin[1:])
         psp = _pspFunction.apply(spike, self.srmKernel, self.simulation["Ts"], alpha)
         if PAIR_SPIKE_PSP and alpha is not None and psp.requires_grad and _recursion_serves(spike):
             # for spike(): what this signal was filtered from, and that it has not been touched since
@@ -173,6 +169,9 @@ class spikeLayer(nn.Module):
     def delayShift(self, input, delay, Ts=1):
         """Delays ``input`` in time by ``delay`` (number, one-element tensor, or one value per
         neuron); the gradient flows to ``input`` only."""
+        origin = _fresh_spikes(input) if isinstance(input, torch.Tensor) and input.dim() == 5 else None
+        if origin is not None:
+            return _delayOfSpikeFunction.apply(input, origin[0], delay, Ts, False, *origin[1:])
         return _delayFunctionNoGradient.apply(input, delay, Ts)
 
     def delay(self, inputSize):
@@ -225,7 +224,8 @@ class spikeLayer(nn.Module):
 # two with a tensor in between.  Gradients that reach s from elsewhere still pass through the spike function's
 # own backward pass; the sum at the membrane potential is the same.  Likewise spike(u) of a signal u that psp() has
 # just returned - the ordering of the reference's MLP example, spike(psp(fc(x))) - sends the spikes' gradient past
-# the PSP filter (slayerCuda.spikeBackwardPspAlpha).  False keeps the two Functions apart.
+# the PSP filter (slayerCuda.spikeBackwardPspAlpha), and delay(s) / delayShift(s, d) of fresh spikes sends its gradient
+# past the spike function as well (slayerCuda.spikeBackwardDelayed).  False keeps the Functions apart.
 PAIR_SPIKE_PSP = True
 
 
@@ -471,6 +471,19 @@ class _spikeDelayedFunction(torch.autograd.Function):
         return gradInput, None, None, None, gradDelay, None
 
 
+def _fresh_spikes(spike):
+    """(membranePotential, theta, pdfTimeConstant, pdfScale) when ``spike`` is what ``spikeLayer.spike`` has just
+    returned for that potential - its own output, untouched, with the graph being recorded - else None."""
+    origin = getattr(spike, "_slayerSpikeOf", None) if PAIR_SPIKE_PSP else None
+    if origin is None or not torch.is_grad_enabled() or not spike.requires_grad or spike._version != origin[4] \
+            or type(spike.grad_fn).__name__ != "_spikeFunctionBackward":
+        return None
+    membranePotential = origin[0]()
+    if membranePotential is None or membranePotential.shape != spike.shape or not membranePotential.is_contiguous():
+        return None
+    return membranePotential, origin[1], origin[2], origin[3]
+
+
 def _recursion_serves(x):
     """Shapes that ``slayerCuda.pspAlpha`` runs as a recursion (others it would hand to conv / corr itself): rows of at
     most 512 samples in a tensor of whole 16-byte vectors."""
@@ -660,9 +673,11 @@ class _delayLayer(nn.Module):
 
     def forward(self, input):
         N, C, H, W, Ns = input.shape
-        if input.numel() != self.delay.numel() * Ns * N:
-            return _delayFunction.apply(input, self.delay.repeat((1, H, W)), self.Ts)
-        return _delayFunction.apply(input, self.delay, self.Ts)
+        table = self.delay.repeat((1, H, W)) if input.numel() != self.delay.numel() * Ns * N else self.delay
+        origin = _fresh_spikes(input)
+        if origin is not None:
+            return _delayOfSpikeFunction.apply(input, origin[0], table, self.Ts, True, *origin[1:])
+        return _delayFunction.apply(input, table, self.Ts)
 
 
 class _delayFunction(torch.autograd.Function):
@@ -683,6 +698,38 @@ class _delayFunction(torch.autograd.Function):
         gradDelay = slayerCuda.delayGrad(output, gradOutput, ctx.Ts).reshape(gradOutput.shape[1:-1])
         gradInput = slayerCuda.shift(gradOutput, delay.contiguous(), ctx.Ts, sign=-1.0)
         return gradInput, gradDelay, None
+
+
+class _delayOfSpikeFunction(torch.autograd.Function):
+    """``_delayFunction`` / ``_delayFunctionNoGradient`` (src/slayer.py:930-979) for a spike tensor that
+    ``_spikeFunction`` has just produced from ``membranePotential``.  Forward: the shift.  Backward: the gradient
+    goes to ``membranePotential`` directly - shifted back and multiplied by the spike function's surrogate gradient
+    (src/slayer.py:858-865) in one kernel - and nothing to ``spike``; a learnable delay table (``learn``) gets the
+    delay gradient as in ``_delayFunction``."""
+
+    @staticmethod
+    def forward(ctx, spike, membranePotential, delay, Ts, learn, theta, pdfTimeConstant, pdfScale):
+        table = delay.detach().to(device=spike.device, dtype=spike.dtype).contiguous() \
+            if isinstance(delay, torch.Tensor) else delay
+        output = slayerCuda.shift(spike.contiguous(), table, Ts)
+        ctx.learn = bool(learn)
+        ctx.save_for_backward(membranePotential, *((output,) if ctx.learn else ()))
+        ctx.delay, ctx.Ts = table, float(Ts)
+        ctx.delayShape = tuple(delay.shape) if isinstance(delay, torch.Tensor) else None
+        ctx.theta, ctx.pdfTimeConstant, ctx.pdfScale = theta, pdfTimeConstant, pdfScale
+        return output
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        membranePotential = ctx.saved_tensors[0]
+        gradOutput = gradOutput.contiguous()
+        gradDelay = grad = None
+        if ctx.learn and ctx.needs_input_grad[2]:
+            gradDelay = slayerCuda.delayGrad(ctx.saved_tensors[1], gradOutput, ctx.Ts).reshape(ctx.delayShape)
+        if ctx.needs_input_grad[1]:
+            grad = slayerCuda.spikeBackwardDelayed(gradOutput, membranePotential, ctx.theta, ctx.pdfTimeConstant,
+                                                   ctx.pdfScale, ctx.delay, ctx.Ts)
+        return None, grad, gradDelay, None, None, None, None, None
 
 
 class _delayFunctionNoGradient(torch.autograd.Function):

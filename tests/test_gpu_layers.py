@@ -276,6 +276,37 @@ def test_spike_of_a_fresh_psp_signal_sends_its_gradient_past_the_filter(monkeypa
         assert all(torch.equal(a, b) for a, b in zip(apart[:3], other[:3]))
 
 
+@pytest.mark.parametrize("learnable", [True, False])
+def test_delay_of_fresh_spikes_sends_its_gradient_past_the_spike_function(learnable, monkeypatch):
+    """Reference-style delay(spike(u)) / delayShift(spike(u), d): the delay recognises a tensor that spike() has just
+    returned and runs the gradient's shift and the surrogate gradient as one kernel; same values, same gradients for
+    the membrane potential and the delays, bit for bit."""
+    from slayerpytorch_amd import slayer as slayer_module
+    params = {"type": "SRMALPHA", "theta": 10, "tauSr": 2.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
+    layer = snn.layer(params, {"Ts": 1.0, "tSample": 120}).cuda()
+    torch.manual_seed(4)
+    u0 = (torch.randn((3, 6, 2, 2, 120)) * 6 + 4).cuda()
+    g = torch.randn_like(u0)
+    dl = layer.delay((6, 2, 2)).cuda()
+    with torch.no_grad():
+        dl.delay.mul_(9.0)
+
+    def run(pair):
+        monkeypatch.setattr(slayer_module, "PAIR_SPIKE_PSP", pair)
+        dl.delay.grad = None
+        u = u0.clone().requires_grad_(True)
+        s = layer.spike(u * 1.0)
+        out = dl(s) if learnable else layer.delayShift(s, 3.0)
+        out.backward(g)
+        return out.detach().clone(), u.grad.clone(), (dl.delay.grad.clone() if learnable else None), type(out.grad_fn).__name__
+
+    apart, paired = run(False), run(True)
+    assert paired[3] == "_delayOfSpikeFunctionBackward" and apart[3] != paired[3]
+    assert torch.equal(apart[0], paired[0]) and torch.equal(apart[1], paired[1]) and float(apart[1].abs().sum()) > 0
+    if learnable:
+        assert torch.equal(apart[2], paired[2]) and float(apart[2].abs().sum()) > 0
+
+
 def test_get_spikes_requires_five_dimensions():
     f = torch.ones(3, device=DEV)
     with pytest.raises(IndexError):
