@@ -126,7 +126,7 @@ def cpu_plumbing_baseline(srm, ref, params):
     try:
         g = torch.Generator().manual_seed(0)
         x = (torch.rand((4, 2, 34, 34, 300), generator=g) < 0.02).float()
-        w = torch.randn((512, 2, 34, 34, 1), generator=g) * (100.0 / 2312)
+        w = torch.randn((512, 2, 34, 34, 1), generator=g) * 100.0      # N(0,1) * scale 100, as the case is stated
         k = torch.from_numpy(srm[::-1].copy()).reshape(1, 1, 1, 1, -1)
         times = {"dense_conv3d": [], "psp_conv3d": [], "spike_oracle": []}
         for _ in range(6):
@@ -507,8 +507,8 @@ def other_rows(device, cpu_leg=False):
     """Quick per-op measurements of the scope rows that are not part of the headline chain, each on
     the largest tensor its benchmark configuration gives it (kernel rows: median of 7 event-timed passes of 8
     launches back to back; network steps: median of 7 event-timed steps).  hbm_frac
-    counts the algorithmic bytes of the unfused reference sequence (Loihi forward + delayShift:
-    16 + 8 B, Loihi backward: 12 + 8 B), also where one fused kernel moves fewer."""
+    counts the bytes the row's kernel has to move (for a fused kernel fewer than the reference sequence it
+    replaces: Loihi forward + delayShift 16 + 8 B, Loihi backward 12 + 8 B)."""
     from slayerpytorch_amd import slayerCuda, slayerLoihiCuda
     from slayerpytorch_amd.slayer import alphaKernel
     from slayerpytorch_amd.slayerLoihi import loihiPspKernel
@@ -535,11 +535,39 @@ def other_rows(device, cpu_leg=False):
     K = 8
 
     def row(name, ab, numel, seconds, shape, moved=None):
-        r = {"op": name, "shape": list(shape), "us": seconds * 1e6, "neuron_timesteps_per_s": numel / seconds,
-             "hbm_frac": ab * numel / seconds / 1e9 / HBM_PEAK_GBS}
-        if moved is not None:       # a fused kernel: the bytes it really moves, next to the unfused sequence's
+        """``ab``: algorithmic bytes per neuron-timestep of the reference sequence the row stands for.  A fused
+        kernel (``moved`` given) moves fewer: its roofline fraction ``hbm_frac`` counts the bytes it moves, and the
+        traffic the separate calls would have needed, over the same time, is kept under a name that cannot be read
+        as a roofline fraction (it exceeds 1 where fusion saves traffic)."""
+        r = {"op": name, "shape": list(shape), "us": seconds * 1e6, "neuron_timesteps_per_s": numel / seconds}
+        if moved is None:
+            r["hbm_frac"] = ab * numel / seconds / 1e9 / HBM_PEAK_GBS
+        else:
             r["bytes_per_element_moved"] = moved
-            r["hbm_frac_of_bytes_moved"] = moved * numel / seconds / 1e9 / HBM_PEAK_GBS
+            r["hbm_frac"] = r["hbm_frac_of_bytes_moved"] = moved * numel / seconds / 1e9 / HBM_PEAK_GBS
+            r["bytes_per_element_of_the_separate_calls"] = ab
+            r["separate_calls_traffic_over_this_time_vs_hbm_peak"] = ab * numel / seconds / 1e9 / HBM_PEAK_GBS
+        return r
+
+    def potentials(shape, srm_k, ref_k, tau_sr, rate_target):
+        """A membrane potential of the kind real layers see: the PSP signal of Bernoulli(0.05) spikes - smooth, above
+        the threshold for runs of samples - scaled so that about ``rate_target`` of the samples fire."""
+        gp = torch.Generator(device="cpu").manual_seed(11)
+        a = slayerCuda.pspAlpha((torch.rand(shape, generator=gp) < 0.05).float().to(device), srm_k, tau_sr, 1.0, 1.0, True)
+        lo, hi = 0.05, 2000.0
+        for _ in range(16):
+            gain = (lo * hi) ** 0.5
+            rate = float(slayerCuda.getSpikes(a * gain, ref_k, 10.0, 1.0).mean())
+            lo, hi = (gain, hi) if rate < rate_target else (lo, gain)
+        u = (a * gain).contiguous()
+        return u, rate, float((u >= 10.0).float().mean())
+
+    def spike_on_potentials(name, shape, srm_k, ref_k, tau_sr, rate_target):
+        u_real, rate, above = potentials(shape, srm_k, ref_k, tau_sr, rate_target)
+        pool = [u_real.clone() for _ in range(K)]
+        restore = lambda: [p.copy_(u_real) for p in pool]
+        r = row(name, 12, u_real.numel(), timed(lambda u: slayerCuda.getSpikes(u, ref_k, 10.0, 1.0), K, (pool, restore)), shape)
+        r["spike_rate"], r["samples_at_or_above_theta_before_the_walk"] = round(rate, 4), round(above, 4)
         return r
 
     out = []
@@ -565,6 +593,13 @@ def other_rows(device, cpu_leg=False):
     out.append(row("spike_T2000_then_per_neuron_delay_fused", 20, n,
                    timed(lambda u: slayerCuda.getSpikesDelayed(u, ref, 10.0, 1.0, lut, 1.0), K, (pool, restore)), shape, moved=12))
     del x, grad, u0, ub, y, pool
+    # the spike kernel's time depends on its input: the rows above (and the headline) feed independent normal samples
+    # (2.3 % isolated samples at or above the threshold); real potentials are smooth and stay above it for runs of samples
+    out.append(spike_on_potentials("spike_T2000_on_psp_shaped_potential_firing_4_percent", shape, srm8, ref, 1.0, 0.04))
+    srm77, ref11 = (torch.tensor(alphaKernel(tau, 1.0, 300, mult=m), dtype=torch.float32, device=device) for tau, m in ((10.0, 1.0), (1.0, -20.0)))
+    for target in (0.04, 0.30):
+        out.append(spike_on_potentials("spike_on_psp_shaped_potential_firing_%d_percent" % round(100 * target),
+                                       (12, 16, 32, 32, 300), srm77, ref11, 10.0, target))
     # the 77-tap PSP filter over the density of its input, as the sum over the taps (slayerCuda.conv: spike trains
     # take the event-driven path tile by tile, denser tiles the matrix cores) and as the recursion that the layers
     # run for their own alpha kernel

@@ -25,6 +25,7 @@ import numpy as np
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
+from torch.utils.weak import WeakTensorKeyDictionary
 
 from . import slayerCuda
 from . import synapse
@@ -91,7 +92,7 @@ class spikeLayer(nn.Module):
         psp = _pspFunction.apply(spike, self.srmKernel, self.simulation["Ts"], alpha)
         if PAIR_SPIKE_PSP and alpha is not None and psp.requires_grad and _recursion_serves(spike):
             # for spike(): what this signal was filtered from, and that it has not been touched since
-            psp._slayerPspOf = (spike, self.srmKernel, alpha, psp._version)
+            _pspNotes[psp] = (spike, self.srmKernel, alpha, psp._version)
         return psp
 
     def _srmKernelIsAlpha(self):
@@ -116,23 +117,22 @@ class spikeLayer(nn.Module):
     def spike(self, membranePotential):
         """Spike function with refractory response.  A contiguous ``membranePotential`` is
         updated in place with the refractory response, as in the reference."""
-        origin = getattr(membranePotential, "_slayerPspOf", None) if PAIR_SPIKE_PSP else None
+        origin = _pspNotes.pop(membranePotential, None) if PAIR_SPIKE_PSP else None   # (the note is what keeps x alive)
         if origin is not None and torch.is_grad_enabled() and membranePotential.requires_grad \
                 and membranePotential.is_contiguous() and membranePotential._version == origin[3] \
-                and type(membranePotential.grad_fn).__name__ == "_pspFunctionBackward" \
-                and origin[0].shape == membranePotential.shape:
+                and isinstance(membranePotential.grad_fn, _pspFunction._backward_cls) \
+                and _unobserved(membranePotential) and origin[0].shape == membranePotential.shape:
             # spike(psp(x)), the ordering of the reference's MLP example: the spikes' gradient goes past the PSP
             # filter straight to x, surrogate gradient and correlation in one kernel
-            del membranePotential._slayerPspOf     # (the note is what keeps x alive; the Function only needs its place in the graph)
             return _spikeOfPspFunction.apply(membranePotential, origin[0], self.refKernel, origin[1], self.neuron,
                                              self.simulation["Ts"], origin[2])
         spikes = _spikeFunction.apply(membranePotential, self.refKernel, self.neuron, self.simulation["Ts"])
         if PAIR_SPIKE_PSP and spikes.requires_grad:
             # for psp(): which potential these spikes came from (kept alive by the spike function's own record for the
-            # backward pass, not by this note), and that they have not been touched since
-            spikes._slayerSpikeOf = (weakref.ref(membranePotential), float(self.neuron["theta"]),
-                                     float(self.neuron["tauRho"] * self.neuron["theta"]), float(self.neuron["scaleRho"]),
-                                     spikes._version)
+            # backward pass, not by this note), and that neither has been touched since
+            _spikeNotes[spikes] = (weakref.ref(membranePotential), float(self.neuron["theta"]),
+                                   float(self.neuron["tauRho"] * self.neuron["theta"]), float(self.neuron["scaleRho"]),
+                                   spikes._version, membranePotential._version)
         return spikes
 
     def spikeDelayed(self, membranePotential, delay, Ts=None):
@@ -231,14 +231,15 @@ PAIR_SPIKE_PSP = True
 
 # The dense layer's product and weight gradient event by event (synapse.denseEvents, denseEventsGradWeight)
 # when its input is sparse enough and has enough channels for that to pay: True / False force the choice,
-# "auto" measures the fraction of non-zero inputs of a layer at its first call and at every
-# DENSE_EVENTS_CHECK_EVERY-th one after that (a device-to-host read, so not at every call, and never while a
-# HIP graph is being captured: the last measurement decides then).
+# "auto" counts the non-zero inputs of a layer on the device - at its first two calls, whenever the input's shape
+# changes and at every DENSE_EVENTS_CHECK_EVERY-th call - and copies the count to pinned host memory without
+# waiting for it: a call uses the latest count that has arrived (at most a few calls old), and only a layer's very
+# first call waits.  Nothing is measured while a HIP graph is being captured: the last count decides then.
 DENSE_EVENTS = "auto"
 DENSE_EVENTS_MAX_DENSITY = 0.05           # weight gradient
 DENSE_EVENTS_MAX_DENSITY_FORWARD = 0.03   # product (its input has to be transposed first)
 DENSE_EVENTS_MIN_CHANNELS = 1024
-DENSE_EVENTS_CHECK_EVERY = 64
+DENSE_EVENTS_CHECK_EVERY = 4
 
 
 class _denseLayer(nn.Conv3d):
@@ -261,7 +262,28 @@ class _denseLayer(nn.Conv3d):
             self.weight = nn.Parameter(weightScale * self.weight)
         self.preHookFx = preHookFx
         self._eventCalls = 0
-        self._eventDensity = None
+        self._eventDensity = None     # latest fraction of non-zero inputs that has arrived on the host
+        self._eventShape = None
+        self._eventPending = None     # (pinned host count, event recorded after its copy, numel)
+
+    def _measureDensity(self, x):
+        """Keeps ``_eventDensity`` current without stalling the stream (see DENSE_EVENTS)."""
+        shape = tuple(x.shape)
+        if shape != self._eventShape:
+            self._eventShape, self._eventCalls, self._eventDensity, self._eventPending = shape, 0, None, None
+        if self._eventPending is not None and self._eventPending[1].query():
+            self._eventDensity = int(self._eventPending[0]) / self._eventPending[2]
+            self._eventPending = None
+        if self._eventPending is None and (self._eventCalls < 2 or self._eventCalls % DENSE_EVENTS_CHECK_EVERY == 0):
+            count = torch.empty((), dtype=torch.int64, pin_memory=True)
+            count.copy_(torch.count_nonzero(x), non_blocking=True)
+            arrived = torch.cuda.Event()
+            arrived.record()
+            self._eventPending = (count, arrived, x.numel())
+            if self._eventDensity is None:      # the first call of this shape has nothing older to go by
+                arrived.synchronize()
+                self._eventDensity, self._eventPending = int(count) / x.numel(), None
+        self._eventCalls += 1
 
     def _inputIsSparse(self, x):
         """(product, weight gradient): which of the two are summed over the events in this call (see DENSE_EVENTS)."""
@@ -274,9 +296,7 @@ class _denseLayer(nn.Conv3d):
         if K < DENSE_EVENTS_MIN_CHANNELS:
             return False, False
         if not torch.cuda.is_current_stream_capturing():
-            if self._eventDensity is None or self._eventCalls % DENSE_EVENTS_CHECK_EVERY == 0:
-                self._eventDensity = int(torch.count_nonzero(x)) / x.numel()
-            self._eventCalls += 1
+            self._measureDensity(x)
         if self._eventDensity is None:
             return False, False
         return self._eventDensity <= DENSE_EVENTS_MAX_DENSITY_FORWARD, self._eventDensity <= DENSE_EVENTS_MAX_DENSITY
@@ -474,14 +494,29 @@ class _spikeDelayedFunction(torch.autograd.Function):
 def _fresh_spikes(spike):
     """(membranePotential, theta, pdfTimeConstant, pdfScale) when ``spike`` is what ``spikeLayer.spike`` has just
     returned for that potential - its own output, untouched, with the graph being recorded - else None."""
-    origin = getattr(spike, "_slayerSpikeOf", None) if PAIR_SPIKE_PSP else None
+    origin = _spikeNotes.get(spike) if PAIR_SPIKE_PSP else None
     if origin is None or not torch.is_grad_enabled() or not spike.requires_grad or spike._version != origin[4] \
-            or type(spike.grad_fn).__name__ != "_spikeFunctionBackward":
+            or not isinstance(spike.grad_fn, _spikeFunction._backward_cls) or not _unobserved(spike):
         return None
     membranePotential = origin[0]()
-    if membranePotential is None or membranePotential.shape != spike.shape or not membranePotential.is_contiguous():
+    # (a potential changed in place after spike() must reach the spike function's own backward pass, whose saved
+    # tensor then raises; the paired kernel would silently use the changed values)
+    if membranePotential is None or membranePotential.shape != spike.shape or not membranePotential.is_contiguous() \
+            or membranePotential._version != origin[5]:
         return None
     return membranePotential, origin[1], origin[2], origin[3]
+
+
+# The pairing notes live beside the tensors, not on them: a tensor with Python attributes is pickled with them
+# (torch.save of a layer's output would carry the note, or fail on it), and an entry goes when its tensor does.
+_pspNotes = WeakTensorKeyDictionary()     # psp() output -> (its input, kernel, (tau, mult), version)
+_spikeNotes = WeakTensorKeyDictionary()   # spike() output -> (weak potential, theta, pdf tau, pdf scale, versions)
+
+
+def _unobserved(tensor):
+    """False when the caller watches this tensor's gradient (``retain_grad`` or a hook registered on it): the paired
+    kernels route the gradient around the tensor, so such a tensor keeps the separate Functions."""
+    return not tensor.retains_grad and not tensor._backward_hooks
 
 
 def _recursion_serves(x):

@@ -803,61 +803,6 @@ def test_spike_delayed_layer_matches_spike_then_delay(learnable):
         assert torch.equal(dl.delay.grad, dl2.delay.grad) and float(dl.delay.grad.abs().sum()) > 0
 
 
-def test_training_step_replayed_from_a_hip_graph():
-    """The entry points only enqueue on the stream they are given (no allocation, no host
-    synchronisation), so a whole training step - psp, spike, delay, dense, loss, backward - can be
-    captured in a HIP graph.  Every replay, with eager work and synchronisations in between, must
-    reproduce the eager step bit for bit."""
-    params = {"type": "SRMALPHA", "theta": 10, "tauSr": 4.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
-    sim = {"Ts": 1.0, "tSample": 100}
-    layer = snn.layer(params, sim).cuda()
-    error = snn.loss({"neuron": params, "simulation": sim, "training": {"error": {"type": "SpikeTime"}}}).cuda()
-    torch.manual_seed(2)
-    fc1, fc2 = layer.dense(40, 32, weightScale=30).cuda(), layer.dense(32, 6, weightScale=30).cuda()
-    delay = layer.delay(32).cuda()
-    x = (torch.rand((3, 40, 1, 1, 100)) < 0.1).float().cuda()
-    target = (torch.rand((3, 6, 1, 1, 100)) < 0.05).float().cuda()
-    leaves = [fc1.weight, fc2.weight, delay.delay]
-    for p in leaves:
-        p.grad = torch.zeros_like(p)
-
-    def step():
-        for p in leaves:
-            p.grad.zero_()
-        s1 = layer.spikeDelayed(layer.psp(fc1(x)), delay)
-        s2 = layer.spike(layer.psp(fc2(s1)))
-        loss = error.spikeTime(s2, target)
-        loss.backward()
-        return loss
-
-    def eager():
-        loss = step()
-        torch.cuda.synchronize()
-        return [loss.detach().clone()] + [p.grad.clone() for p in leaves]
-
-    ref = eager()
-    assert float(ref[0]) > 0 and all(float(r.abs().sum()) > 0 for r in ref[1:])
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        for _ in range(3):
-            step()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        static_loss = step()
-    for _ in range(4):
-        graph.replay()
-        torch.cuda.synchronize()
-        got = [static_loss.detach()] + [p.grad for p in leaves]
-        for a, b in zip(got, ref):
-            assert torch.equal(a, b)
-        again = eager()                      # the program's own eager work between replays
-        for a, b in zip(again, ref):
-            assert torch.equal(a, b)
-
-
 @pytest.mark.parametrize("Ts,T,shape", [(1.0, 300, (4, 10, 1, 1)), (0.5, 128, (2, 3, 2, 2)), (1.0, 20000, (1, 2, 1, 1))])
 def test_spike_time_loss_kernel_matches_tensor_expression(Ts, T, shape):
     """The fused loss (error signal + squared sum in two launches) against the reference's expression
@@ -889,9 +834,12 @@ def test_spike_time_loss_kernel_matches_tensor_expression(Ts, T, shape):
     assert abs(float(loss) - 0.5 * float((eo.astype(np.float64) ** 2).sum()) * Ts) <= 1e-5 * abs(float(ref))
 
 
-def test_cpu_plumbing_configuration():
+@pytest.mark.parametrize("scale", [100.0, 0.5])
+def test_cpu_plumbing_configuration(scale):
     """The reference's CPU-runnable case: Bernoulli(0.02) spikes (4, 2, 34, 34, 300), dense 2312 -> 512 as a
-    conv3d with N(0,1) weights, a pspLayer-style conv3d PSP (left-padded, flipped SRM kernel, tauSr = 10) on the
+    conv3d with N(0,1) * scale weights - scale 100 as that configuration is stated (every neuron with a positive
+    drive then fires at each step), and 0.5, where the layer fires a few per cent of the time and the potentials
+    cross the threshold slowly - a pspLayer-style conv3d PSP (left-padded, flipped SRM kernel, tauSr = 10) on the
     CPU with torch, threshold / refractory spikes by the oracle - against dense -> psp -> spike of this package on
     the GPU.  The membrane potentials agree to fp32 rounding; spikes may flip only where the potential sits
     within that rounding of the threshold."""
@@ -901,7 +849,7 @@ def test_cpu_plumbing_configuration():
     x = (torch.rand((4, 2, 34, 34, 300)) < 0.02).float()
     fc = layer.dense((34, 34, 2), 512)
     with torch.no_grad():
-        fc.weight.copy_(torch.randn(fc.weight.shape) * 0.5)
+        fc.weight.copy_(torch.randn(fc.weight.shape) * scale)
     srm = layer.srmKernel.clone()
     # CPU: conv3d dense, then the PSP as a conv3d over time with the flipped kernel (src/slayer.py:760-791)
     with torch.no_grad():
@@ -917,5 +865,5 @@ def test_cpu_plumbing_configuration():
         assert rel_err(a_gpu.cpu().numpy(), a_cpu.numpy()) <= 1e-5
         s_gpu = layer.spike(a_gpu)
     flips = float((s_gpu.cpu().numpy() != s_cpu).mean())
-    assert 0.005 < float(s_cpu.mean()) < 0.5
+    assert 0.005 < float(s_cpu.mean()) < (0.5 if scale < 1 else 0.9)
     assert flips <= 1e-4, "spike flip rate %g" % flips
