@@ -593,6 +593,17 @@ def other_rows(device, cpu_leg=False):
     out.append(row("spike_T2000_then_per_neuron_delay_fused", 20, n,
                    timed(lambda u: slayerCuda.getSpikesDelayed(u, ref, 10.0, 1.0, lut, 1.0), K, (pool, restore)), shape, moved=12))
     del x, grad, u0, ub, y, pool
+    # the 77-tap alpha kernel on these long rows: as a recursion carried from piece to piece, and as sums over the taps
+    srm77 = torch.tensor(alphaKernel(10.0, 1.0, 2000), dtype=torch.float32, device=device)
+    xg = torch.randn(shape, generator=g).to(device)
+    for nm, src in (("spikes", (torch.rand(shape, generator=g) < 0.02).float().to(device)), ("dense", xg)):
+        for causal in (True, False):
+            r = row("psp_%s77_T2000_as_recursion_%s_input" % ("conv" if causal else "corr", nm), 8, n,
+                    timed(lambda: slayerCuda.pspAlpha(src, srm77, 10.0, 1.0, 1.0, causal), K), shape)
+            taps = timed(lambda: (slayerCuda.conv if causal else slayerCuda.corr)(src, srm77, 1.0), K)
+            r["us_as_sums_over_the_taps"], r["hbm_frac_as_sums_over_the_taps"] = taps * 1e6, 8 * n / taps / 1e9 / HBM_PEAK_GBS
+            out.append(r)
+    del xg, src
     # the spike kernel's time depends on its input: the rows above (and the headline) feed independent normal samples
     # (2.3 % isolated samples at or above the threshold); real potentials are smooth and stay above it for runs of samples
     out.append(spike_on_potentials("spike_T2000_on_psp_shaped_potential_firing_4_percent", shape, srm8, ref, 1.0, 0.04))

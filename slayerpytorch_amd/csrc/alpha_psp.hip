@@ -274,6 +274,235 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
     }
 }
 
+// ---- rows longer than kAlphaMaxT: the same recursion piece by piece ---------------------------------------------
+// A wavefront owns 4 rows and walks them in pieces of kPieceT samples along the logical time axis (forward for the
+// convolution, backward for the correlation).  What a piece needs from the ones before it is three numbers per row -
+// the running sums p and q at its start, composed into the lanes' scan like one more segment - and the last H >= L
+// values of r, kept in front of the piece's own r in LDS, so that r[t - L] is read the same way everywhere (zeros in
+// front of the row).  LDS holds a piece in logical order: for the correlation the vectors and their elements are
+// mirrored between memory and LDS, which costs nothing (a lane loads and stores the same memory vector either way)
+// and leaves one form of the passes.  The loads of the next piece are issued before the passes over this one.
+constexpr int kPieceT = 256;              // samples per row and piece: 64 vectors, 4 per lane of a row
+constexpr int kPieceMaxL = kPieceT;       // r[t - L] lies in this piece or the one before
+
+struct AlphaPieces {
+    int H;              // history samples of r per row: L rounded up to whole vectors
+    float aSegFull;     // a^16: a lane's segment of a full piece
+    float aSegLast[2];  // a^n for the last piece's segments of units / 16 and units / 16 + 1 vectors
+};
+
+template <bool CAUSAL, int GATE>
+__global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, AlphaPieces pc)
+{
+    constexpr bool GATED = GATE == 1, GATED_OUT = GATE == 2;
+    constexpr int R = kAlphaRows, kParts = kWave / R, PT = kPieceT, PV = PT / 4;
+    static_assert(R == 4 && PV == kWave, "lane c moves vector c of every row's piece");
+    extern __shared__ __align__(16) float lds[];
+    const int T = p.T, L = p.L, H = pc.H;
+    const int pitch = H + PT;
+    float *Q = lds;             // [R][PT]: x, then q, logical order
+    float *Rr = lds + R * PT;   // [R][H + PT]: the last H values of r of the piece before, then this piece's
+
+    const int lane = threadIdx.x;
+    const int perRow = T >> 2;
+    const int nPieces = (perRow + PV - 1) / PV;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
+    const int nRows = static_cast<int>(min(static_cast<int64_t>(R), p.rows - row0));
+    const int rowBytes = T * 4;
+    const int tileBytes = nRows * rowBytes;   // rows behind the last one read zeros, their stores are dropped
+    const BufferRsrc bufIn = make_buffer(p.in + row0 * static_cast<int64_t>(T), tileBytes);
+    const BufferRsrc bufU = make_buffer((GATE != 0 ? p.u : p.in) + row0 * static_cast<int64_t>(T), tileBytes);
+    const BufferRsrc bufAdd = make_buffer((GATED_OUT && p.add ? p.add : p.in) + row0 * static_cast<int64_t>(T), tileBytes);
+    const BufferRsrc bufOut = make_buffer(p.out + row0 * static_cast<int64_t>(T), tileBytes);
+    const bool hasAdd = GATED_OUT && p.add != nullptr;
+
+    // byte offset of this lane's vector of piece k inside a row (the same on the way in and on the way out)
+    auto lane_offset = [&](int k) {
+        const int V = k * PV + lane;
+        return masked_offset(V < perRow, (CAUSAL ? V : perRow - 1 - V) * 16);
+    };
+    auto mirrored = [](float4 v) { return CAUSAL ? v : make_float4(v.w, v.z, v.y, v.x); };
+
+    for (int b = 0; b < R; ++b)
+        for (int c = lane; c < (H >> 2); c += kWave)
+            *reinterpret_cast<float4 *>(Rr + b * pitch + 4 * c) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+
+    float4 x[R], gu[GATE != 0 ? R : 1], more[GATED_OUT ? R : 1];
+    {
+        const int at = lane_offset(0);
+#pragma unroll
+        for (int b = 0; b < R; ++b) {
+            x[b] = buffer_load4(bufIn, at, b * rowBytes);
+            if (GATE != 0) gu[b] = buffer_load4(bufU, at, b * rowBytes);
+            if (GATED_OUT) more[b] = hasAdd ? buffer_load4(bufAdd, at, b * rowBytes) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+    }
+    const int r = lane / kParts, j = lane - r * kParts;
+    const float a = p.a, fL = static_cast<float>(L);
+    float carryP = 0.0f, carryQ = 0.0f;   // the row's running sums in front of the piece (the same in all its lanes)
+    auto step = [&](float &pp, float &qq, float xe) {
+        qq = a * (qq + pp);
+        pp = __builtin_fmaf(a, pp, xe);
+    };
+
+    for (int k = 0; k < nPieces; ++k) {
+        const int units = min(PV, perRow - k * PV);   // vectors per row in this piece
+        const int at = lane_offset(k);
+        // ---- this piece into LDS, then the next one's loads
+        bool bad = false;
+        float4 guOut[GATED_OUT ? R : 1], moreOut[GATED_OUT ? R : 1];
+#pragma unroll
+        for (int b = 0; b < R; ++b) {
+            float4 v = x[b];
+            if (GATED)
+                v = make_float4(v.x * spike_pdf(gu[b].x, p.theta, p.tauRho, p.gain), v.y * spike_pdf(gu[b].y, p.theta, p.tauRho, p.gain),
+                                v.z * spike_pdf(gu[b].z, p.theta, p.tauRho, p.gain), v.w * spike_pdf(gu[b].w, p.theta, p.tauRho, p.gain));
+            if (lane < units) {
+                *reinterpret_cast<float4 *>(Q + b * PT + 4 * lane) = mirrored(v);
+                bad |= ((v.x + v.y) + (v.z + v.w)) * 0.0f != 0.0f;   // infinite or NaN
+            }
+            if (GATED_OUT) { guOut[b] = gu[b]; moreOut[b] = more[b]; }
+        }
+        if (k + 1 < nPieces) {
+            const int next = lane_offset(k + 1);
+#pragma unroll
+            for (int b = 0; b < R; ++b) {
+                x[b] = buffer_load4(bufIn, next, b * rowBytes);
+                if (GATE != 0) gu[b] = buffer_load4(bufU, next, b * rowBytes);
+                if (GATED_OUT && hasAdd) more[b] = buffer_load4(bufAdd, next, b * rowBytes);
+            }
+        }
+        const bool chains = __builtin_amdgcn_ballot_w64(bad) != 0;
+        wave_sync();
+        if (chains) {
+            // a non-finite sample: from this piece on the running sums would carry it to the end of the row, where the
+            // sum over the taps lets it go after L samples; the rest of the tile as chains over the valid taps, from memory
+            const int done = k * PT, left = T - done;          // logical samples [done, T) remain
+            for (int e = lane; e < nRows * left; e += kWave) {
+                const int rr = e / left, i = done + (e - rr * left);
+                const int t = CAUSAL ? i : T - 1 - i;
+                const int64_t base = (row0 + rr) * static_cast<int64_t>(T);
+                const float *xr = p.in + base;
+                const int taps = CAUSAL ? min(t + 1, L) : min(T - t, L);
+                auto sample = [&](int s) { return GATED ? xr[s] * spike_pdf(p.u[base + s], p.theta, p.tauRho, p.gain) : xr[s]; };
+                float acc = 0.0f;
+                for (int q = 0; q < taps; ++q) acc = __builtin_fmaf(sample(CAUSAL ? t - q : t + q), p.filt[q], acc);
+                acc *= p.Ts;
+                if (GATED_OUT) {
+                    if (p.add) acc += p.add[base + t];
+                    acc *= spike_pdf(p.u[base + t], p.theta, p.tauRho, p.gain);
+                }
+                p.out[base + t] = acc;
+            }
+            return;
+        }
+        // ---- lane (row r, part j): vectors [v0, v1) of the row's piece; pass 1 from a zero state
+        const int v0 = (j * units) / kParts, v1 = ((j + 1) * units) / kParts;
+        float *q4 = Q + r * PT, *r4 = Rr + r * pitch + H;
+        float sp = 0.0f, sq = 0.0f;
+        for (int V = v0; V < v1; ++V) {
+            const float4 v = *reinterpret_cast<const float4 *>(q4 + 4 * V);
+            step(sp, sq, v.x);
+            step(sp, sq, v.y);
+            step(sp, sq, v.z);
+            step(sp, sq, v.w);
+        }
+        // ---- the state in front of every segment: inclusive scan over the row's lanes, the lane below hands its
+        //      result up, and the state in front of the piece passes through the samples in between
+        float cp, cq;
+        {
+            float rA = units == PV ? pc.aSegFull : pc.aSegLast[(v1 - v0) - units / kParts];
+            float rN = static_cast<float>((v1 - v0) << 2), rP = sp, rQ = sq;
+            auto below = [&](float own, float identity, auto ctrlTag) {
+                return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity),
+                                                                             __builtin_bit_cast(int, own), decltype(ctrlTag)::value,
+                                                                             0xf, 0xf, false));
+            };
+            auto take_in = [&](auto ctrlTag) {
+                const float lA = below(rA, 1.0f, ctrlTag), lN = below(rN, 0.0f, ctrlTag), lP = below(rP, 0.0f, ctrlTag),
+                            lQ = below(rQ, 0.0f, ctrlTag);
+                rQ = __builtin_fmaf(rA, __builtin_fmaf(rN, lP, lQ), rQ);
+                rP = __builtin_fmaf(rA, lP, rP);
+                rA *= lA;
+                rN += lN;
+            };
+            static_assert(kParts == 16, "a row's lanes are one row of the lane-shifting moves");
+            take_in(std::integral_constant<int, 0x111>{});
+            take_in(std::integral_constant<int, 0x112>{});
+            take_in(std::integral_constant<int, 0x114>{});
+            take_in(std::integral_constant<int, 0x118>{});
+            const float eA = below(rA, 1.0f, std::integral_constant<int, 0x111>{}), eN = below(rN, 0.0f, std::integral_constant<int, 0x111>{});
+            cp = __builtin_fmaf(eA, carryP, below(rP, 0.0f, std::integral_constant<int, 0x111>{}));
+            cq = __builtin_fmaf(eA, __builtin_fmaf(eN, carryP, carryQ), below(rQ, 0.0f, std::integral_constant<int, 0x111>{}));
+            // the state behind the piece, from the row's last lane
+            const int last = lane | (kParts - 1);
+            const float tA = __shfl(rA, last), tN = __shfl(rN, last), tP = __shfl(rP, last), tQ = __shfl(rQ, last);
+            const float nextQ = __builtin_fmaf(tA, __builtin_fmaf(tN, carryP, carryQ), tQ);
+            carryP = __builtin_fmaf(tA, carryP, tP);
+            carryQ = nextQ;
+        }
+        // ---- pass 2: q over x, r behind the history
+        {
+            float pp = cp, qq = cq;
+            for (int V = v0; V < v1; ++V) {
+                const float4 v = *reinterpret_cast<const float4 *>(q4 + 4 * V);
+                float4 qv, rv;
+                step(pp, qq, v.x); qv.x = qq; rv.x = __builtin_fmaf(fL, pp, qq);
+                step(pp, qq, v.y); qv.y = qq; rv.y = __builtin_fmaf(fL, pp, qq);
+                step(pp, qq, v.z); qv.z = qq; rv.z = __builtin_fmaf(fL, pp, qq);
+                step(pp, qq, v.w); qv.w = qq; rv.w = __builtin_fmaf(fL, pp, qq);
+                *reinterpret_cast<float4 *>(q4 + 4 * V) = qv;
+                *reinterpret_cast<float4 *>(r4 + 4 * V) = rv;
+            }
+        }
+        wave_sync();
+        // ---- out: y[i] = scale (q[i] - a^L r[i - L]); r[i - L] for the four samples of a vector lies in two aligned
+        //      vectors of the row's r (history included), (-L) & 3 samples off
+        {
+            const float aL = p.aL, scale = p.scale;
+            const int lo = (H - L) >> 2, off = (H - L) & 3;    // r[i - L] of local sample i is Rr[row][H - L + i]
+#pragma unroll
+            for (int b = 0; b < R; ++b) {
+                const int c = min(lane, units - 1);                 // (lanes behind the piece: their stores are dropped)
+                const float4 qv = *reinterpret_cast<const float4 *>(Q + b * PT + 4 * c);
+                const float *rrow = Rr + b * pitch + 4 * (c + lo);
+                const float4 ra = *reinterpret_cast<const float4 *>(rrow);
+                float4 rs;
+                if (off == 0) rs = ra;
+                else {
+                    const float4 rb = *reinterpret_cast<const float4 *>(rrow + 4);
+                    if (off == 1) rs = make_float4(ra.y, ra.z, ra.w, rb.x);
+                    else if (off == 2) rs = make_float4(ra.z, ra.w, rb.x, rb.y);
+                    else rs = make_float4(ra.w, rb.x, rb.y, rb.z);
+                }
+                float4 y = make_float4(scale * __builtin_fmaf(-aL, rs.x, qv.x), scale * __builtin_fmaf(-aL, rs.y, qv.y),
+                                       scale * __builtin_fmaf(-aL, rs.z, qv.z), scale * __builtin_fmaf(-aL, rs.w, qv.w));
+                y = mirrored(y);
+                if (GATED_OUT) {
+                    if (hasAdd) y = make_float4(y.x + moreOut[b].x, y.y + moreOut[b].y, y.z + moreOut[b].z, y.w + moreOut[b].w);
+                    y = make_float4(y.x * spike_pdf(guOut[b].x, p.theta, p.tauRho, p.gain), y.y * spike_pdf(guOut[b].y, p.theta, p.tauRho, p.gain),
+                                    y.z * spike_pdf(guOut[b].z, p.theta, p.tauRho, p.gain), y.w * spike_pdf(guOut[b].w, p.theta, p.tauRho, p.gain));
+                }
+                buffer_store4(bufOut, at, b * rowBytes, y);
+            }
+        }
+        // ---- the last H values of this piece's r become the history of the next
+        if (k + 1 < nPieces) {
+            wave_sync();
+            float4 keep[R];
+            const int c = min(lane, (H >> 2) - 1);
+#pragma unroll
+            for (int b = 0; b < R; ++b) keep[b] = *reinterpret_cast<const float4 *>(Rr + b * pitch + PT + 4 * c);
+            wave_sync();
+            if (lane < (H >> 2)) {
+#pragma unroll
+                for (int b = 0; b < R; ++b) *reinterpret_cast<float4 *>(Rr + b * pitch + 4 * c) = keep[b];
+            }
+            wave_sync();
+        }
+    }
+}
+
 }  // namespace slayer
 
 namespace slayer {
@@ -287,9 +516,12 @@ static bool launch_alpha(float *out, const float *in, const float *filt, int64_t
     const int64_t tiles = ceil_div(nNeurons, R);
     // rows of whole vectors, or at least a tensor of whole vectors (then every tile of 4 rows is one, too)
     const bool vec = T % 4 == 0;
-    if (generic_forced() || (!vec && (nNeurons * T) % 4 != 0) || T > kAlphaMaxT || !aligned16(out) || !aligned16(in) ||
+    if (generic_forced() || (!vec && (nNeurons * T) % 4 != 0) || !aligned16(out) || !aligned16(in) ||
         (u && !aligned16(u)) || (add && !aligned16(add)) || tiles >= (1LL << 31) || F >= (1 << 20))
         return false;
+    // longer rows go piece by piece: rows of whole vectors, a kernel no longer than a piece
+    const bool pieces = T > kAlphaMaxT;
+    if (pieces && (!vec || F > kPieceMaxL || T > kBufferMaxT)) return false;
     AlphaArgs a{};
     a.out = out; a.in = in; a.filt = filt;
     a.rows = nNeurons;
@@ -307,8 +539,23 @@ static bool launch_alpha(float *out, const float *in, const float *filt, int64_t
     a.Ts = Ts;
     a.u = u; a.theta = theta; a.tauRho = tauRho; a.gain = gain;
     a.add = add;
-    const size_t lds = static_cast<size_t>(2) * R * T * sizeof(float);
     const dim3 grid(static_cast<unsigned>(tiles));
+    if (pieces) {
+        AlphaPieces pc{};
+        pc.H = static_cast<int>((F + 3) / 4 * 4);
+        const int64_t lastUnits = (T / 4) % (kPieceT / 4);      // vectors per row in a shorter last piece (0: none)
+        const double ad = static_cast<double>(a.a);
+        pc.aSegFull = static_cast<float>(pow(ad, 4.0 * (kPieceT / 4 / parts)));
+        pc.aSegLast[0] = static_cast<float>(pow(ad, 4.0 * static_cast<double>(lastUnits / parts)));
+        pc.aSegLast[1] = static_cast<float>(pow(ad, 4.0 * static_cast<double>(lastUnits / parts + 1)));
+        const size_t ldsPieces = static_cast<size_t>(R) * (2 * kPieceT + pc.H) * sizeof(float);
+        if (u && gateOut) hipLaunchKernelGGL((alpha_psp_pieces_kernel<false, 2>), grid, dim3(kWave), ldsPieces, st, a, pc);
+        else if (u) hipLaunchKernelGGL((alpha_psp_pieces_kernel<false, 1>), grid, dim3(kWave), ldsPieces, st, a, pc);
+        else if (causal) hipLaunchKernelGGL((alpha_psp_pieces_kernel<true, 0>), grid, dim3(kWave), ldsPieces, st, a, pc);
+        else hipLaunchKernelGGL((alpha_psp_pieces_kernel<false, 0>), grid, dim3(kWave), ldsPieces, st, a, pc);
+        return true;
+    }
+    const size_t lds = static_cast<size_t>(2) * R * T * sizeof(float);
 #define SLAYER_ALPHA_LAUNCH(VEC)                                                                                       \
     do {                                                                                                              \
         if (u && gateOut) hipLaunchKernelGGL((alpha_psp_kernel<false, R, 2, VEC>), grid, dim3(kWave), lds, st, a);    \

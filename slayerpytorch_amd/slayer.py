@@ -520,9 +520,10 @@ def _unobserved(tensor):
 
 
 def _recursion_serves(x):
-    """Shapes that ``slayerCuda.pspAlpha`` runs as a recursion (others it would hand to conv / corr itself): rows of at
-    most 512 samples in a tensor of whole 16-byte vectors."""
-    return x.shape[-1] <= 512 and x.numel() % 4 == 0
+    """Shapes that ``slayerCuda.pspAlpha`` runs as a recursion (others it hands to conv / corr itself): rows of at most
+    512 samples in a tensor of whole 16-byte vectors, and longer rows of whole vectors (taken in pieces)."""
+    T = x.shape[-1]
+    return x.numel() % 4 == 0 if T <= 512 else T % 4 == 0
 
 
 class _pspSpikeFunction(torch.autograd.Function):

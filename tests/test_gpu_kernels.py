@@ -277,7 +277,12 @@ def close_to_alpha_sum(got, x, f, tau, mult, Ts, causal):
                                                # rows that are not whole vectors in a tensor that is: tiles of 4 rows travel whole
                                                ((2, 6, 1, 1, 350), 10.0, 1.0, 1.0), ((1, 4, 1, 1, 33), 10.0, 1.0, 1.0),
                                                ((1, 2, 1, 1, 7), 2.0, 1.0, 1.0), ((3, 4, 1, 1, 1), 10.0, 1.0, 1.0),
-                                               ((1, 10, 1, 1, 478), 25.0, 2.0, 0.5)])
+                                               ((1, 10, 1, 1, 478), 25.0, 2.0, 0.5),
+                                               # rows of more than 512 samples: pieces of 256 with the state carried along
+                                               ((2, 5, 1, 1, 2000), 10.0, 1.0, 1.0), ((1, 6, 1, 1, 1000), 10.0, 1.0, 1.0),
+                                               ((1, 3, 1, 1, 516), 4.0, 1.0, 1.0), ((1, 9, 1, 1, 1280), 10.0, -2.0, 1.0),
+                                               ((1, 2, 1, 1, 4100), 30.0, 1.0, 1.0), ((1, 7, 1, 1, 772), 1.0, 1.0, 0.1),
+                                               ((1, 4, 1, 1, 1028), 12.0, 1.0, 0.5)])
 @pytest.mark.parametrize("kind", ["dense", "spikes"])
 def test_psp_alpha_is_the_sum_over_the_taps_to_rounding(shape, tau, mult, Ts, kind):
     rng = np.random.default_rng(shape[-1] + int(tau))
@@ -328,12 +333,36 @@ def test_psp_alpha_filters_a_tile_with_a_non_finite_sample_with_the_taps(kind):
         assert rel_err(np.delete(got, slice(4, 8), 0), np.delete(want, slice(4, 8), 0)) <= REL_TOL
 
 
-@pytest.mark.parametrize("shape", [(1, 3, 1, 1, 350), (1, 2, 1, 1, 1000), (1, 3, 1, 1, 7)])
-def test_psp_alpha_outside_its_shapes_is_conv_and_corr(impl, shape):
-    # tensors that are not whole vectors, rows longer than 512 samples, and forced generic kernels: the taps
-    rng = np.random.default_rng(shape[-1])
-    tau, Ts = 10.0, 1.0
+@pytest.mark.parametrize("kind", ["infinity", "nan"])
+def test_psp_alpha_long_rows_switch_to_the_taps_at_a_non_finite_sample(kind):
+    # rows in pieces: the pieces in front of the sample (in the direction the filter runs) are the recursion's, from
+    # the sample's piece on the tile of 4 rows is the chain over the taps, bit for bit
+    rng = np.random.default_rng(10)
+    tau, Ts, T = 10.0, 1.0, 1200
     f = np.array(alphaKernel(tau, Ts, 300), dtype=np.float32)
+    x = rng.standard_normal((1, 12, 1, 1, T)).astype(np.float32)
+    x[0, 5, 0, 0, 700] = np.inf if kind == "infinity" else np.nan
+    for causal, op in ((True, "conv"), (False, "corr")):
+        got = host(slayerCuda.pspAlpha(dev(x), dev(f), tau, 1.0, Ts, causal)).reshape(12, T)
+        want = getattr(O, op)(x, f, Ts, fused=True).reshape(12, T)
+        # pieces of 256 from the end the filter starts at: the sample lies in the third one forward, the second one backward
+        chain = slice(512, T) if causal else slice(0, T - 256)
+        rest = slice(0, 512) if causal else slice(T - 256, T)
+        assert np.array_equal(bits(got[4:8, chain]), bits(want[4:8, chain]))
+        assert np.all(np.isfinite(got[4:8, rest])) and rel_err(got[4:8, rest], want[4:8, rest]) <= REL_TOL
+        assert np.all(np.isfinite(got[:4])) and np.all(np.isfinite(got[8:]))
+        assert rel_err(np.delete(got, slice(4, 8), 0), np.delete(want, slice(4, 8), 0)) <= REL_TOL
+
+
+@pytest.mark.parametrize("shape,tau", [((1, 3, 1, 1, 350), 10.0), ((1, 2, 1, 1, 1002), 10.0), ((1, 3, 1, 1, 7), 10.0),
+                                       ((1, 4, 1, 1, 1000), 40.0)])
+def test_psp_alpha_outside_its_shapes_is_conv_and_corr(impl, shape, tau):
+    # tensors that are not whole vectors, rows longer than 512 samples that are not whole vectors or whose kernel is
+    # longer than a piece (256 taps), and forced generic kernels: the taps
+    rng = np.random.default_rng(shape[-1])
+    Ts = 1.0
+    f = np.array(alphaKernel(tau, Ts, 1000), dtype=np.float32)
+    assert tau < 40 or f.size > 256
     x = (rng.random(shape) < 0.1).astype(np.float32)
     assert torch.equal(slayerCuda.pspAlpha(dev(x), dev(f), tau, 1.0, Ts, True), slayerCuda.conv(dev(x), dev(f), Ts))
     assert torch.equal(slayerCuda.pspAlpha(dev(x), dev(f), tau, 1.0, Ts, False), slayerCuda.corr(dev(x), dev(f), Ts))
@@ -341,7 +370,8 @@ def test_psp_alpha_outside_its_shapes_is_conv_and_corr(impl, shape):
 
 @pytest.mark.parametrize("shape,tau", [((2, 6, 5, 3, 300), 10.0), ((1, 9, 1, 1, 352), 4.0), ((3, 7, 1, 1, 64), 10.0),
                                        ((1, 1, 1, 1, 4), 1.0), ((2, 5, 1, 1, 512), 20.0), ((1, 3, 1, 1, 350), 10.0),
-                                       ((1, 2, 1, 1, 1000), 10.0), ((2, 6, 1, 1, 350), 10.0)])
+                                       ((1, 2, 1, 1, 1000), 10.0), ((2, 6, 1, 1, 350), 10.0), ((2, 5, 1, 1, 2000), 10.0),
+                                       ((1, 3, 1, 1, 1002), 10.0)])
 def test_spike_backward_psp_alpha_is_spikeBackward_then_corr(impl, shape, tau):
     # the surrogate gradient on the way in, then the correlation with the alpha kernel as a recursion: the values of
     # spikeBackward followed by pspAlpha bit for bit (the same products enter the same recursion), which is the sum over
@@ -353,7 +383,7 @@ def test_spike_backward_psp_alpha_is_spikeBackward_then_corr(impl, shape, tau):
     v = (rng.standard_normal(shape) * 4 + 8).astype(np.float32)
     got = slayerCuda.spikeBackwardPspAlpha(dev(g), dev(v), dev(f), tau, 1.0, theta, tauRho, scale, Ts)
     T = shape[-1]
-    if not impl and g.size % 4 == 0 and T <= 512:
+    if not impl and (g.size % 4 == 0 if T <= 512 else T % 4 == 0):
         two = slayerCuda.pspAlpha(slayerCuda.spikeBackward(dev(g), dev(v), theta, tauRho, scale), dev(f), tau, 1.0, Ts, False)
         assert np.array_equal(bits(host(got)), bits(host(two)))
     else:
@@ -365,7 +395,8 @@ def test_spike_backward_psp_alpha_is_spikeBackward_then_corr(impl, shape, tau):
 
 @pytest.mark.parametrize("shape,tau", [((2, 6, 5, 3, 300), 10.0), ((1, 9, 1, 1, 352), 4.0), ((3, 7, 1, 1, 64), 10.0),
                                        ((1, 1, 1, 1, 4), 1.0), ((2, 5, 1, 1, 512), 20.0), ((1, 3, 1, 1, 350), 10.0),
-                                       ((1, 2, 1, 1, 1000), 10.0), ((2, 6, 1, 1, 350), 10.0)])
+                                       ((1, 2, 1, 1, 1000), 10.0), ((2, 6, 1, 1, 350), 10.0), ((2, 5, 1, 1, 2000), 10.0),
+                                       ((1, 3, 1, 1, 1002), 10.0)])
 @pytest.mark.parametrize("direct", [False, True])
 def test_psp_spike_backward_alpha_is_corr_then_spikeBackward(impl, shape, tau, direct):
     # the other order: the correlation with the alpha kernel as a recursion, plus the gradient that reaches the spikes
@@ -380,7 +411,7 @@ def test_psp_spike_backward_alpha_is_corr_then_spikeBackward(impl, shape, tau, d
     v = (rng.standard_normal(shape) * 4 + 8).astype(np.float32)
     got = slayerCuda.pspSpikeBackwardAlpha(dev(g), dev(gs) if direct else None, dev(v), dev(f), tau, 1.0, theta, tauRho, scale, Ts)
     T = shape[-1]
-    recursion = not impl and g.size % 4 == 0 and T <= 512
+    recursion = not impl and (g.size % 4 == 0 if T <= 512 else T % 4 == 0)
     inner = slayerCuda.pspAlpha(dev(g), dev(f), tau, 1.0, Ts, False) if recursion else slayerCuda.corr(dev(g), dev(f), Ts)
     if direct:
         inner = inner + dev(gs)
