@@ -282,30 +282,34 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
 // front of the row).  LDS holds a piece in logical order: for the correlation the vectors and their elements are
 // mirrored between memory and LDS, which costs nothing (a lane loads and stores the same memory vector either way)
 // and leaves one form of the passes.  The loads of the next piece are issued before the passes over this one.
-constexpr int kPieceT = 256;              // samples per row and piece: 64 vectors, 4 per lane of a row
+constexpr int kPieceT = 256;              // samples per row and piece: 64 vectors, one per lane on the way in and out
 constexpr int kPieceMaxL = kPieceT;       // r[t - L] lies in this piece or the one before
 
 struct AlphaPieces {
     int H;              // history samples of r per row: L rounded up to whole vectors
-    float aSegFull;     // a^16: a lane's segment of a full piece
+    float aPow[5];      // a^16, a^32, a^64, a^128, a^256: runs of 1, 2, 4, 8 and 16 of a full piece's segments
     float aSegLast[2];  // a^n for the last piece's segments of units / 16 and units / 16 + 1 vectors
 };
 
-template <bool CAUSAL, int GATE>
+// OFF = H - L (0 .. 3): how far r[t - L] lies from a vector boundary - a template parameter, so that the way out is
+// straight-line code: together with loads and stores that are masked instead of branched around, every trip of the
+// piece loop issues the same memory instructions, and the wait for a piece's loads can leave the younger stores of the
+// piece before it in flight.
+template <bool CAUSAL, int GATE, int OFF>
 __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, AlphaPieces pc)
 {
     constexpr bool GATED = GATE == 1, GATED_OUT = GATE == 2;
-    constexpr int R = kAlphaRows, kParts = kWave / R, PT = kPieceT, PV = PT / 4;
-    static_assert(R == 4 && PV == kWave, "lane c moves vector c of every row's piece");
+    constexpr int R = kAlphaRows, kParts = kWave / R, PT = kPieceT, PV = PT / 4, SEG = PV / kParts;
+    static_assert(R == 4 && PV == kWave && SEG == 4, "lane c moves vector c of every row's piece; segments of 4 vectors");
     extern __shared__ __align__(16) float lds[];
-    const int T = p.T, L = p.L, H = pc.H;
+    const int T = p.T, L = p.L, H = pc.H, HV = H >> 2;
     const int pitch = H + PT;
     float *Q = lds;             // [R][PT]: x, then q, logical order
     float *Rr = lds + R * PT;   // [R][H + PT]: the last H values of r of the piece before, then this piece's
 
     const int lane = threadIdx.x;
     const int perRow = T >> 2;
-    const int nPieces = (perRow + PV - 1) / PV;
+    const int nFull = perRow / PV, lastUnits = perRow - nFull * PV;   // full pieces, vectors per row of a shorter last one
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
     const int nRows = static_cast<int>(min(static_cast<int64_t>(R), p.rows - row0));
     const int rowBytes = T * 4;
@@ -316,15 +320,22 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
     const BufferRsrc bufOut = make_buffer(p.out + row0 * static_cast<int64_t>(T), tileBytes);
     const bool hasAdd = GATED_OUT && p.add != nullptr;
 
-    // byte offset of this lane's vector of piece k inside a row (the same on the way in and on the way out)
+    // byte offset of this lane's vector of piece k inside a row (the same on the way in and on the way out; behind the
+    // row's end: out of range, which reads zeros and drops stores)
     auto lane_offset = [&](int k) {
         const int V = k * PV + lane;
         return masked_offset(V < perRow, (CAUSAL ? V : perRow - 1 - V) * 16);
     };
     auto mirrored = [](float4 v) { return CAUSAL ? v : make_float4(v.w, v.z, v.y, v.x); };
+    // Where vector V of a row's piece lies in LDS.  The lanes of a row walk segments of 4 vectors: laid out as they
+    // come, the vectors that 8 lanes read together would fall into two of the 8 groups of banks.  Exchanging the low
+    // bits of the position with the segment's number spreads them over all 8, for the lanes that walk segments and for
+    // the lanes that move consecutive vectors alike.
+    auto swz = [](int V) { return V ^ ((V >> 3) & 7); };
+    auto r_at = [&](int w) { return 4 * (w < HV ? w : HV + swz(w - HV)); };   // vector w of a row's r, history included
 
     for (int b = 0; b < R; ++b)
-        for (int c = lane; c < (H >> 2); c += kWave)
+        for (int c = lane; c < HV; c += kWave)
             *reinterpret_cast<float4 *>(Rr + b * pitch + 4 * c) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 
     float4 x[R], gu[GATE != 0 ? R : 1], more[GATED_OUT ? R : 1];
@@ -334,8 +345,12 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
         for (int b = 0; b < R; ++b) {
             x[b] = buffer_load4(bufIn, at, b * rowBytes);
             if (GATE != 0) gu[b] = buffer_load4(bufU, at, b * rowBytes);
-            if (GATED_OUT) more[b] = hasAdd ? buffer_load4(bufAdd, at, b * rowBytes) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (GATED_OUT) more[b] = buffer_load4(bufAdd, hasAdd ? at : kOutOfRange, b * rowBytes);
         }
+        // (stores that the range check drops: the first trip then finds the same instructions in flight as the later
+        // ones, which is what lets the compiler count them)
+#pragma unroll
+        for (int b = 0; b < R; ++b) buffer_store4(bufOut, kOutOfRange, b * rowBytes, make_float4(0.0f, 0.0f, 0.0f, 0.0f));
     }
     const int r = lane / kParts, j = lane - r * kParts;
     const float a = p.a, fL = static_cast<float>(L);
@@ -344,12 +359,32 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
         qq = a * (qq + pp);
         pp = __builtin_fmaf(a, pp, xe);
     };
+    auto below = [&](float own, float identity, auto ctrlTag) {   // row_shr:d as a compile-time constant
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity), __builtin_bit_cast(int, own),
+                                                                     decltype(ctrlTag)::value, 0xf, 0xf, false));
+    };
+    using Shr1 = std::integral_constant<int, 0x111>;
+    using Shr2 = std::integral_constant<int, 0x112>;
+    using Shr4 = std::integral_constant<int, 0x114>;
+    using Shr8 = std::integral_constant<int, 0x118>;
+    static_assert(kParts == 16, "a row's lanes are one row of the lane-shifting moves");
+    // what stays the same from one full piece to the next: where this lane's vectors lie in LDS (on the way in and out:
+    // vector `lane` of every row; in the passes: vectors 4 j .. 4 j + 3 of row r) and the decay over the 16 j samples
+    // between the piece's start and this lane's segment
+    const int mine = 4 * swz(lane), rMine = r_at(lane), rNext = r_at(lane + 1);
+    int seg[SEG];
+#pragma unroll
+    for (int i = 0; i < SEG; ++i) seg[i] = 4 * swz(SEG * j + i);
+    const float frontA = ((j & 1) ? pc.aPow[0] : 1.0f) * ((j & 2) ? pc.aPow[1] : 1.0f) * ((j & 4) ? pc.aPow[2] : 1.0f) *
+                         ((j & 8) ? pc.aPow[3] : 1.0f);
+    const float frontN = static_cast<float>(4 * SEG * j);
 
-    for (int k = 0; k < nPieces; ++k) {
-        const int units = min(PV, perRow - k * PV);   // vectors per row in this piece
+    // One piece.  FULL: all 64 vectors per row, every lane a segment of 4 - the shape of all pieces but possibly the last.
+    auto piece = [&](auto fullTag, int k) -> bool {
+        constexpr bool FULL = decltype(fullTag)::value;
+        const int units = FULL ? PV : lastUnits;
         const int at = lane_offset(k);
         // ---- this piece into LDS, then the next one's loads
-        bool bad = false;
         float4 guOut[GATED_OUT ? R : 1], moreOut[GATED_OUT ? R : 1];
 #pragma unroll
         for (int b = 0; b < R; ++b) {
@@ -357,67 +392,59 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
             if (GATED)
                 v = make_float4(v.x * spike_pdf(gu[b].x, p.theta, p.tauRho, p.gain), v.y * spike_pdf(gu[b].y, p.theta, p.tauRho, p.gain),
                                 v.z * spike_pdf(gu[b].z, p.theta, p.tauRho, p.gain), v.w * spike_pdf(gu[b].w, p.theta, p.tauRho, p.gain));
-            if (lane < units) {
-                *reinterpret_cast<float4 *>(Q + b * PT + 4 * lane) = mirrored(v);
-                bad |= ((v.x + v.y) + (v.z + v.w)) * 0.0f != 0.0f;   // infinite or NaN
-            }
+            // (lanes behind a shorter last piece hold zeros, which nobody reads)
+            *reinterpret_cast<float4 *>(Q + b * PT + mine) = mirrored(v);
             if (GATED_OUT) { guOut[b] = gu[b]; moreOut[b] = more[b]; }
         }
-        if (k + 1 < nPieces) {
-            const int next = lane_offset(k + 1);
+        {
+            const int next = lane_offset(k + 1);   // (behind the last piece: out of range, zeros that nobody uses)
 #pragma unroll
             for (int b = 0; b < R; ++b) {
                 x[b] = buffer_load4(bufIn, next, b * rowBytes);
                 if (GATE != 0) gu[b] = buffer_load4(bufU, next, b * rowBytes);
-                if (GATED_OUT && hasAdd) more[b] = buffer_load4(bufAdd, next, b * rowBytes);
+                if (GATED_OUT) more[b] = buffer_load4(bufAdd, hasAdd ? next : kOutOfRange, b * rowBytes);
             }
         }
-        const bool chains = __builtin_amdgcn_ballot_w64(bad) != 0;
         wave_sync();
-        if (chains) {
-            // a non-finite sample: from this piece on the running sums would carry it to the end of the row, where the
-            // sum over the taps lets it go after L samples; the rest of the tile as chains over the valid taps, from memory
-            const int done = k * PT, left = T - done;          // logical samples [done, T) remain
-            for (int e = lane; e < nRows * left; e += kWave) {
-                const int rr = e / left, i = done + (e - rr * left);
-                const int t = CAUSAL ? i : T - 1 - i;
-                const int64_t base = (row0 + rr) * static_cast<int64_t>(T);
-                const float *xr = p.in + base;
-                const int taps = CAUSAL ? min(t + 1, L) : min(T - t, L);
-                auto sample = [&](int s) { return GATED ? xr[s] * spike_pdf(p.u[base + s], p.theta, p.tauRho, p.gain) : xr[s]; };
-                float acc = 0.0f;
-                for (int q = 0; q < taps; ++q) acc = __builtin_fmaf(sample(CAUSAL ? t - q : t + q), p.filt[q], acc);
-                acc *= p.Ts;
-                if (GATED_OUT) {
-                    if (p.add) acc += p.add[base + t];
-                    acc *= spike_pdf(p.u[base + t], p.theta, p.tauRho, p.gain);
-                }
-                p.out[base + t] = acc;
-            }
-            return;
-        }
         // ---- lane (row r, part j): vectors [v0, v1) of the row's piece; pass 1 from a zero state
-        const int v0 = (j * units) / kParts, v1 = ((j + 1) * units) / kParts;
+        const int v0 = FULL ? SEG * j : (j * units) / kParts, v1 = FULL ? SEG * j + SEG : ((j + 1) * units) / kParts;
         float *q4 = Q + r * PT, *r4 = Rr + r * pitch + H;
         float sp = 0.0f, sq = 0.0f;
-        for (int V = v0; V < v1; ++V) {
-            const float4 v = *reinterpret_cast<const float4 *>(q4 + 4 * V);
+        auto pass1 = [&](int at4) {
+            const float4 v = *reinterpret_cast<const float4 *>(q4 + at4);
             step(sp, sq, v.x);
             step(sp, sq, v.y);
             step(sp, sq, v.z);
             step(sp, sq, v.w);
+        };
+        if constexpr (FULL) {
+#pragma unroll
+            for (int i = 0; i < SEG; ++i) pass1(seg[i]);
+        } else {
+            for (int V = v0; V < v1; ++V) pass1(4 * swz(V));
         }
-        // ---- the state in front of every segment: inclusive scan over the row's lanes, the lane below hands its
-        //      result up, and the state in front of the piece passes through the samples in between
-        float cp, cq;
-        {
-            float rA = units == PV ? pc.aSegFull : pc.aSegLast[(v1 - v0) - units / kParts];
-            float rN = static_cast<float>((v1 - v0) << 2), rP = sp, rQ = sq;
-            auto below = [&](float own, float identity, auto ctrlTag) {
-                return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity),
-                                                                             __builtin_bit_cast(int, own), decltype(ctrlTag)::value,
-                                                                             0xf, 0xf, false));
+        // ---- the state in front of every segment: an inclusive scan over the row's lanes (a run of n samples takes a
+        //      state (p, q) to (a^n p, a^n (q + n p)) plus the run's own sums; each lane takes in the run that ends d
+        //      lanes below it), the lane below hands its result up, and the state in front of the piece passes through
+        //      the samples in between.  In a full piece the run a lane has gathered before the step over d lanes is d
+        //      segments long wherever there is something to take in, so a^n and n are the same for the whole wavefront.
+        float cp, cq, tA, tN, rP = sp, rQ = sq;
+        if constexpr (FULL) {
+            auto take_in = [&](auto ctrlTag, float A, float N) {
+                const float lP = below(rP, 0.0f, ctrlTag), lQ = below(rQ, 0.0f, ctrlTag);
+                rQ = __builtin_fmaf(A, __builtin_fmaf(N, lP, lQ), rQ);
+                rP = __builtin_fmaf(A, lP, rP);
             };
+            take_in(Shr1{}, pc.aPow[0], 4.0f * SEG);
+            take_in(Shr2{}, pc.aPow[1], 8.0f * SEG);
+            take_in(Shr4{}, pc.aPow[2], 16.0f * SEG);
+            take_in(Shr8{}, pc.aPow[3], 32.0f * SEG);
+            cp = __builtin_fmaf(frontA, carryP, below(rP, 0.0f, Shr1{}));
+            cq = __builtin_fmaf(frontA, __builtin_fmaf(frontN, carryP, carryQ), below(rQ, 0.0f, Shr1{}));
+            tA = pc.aPow[4];
+            tN = static_cast<float>(PT);
+        } else {
+            float rA = (v1 - v0) > units / kParts ? pc.aSegLast[1] : pc.aSegLast[0], rN = static_cast<float>((v1 - v0) << 2);
             auto take_in = [&](auto ctrlTag) {
                 const float lA = below(rA, 1.0f, ctrlTag), lN = below(rN, 0.0f, ctrlTag), lP = below(rP, 0.0f, ctrlTag),
                             lQ = below(rQ, 0.0f, ctrlTag);
@@ -426,53 +453,63 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
                 rA *= lA;
                 rN += lN;
             };
-            static_assert(kParts == 16, "a row's lanes are one row of the lane-shifting moves");
-            take_in(std::integral_constant<int, 0x111>{});
-            take_in(std::integral_constant<int, 0x112>{});
-            take_in(std::integral_constant<int, 0x114>{});
-            take_in(std::integral_constant<int, 0x118>{});
-            const float eA = below(rA, 1.0f, std::integral_constant<int, 0x111>{}), eN = below(rN, 0.0f, std::integral_constant<int, 0x111>{});
-            cp = __builtin_fmaf(eA, carryP, below(rP, 0.0f, std::integral_constant<int, 0x111>{}));
-            cq = __builtin_fmaf(eA, __builtin_fmaf(eN, carryP, carryQ), below(rQ, 0.0f, std::integral_constant<int, 0x111>{}));
-            // the state behind the piece, from the row's last lane
-            const int last = lane | (kParts - 1);
-            const float tA = __shfl(rA, last), tN = __shfl(rN, last), tP = __shfl(rP, last), tQ = __shfl(rQ, last);
+            take_in(Shr1{});
+            take_in(Shr2{});
+            take_in(Shr4{});
+            take_in(Shr8{});
+            const float eA = below(rA, 1.0f, Shr1{}), eN = below(rN, 0.0f, Shr1{});
+            cp = __builtin_fmaf(eA, carryP, below(rP, 0.0f, Shr1{}));
+            cq = __builtin_fmaf(eA, __builtin_fmaf(eN, carryP, carryQ), below(rQ, 0.0f, Shr1{}));
+            tA = __shfl(rA, lane | (kParts - 1));
+            tN = __shfl(rN, lane | (kParts - 1));
+        }
+        {   // the state behind the piece, from the row's last lane
+            const float tP = __shfl(rP, lane | (kParts - 1)), tQ = __shfl(rQ, lane | (kParts - 1));
             const float nextQ = __builtin_fmaf(tA, __builtin_fmaf(tN, carryP, carryQ), tQ);
             carryP = __builtin_fmaf(tA, carryP, tP);
             carryQ = nextQ;
         }
+        // An infinite or NaN sample (or sums that outgrow fp32) shows in the running sums behind the piece, and would stay
+        // in them to the end of the row, where the sum over the taps lets it go after L samples: the caller then takes
+        // this piece and the rest of the tile as chains over the taps.
+        if (__builtin_amdgcn_ballot_w64((carryP + carryQ) * 0.0f != 0.0f) != 0) return false;
         // ---- pass 2: q over x, r behind the history
         {
             float pp = cp, qq = cq;
-            for (int V = v0; V < v1; ++V) {
-                const float4 v = *reinterpret_cast<const float4 *>(q4 + 4 * V);
+            auto pass2 = [&](int at4) {
+                const float4 v = *reinterpret_cast<const float4 *>(q4 + at4);
                 float4 qv, rv;
                 step(pp, qq, v.x); qv.x = qq; rv.x = __builtin_fmaf(fL, pp, qq);
                 step(pp, qq, v.y); qv.y = qq; rv.y = __builtin_fmaf(fL, pp, qq);
                 step(pp, qq, v.z); qv.z = qq; rv.z = __builtin_fmaf(fL, pp, qq);
                 step(pp, qq, v.w); qv.w = qq; rv.w = __builtin_fmaf(fL, pp, qq);
-                *reinterpret_cast<float4 *>(q4 + 4 * V) = qv;
-                *reinterpret_cast<float4 *>(r4 + 4 * V) = rv;
+                *reinterpret_cast<float4 *>(q4 + at4) = qv;
+                *reinterpret_cast<float4 *>(r4 + at4) = rv;
+            };
+            if constexpr (FULL) {
+#pragma unroll
+                for (int i = 0; i < SEG; ++i) pass2(seg[i]);
+            } else {
+                for (int V = v0; V < v1; ++V) pass2(4 * swz(V));
             }
         }
         wave_sync();
-        // ---- out: y[i] = scale (q[i] - a^L r[i - L]); r[i - L] for the four samples of a vector lies in two aligned
-        //      vectors of the row's r (history included), (-L) & 3 samples off
+        // ---- out: y[i] = scale (q[i] - a^L r[i - L]); r[i - L] of a row's local sample i is Rr[row][OFF + i]: the four
+        //      of a vector lie in two aligned vectors of the row's r (history included), OFF samples off
         {
             const float aL = p.aL, scale = p.scale;
-            const int lo = (H - L) >> 2, off = (H - L) & 3;    // r[i - L] of local sample i is Rr[row][H - L + i]
+            const int c = FULL ? lane : min(lane, units - 1);    // (lanes behind the piece: their stores are dropped)
+            const int qAt = FULL ? mine : 4 * swz(c), raAt = FULL ? rMine : r_at(c), rbAt = FULL ? rNext : r_at(c + 1);
 #pragma unroll
             for (int b = 0; b < R; ++b) {
-                const int c = min(lane, units - 1);                 // (lanes behind the piece: their stores are dropped)
-                const float4 qv = *reinterpret_cast<const float4 *>(Q + b * PT + 4 * c);
-                const float *rrow = Rr + b * pitch + 4 * (c + lo);
-                const float4 ra = *reinterpret_cast<const float4 *>(rrow);
-                float4 rs;
-                if (off == 0) rs = ra;
-                else {
-                    const float4 rb = *reinterpret_cast<const float4 *>(rrow + 4);
-                    if (off == 1) rs = make_float4(ra.y, ra.z, ra.w, rb.x);
-                    else if (off == 2) rs = make_float4(ra.z, ra.w, rb.x, rb.y);
+                const float4 qv = *reinterpret_cast<const float4 *>(Q + b * PT + qAt);
+                const float *rrow = Rr + b * pitch;
+                const float4 ra = *reinterpret_cast<const float4 *>(rrow + raAt);
+                float4 rs = ra;
+                if constexpr (OFF != 0) {
+                    const float4 rb = *reinterpret_cast<const float4 *>(rrow + rbAt);
+                    if constexpr (OFF == 1) rs = make_float4(ra.y, ra.z, ra.w, rb.x);
+                    else if constexpr (OFF == 2) rs = make_float4(ra.z, ra.w, rb.x, rb.y);
                     else rs = make_float4(ra.w, rb.x, rb.y, rb.z);
                 }
                 float4 y = make_float4(scale * __builtin_fmaf(-aL, rs.x, qv.x), scale * __builtin_fmaf(-aL, rs.y, qv.y),
@@ -486,19 +523,47 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
                 buffer_store4(bufOut, at, b * rowBytes, y);
             }
         }
-        // ---- the last H values of this piece's r become the history of the next
-        if (k + 1 < nPieces) {
+        // ---- the last H values of this piece's r become the history of the next.  They lie behind the history, so
+        //      reading and writing need no synchronisation in between - and nothing may sit in a local array across a
+        //      wave_sync: its fence sends such an array through scratch memory, and the wait for that stalls on every
+        //      load and store in flight.
+        if constexpr (FULL) {
             wave_sync();
-            float4 keep[R];
-            const int c = min(lane, (H >> 2) - 1);
+            if (lane < HV) {
 #pragma unroll
-            for (int b = 0; b < R; ++b) keep[b] = *reinterpret_cast<const float4 *>(Rr + b * pitch + PT + 4 * c);
-            wave_sync();
-            if (lane < (H >> 2)) {
-#pragma unroll
-                for (int b = 0; b < R; ++b) *reinterpret_cast<float4 *>(Rr + b * pitch + 4 * c) = keep[b];
+                for (int b = 0; b < R; ++b)
+                    *reinterpret_cast<float4 *>(Rr + b * pitch + 4 * lane) = *reinterpret_cast<const float4 *>(Rr + b * pitch + r_at(PV + lane));
             }
             wave_sync();
+        }
+        return true;
+    };
+
+    int k = 0;
+    bool finite = true;
+    for (; k < nFull && finite; ++k) finite = piece(std::true_type{}, k);
+    if (finite && lastUnits != 0) {
+        finite = piece(std::false_type{}, k);
+        ++k;
+    }
+    if (!finite) {
+        // the piece that found the non-finite sample (k - 1) and everything behind it, from memory
+        const int done = (k - 1) * PT, left = T - done;          // logical samples [done, T) remain
+        for (int e = lane; e < nRows * left; e += kWave) {
+            const int rr = e / left, i = done + (e - rr * left);
+            const int t = CAUSAL ? i : T - 1 - i;
+            const int64_t base = (row0 + rr) * static_cast<int64_t>(T);
+            const float *xr = p.in + base;
+            const int taps = CAUSAL ? min(t + 1, L) : min(T - t, L);
+            auto sample = [&](int s) { return GATED ? xr[s] * spike_pdf(p.u[base + s], p.theta, p.tauRho, p.gain) : xr[s]; };
+            float acc = 0.0f;
+            for (int q = 0; q < taps; ++q) acc = __builtin_fmaf(sample(CAUSAL ? t - q : t + q), p.filt[q], acc);
+            acc *= p.Ts;
+            if (GATED_OUT) {
+                if (p.add) acc += p.add[base + t];
+                acc *= spike_pdf(p.u[base + t], p.theta, p.tauRho, p.gain);
+            }
+            p.out[base + t] = acc;
         }
     }
 }
@@ -545,14 +610,24 @@ static bool launch_alpha(float *out, const float *in, const float *filt, int64_t
         pc.H = static_cast<int>((F + 3) / 4 * 4);
         const int64_t lastUnits = (T / 4) % (kPieceT / 4);      // vectors per row in a shorter last piece (0: none)
         const double ad = static_cast<double>(a.a);
-        pc.aSegFull = static_cast<float>(pow(ad, 4.0 * (kPieceT / 4 / parts)));
+        for (int i = 0; i < 5; ++i) pc.aPow[i] = static_cast<float>(pow(ad, 16.0 * static_cast<double>(1 << i)));
         pc.aSegLast[0] = static_cast<float>(pow(ad, 4.0 * static_cast<double>(lastUnits / parts)));
         pc.aSegLast[1] = static_cast<float>(pow(ad, 4.0 * static_cast<double>(lastUnits / parts + 1)));
         const size_t ldsPieces = static_cast<size_t>(R) * (2 * kPieceT + pc.H) * sizeof(float);
-        if (u && gateOut) hipLaunchKernelGGL((alpha_psp_pieces_kernel<false, 2>), grid, dim3(kWave), ldsPieces, st, a, pc);
-        else if (u) hipLaunchKernelGGL((alpha_psp_pieces_kernel<false, 1>), grid, dim3(kWave), ldsPieces, st, a, pc);
-        else if (causal) hipLaunchKernelGGL((alpha_psp_pieces_kernel<true, 0>), grid, dim3(kWave), ldsPieces, st, a, pc);
-        else hipLaunchKernelGGL((alpha_psp_pieces_kernel<false, 0>), grid, dim3(kWave), ldsPieces, st, a, pc);
+#define SLAYER_PIECES_LAUNCH(OFFV)                                                                                      \
+        do {                                                                                                           \
+            if (u && gateOut) hipLaunchKernelGGL((alpha_psp_pieces_kernel<false, 2, OFFV>), grid, dim3(kWave), ldsPieces, st, a, pc); \
+            else if (u) hipLaunchKernelGGL((alpha_psp_pieces_kernel<false, 1, OFFV>), grid, dim3(kWave), ldsPieces, st, a, pc);       \
+            else if (causal) hipLaunchKernelGGL((alpha_psp_pieces_kernel<true, 0, OFFV>), grid, dim3(kWave), ldsPieces, st, a, pc);   \
+            else hipLaunchKernelGGL((alpha_psp_pieces_kernel<false, 0, OFFV>), grid, dim3(kWave), ldsPieces, st, a, pc);              \
+        } while (0)
+        switch (pc.H - static_cast<int>(F)) {
+            case 0: SLAYER_PIECES_LAUNCH(0); break;
+            case 1: SLAYER_PIECES_LAUNCH(1); break;
+            case 2: SLAYER_PIECES_LAUNCH(2); break;
+            default: SLAYER_PIECES_LAUNCH(3); break;
+        }
+#undef SLAYER_PIECES_LAUNCH
         return true;
     }
     const size_t lds = static_cast<size_t>(2) * R * T * sizeof(float);
