@@ -549,6 +549,17 @@ def other_rows(device, cpu_leg=False):
             r["separate_calls_traffic_over_this_time_vs_hbm_peak"] = ab * numel / seconds / 1e9 / HBM_PEAK_GBS
         return r
 
+    def cold(r, ab, src, fn):
+        """Adds to row ``r`` the time of ``fn(input)`` when the input is not in the 256 MB last-level cache: a different
+        copy of ``src`` per launch, more than 512 MB of copies in turn.  The row's own figure re-reads one input, which
+        kernels that load with the default cache policy find in that cache when the tensor fits it."""
+        copies = [src.clone() for _ in range(max(2, -(-(640 << 20) // (src.numel() * 4))))]
+        burst = [copies[i % len(copies)] for i in range(K)]
+        t = timed(lambda x: fn(x), K, (burst, lambda: None))
+        r["us_with_input_not_in_cache"] = t * 1e6
+        r["hbm_frac_with_input_not_in_cache"] = ab * src.numel() / t / 1e9 / HBM_PEAK_GBS
+        return r
+
     def potentials(shape, srm_k, ref_k, tau_sr, rate_target):
         """A membrane potential of the kind real layers see: the PSP signal of Bernoulli(0.05) spikes - smooth, above
         the threshold for runs of samples - scaled so that about ``rate_target`` of the samples fire."""
@@ -602,6 +613,8 @@ def other_rows(device, cpu_leg=False):
                     timed(lambda: slayerCuda.pspAlpha(src, srm77, 10.0, 1.0, 1.0, causal), K), shape)
             taps = timed(lambda: (slayerCuda.conv if causal else slayerCuda.corr)(src, srm77, 1.0), K)
             r["us_as_sums_over_the_taps"], r["hbm_frac_as_sums_over_the_taps"] = taps * 1e6, 8 * n / taps / 1e9 / HBM_PEAK_GBS
+            if nm == "dense":
+                cold(r, 8, src, lambda x: slayerCuda.pspAlpha(x, srm77, 10.0, 1.0, 1.0, causal))
             out.append(r)
     del xg, src
     # the spike kernel's time depends on its input: the rows above (and the headline) feed independent normal samples
@@ -659,13 +672,15 @@ def other_rows(device, cpu_leg=False):
     psp = torch.tensor(loihiPspKernel(1024, 128, 0), dtype=torch.float32, device=device)
     n = w.numel()
     s, v, u = slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1)
-    out.append(row("loihi_forward", 16, n, timed(lambda: slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1), K), shape))
+    out.append(cold(row("loihi_forward", 16, n, timed(lambda: slayerLoihiCuda.getSpikes(w, 0, 5120, 1024, 128, 1), K), shape),
+                    16, w, lambda x: slayerLoihiCuda.getSpikes(x, 0, 5120, 1024, 128, 1)))
     out.append(row("loihi_forward_spike_and_voltage_delay1_fused", 24, n,
                    timed(lambda: slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 1, voltage=True, current=False), K),
                    shape, moved=12))
     out.append(row("loihi_forward_spike_only_delay1_fused", 24, n,
                    timed(lambda: slayerLoihiCuda.getSpikesDelayed(w, 0, 5120, 1024, 128, 1, 1, voltage=False, current=False), K),
                    shape, moved=8))
+    cold(out[-1], 8, w, lambda x: slayerLoihiCuda.getSpikesDelayed(x, 0, 5120, 1024, 128, 1, 1, voltage=False, current=False))
     out.append(row("loihi_backward_pdf_plus_corr110", 20, n,
                    timed(lambda: slayerCuda.spikeBackwardCorr(gl, v, psp, 5120.0, 5120.0, 1 / 195.0, 1.0), K),
                    shape, moved=12))

@@ -88,8 +88,8 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             if (b * kWave < tileVec) {
-                x[b] = buffer_load4(bufIn, (lane + b * kWave) * 16, 0);
-                if (GATE != 0) gu[b] = buffer_load4(bufU, (lane + b * kWave) * 16, 0);
+                x[b] = buffer_load4<kCached>(bufIn, (lane + b * kWave) * 16, 0);
+                if (GATE != 0) gu[b] = buffer_load4<kCached>(bufU, (lane + b * kWave) * 16, 0);
             }
         }
 #pragma unroll
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(64) void alpha_psp_kernel(AlphaArgs p)
                 if (GATED_OUT) {
                     if (p.add) {
                         const BufferRsrc bufAdd = make_buffer(p.add + row0 * static_cast<int64_t>(T), nVec * 16);
-                        const float4 more = buffer_load4(bufAdd, (lane + b * kWave) * 16, 0);
+                        const float4 more = buffer_load4<kCached>(bufAdd, (lane + b * kWave) * 16, 0);
                         y = make_float4(y.x + more.x, y.y + more.y, y.z + more.z, y.w + more.w);
                     }
                     y = make_float4(y.x * spike_pdf(gu[b].x, p.theta, p.tauRho, p.gain), y.y * spike_pdf(gu[b].y, p.theta, p.tauRho, p.gain),
@@ -338,20 +338,25 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
         for (int c = lane; c < HV; c += kWave)
             *reinterpret_cast<float4 *>(Rr + b * pitch + 4 * c) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 
-    float4 x[R], gu[GATE != 0 ? R : 1], more[GATED_OUT ? R : 1];
-    {
-        const int at = lane_offset(0);
+    // Two sets of registers take turns: a piece's loads are issued two pieces ahead, behind the stores of the piece that
+    // has just left the set, so a piece and a half of loads is in flight while a piece is worked on.
+    constexpr int NG = GATE != 0 ? R : 1, NM = GATED_OUT ? R : 1;
+    float4 xA[R], guA[NG], moreA[NM], xB[R], guB[NG], moreB[NM];
+    auto load_piece = [&](int k, float4 (&x)[R], float4 (&gu)[NG], float4 (&more)[NM]) {
+        const int at = lane_offset(k);      // (behind the last piece: out of range, zeros that nobody uses)
 #pragma unroll
         for (int b = 0; b < R; ++b) {
-            x[b] = buffer_load4(bufIn, at, b * rowBytes);
-            if (GATE != 0) gu[b] = buffer_load4(bufU, at, b * rowBytes);
-            if (GATED_OUT) more[b] = buffer_load4(bufAdd, hasAdd ? at : kOutOfRange, b * rowBytes);
+            x[b] = buffer_load4<kCached>(bufIn, at, b * rowBytes);
+            if (GATE != 0) gu[b] = buffer_load4<kCached>(bufU, at, b * rowBytes);
+            if (GATED_OUT) more[b] = buffer_load4<kCached>(bufAdd, hasAdd ? at : kOutOfRange, b * rowBytes);
         }
-        // (stores that the range check drops: the first trip then finds the same instructions in flight as the later
-        // ones, which is what lets the compiler count them)
+    };
+    load_piece(0, xA, guA, moreA);
+    // (stores that the range check drops: the first trip then finds the same instructions in flight as the later ones -
+    // a piece's loads, the stores of the piece before, the next piece's loads - which is what lets the compiler count them)
 #pragma unroll
-        for (int b = 0; b < R; ++b) buffer_store4(bufOut, kOutOfRange, b * rowBytes, make_float4(0.0f, 0.0f, 0.0f, 0.0f));
-    }
+    for (int b = 0; b < R; ++b) buffer_store4(bufOut, kOutOfRange, b * rowBytes, make_float4(0.0f, 0.0f, 0.0f, 0.0f));
+    load_piece(1, xB, guB, moreB);
     const int r = lane / kParts, j = lane - r * kParts;
     const float a = p.a, fL = static_cast<float>(L);
     float carryP = 0.0f, carryQ = 0.0f;   // the row's running sums in front of the piece (the same in all its lanes)
@@ -380,12 +385,13 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
     const float frontN = static_cast<float>(4 * SEG * j);
 
     // One piece.  FULL: all 64 vectors per row, every lane a segment of 4 - the shape of all pieces but possibly the last.
-    auto piece = [&](auto fullTag, int k) -> bool {
+    constexpr int kNone = 0x7fffffff;
+    int firstBad = kNone;
+    auto piece = [&](auto fullTag, int k, float4 (&x)[R], float4 (&gu)[NG], float4 (&more)[NM]) {
         constexpr bool FULL = decltype(fullTag)::value;
         const int units = FULL ? PV : lastUnits;
         const int at = lane_offset(k);
-        // ---- this piece into LDS, then the next one's loads
-        float4 guOut[GATED_OUT ? R : 1], moreOut[GATED_OUT ? R : 1];
+        // ---- this piece into LDS
 #pragma unroll
         for (int b = 0; b < R; ++b) {
             float4 v = x[b];
@@ -394,16 +400,6 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
                                 v.z * spike_pdf(gu[b].z, p.theta, p.tauRho, p.gain), v.w * spike_pdf(gu[b].w, p.theta, p.tauRho, p.gain));
             // (lanes behind a shorter last piece hold zeros, which nobody reads)
             *reinterpret_cast<float4 *>(Q + b * PT + mine) = mirrored(v);
-            if (GATED_OUT) { guOut[b] = gu[b]; moreOut[b] = more[b]; }
-        }
-        {
-            const int next = lane_offset(k + 1);   // (behind the last piece: out of range, zeros that nobody uses)
-#pragma unroll
-            for (int b = 0; b < R; ++b) {
-                x[b] = buffer_load4(bufIn, next, b * rowBytes);
-                if (GATE != 0) gu[b] = buffer_load4(bufU, next, b * rowBytes);
-                if (GATED_OUT) more[b] = buffer_load4(bufAdd, hasAdd ? next : kOutOfRange, b * rowBytes);
-            }
         }
         wave_sync();
         // ---- lane (row r, part j): vectors [v0, v1) of the row's piece; pass 1 from a zero state
@@ -469,10 +465,12 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
             carryP = __builtin_fmaf(tA, carryP, tP);
             carryQ = nextQ;
         }
-        // An infinite or NaN sample (or sums that outgrow fp32) shows in the running sums behind the piece, and would stay
-        // in them to the end of the row, where the sum over the taps lets it go after L samples: the caller then takes
-        // this piece and the rest of the tile as chains over the taps.
-        if (__builtin_amdgcn_ballot_w64((carryP + carryQ) * 0.0f != 0.0f) != 0) return false;
+        // An infinite or NaN sample (or sums that outgrow fp32) shows in the running sums behind the piece, and stays in
+        // them to the end of the row, where the sum over the taps lets it go after L samples: the first such piece is
+        // noted, and the tile is redone from there as chains over the taps once the walk is over.  (Leaving the walk
+        // here instead costs every tile: with a way out of the loop the compiler no longer counts the stores in flight
+        // and waits for all of them at every piece.)
+        firstBad = (firstBad == kNone && __builtin_amdgcn_ballot_w64((carryP + carryQ) * 0.0f != 0.0f) != 0) ? k : firstBad;
         // ---- pass 2: q over x, r behind the history
         {
             float pp = cp, qq = cq;
@@ -516,13 +514,14 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
                                        scale * __builtin_fmaf(-aL, rs.z, qv.z), scale * __builtin_fmaf(-aL, rs.w, qv.w));
                 y = mirrored(y);
                 if (GATED_OUT) {
-                    if (hasAdd) y = make_float4(y.x + moreOut[b].x, y.y + moreOut[b].y, y.z + moreOut[b].z, y.w + moreOut[b].w);
-                    y = make_float4(y.x * spike_pdf(guOut[b].x, p.theta, p.tauRho, p.gain), y.y * spike_pdf(guOut[b].y, p.theta, p.tauRho, p.gain),
-                                    y.z * spike_pdf(guOut[b].z, p.theta, p.tauRho, p.gain), y.w * spike_pdf(guOut[b].w, p.theta, p.tauRho, p.gain));
+                    if (hasAdd) y = make_float4(y.x + more[b].x, y.y + more[b].y, y.z + more[b].z, y.w + more[b].w);
+                    y = make_float4(y.x * spike_pdf(gu[b].x, p.theta, p.tauRho, p.gain), y.y * spike_pdf(gu[b].y, p.theta, p.tauRho, p.gain),
+                                    y.z * spike_pdf(gu[b].z, p.theta, p.tauRho, p.gain), y.w * spike_pdf(gu[b].w, p.theta, p.tauRho, p.gain));
                 }
                 buffer_store4(bufOut, at, b * rowBytes, y);
             }
         }
+        load_piece(k + 2, x, gu, more);
         // ---- the last H values of this piece's r become the history of the next.  They lie behind the history, so
         //      reading and writing need no synchronisation in between - and nothing may sit in a local array across a
         //      wave_sync: its fence sends such an array through scratch memory, and the wait for that stalls on every
@@ -536,19 +535,24 @@ __global__ __launch_bounds__(64) void alpha_psp_pieces_kernel(AlphaArgs p, Alpha
             }
             wave_sync();
         }
-        return true;
     };
 
     int k = 0;
-    bool finite = true;
-    for (; k < nFull && finite; ++k) finite = piece(std::true_type{}, k);
-    if (finite && lastUnits != 0) {
-        finite = piece(std::false_type{}, k);
-        ++k;
+    for (; k + 1 < nFull; k += 2) {
+        piece(std::true_type{}, k, xA, guA, moreA);
+        piece(std::true_type{}, k + 1, xB, guB, moreB);
     }
-    if (!finite) {
-        // the piece that found the non-finite sample (k - 1) and everything behind it, from memory
-        const int done = (k - 1) * PT, left = T - done;          // logical samples [done, T) remain
+    if (k < nFull) {
+        piece(std::true_type{}, k, xA, guA, moreA);
+        if (lastUnits != 0) piece(std::false_type{}, nFull, xB, guB, moreB);
+    } else if (lastUnits != 0) {
+        piece(std::false_type{}, nFull, xA, guA, moreA);
+    }
+    if (firstBad != kNone) {
+        // from the piece that met the non-finite sample on, from memory - once the stores of the walk have landed, so
+        // that what the chains write is what stays
+        __builtin_amdgcn_s_waitcnt(0);
+        const int done = firstBad * PT, left = T - done;          // logical samples [done, T) remain
         for (int e = lane; e < nRows * left; e += kWave) {
             const int rr = e / left, i = done + (e - rr * left);
             const int t = CAUSAL ? i : T - 1 - i;

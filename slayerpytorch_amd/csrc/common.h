@@ -144,10 +144,18 @@ __device__ __forceinline__ BufferRsrc make_buffer(const void *base)
 // once per kernel, so the "non-temporal" hint keeps them from displacing each other in L2
 // (measured on MI355X: a 16-byte-per-lane copy runs at 6.5 TB/s with the hint, 6.0 without).
 constexpr int kStream = 2;  // "nt" bit of the buffer instruction's cache-policy field
+// Loads of kernels that walk along rows whose input is typically another kernel's recent output or a tensor that is
+// read again soon (the PSP recursion, the Loihi neuron) keep the default policy.  Measured with plain copies of the
+// walking pattern: the hint on loads gains nothing on tensors beyond the 256 MB last-level cache (1 GB moved: 202 us
+// with the hint on stores only, 205 us on both) and costs a third when the input fits that cache and was touched
+// recently (262 MB moved: 36 us against 54 us), because the hint keeps it from being found there.  Stores keep the
+// hint at every size; kernels whose loads are one flat stream keep it on loads too (6 % on large tensors).
+constexpr int kCached = 0;
 
+template <int POLICY = kStream>
 __device__ __forceinline__ float buffer_load(BufferRsrc b, int laneBytes, int uniformBytes)
 {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(b, laneBytes, uniformBytes, kStream));
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(b, laneBytes, uniformBytes, POLICY));
 }
 
 typedef float float4_ext __attribute__((ext_vector_type(4)));

@@ -181,10 +181,10 @@ __global__ __launch_bounds__(64) void loihi_tile_kernel(float *__restrict__ s, f
             if (lane + b * kWave < total) {
                 const int off = (rc.r * T + tL + rc.c * V) * 4;
                 if (VEC) {
-                    const float4 q = buffer_load4(bufW, off, 0);
+                    const float4 q = buffer_load4<kCached>(bufW, off, 0);
                     x[4 * b] = q.x; x[4 * b + 1] = q.y; x[4 * b + 2] = q.z; x[4 * b + 3] = q.w;
                 } else {
-                    x[b] = buffer_load(bufW, off, 0);
+                    x[b] = buffer_load<kCached>(bufW, off, 0);
                 }
             }
             rc.advance(dr, dc, perRow);
@@ -368,7 +368,7 @@ __global__ __launch_bounds__(64, 2) void loihi_lines_kernel(float *__restrict__ 
             const int r = b * RPI + subRow;
             const int time = TC * j - ((o0 + r * T) & 31) + col;
             // any sample of the vector inside the row (with whole-vector rows: all or none)
-            x[b] = buffer_load4(bufW, masked_offset(r < nRows && time + 3 >= 0 && time < T, (r * T + time) * 4), 0);
+            x[b] = buffer_load4<kCached>(bufW, masked_offset(r < nRows && time + 3 >= 0 && time < T, (r * T + time) * 4), 0);
         }
     };
 
