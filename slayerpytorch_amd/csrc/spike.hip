@@ -143,8 +143,9 @@ __global__ __launch_bounds__(64) void spike_stream_kernel(float *__restrict__ s,
 //    that arrives below the threshold never fires.  All 64 lanes mark the samples at or above it
 //    ("candidates", a few per cent) while the piece is staged, one bit per sample, and the walking lanes go from
 //    candidate to candidate: test the sample's current value and, on a spike, add nu[0..NU) onto the NU samples
-//    from it on, in place - the same fp32 additions in the same order as the sequential loop;
-//  * any other kernel, and tiles with a row that is above the threshold more than one sample in 12: every
+//    from it on, in place - the same fp32 additions in the same order as the sequential loop - and strike the
+//    samples that the response has taken below the threshold from the candidates;
+//  * any other kernel, and tiles with a row that is above the threshold half of the time or more: every
 //    sample in turn through a register window that is spread over the lanes of the row (further down).
 // The last LAG samples of a piece are not final until the next piece arrives: they (and their candidate bits)
 // are copied to the front of the tile and open the next piece.  Taps beyond nuSize are -0.0f, whose addition
@@ -397,8 +398,6 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 
         // ---- walk: lane = row.  Columns [0, W) become final in this step.
         const int W = last ? n + LAG : n;
-        // going from candidate to candidate costs a round trip through LDS each, and the wavefront stays as long as
-        // its busiest row: it pays while no row of the tile has more than a candidate per 24 samples
         // The walking wavefront shares its SIMD's issue slots with the wavefronts that move data, so what counts
         // here is the number of instructions, not the active lanes: all 64 lanes take part, kParts = 64 / R per
         // row.  They count the row's candidates and note its non-empty candidate words together; in the walk every
@@ -420,11 +419,13 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
                 mine += __shfl_xor(mine, off, kWave);
                 nzw |= __shfl_xor(nzw, off, kWave);
             }
-            // going from candidate to candidate pays while no row of the tile has more than a candidate per 12 samples:
-            // the wavefront stays as long as its busiest row (1 in 24: 102 us, 1 in 12: 92 us, 1 in 4: 91 us on
-            // (64,256,1,1,2000) with 2.3 % candidates, where a few rows per launch exceed 1 in 24; tensors whose
-            // busiest rows are above the threshold most of the time take the window walk at any of these settings)
-            hop = __builtin_amdgcn_ballot_w64(mine * 12 > W) == 0;
+            // Going from candidate to candidate costs a round trip through LDS per visit, and the wavefront stays as long
+            // as its busiest row.  Visits are spikes plus the candidates that no response has removed (below), so the
+            // count of candidates on arrival only bounds them: a smooth potential that fires 4 % of the time arrives with
+            // 19 % candidates (137 us this way, 156 us sample by sample, on (12,16,32,32,300)), one that fires 12 % of
+            // the time with 45 % (198 us against 170 us).  Tiles with a row above the threshold half of the time or more
+            // take the walk over every sample (a third: 145 us on the first of the two tensors).
+            hop = __builtin_amdgcn_ballot_w64(mine * 2 > W) == 0;
         }
         if (hop) {
             const int words = (W + 31) >> 5;
@@ -452,12 +453,28 @@ __global__ __launch_bounds__(64) void spike_tile_kernel(float *__restrict__ s, f
 #pragma unroll
                     for (int j = 0; j < kRounds; ++j)
                         if ((j + 1) * kParts <= NU || part + j * kParts < NU) val[j] = q[j * kParts];
-                    const float x0 = __shfl(val[0], cr * kParts, kWave);   // the candidate itself: the value lane 0 of the row read
+                    const float x0 = q[-part];   // the candidate itself (one address per row: a broadcast, no shuffle)
                     if (x0 >= theta) {
                         fired |= 1u << k;
+                        // The response only lowers the potential: a sample it takes below the threshold will never
+                        // fire and stops being a candidate.  A potential that stays above the threshold for many
+                        // samples (the output of a PSP filter) is then visited once per spike, not once per sample.
+                        // Each lane knows the new value of its own samples; a ballot collects the row's verdicts
+                        // (bit p of the row's field: sample k + j kParts + p), and what falls into the next word
+                        // of candidates is cleared there by one lane.
+                        uint64_t gone = 0u;
 #pragma unroll
-                        for (int j = 0; j < kRounds; ++j)
-                            if ((j + 1) * kParts <= NU || part + j * kParts < NU) q[j * kParts] = val[j] + myTap[j];
+                        for (int j = 0; j < kRounds; ++j) {
+                            const bool mineToo = (j + 1) * kParts <= NU || part + j * kParts < NU;
+                            const float now = val[j] + myTap[j];
+                            if (mineToo) q[j * kParts] = now;
+                            const uint64_t below = __builtin_amdgcn_ballot_w64(mineToo && now < theta);
+                            gone |= ((below >> (lane - part)) & ((1ull << kParts) - 1ull)) << (j * kParts);
+                        }
+                        gone <<= k;
+                        cm &= ~static_cast<uint32_t>(gone);
+                        const uint32_t over = static_cast<uint32_t>(gone >> 32);
+                        if (over != 0u && part == 0 && w + 1 < words) cand[cr * MP + w + 1] &= ~over;
                     }
                 }
             }
