@@ -523,9 +523,11 @@ __global__ __launch_bounds__(64, 2) void loihi_lines_kernel(float *__restrict__ 
                 }
                 const int off = masked_offset(ok, (r * T + time) * 4);
                 const uint32_t m = masks[r * LPP + (col >> 5)] >> (col & 31);
-                if (OUTS == 0 && u) buffer_store4(bufU, off, 0, *reinterpret_cast<const float4 *>(tileC + r * P + col));
-                if (OUTS == 2 || (OUTS == 0 && v))
-                    buffer_store4(bufV, off, 0, *reinterpret_cast<const float4 *>(tileV + (kVol ? r * P + col : 0)));
+                // (OUTS = 0: an output that is not wanted is masked, not skipped - with a fixed number of stores per trip
+                // the wait for the next piece's loads can leave all of them in flight, not just the spikes')
+                if (OUTS == 0) buffer_store4(bufU, u ? off : kOutOfRange, 0, *reinterpret_cast<const float4 *>(tileC + r * P + col));
+                if (OUTS == 2 || OUTS == 0)
+                    buffer_store4(bufV, (OUTS == 2 || v) ? off : kOutOfRange, 0, *reinterpret_cast<const float4 *>(tileV + (kVol ? r * P + col : 0)));
                 buffer_store4(bufS, off, 0,
                               make_float4((m & 1u) ? 1.0f : 0.0f, (m & 2u) ? 1.0f : 0.0f,
                                           (m & 4u) ? 1.0f : 0.0f, (m & 8u) ? 1.0f : 0.0f));
