@@ -55,6 +55,7 @@ class event():
     def __init__(self, xEvent, yEvent, pEvent, tEvent):
         self._raw = None
         self._format = None
+        self._decoded = None
         self.dim = 1 if yEvent is None else 2
         self.x = np.asarray(xEvent)
         self.y = yEvent if yEvent is None else np.asarray(yEvent)
@@ -75,13 +76,24 @@ class event():
         raw = raw[:n * _EVENT_BYTES[fmt]]
         x, y, p, t = _decode(raw, fmt)
         self = cls(x, y, p, t / 1000)          # spike times in ms
-        # the decoded arrays are handed out read-only: an in-place edit would not be seen by the packed path (assign
-        # a new array, e.g. ev.t = ev.t + 5, to change the events)
-        for a in (self.x, self.y, self.p, self.t):
-            if a is not None:
-                a.setflags(write=False)
+        # The members are ordinary writable arrays, as in the reference.  An edit in place (ev.t -= ev.t.min(),
+        # ev.x[:] = W - 1 - ev.x) is not seen by __setattr__, so a private copy of what the file bytes decode to
+        # is kept, and the bytes only stand for the events while the members still equal it (_packed).
+        self._decoded = tuple(None if a is None else a.copy() for a in (self.x, self.y, self.p, self.t))
         self._raw, self._format = raw, fmt
         return self
+
+    def _packed(self):
+        """The layout of the file bytes while they still describe the events, else None."""
+        if self._raw is None:
+            return None
+        now = (self.x, self.y, self.p, self.t)
+        same = all((a is None and b is None) or (a is not None and b is not None and a.shape == b.shape and
+                                                  a.dtype == b.dtype and np.array_equal(a, b))
+                   for a, b in zip(now, self._decoded))
+        if not same:       # edited in place: from now on the members are what counts
+            self._raw = self._format = None
+        return self._format
 
     def _shift(self, samplingTime, T, randomShift):
         """The reference's random start bin (src/spikeFileIO.py:80-90), drawn on the host."""
@@ -120,7 +132,7 @@ def toSpikeTensorBatch(events, emptyTensor, samplingTime=1, randomShift=False, b
     lib = _lib.load()
     base = emptyTensor.clone() if mode == 1 else None
     shifts = [ev._shift(samplingTime, T, randomShift) for ev in events]
-    formats = {ev._format for ev in events}
+    formats = {ev._packed() for ev in events}
     packed = None not in formats and len(formats) == 1 and all(ev.dim == (1 if ev._format == 1 else 2) for ev in events)
     if packed and events[0]._format == 1 and H != 1:
         raise RuntimeError("1-D events need a tensor of height 1, got %d" % H)

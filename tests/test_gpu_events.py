@@ -125,17 +125,26 @@ def test_events_changed_after_reading_are_binned_as_changed():
     # an augmentation between read and bin (a flip, a time offset): the members are binned, as in the reference,
     # not the file's bytes
     raw, shape = GOLD["nmnist_bs2"], (2, 34, 34, 350)
-    ev = snn.io.event._fromBytes(raw, 2)
-    with pytest.raises(ValueError):
-        ev.x[0] = 3                                   # the decoded arrays are read-only: assign new ones
-    ev.x = 33 - ev.x
-    ev.t = ev.t + 20.0
-    got = ev.toSpikeTensor(torch.zeros(shape, device="cuda"), 1.0).cpu().numpy()
     x, y, p, t = O.decode_events(raw, 2)
     want = O.bin_events(np.zeros(shape, np.float32), 33 - x, y, p - p.min(), t / 1000 + 20.0, 1.0)
-    assert np.array_equal(got, want)
     same = snn.io.event._fromBytes(raw, 2).toSpikeTensor(torch.zeros(shape, device="cuda"), 1.0).cpu().numpy()
-    assert not np.array_equal(got, same)
+    assert not np.array_equal(want, same)
+    ev = snn.io.event._fromBytes(raw, 2)             # new arrays assigned
+    ev.x = 33 - ev.x
+    ev.t = ev.t + 20.0
+    assert np.array_equal(ev.toSpikeTensor(torch.zeros(shape, device="cuda"), 1.0).cpu().numpy(), want)
+    ev = snn.io.event._fromBytes(raw, 2)             # the same edits in place, as the reference's writable arrays allow
+    assert ev._packed() == 2
+    ev.x[:] = 33 - ev.x
+    ev.t += 20.0
+    assert np.array_equal(ev.toSpikeTensor(torch.zeros(shape, device="cuda"), 1.0).cpu().numpy(), want)
+    assert ev._packed() is None
+    ev = snn.io.event._fromBytes(raw, 2)             # a single element
+    ev.p[7] = 1 - ev.p[7]
+    pp = p - p.min()
+    pp[7] = 1 - pp[7]
+    assert np.array_equal(ev.toSpikeTensor(torch.zeros(shape, device="cuda"), 1.0).cpu().numpy(),
+                          O.bin_events(np.zeros(shape, np.float32), x, y, pp, t / 1000, 1.0))
 
 
 def test_argument_errors():
