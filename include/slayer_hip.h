@@ -184,9 +184,12 @@ int slayer_psp_spike_f32(float *s, float *u, const float *a, const float *srm, c
  * kernel that the reference's layers build (src/slayer.py:98-123) and hand to slayerCuda.conv / corr
  * (src/slayer.py:878-899, src/cuda/slayerKernels.cu:41-75) - computed as a two-term recursion over time instead of
  * an F-tap sum: about 10 operations per sample whatever F is.  causal != 0: the convolution of slayer_conv_f32;
- * causal == 0: the correlation of slayer_corr_f32.  `filt` must hold exactly that kernel (it is what a tile with a
- * non-finite sample, and every shape outside rows of at most 512 samples in a 16-byte aligned tensor of whole
- * 16-byte vectors, is filtered with, through the F-tap kernels); the caller states tau and mult.  The result agrees with the F-tap chain to
+ * causal == 0: the correlation of slayer_corr_f32.  The recursion serves rows of at most 512 samples in a 16-byte
+ * aligned tensor of whole 16-byte vectors, and longer rows of whole vectors (T % 4 == 0) with F <= 256, which it
+ * takes in pieces of 256 samples with the state carried from piece to piece.  `filt` must hold exactly that kernel:
+ * it is what every other shape is filtered with (through the F-tap kernels), and what a tile of four rows that holds
+ * a non-finite sample is filtered with (a long row: from the piece with that sample on), so that infinities and NaNs
+ * reach the samples the reference lets them reach.  The caller states tau and mult.  The result agrees with the F-tap chain to
  * rounding, relative to the sum of the magnitudes of the terms of the UNTRUNCATED response
  * (sum_k |x[t -+ k]| |mult| (k Ts / tau) exp(1 - k Ts / tau) over all k): 1e-5 of that sum at most, about 1e-6
  * measured.  Optional: a caller that does not know its filter to be an alpha kernel keeps calling
