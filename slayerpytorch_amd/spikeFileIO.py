@@ -44,30 +44,43 @@ class event():
     and time stamps ``t`` in ms (src/spikeFileIO.py:6-34).  As in the reference the polarity is
     shifted so that its minimum is 0."""
 
-    def __setattr__(self, name, value):
-        # the file bytes stand for the events only as long as nobody reassigns them (a flip, a time offset, any
-        # augmentation): after that the members are binned, as in the reference
-        if name in ("x", "y", "p", "t"):
-            object.__setattr__(self, "_raw", None)
-            object.__setattr__(self, "_format", None)
-        object.__setattr__(self, name, value)
+    # The events of a file are binned from the file's bytes (one launch decodes and bins a whole batch) for as long as
+    # nobody outside this module has touched the decoded arrays: x, y, p and t are properties over private members,
+    # and reading one of them - the only way to edit it in place, ev.t -= ev.t.min(), ev.x[:] = W - 1 - ev.x - or
+    # assigning a new array makes the members what is binned from then on, as in the reference.  The arrays
+    # themselves are ordinary writable arrays.
+    def _touched(self):
+        self._raw = None
+        self._format = None
+
+    def _member(name):
+        def get(self):
+            self._touched()
+            return getattr(self, "_" + name)
+
+        def put(self, value):
+            self._touched()
+            setattr(self, "_" + name, value)
+        return property(get, put)
+
+    x, y, p, t = _member("x"), _member("y"), _member("p"), _member("t")
+    del _member
 
     def __init__(self, xEvent, yEvent, pEvent, tEvent):
         self._raw = None
         self._format = None
-        self._decoded = None
         self.dim = 1 if yEvent is None else 2
-        self.x = np.asarray(xEvent)
-        self.y = yEvent if yEvent is None else np.asarray(yEvent)
-        self.p = np.asarray(pEvent)
-        self.t = np.asarray(tEvent)
-        if not issubclass(self.x.dtype.type, np.integer):
-            self.x = self.x.astype("int")
-        if not issubclass(self.p.dtype.type, np.integer):
-            self.p = self.p.astype("int")
-        if self.dim == 2 and not issubclass(self.y.dtype.type, np.integer):
-            self.y = self.y.astype("int")
-        self.p = self.p - self.p.min()
+        self._x = np.asarray(xEvent)
+        self._y = yEvent if yEvent is None else np.asarray(yEvent)
+        self._p = np.asarray(pEvent)
+        self._t = np.asarray(tEvent)
+        if not issubclass(self._x.dtype.type, np.integer):
+            self._x = self._x.astype("int")
+        if not issubclass(self._p.dtype.type, np.integer):
+            self._p = self._p.astype("int")
+        if self.dim == 2 and not issubclass(self._y.dtype.type, np.integer):
+            self._y = self._y.astype("int")
+        self._p = self._p - self._p.min()
 
     @classmethod
     def _fromBytes(cls, raw, fmt):
@@ -76,32 +89,20 @@ class event():
         raw = raw[:n * _EVENT_BYTES[fmt]]
         x, y, p, t = _decode(raw, fmt)
         self = cls(x, y, p, t / 1000)          # spike times in ms
-        # The members are ordinary writable arrays, as in the reference.  An edit in place (ev.t -= ev.t.min(),
-        # ev.x[:] = W - 1 - ev.x) is not seen by __setattr__, so a private copy of what the file bytes decode to
-        # is kept, and the bytes only stand for the events while the members still equal it (_packed).
-        self._decoded = tuple(None if a is None else a.copy() for a in (self.x, self.y, self.p, self.t))
         self._raw, self._format = raw, fmt
         return self
 
     def _packed(self):
         """The layout of the file bytes while they still describe the events, else None."""
-        if self._raw is None:
-            return None
-        now = (self.x, self.y, self.p, self.t)
-        same = all((a is None and b is None) or (a is not None and b is not None and a.shape == b.shape and
-                                                  a.dtype == b.dtype and np.array_equal(a, b))
-                   for a, b in zip(now, self._decoded))
-        if not same:       # edited in place: from now on the members are what counts
-            self._raw = self._format = None
         return self._format
 
     def _shift(self, samplingTime, T, randomShift):
         """The reference's random start bin (src/spikeFileIO.py:80-90), drawn on the host."""
         if randomShift is not True:
             return 0
-        return int(np.random.randint(max(int(self.t.min() / samplingTime),
-                                         int(self.t.max() / samplingTime) - T,
-                                         T - int(self.t.max() / samplingTime), 1)))
+        return int(np.random.randint(max(int(self._t.min() / samplingTime),
+                                         int(self._t.max() / samplingTime) - T,
+                                         T - int(self._t.max() / samplingTime), 1)))
 
     def toSpikeTensor(self, emptyTensor, samplingTime=1, randomShift=False, binningMode="OR"):
         """Bins the events into ``emptyTensor`` (C, H, W, T), a float32 tensor on the GPU, in place,
@@ -162,10 +163,10 @@ def toSpikeTensorBatch(events, emptyTensor, samplingTime=1, randomShift=False, b
             if ev.dim == 1 and H != 1:
                 raise RuntimeError("1-D events need a tensor of height 1, got %d" % H)
             dev = emptyTensor.device
-            x = torch.from_numpy(np.ascontiguousarray(ev.x, dtype=np.int32)).to(dev)
-            p = torch.from_numpy(np.ascontiguousarray(ev.p, dtype=np.int32)).to(dev)
-            t = torch.from_numpy(np.ascontiguousarray(ev.t, dtype=np.float64)).to(dev)
-            y = None if ev.dim == 1 else torch.from_numpy(np.ascontiguousarray(ev.y, dtype=np.int32)).to(dev)
+            x = torch.from_numpy(np.ascontiguousarray(ev._x, dtype=np.int32)).to(dev)
+            p = torch.from_numpy(np.ascontiguousarray(ev._p, dtype=np.int32)).to(dev)
+            t = torch.from_numpy(np.ascontiguousarray(ev._t, dtype=np.float64)).to(dev)
+            y = None if ev.dim == 1 else torch.from_numpy(np.ascontiguousarray(ev._y, dtype=np.int32)).to(dev)
             _lib.check(lib.slayer_bin_events_f32(
                 _ptr(emptyTensor[i]), _ptr(base[i]) if base is not None else None, _ptr(x),
                 _ptr(y) if y is not None else None, _ptr(p), _ptr(t), x.numel(), shifts[i], C, H, W, T,
