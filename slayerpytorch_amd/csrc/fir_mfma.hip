@@ -100,6 +100,7 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
     };
     // vector e = lane + 64 k of a tile is vector e % lenIn of row e / lenIn; samples outside the row read as zeros
     float4 pre[NV], preU[GATED ? NV : 1];
+    constexpr int kEarlyU = (GATED && LINEAR) ? NV / 2 : NV;   // potentials fetched ahead with the samples (LINEAR is the only gated layout)
     // the lane index behind a barrier for the optimiser: the (row, vector) sequences below do not depend on the
     // tile, and kept across the walk they would cost 2 registers per vector
     auto lane_again = [&]() {
@@ -111,12 +112,16 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
         if (LINEAR) {
             const BufferRsrc bufIn = make_buffer(p.in + q.row0 * T, q.nRows * T * 4);
             const BufferRsrc bufU = make_buffer(GATED ? p.gate.u + q.row0 * T : p.in, q.nRows * T * 4);
+            // (all NV of them, whatever p.nv is: the vectors behind the 16 rows fail the buffers' range check and cost
+            // nothing, and a fixed number of loads and stores per tile is what lets the wait for a tile's loads leave
+            // the younger stores of the tile before it in flight)
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                if (k < p.nv) {
-                    pre[k] = buffer_load4(bufIn, (lane + kWave * k) * 16, 0);
-                    if (GATED) preU[k] = buffer_load4(bufU, (lane + kWave * k) * 16, 0);
-                }
+                // (the vector's number travels in the instruction's scalar offset: one address register for all of them)
+                pre[k] = buffer_load4(bufIn, lane * 16, kWave * 16 * k);
+                // (the potentials of the tile's second half are fetched by stage(), while it gates the first half: with
+                // both tensors of a whole tile in registers during the walk, the 110-tap kernel spilled)
+                if (GATED && k < kEarlyU) preU[k] = buffer_load4(bufU, lane * 16, kWave * 16 * k);
             }
             return;
         }
@@ -134,8 +139,13 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
             rc.advance(dr, dc, lenIn);
         }
     };
-    auto stage = [&]() {  // the fetched vectors into LDS; true if a sample is not finite
+    auto stage = [&](const Tile &q) {  // the fetched vectors into LDS; true if a sample is not finite
         bool bad = false;
+        if (GATED && LINEAR) {
+            const BufferRsrc bufU = make_buffer(p.gate.u + q.row0 * T, q.nRows * T * 4);
+#pragma unroll
+            for (int k = kEarlyU; k < NV; ++k) preU[k] = buffer_load4(bufU, lane * 16, kWave * 16 * k);
+        }
         RowCol rc;
         if (!LINEAR) rc.init(lane_again(), lenIn, 1.0f / static_cast<float>(lenIn));
         const int dr = kWave / lenIn, dc = kWave % lenIn;
@@ -169,16 +179,24 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
     if (i >= p.nItems) return;
     Tile cur = tile_of(i);
     fetch(cur);
+    {
+        // stores that the range check drops, as many as a tile's: the first trip then finds the same instructions in
+        // flight as the later ones - a tile's loads, then the stores of the tile before - so that one count serves all
+        const BufferRsrc none = make_buffer(p.out, 0);
+#pragma unroll
+        for (int k = 0; k < NV; ++k) buffer_store4(none, (lane + kWave * k) * 16, 0, make_float4(static_cast<float>(k), 0.0f, 0.0f, 0.0f));
+    }
     for (;;) {
-        const bool chains = stage();
+        const bool chains = stage(cur);
         wave_sync();
         const uint32_t iNext = i + gridDim.x;
         const bool more = iNext < p.nItems;
-        Tile next = cur;
-        if (more) {
-            next = tile_of(iNext);
-            fetch(next);
-        }
+        // (the next tile's loads behind every wait of stage(): moved up between them, as the compiler likes to do to
+        // reuse the registers one by one, each of those waits would also wait for the stores of the tile before)
+        // (behind the last tile: a tile without rows, whose loads all fail the range check)
+        Tile next = tile_of(more ? iNext : i);
+        if (!more) next.nRows = 0;
+        fetch(next);
         if (chains) {
             // a non-finite sample: the tile's outputs as sequential chains over the valid taps
             const int width = min(16 * cur.nb, T - cur.t0);
@@ -238,8 +256,8 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
             const BufferRsrc bufOut = make_buffer(p.out + cur.row0 * T, chains ? 0 : cur.nRows * T * 4);
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                if (k < p.nv)
-                    buffer_store4(bufOut, (lane + kWave * k) * 16, 0, *reinterpret_cast<const float4 *>(X + 4 * (lane + kWave * k)));
+                // (vectors from p.nv on lie behind the 16 rows: read from the tile's first bytes, dropped by the range check)
+                buffer_store4(bufOut, lane * 16, kWave * 16 * k, *reinterpret_cast<const float4 *>(X + (k < p.nv ? 4 * (lane + kWave * k) : 0)));
                 if (k % 8 == 7) __builtin_amdgcn_sched_barrier(0);  // a few vectors at a time: they occupy registers
             }
         } else {
