@@ -132,6 +132,8 @@ FIR_CASES = [
     # fewer than 16 rows, a row count that is no multiple of 16, every window size (4..9 blocks)
     ((37,), 300, 77), ((3, 16), 304, 66), ((5,), 2000, 50), ((21,), 1000, 97), ((100,), 28, 45), ((7,), 16, 34),
     ((33,), 20, 40), ((5,), 64, 129), ((18,), 76, 113), ((40,), 44, 82), ((2, 9), 48, 34), ((1,), 300, 100),
+    # whole rows of 13..16 vectors per lane, each size of the bf16 kernel's window (3..5 chunks of 32 samples)
+    ((20,), 252, 120), ((17,), 204, 60), ((35,), 236, 90), ((16,), 220, 36), ((9,), 244, 100),
 ]
 
 
@@ -173,6 +175,61 @@ def test_fir_filter_lengths_around_kernel_choices(Fl, T):
             assert rel_err(np.where(fin, got, 0), np.where(fin, want, 0)) <= REL_TOL, (op, Fl, T)
         else:
             assert np.array_equal(np.where(np.isnan(got), 0, bits(got)), np.where(np.isnan(want), 0, bits(want))), (op, Fl, T)
+
+
+def sum_bounds(x, f):
+    """Per output of corr(x, f): the exact sum, sum |x||f| and the sum of |x| over its window, in double precision."""
+    x64, f64 = np.asarray(x, np.float64), np.asarray(f, np.float64)
+    pad = np.zeros(len(f64) - 1)
+    exact = np.stack([np.correlate(np.concatenate([r, pad]), f64, "valid") for r in x64])
+    mag = np.stack([np.correlate(np.concatenate([np.abs(r), pad]), np.abs(f64), "valid") for r in x64])
+    win = np.stack([np.correlate(np.concatenate([np.abs(r), pad]), np.ones_like(f64), "valid") for r in x64])
+    return exact, mag, win
+
+
+@pytest.mark.parametrize("Fl", [40, 60, 77, 90, 110, 129])
+def test_corr_from_split_operands_is_as_close_as_the_chain(Fl):
+    # Whole rows with T / 4 odd run on bf16 matrix instructions over a three-way split of samples and taps.  The split
+    # leaves out products below 2^-23 of a term and every instruction rounds its accumulator: the result stays within
+    # 1e-6 of the sum of the terms' magnitudes (a tenth of the tolerance; measured: up to 4.4e-7 where one term
+    # dominates a sum, 2.8e-7 on samples of one size), for samples and taps of every size and mixed signs ...
+    rng = np.random.default_rng(Fl)
+    T = 300
+    f = (rng.standard_normal(Fl) * np.exp2(rng.integers(-20, 20, Fl))).astype(np.float32)
+    for lo, hi in [(0, 1), (-60, 60), (-30, -29), (90, 100)]:
+        x = (rng.standard_normal((48, T)) * np.exp2(rng.integers(lo, hi, (48, T)))).astype(np.float32)
+        got = host(slayerCuda.corr(dev(x), dev(f), 1.0)).astype(np.float64)
+        exact, mag, _ = sum_bounds(x, f)
+        assert np.all(np.abs(got - exact) <= 1e-6 * mag), (Fl, lo, hi, np.max(np.abs(got - exact) / mag))
+    # ... down to where the instruction reads a bf16 operand below 2^-126 as zero: parts of samples and taps below
+    # 2^-102, at most 2^-124 * (sum |f| + sum |x| over the window) in absolute terms
+    for scale in [1e-30, 1e-33, 1e-36, 1e-38, 1e-42]:
+        x = (rng.standard_normal((32, T)) * scale).astype(np.float32)
+        for xx, ff in [(x, f), (rng.standard_normal((32, T)).astype(np.float32), (f * np.float32(scale)).astype(np.float32))]:
+            got = host(slayerCuda.corr(dev(xx), dev(ff), 1.0)).astype(np.float64)
+            exact, mag, win = sum_bounds(xx, ff)
+            floor = 2.0 ** -124 * (np.sum(np.abs(ff.astype(np.float64))) + win)
+            assert np.all(np.abs(got - exact) <= 1e-6 * mag + floor), scale
+
+
+def test_corr_from_split_operands_with_a_tap_that_is_not_finite():
+    # such a tap has no split: every tile takes the chains, whose bits are the oracle's
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((40, 300)).astype(np.float32)
+    v = (rng.standard_normal((40, 300)) * 3 + 8).astype(np.float32)
+    for bad in [np.inf, -np.inf, np.nan]:
+        f = rng.standard_normal(77).astype(np.float32)
+        f[33] = bad
+        got = host(slayerCuda.corr(dev(x), dev(f), 0.5))
+        want = O.corr(x, f, 0.5, fused=True)
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(np.where(np.isnan(got), 0, bits(got)), np.where(np.isnan(want), 0, bits(want)))
+        gated = host(slayerCuda.spikeBackwardCorr(dev(x), dev(v), dev(f), 10.0, 5.0, 1.0, 0.5))
+        want = O.corr(O.spike_bwd(x, v, 10.0, 5.0, 1.0), f, 0.5, fused=True)
+        assert np.array_equal(np.isnan(gated), np.isnan(want))
+        fin = np.isfinite(want)
+        assert np.array_equal(gated[~fin], want[~fin], equal_nan=True)
+        assert rel_err(np.where(fin, gated, 0), np.where(fin, want, 0)) <= REL_TOL
 
 
 def test_fir_sparse_spike_input_and_alpha_kernel(impl):
@@ -616,7 +673,8 @@ def test_spike_bwd(n):
 @pytest.mark.parametrize("shape,Fl", [((2, 3, 5, 7, 300), 110), ((3, 41, 350), 110), ((2, 9, 64), 8), ((1, 5, 2000), 77),
                                       ((1, 2, 50), 500), ((4, 7, 1), 3),
                                       # the fused kernel on the matrix cores (rows kept as they lie in memory: T / 4 odd)
-                                      ((37, 300), 77), ((3, 44), 40), ((18, 76), 113), ((100, 28), 45), ((5, 316), 129)])
+                                      ((37, 300), 77), ((3, 44), 40), ((18, 76), 113), ((100, 28), 45), ((5, 316), 129),
+                                      ((19, 220), 100), ((33, 252), 60), ((40, 300), 50), ((8, 16, 300), 110)])
 def test_spike_bwd_corr_is_the_two_ops_in_one(impl, shape, Fl):
     # the Loihi neuron's backward pass: pdf(voltage) * gradOut, then corr with the PSP kernel
     rng = np.random.default_rng(shape[-1] + Fl)
