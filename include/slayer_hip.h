@@ -99,8 +99,12 @@ int slayer_conv_f32(float *out, const float *in, const float *filt, int64_t nNeu
  * out[n][t] = Ts * sum_{i=0..F-1, t+i<T} in[n][t+i] * filt[i].
  *
  * Rows of whole 16-byte vectors with 34 to 129 taps are computed on the matrix cores, which add the
- * terms in another order than the sequential loop: those results agree with it to rounding (1e-7 of
- * the largest output), all others bit for bit with the fused-multiply-add loop.
+ * terms in another order than the sequential loop - whole rows of up to 316 samples whose T / 4 is odd
+ * (T = 300) with bf16 instructions over a three-way split of samples and taps, the others with fp32
+ * instructions: those results agree with the loop to rounding (every output within 1e-6 of the sum of the
+ * magnitudes of its own terms; parts of samples and taps below 2^-126 are read as zero, at most
+ * 2^-124 * (sum |filt| + sum |in| over an output's window) in absolute terms), all others bit for bit
+ * with the fused-multiply-add loop.
  */
 int slayer_corr_f32(float *out, const float *in, const float *filt, int64_t nNeurons, int64_t T,
                     int64_t F, float Ts, void *stream);
@@ -167,8 +171,10 @@ int slayer_spike_bwd_corr_f32(float *gradIn, const float *gradOut, const float *
  *
  * u = Ts * conv(a, srm), then s and the refractory update of u as in slayer_get_spikes_f32, without
  * the round trip of u through memory when rows are whole 16-byte vectors of at most 352 samples,
- * nuSize <= 24 and F <= 160.  Filters of 34 to 129 taps (on rows of at least 16 samples) are summed on the
- * matrix cores, which add the terms in another order than the sequential fused-multiply-add loop: the
+ * nuSize <= 24 and F <= 160.  Filters of 34 to 113 taps (on rows of at least 16 samples) are summed on the
+ * matrix cores (bf16 instructions over a three-way split of samples and taps, as in slayer_corr_f32; 114 to
+ * 129 taps: slayer_conv_f32, then slayer_get_spikes_f32), which add the terms in another order than the
+ * sequential fused-multiply-add loop: the
  * potentials agree with the reference's to rounding (1e-5 of the sum of each output's terms' magnitudes), the
  * spikes are the spike function of exactly these potentials, and a tile of 16 rows that holds a non-finite
  * sample is filtered with the sequential loop (the reference's bits, infinities and NaNs where it puts them).

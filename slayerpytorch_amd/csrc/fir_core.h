@@ -22,6 +22,40 @@ bool launch_fir_corr_mfma(float *out, const float *in, const float *filt, int64_
 // the tiled kernel of fir.hip).
 constexpr int kFirMfmaMinTaps = 34, kFirMfmaMaxTaps = 129;
 
+// ---- operands of the bf16 matrix instruction from fp32 numbers (the three-way split that fir_mfma.hip describes) ----
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+struct SplitPlanes {
+    uint4_ext hi, mid, lo;  // 8 bf16 each: element e in the lower (even e) or upper half of word e / 2
+};
+
+__device__ __forceinline__ SplitPlanes split_bf16(const float (&x)[8])
+{
+    uint32_t a[8], b[8], cc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        a[e] = __builtin_bit_cast(uint32_t, x[e]);
+        const float r1 = x[e] - __builtin_bit_cast(float, a[e] & 0xffff0000u);  // exact
+        b[e] = __builtin_bit_cast(uint32_t, r1);
+        const float r2 = r1 - __builtin_bit_cast(float, b[e] & 0xffff0000u);  // exact
+        cc[e] = __builtin_bit_cast(uint32_t, r2);
+    }
+    SplitPlanes s;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {  // the upper halves of two words into one
+        s.hi[w] = __builtin_amdgcn_perm(a[2 * w + 1], a[2 * w], 0x07060302u);
+        s.mid[w] = __builtin_amdgcn_perm(b[2 * w + 1], b[2 * w], 0x07060302u);
+        s.lo[w] = __builtin_amdgcn_perm(cc[2 * w + 1], cc[2 * w], 0x07060302u);
+    }
+    return s;
+}
+
+__device__ __forceinline__ f32x4 mfma_bf16(const uint4_ext &a, const uint4_ext &b, f32x4 acc)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+}
+
 // A lane produces U consecutive outputs from a register window of U + 4 samples held as
 // NQ = U/4 + 1 16-byte vectors q[].  ROT says which vector currently holds the oldest samples:
 // window sample e is component e % 4 of q[(ROT + e / 4) % NQ].  After a 4-tap block the oldest

@@ -31,8 +31,6 @@
 
 namespace slayer {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
 constexpr int kMfmaLdsBytes = 160 * 1024 / 8;  // per wavefront: 8 of them on a compute unit
 
 struct MfmaFirArgs {
@@ -250,38 +248,6 @@ __global__ __launch_bounds__(64, 2) void fir_mfma_kernel(MfmaFirArgs p)
 // The tile: vector e of the 16 rows' memory is vector e of LDS, no index arithmetic; the range check of the buffers
 // masks what lies behind the last row of the tensor.  The last chunk of a row ends in the first samples of the next
 // row, which the walk masks.
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-
-struct SplitPlanes {
-    uint4_ext hi, mid, lo;  // 8 bf16 each: element e in the lower (even e) or upper half of word e / 2
-};
-
-__device__ __forceinline__ SplitPlanes split_bf16(const float (&x)[8])
-{
-    uint32_t a[8], b[8], cc[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        a[e] = __builtin_bit_cast(uint32_t, x[e]);
-        const float r1 = x[e] - __builtin_bit_cast(float, a[e] & 0xffff0000u);  // exact
-        b[e] = __builtin_bit_cast(uint32_t, r1);
-        const float r2 = r1 - __builtin_bit_cast(float, b[e] & 0xffff0000u);  // exact
-        cc[e] = __builtin_bit_cast(uint32_t, r2);
-    }
-    SplitPlanes s;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {  // the upper halves of two words into one
-        s.hi[w] = __builtin_amdgcn_perm(a[2 * w + 1], a[2 * w], 0x07060302u);
-        s.mid[w] = __builtin_amdgcn_perm(b[2 * w + 1], b[2 * w], 0x07060302u);
-        s.lo[w] = __builtin_amdgcn_perm(cc[2 * w + 1], cc[2 * w], 0x07060302u);
-    }
-    return s;
-}
-
-__device__ __forceinline__ f32x4 mfma_bf16(const uint4_ext &a, const uint4_ext &b, f32x4 acc)
-{
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
-}
-
 // NC: chunks in the window (the second block of a chunk reaches 31 + F samples from the chunk's start); NCE: chunks
 // that the first block reaches.  NV: 16-byte vectors per lane and tile.
 template <int NCE, int NC, int NV, bool GATED>

@@ -199,30 +199,30 @@ __global__ __launch_bounds__(64) void psp_spike_kernel(float *__restrict__ s, fl
 
 // ---- the same on the matrix cores, for filters of 34 to 129 taps ---------------------------------------------------
 // Above about 33 taps the register-window chain is bound by FMA issue.  Here a wavefront owns 16 whole rows and
-// filters them as products of a banded Toeplitz matrix of the filter with blocks of 16 samples
-// (v_mfma_f32_16x16x4_f32; the formulation of fir_mfma.hip on the reversed time axis, where the convolution is
-// a correlation): with m = 16 nBlk - 1 - t, output block j (in m) is the product of the filter band with the D
-// input blocks j .. j + D - 1, i.e. with time blocks q = nBlk - 1 - j down to q - D + 1.  Lane (c = lane % 16,
-// h = lane / 16) supplies, for instruction v of a block, component 3 - v of vector 3 - h of row c's time block
-// and filt[16d + 4h + v - i] for i = lane % 16; its accumulator holds the four outputs of that same vector
-// in descending time.  So a lane only ever reads and writes its own vectors of LDS: the walk goes down in time,
-// writes every output block over the input block that has just left the window, and leaves the membrane
-// potential where the spike walk wants it, tile[r][LAG + t].  The candidate bits of the spike walk are set as
-// the outputs are written; the walk (all 64 lanes, four per row) and the stores are those of spike.hip's
-// row tiles.  The matrix instruction sums four products per step in its own order: the potentials agree with
-// the sequential chain to rounding, and the spikes are the spike function of exactly these potentials.  A tile
-// with a non-finite sample is filtered as sequential chains instead (a structural zero of the band times an
-// infinity would put NaNs where the reference has none).
+// filters them as products of a banded Toeplitz matrix of the filter with chunks of 32 samples, on bf16 matrix
+// instructions over a three-way split of samples and taps (fir_mfma.hip has the formulation and its error: a few
+// 1e-7 of sum |a| |srm|).  The walk goes down in time: the window is the NC chunks up to the one whose 32 outputs
+// are made - split once per sample, when the chunk enters - and lane (c = lane % 16, h = lane / 16) supplies samples
+// 8h .. 8h + 7 of each chunk of row c and, for block p (16 outputs) of a chunk and the chunk s before it,
+// srm[32 s + 16 p + c - (8h + e)].  Its accumulators hold outputs 4h .. 4h + 3 of either block of row c, which it
+// writes over the chunk that has just left the window: the membrane potential ends up where the spike walk wants
+// it, tile[r][LAG + t].  The candidate bits of the spike walk are set as the outputs are written; the walk (all 64
+// lanes, four per row) and the stores are those of spike.hip's row tiles.  The potentials agree with the
+// sequential chain to rounding, and the spikes are the spike function of exactly these potentials.  A tile with a
+// non-finite sample is filtered as sequential chains instead (a structural zero of the band times an infinity would
+// put NaNs where the reference has none), and so is every tile when a tap is not finite.
 constexpr int kFusedMfmaRows = 16;
+constexpr int kFusedMfmaMaxTaps = 113;  // the first block of a chunk reaches four chunks, the second five
 
-template <int D, int NU>
+// NC: chunks in the window (the first block of a chunk reaches back 31 + F samples from the chunk's end), NCE: chunks
+// that the second block reaches
+template <int NCE, int NC, int NU>
 __global__ __launch_bounds__(64, 2) void psp_spike_mfma_kernel(float *__restrict__ s, float *__restrict__ u,
                                                             const float *__restrict__ a, const float *__restrict__ srm,
                                                             const float *__restrict__ nu, int64_t rows, int T, int F,
                                                             int nuSize, int P, int MP, float theta, float Ts)
 {
-    typedef float f32x4 __attribute__((ext_vector_type(4)));
-    constexpr int R = kFusedMfmaRows, G = 32, W = D + 1;
+    constexpr int R = kFusedMfmaRows, G = 32;
     constexpr int LAG = (NU + 2) & ~3;
     constexpr int NBV = (R * (kFusedMaxT / 4) + kWave - 1) / kWave;  // vectors per lane of a tile, at most
     constexpr int kParts = kWave / R, kRounds = (NU + kParts - 1) / kParts;
@@ -243,15 +243,28 @@ __global__ __launch_bounds__(64, 2) void psp_spike_mfma_kernel(float *__restrict
 
     // A tile is one contiguous run of vectors (rows behind the last one arrive as zeros).  A wavefront walks over
     // tiles; the next tile's samples are on their way into registers while this one is filtered, walked and stored.
+    // In three parts.  As many vectors as the registers hold beside the filter's operands and the window (12
+    // registers per chunk each) travel during the filter; more of them from then on, during the spike walk, beside
+    // the filter's operands and the walk's registers; what is left is fetched while the tile before is stored away
+    // and this one is staged, one vector for each one that has been put into LDS.
+    constexpr int kWalkRegs = 96 + (NU > 12 ? 16 : 0);   // (measured: the largest counts that leave nothing in scratch)
+    constexpr int kRoomWalk = (236 - kWalkRegs - 12 * (NCE + NC)) / 4;
+    constexpr int kAhead = kRoomWalk < 1 ? 1 : kRoomWalk < NBV ? kRoomWalk : NBV;
+    constexpr int kRoom = (236 - 68 - 12 * (NCE + 2 * NC)) / 4;
+    constexpr int kEarly = kRoom < 0 ? 0 : kRoom < kAhead ? kRoom : kAhead;
     float4 x[NBV];
-    auto fetch = [&](int64_t t) {
-        const int64_t r0 = t * R;
-        const int n = static_cast<int>(min(static_cast<int64_t>(R), rows - r0)) * perRow;
-        const BufferRsrc bufA = make_buffer(a + r0 * static_cast<int64_t>(T), n * 16);
-        // (always NBV loads, those behind the tile masked by the range check: a fixed number of memory instructions
-        // lets the wait for these loads leave the stores that are issued behind them in flight)
+    auto buffer_of = [&](int64_t t) {
+        // (behind the tile - or behind the last tile: everything - masked by the range check: a fixed number of
+        // memory instructions lets the wait for these loads leave the stores that are issued behind them in flight)
+        const int64_t r0 = t < tiles ? t * R : 0;
+        const int n = t < tiles ? static_cast<int>(min(static_cast<int64_t>(R), rows - r0)) * perRow : 0;
+        return make_buffer(a + r0 * static_cast<int64_t>(T), n * 16);
+    };
+    auto fetch = [&](int64_t t, bool rest) {
+        const BufferRsrc bufA = buffer_of(t);
 #pragma unroll
-        for (int b = 0; b < NBV; ++b) x[b] = buffer_load4(bufA, (lane + b * kWave) * 16, 0);
+        for (int b = 0; b < kAhead; ++b)
+            if ((b >= kEarly) == rest) x[b] = buffer_load4(bufA, (lane + b * kWave) * 16, 0);
     };
     // the lane index behind a barrier for the optimiser: the (row, vector) sequences of the staging and storing
     // loops do not depend on the tile, and kept across the filter and the walk they would cost 2 registers per vector
@@ -262,20 +275,30 @@ __global__ __launch_bounds__(64, 2) void psp_spike_mfma_kernel(float *__restrict
     };
     int64_t tileIdx = blockIdx.x;
     if (tileIdx >= tiles) return;
-    fetch(tileIdx);
-    // the lane's column of the Toeplitz factor; the range check of a buffer that ends with the filter turns every
-    // index that is not a tap into a zero
-    float fa[D][4];
+    fetch(tileIdx, false);
+    fetch(tileIdx, true);
+    // the lane's part of the Toeplitz factor, split; the range check of a buffer that ends with the filter turns every
+    // index that is not a tap into a zero.  aE: the operand of a chunk's second block, which reaches NCE chunks; aO:
+    // of its first block, which reaches all NC.
+    SplitPlanes aE[NCE], aO[NC];
+    bool chainsAlways = false;
     {
         const BufferRsrc bufF = make_buffer(srm, F * 4);
+        bool badTap = false;
 #pragma unroll
-        for (int d = 0; d < D; ++d)
+        for (int sc = 0; sc < NC; ++sc) {
+            float fe[8], fo[8];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int tap = 16 * d + 4 * h + v - c;
-                fa[d][v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                                         bufF, masked_offset(tap >= 0 && tap < F, tap * 4), 0, 0));
+            for (int e = 0; e < 8; ++e) {
+                const int tapE = 32 * sc + 16 + c - (8 * h + e), tapO = tapE - 16;
+                fe[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bufF, masked_offset(tapE >= 0 && tapE < F, tapE * 4), 0, 0));
+                fo[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bufF, masked_offset(tapO >= 0 && tapO < F, tapO * 4), 0, 0));
+                badTap |= fe[e] * 0.0f != 0.0f || fo[e] * 0.0f != 0.0f;
             }
+            if (sc < NCE) aE[sc] = split_bf16(fe);
+            aO[sc] = split_bf16(fo);
+        }
+        chainsAlways = __builtin_amdgcn_ballot_w64(badTap) != 0;
     }
     float tap[NU];
 #pragma unroll
@@ -300,6 +323,7 @@ __global__ __launch_bounds__(64, 2) void psp_spike_mfma_kernel(float *__restrict
     for (int i = lane; i < R * MP; i += kWave) cand[i] = 0u;
     bool bad = false;
     {
+        const BufferRsrc bufCur = buffer_of(tileIdx);
         RowCol rc;
         rc.init(lane_again(), perRow, 1.0f / static_cast<float>(perRow));
         const int dr = kWave / perRow, dc = kWave % perRow;
@@ -310,13 +334,14 @@ __global__ __launch_bounds__(64, 2) void psp_spike_mfma_kernel(float *__restrict
                 // infinite or NaN (or four samples that add up to more than fp32 holds, which only costs time)
                 bad |= ((x[b].x + x[b].y) + (x[b].z + x[b].w)) * 0.0f != 0.0f;
             }
+            if (b + kAhead < NBV) x[b + kAhead] = buffer_load4(bufCur, (lane + (b + kAhead) * kWave) * 16, 0);
             rc.advance(dr, dc, perRow);
         }
     }
-    const bool chains = __builtin_amdgcn_ballot_w64(bad) != 0;
+    const bool chains = __builtin_amdgcn_ballot_w64(bad) != 0 || chainsAlways;
     wave_sync();
     const int64_t tileNext = tileIdx + gridDim.x;
-    if (tileNext < tiles) fetch(tileNext);
+    fetch(tileNext, false);
 
     auto mark4 = [&](int r, int col, const float4 &y) {  // col is a multiple of 4: the four bits lie in one word
         const uint32_t bits = (y.x >= theta ? 1u : 0u) | (y.y >= theta ? 2u : 0u) | (y.z >= theta ? 4u : 0u) |
@@ -342,45 +367,70 @@ __global__ __launch_bounds__(64, 2) void psp_spike_mfma_kernel(float *__restrict
             if (monotone) mark4(r, LAG + t0, q);
         }
     } else {
-        // walk down in time: step j makes time block q = nBlk - 1 - j from time blocks q .. q - D + 1
-        const int nBlk = (T + 15) >> 4;
-        const int vecT = 4 * (3 - h);  // this lane's vector of a block, as a time offset
-        float *col = tile + c * P + LAG + vecT;
-        const float *zr = zeros + 4 * h;
-        auto block = [&](int jm) {  // block jm of the reversed axis; zeros before the row's start and behind its end
-            const int q = nBlk - 1 - jm;
-            const bool keep = q >= 0 && 16 * q + vecT < T;
-            return *reinterpret_cast<const float4 *>(keep ? col + 16 * q : zr);
+        // walk down in time: a step makes outputs 32 m .. 32 m + 31 from chunks m - NC + 1 .. m and writes them over
+        // chunk m
+        const int nCh = (T + 31) >> 5;
+        float *col = tile + c * P + LAG + 8 * h;
+        // chunk q of the lane's row; zeros before the row's start and behind its end
+        auto raw = [&](int q, float4 &v0, float4 &v1) {
+            const int t = 32 * q + 8 * h;
+            v0 = *reinterpret_cast<const float4 *>(q >= 0 && t < T ? col + 32 * q : zeros);
+            v1 = *reinterpret_cast<const float4 *>(q >= 0 && t + 4 < T ? col + 32 * q + 4 : zeros);
         };
-        float4 w[W];
+        auto split = [&](const float4 &v0, const float4 &v1) {
+            const float xs[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+            return split_bf16(xs);
+        };
+        SplitPlanes w[NC];  // at step k of a round, w[(k + sc) % NC] holds chunk m - sc
 #pragma unroll
-        for (int d = 0; d < D; ++d) w[d] = block(d);
-        for (int j0 = 0; j0 < nBlk; j0 += W) {
+        for (int sc = 0; sc < NC; ++sc) {
+            float4 v0, v1;
+            raw(nCh - 1 - sc, v0, v1);
+            w[sc] = split(v0, v1);
+        }
+        for (int j0 = 0; j0 < nCh; j0 += NC) {
 #pragma unroll
-            for (int k = 0; k < W; ++k) {
-                const int j = j0 + k;
-                if (j < nBlk) {
-                    w[(k + D) % W] = block(j + D);       // the block the next step adds
+            for (int k = 0; k < NC; ++k) {
+                if (j0 + k < nCh) {
+                    const int m = nCh - 1 - (j0 + k);
+                    float4 v0, v1;
+                    raw(m - NC, v0, v1);                // the chunk that the next step adds
                     __builtin_amdgcn_sched_barrier(0);  // (issued here, not after the step's matrix work)
-                    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+                    // four sums: the leading products and the five smaller ones, of either block
+                    f32x4 e0 = {0.0f, 0.0f, 0.0f, 0.0f}, e1 = e0, o0 = e0, o1 = e0;
 #pragma unroll
-                    for (int d = 0; d < D; ++d) {
-                        const float4 &xv = w[(k + d) % W];
-                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[d][0], xv.w, acc, 0, 0, 0);
-                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[d][1], xv.z, acc, 0, 0, 0);
-                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[d][2], xv.y, acc, 0, 0, 0);
-                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[d][3], xv.x, acc, 0, 0, 0);
+                    for (int sc = 0; sc < NC; ++sc) {
+                        const SplitPlanes &xs = w[(k + sc) % NC];
+                        if (sc < NCE) e1 = mfma_bf16(aE[sc].lo, xs.hi, e1);
+                        o1 = mfma_bf16(aO[sc].lo, xs.hi, o1);
+                        if (sc < NCE) e1 = mfma_bf16(aE[sc].hi, xs.lo, e1);
+                        o1 = mfma_bf16(aO[sc].hi, xs.lo, o1);
+                        if (sc < NCE) e1 = mfma_bf16(aE[sc].mid, xs.mid, e1);
+                        o1 = mfma_bf16(aO[sc].mid, xs.mid, o1);
+                        if (sc < NCE) e1 = mfma_bf16(aE[sc].mid, xs.hi, e1);
+                        o1 = mfma_bf16(aO[sc].mid, xs.hi, o1);
+                        if (sc < NCE) e1 = mfma_bf16(aE[sc].hi, xs.mid, e1);
+                        o1 = mfma_bf16(aO[sc].hi, xs.mid, o1);
+                        if (sc < NCE) e0 = mfma_bf16(aE[sc].hi, xs.hi, e0);
+                        o0 = mfma_bf16(aO[sc].hi, xs.hi, o0);
                     }
-                    const int q = nBlk - 1 - j;
-                    if (16 * q + vecT < T) {
-                        const float4 y = make_float4(acc.w * Ts, acc.z * Ts, acc.y * Ts, acc.x * Ts);
-                        *reinterpret_cast<float4 *>(col + 16 * q) = y;
-                        if (monotone) mark4(c, LAG + 16 * q + vecT, y);
+                    const int t = 32 * m + 4 * h;   // the lane's outputs: t .. t + 3 (first block), t + 16 .. (second)
+                    if (t < T) {
+                        const float4 y = make_float4((o0.x + o1.x) * Ts, (o0.y + o1.y) * Ts, (o0.z + o1.z) * Ts, (o0.w + o1.w) * Ts);
+                        *reinterpret_cast<float4 *>(col + 32 * m - 4 * h) = y;
+                        if (monotone) mark4(c, LAG + t, y);
                     }
+                    if (t + 16 < T) {
+                        const float4 y = make_float4((e0.x + e1.x) * Ts, (e0.y + e1.y) * Ts, (e0.z + e1.z) * Ts, (e0.w + e1.w) * Ts);
+                        *reinterpret_cast<float4 *>(col + 32 * m + 16 - 4 * h) = y;
+                        if (monotone) mark4(c, LAG + t + 16, y);
+                    }
+                    w[k] = split(v0, v1);
                 }
             }
         }
     }
+    fetch(tileNext, true);
     wave_sync();
 
     // ---- walk: columns [0, T + LAG) of the tile become final
@@ -554,21 +604,15 @@ static int launch_psp_spike_mfma(float *s, float *u, const float *a, const float
     const int64_t resident = static_cast<int64_t>(compute_units()) * (perUnit < 8 ? perUnit : 8);
     const int64_t trips = ceil_div(tiles, resident);
     const dim3 grid(static_cast<unsigned>(ceil_div(tiles, trips)));
-    const int D = (F + 14) / 16 + 1;
-#define SLAYER_PSP_SPIKE_MFMA(DD)                                                                                     \
-    case DD:                                                                                                          \
-        hipLaunchKernelGGL((psp_spike_mfma_kernel<DD, NU>), grid, dim3(kWave), lds, st, s, u, a, srm, nu, rows, T, F, \
-                           nuSize, P, MP, theta, Ts);                                                                 \
-        break
-    switch (D) {
-        SLAYER_PSP_SPIKE_MFMA(4);
-        SLAYER_PSP_SPIKE_MFMA(5);
-        SLAYER_PSP_SPIKE_MFMA(6);
-        SLAYER_PSP_SPIKE_MFMA(7);
-        SLAYER_PSP_SPIKE_MFMA(8);
-        default:
-            SLAYER_PSP_SPIKE_MFMA(9);
-    }
+    const int nce = (15 + F + 31) / 32, nc = (31 + F + 31) / 32;
+#define SLAYER_PSP_SPIKE_MFMA(E, C)                                                                                   \
+    hipLaunchKernelGGL((psp_spike_mfma_kernel<E, C, NU>), grid, dim3(kWave), lds, st, s, u, a, srm, nu, rows, T, F,   \
+                       nuSize, P, MP, theta, Ts)
+    if (nc == 3 && nce == 2) SLAYER_PSP_SPIKE_MFMA(2, 3);
+    else if (nc == 3) SLAYER_PSP_SPIKE_MFMA(3, 3);
+    else if (nc == 4 && nce == 3) SLAYER_PSP_SPIKE_MFMA(3, 4);
+    else if (nc == 4) SLAYER_PSP_SPIKE_MFMA(4, 4);
+    else SLAYER_PSP_SPIKE_MFMA(4, 5);
 #undef SLAYER_PSP_SPIKE_MFMA
     return launch_status();
 }
@@ -593,7 +637,14 @@ extern "C" int slayer_psp_spike_f32(float *s, float *u, const float *a, const fl
         if (status != SLAYER_OK) return status;
         return slayer_get_spikes_f32(s, u, nu, nNeurons, T, nuSize, theta, Ts, stream);
     }
-    if (F >= kFirMfmaMinTaps && F <= kFirMfmaMaxTaps && T >= 16) {  // filters that pay on the matrix cores
+    // (from 114 taps on the filter's operands, five chunks for either block, leave the fused kernel no registers for a
+    // tile in flight: the two kernels then)
+    if (F > kFusedMfmaMaxTaps && F <= kFirMfmaMaxTaps && T >= 16) {
+        const int status = slayer_conv_f32(u, a, srm, nNeurons, T, F, Ts, stream);
+        if (status != SLAYER_OK) return status;
+        return slayer_get_spikes_f32(s, u, nu, nNeurons, T, nuSize, theta, Ts, stream);
+    }
+    if (F >= kFirMfmaMinTaps && F <= kFusedMfmaMaxTaps && T >= 16) {  // filters that pay on the matrix cores
         if (nuSize <= 12)
             return launch_psp_spike_mfma<12>(s, u, a, srm, nu, nNeurons, static_cast<int>(T), static_cast<int>(F),
                                              static_cast<int>(nuSize), theta, Ts, st);

@@ -354,7 +354,7 @@ def spikeBackward(gradOutput, membranePotential, theta, tau, scale):
 
 def pspSpike(input, srmKernel, refKernel, theta, Ts):
     """``conv(input, srmKernel, Ts)`` followed by ``getSpikes`` on the result, in one kernel where
-    the shape allows (filters of 34 to 129 taps then run on the matrix cores, like ``conv`` on dense
+    the shape allows (filters of 34 to 113 taps then run on the matrix cores, like ``conv`` on dense
     input).  Returns ``(spike, membranePotential)``; the membrane potential is the one after the
     refractory updates, as ``getSpikes`` leaves it."""
     _check_input(input, "input")
