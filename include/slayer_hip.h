@@ -425,6 +425,27 @@ int slayer_dense_events_grad_weight_f32(float *gradW, const float *gradOut, cons
                                         void *stream);
 
 /*
+ * ---- Fully connected synapse with few inputs, on the matrix cores --------------------------------
+ * out[n][o][t] = sum_{k<K} W[o][k] * x[n][k][t] with W[o][k] = w[o * wRow + k * wCol]: per batch item the
+ * matrix product W[O x K] * x[K x T] of _denseLayer.forward (src/slayer.py:435-440, see above) with
+ * wRow = K, wCol = 1, and its input gradient W^T * gradOut (the one autograd derives for that call) with
+ * w the same weight, wRow = 1, wCol = the layer's input count, and the roles of K and O exchanged.  x is
+ * [N][K][T], out [N][O][T] (every element is written); T a multiple of 4, x and out 16-byte aligned, K * T
+ * and O * T below 2^29, else SLAYER_EUNSUPPORTED (slayer_dense_rows_supported says so beforehand).
+ * `workspace` holds slayer_dense_rows_workspace_bytes(K, O) bytes, 16-byte aligned (the weights, split).
+ * One launch per 224 inputs (and a small one that splits the weights): the rows of W stay in registers, split into three bf16 parts each, the tiles of
+ * x are split on their way into LDS, and the products run on bf16 matrix instructions (six of the nine partial
+ * products, each exact in the fp32 accumulator; three when a tile of x holds spikes, i.e. values with at most 8
+ * significant bits).  The result is the product up to the order of the additions and 2^-23 of each term: within
+ * 1e-6 of sum_k |W[o][k]| |x[n][k][t]|.  Weights and samples must be finite.  Meant for layers with up to a
+ * few hundred inputs, where a library product spends its time on fp32 matrix instructions.
+ */
+int slayer_dense_rows_supported(int64_t N, int64_t K, int64_t O, int64_t T);
+int64_t slayer_dense_rows_workspace_bytes(int64_t K, int64_t O);
+int slayer_dense_rows_f32(float *out, const float *w, const float *x, void *workspace, int64_t N, int64_t K, int64_t O,
+                          int64_t T, int64_t wRow, int64_t wCol, void *stream);
+
+/*
  * ---- Weight quantisation of the Loihi layers ---------------------------------------------------
  * out[i] = round(in[i] / step) * step the way torch evaluates the expression on the GPU for a Python number
  * `step`: in[i] times the fp32 rounding of the double-precision reciprocal of step, to the nearest integer with

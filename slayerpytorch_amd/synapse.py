@@ -15,7 +15,8 @@ from . import _lib
 from .slayerCuda import _check_device, _check_input, _on_device_of, _ptr
 
 __all__ = ["conv", "convGradInput", "convGradWeight", "outShape", "supported", "synapseConv", "synapseConvTranspose",
-           "denseEvents", "denseEventsGradWeight", "denseEventsSupported", "synapseDenseEvents"]
+           "denseEvents", "denseEventsGradWeight", "denseEventsSupported", "synapseDenseEvents", "denseRows",
+           "denseRowsSupported", "denseRowsPays", "synapseDenseRows"]
 
 
 def _pair(v, name):
@@ -264,6 +265,34 @@ def denseEventsGradWeight(gradOutput, input):
     return gradW
 
 
+def denseRowsSupported(N, K, O, T):
+    """Whether ``denseRows`` takes these extents (the limits the header states)."""
+    return bool(_lib.load().slayer_dense_rows_supported(N, K, O, T))
+
+
+def denseRows(input, weight, transposed=False):
+    """``weight @ input[n]`` for every batch item, ``input`` (N, K, T), ``weight`` (O, K) - or, ``transposed``,
+    ``weight.T @ input[n]`` with ``weight`` (K, O): the dense layer's product and its input gradient on bf16
+    matrix instructions over split operands (``slayer_dense_rows_f32``), for layers with up to a few hundred
+    inputs."""
+    _check_input(input, "input")
+    _check_input(weight, "weight")
+    _check_device(input, weight, "input", "weight")
+    if input.dim() != 3 or weight.dim() != 2 or weight.shape[0 if transposed else 1] != input.shape[1]:
+        raise RuntimeError("denseRows takes input (N, K, T) and weight (O, K), or (K, O) transposed; got %r and %r"
+                           % (tuple(input.shape), tuple(weight.shape)))
+    N, K, T = (int(v) for v in input.shape)
+    O = int(weight.shape[1 if transposed else 0])
+    lib = _lib.load()
+    out = torch.empty((N, O, T), dtype=input.dtype, device=input.device)
+    wRow, wCol = (1, O) if transposed else (K, 1)
+    workspace = torch.empty((lib.slayer_dense_rows_workspace_bytes(K, O) + 3) // 4, dtype=torch.float32, device=input.device)
+    with _on_device_of(input) as stream:
+        _lib.check(lib.slayer_dense_rows_f32(_ptr(out), _ptr(weight), _ptr(input), _ptr(workspace), N, K, O, T, wRow, wCol,
+                                             stream), "slayer_dense_rows_f32")
+    return out
+
+
 class _synapseDenseEventsFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, weight, product, gradient):
@@ -288,6 +317,45 @@ class _synapseDenseEventsFunction(torch.autograd.Function):
             else:
                 gradWeight = torch.bmm(gradOutput, input.transpose(1, 2)).sum(0)
         return gradInput, gradWeight, None, None
+
+
+DENSE_ROWS_MAX_INPUTS = 448   # two launches of slayer_dense_rows_f32; beyond that the library product
+
+
+def denseRowsPays(N, K, O, T):
+    """Whether the dense layer's product (N, K, T) -> (N, O, T) is taken by ``denseRows``: few enough inputs, and enough
+    work for a kernel that keeps the weights in registers (a library product is as fast on small problems)."""
+    return K <= DENSE_ROWS_MAX_INPUTS and N * T >= 2048 and O >= 16 and denseRowsSupported(N, K, O, T)
+
+
+class _synapseDenseRowsFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, weight):
+        ctx.save_for_backward(input, weight)
+        return denseRows(input, weight.contiguous())
+
+    @staticmethod
+    def backward(ctx, gradOutput):
+        input, weight = ctx.saved_tensors
+        gradOutput = gradOutput.contiguous()
+        gradInput = gradWeight = None
+        N, K, T = input.shape
+        O = weight.shape[0]
+        if ctx.needs_input_grad[0]:
+            if denseRowsPays(N, O, K, T):     # (the outputs are what is summed over now)
+                gradInput = denseRows(gradOutput, weight.contiguous(), transposed=True)
+            else:
+                gradInput = torch.bmm(weight.t().unsqueeze(0).expand(N, K, O), gradOutput)
+        if ctx.needs_input_grad[1]:
+            gradWeight = torch.bmm(gradOutput, input.transpose(1, 2)).sum(0)
+        return gradInput, gradWeight
+
+
+def synapseDenseRows(input, weight):
+    """``weight @ input[n]`` for every batch item (``input`` (N, K, T), ``weight`` (O, K)) with its gradients, for
+    layers with few inputs: product and input gradient from ``denseRows`` (bf16 matrix instructions over split
+    operands, weights in registers), the weight gradient from the library."""
+    return _synapseDenseRowsFunction.apply(input.contiguous(), weight)
 
 
 def synapseDenseEvents(input, weight, product=True, gradient=True):

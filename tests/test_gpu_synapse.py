@@ -11,6 +11,7 @@ import pytest
 import torch
 
 from oracle import oracle as O
+from _util import rel_err
 from slayerpytorch_amd import _lib, synapse
 import slayerpytorch_amd as snn
 
@@ -379,6 +380,89 @@ def test_dense_events_status_codes():
     assert lib.slayer_dense_events_grad_weight_f32(p, p, p, p, -1, 5, 5, 8, None) == 1
     with pytest.raises(_lib.SlayerHipError, match="not supported"):
         synapse.denseEventsGradWeight(torch.zeros((1, 1025, 8), device="cuda"), torch.zeros((1, 5, 8), device="cuda"))
+
+
+# (N, K, O, T, spike input)
+DENSE_ROWS_CASES = [
+    (2, 200, 256, 64, True),       # the long-sequence network's first layer: seven chunks of inputs, all eight wavefronts
+    (2, 200, 256, 64, False),      # the same on a dense input: all six products
+    (3, 7, 5, 36, False),          # tiny: one chunk, one wavefront at work, a tile of 4 samples at the end
+    (2, 256, 200, 100, True),      # more than 224 inputs: two launches that add up; 200 outputs: a wavefront with 8 rows
+    (2, 300, 40, 2000, False),     # long rows: many tiles per work-group
+    (1, 32, 16, 4, False),         # a single tile of four samples
+    (2, 224, 300, 96, True),       # more than 256 outputs: two groups of wavefronts
+    (1, 448, 33, 68, False),       # the most inputs the layer sends here
+    (70, 96, 64, 32, True),        # more tiles than one per batch item... one tile each, 70 items
+]
+
+
+@pytest.mark.parametrize("case", DENSE_ROWS_CASES)
+@pytest.mark.parametrize("transposed", [False, True])
+def test_dense_rows_product(case, transposed):
+    # the dense layer's product and (transposed) input gradient on bf16 matrix instructions over split operands: every
+    # output within 1e-6 of the sum of its terms' magnitudes (the bound the header states; SUM_TOL for all synapse
+    # kernels is the north star's 1e-5), on spikes and on dense inputs of mixed magnitude
+    N, K, O, T, spikes = case
+    rng = np.random.default_rng(N + K + O + T)
+    x = dense_input(rng, (N, K, T), 0.04, True) if spikes else \
+        (rng.standard_normal((N, K, T)) * np.exp2(rng.integers(-8, 8, (N, K, T)))).astype(np.float32)
+    w = (rng.standard_normal((K, O) if transposed else (O, K)) * np.exp2(rng.integers(-6, 6, (K, O) if transposed else (O, K)))).astype(np.float32)
+    W = (w.T if transposed else w).astype(np.float64)
+    ref = np.einsum("ok,nkt->not", W, x.astype(np.float64))
+    scale = np.einsum("ok,nkt->not", np.abs(W), np.abs(x).astype(np.float64))
+    got = synapse.denseRows(dev(x), dev(w), transposed)
+    err = np.abs(host(got).astype(np.float64) - ref)
+    assert np.all(err <= 1e-6 * scale + 1e-30), float((err / (scale + 1e-30)).max())
+    assert torch.equal(got, synapse.denseRows(dev(x), dev(w), transposed))            # the same bits every time
+
+
+def test_dense_rows_status_codes_and_limits():
+    lib = _lib.load()
+    t = torch.full((4096,), 7.0, device="cuda")
+    p = t.data_ptr()
+    assert lib.slayer_dense_rows_f32(None, None, None, None, 0, 5, 5, 8, 5, 1, None) == 0                 # empty: nothing to do
+    assert lib.slayer_dense_rows_f32(None, p, p, p, 1, 5, 5, 8, 5, 1, None) == 1
+    assert lib.slayer_dense_rows_f32(p, p, p, None, 1, 5, 5, 8, 5, 1, None) == 1
+    assert lib.slayer_dense_rows_f32(p, p, p, p, 1, 5, 5, 6, 5, 1, None) == 2                             # T % 4 != 0
+    assert lib.slayer_dense_rows_f32(p, p, p + 4, p, 1, 5, 5, 8, 5, 1, None) == 2                         # x not 16-byte aligned
+    assert lib.slayer_dense_rows_f32(p, p, p, p, 1, 5, 5, 1 << 30, 5, 1, None) == 2                       # rows over 2 GiB
+    assert not lib.slayer_dense_rows_supported(1, 5, 5, 6) and lib.slayer_dense_rows_supported(1, 5, 5, 8)
+    assert lib.slayer_dense_rows_workspace_bytes(0, 5) == 0
+    # eight wavefronts x two halves x seven chunks x three parts of 1 KiB
+    assert lib.slayer_dense_rows_workspace_bytes(200, 256) == 8 * 2 * 7 * 3 * 1024
+    assert synapse.denseRowsPays(64, 200, 256, 2000) and not synapse.denseRowsPays(64, 449, 256, 2000)
+    assert not synapse.denseRowsPays(64, 200, 256, 2001) and not synapse.denseRowsPays(1, 200, 256, 64)
+    with pytest.raises(RuntimeError, match="denseRows takes"):
+        synapse.denseRows(torch.zeros((1, 5, 8), device="cuda"), torch.zeros((4, 6), device="cuda"))
+
+
+def test_dense_layer_with_few_inputs_runs_dense_rows(monkeypatch):
+    """_denseLayer with 200 inputs: product and input gradient from synapse.denseRows, against the library products
+    (DENSE_ROWS = False): outputs and all gradients to rounding."""
+    from slayerpytorch_amd import slayer as slayer_module
+    params = {"type": "SRMALPHA", "theta": 10, "tauSr": 10.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
+    T = 512
+    layer = snn.layer(params, {"Ts": 1.0, "tSample": T}).cuda()
+    torch.manual_seed(5)
+    fc = layer.dense(200, 96).cuda()
+    rng = np.random.default_rng(11)
+    g = dev(rng.standard_normal((4, 96, 1, 1, T)).astype(np.float32))
+    calls = []
+    real = synapse.denseRows
+    monkeypatch.setattr(synapse, "denseRows", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    for x0 in (dense_input(rng, (4, 200, 1, 1, T), 0.03, True), rng.standard_normal((4, 200, 1, 1, T)).astype(np.float32)):
+        results = []
+        for mode in (True, False):
+            monkeypatch.setattr(slayer_module, "DENSE_ROWS", mode)
+            x = dev(x0).requires_grad_(True)
+            fc.weight.grad = None
+            n = len(calls)
+            y = fc(x)
+            y.backward(g)
+            assert (len(calls) - n) == (2 if mode else 0)        # the product and the input gradient
+            results.append((host(y), host(x.grad), host(fc.weight.grad)))
+        for a, b in zip(*results):
+            assert rel_err(a, b) <= 1e-5
 
 
 @pytest.mark.parametrize("shape", [((34, 34, 2), 40, 12), (50, 10, 33)])
