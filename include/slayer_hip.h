@@ -446,6 +446,20 @@ int slayer_dense_rows_f32(float *out, const float *w, const float *x, void *work
                           int64_t T, int64_t wRow, int64_t wCol, void *stream);
 
 /*
+ * gradW[o][k] = sum_{n,t} gradOut[n][o][t] * x[n][k][t]: the weight gradient of the same layers (the one autograd
+ * derives for the F.conv3d of _denseLayer.forward, src/slayer.py:435-440), for up to 448 inputs and 256 outputs.
+ * x is [N][K][T], gradOut [N][O][T], gradW [O][K] (every element is written); T a multiple of 4, both tensors
+ * 16-byte aligned.  `workspace` holds slayer_dense_rows_grad_weight_workspace_bytes(N, K, O, T) bytes: every
+ * work-group sums a range of the batch's samples for all weights - on bf16 matrix instructions over split operands,
+ * as slayer_dense_rows_f32 - and a second launch adds the work-groups' sums in a fixed order.  Within 1e-6 of
+ * sum_{n,t} |gradOut| |x|.
+ */
+int slayer_dense_rows_grad_weight_supported(int64_t N, int64_t K, int64_t O, int64_t T);
+int64_t slayer_dense_rows_grad_weight_workspace_bytes(int64_t N, int64_t K, int64_t O, int64_t T);
+int slayer_dense_rows_grad_weight_f32(float *gradW, const float *gradOut, const float *x, void *workspace, int64_t N,
+                                      int64_t K, int64_t O, int64_t T, void *stream);
+
+/*
  * ---- Weight quantisation of the Loihi layers ---------------------------------------------------
  * out[i] = round(in[i] / step) * step the way torch evaluates the expression on the GPU for a Python number
  * `step`: in[i] times the fp32 rounding of the double-precision reciprocal of step, to the nearest integer with

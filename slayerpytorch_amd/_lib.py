@@ -80,6 +80,9 @@ SIGNATURES = {
     "slayer_dense_events_grad_weight_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _i64, _i64, _i64, _i64, _stream]),
     "slayer_dense_rows_supported": (ctypes.c_int, [_i64, _i64, _i64, _i64]),
     "slayer_dense_rows_workspace_bytes": (_i64, [_i64, _i64]),
+    "slayer_dense_rows_grad_weight_supported": (ctypes.c_int, [_i64, _i64, _i64, _i64]),
+    "slayer_dense_rows_grad_weight_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
+    "slayer_dense_rows_grad_weight_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _i64, _i64, _i64, _i64, _stream]),
     "slayer_dense_rows_f32": (ctypes.c_int, [_f32p, _f32p, _f32p, _f32p, _i64, _i64, _i64, _i64, _i64, _i64, _stream]),
 }
 

@@ -380,3 +380,316 @@ extern "C" int slayer_dense_rows_f32(float *out, const float *w, const float *x,
     }
     return launch_status();
 }
+
+// ---- the weight gradient of the same layers -------------------------------------------------------------------------
+//
+//     gradW[o][k] = sum_{n, t} gradOut[n][o][t] * x[n][k][t]
+//
+// Both operands have the reduction axis, time, innermost: a lane's operand of v_mfma_f32_16x16x32_bf16 - 8 consecutive
+// samples of one row - is 32 contiguous bytes of either tensor.  A work-group of 8 wavefronts owns ALL outputs and up
+// to 208 inputs (16 x 13 tiles of 16 x 16, wavefront w the tiles of output rows 32 w .. 32 w + 31: at most 104
+// accumulator registers; layers with more inputs take a launch per block of inputs) and a contiguous range of chunks
+// of 32 samples.  Per chunk the rows of x travel into a ring in LDS and are split into three planes [k][t] of bf16
+// there, once, for all wavefronts (pitch 80 bytes: the 16 rows of an operand read spread over the banks); a
+// wavefront's own 32 rows of gradOut come straight from memory into registers, one chunk ahead, and are split there.
+// Spike tiles of x take three of the six products, as in the kernel above.  Every work-group writes its sums to a row
+// of `partial`; a second kernel adds the
+// rows in a fixed order.
+namespace slayer {
+
+// floats between the work-groups' sums in the workspace: a multiple of four, for the sum kernel's 16-byte loads
+__host__ __device__ inline int64_t dense_wgrad_pitch(int64_t O, int64_t K) { return (O * K + 3) / 4 * 4; }
+
+constexpr int kWgradMaxInputs = 208;   // per launch: 13 tiles of 16, what the planes of a chunk leave room for in LDS
+constexpr int kWgradPitch = 80;   // bytes per input row of a plane: 32 samples of bf16 and 16 bytes of padding
+
+struct DenseWgradArgs {
+    float *partial;
+    const float *gradOut, *x;
+    int N, O, K, T;
+    int k0, kEnd;            // the inputs this launch covers
+    int chunksPerItem;
+    uint32_t chunks;
+};
+
+template <int KT>   // tiles of 16 inputs
+__global__ __launch_bounds__(64 * kDenseWaves) void dense_wgrad_split_kernel(DenseWgradArgs g)
+{
+    extern __shared__ __align__(16) char lds[];
+    constexpr int PLANE = 16 * KT * kWgradPitch;            // bytes per plane
+    constexpr int GROUPS = 2 * KT;                          // groups of 8 rows (1 KiB) of a raw tile
+    constexpr int RL = (GROUPS + kDenseWaves - 1) / kDenseWaves;   // groups, i.e. load instructions, per wavefront
+    constexpr int RAW = GROUPS * 1024;
+    const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char *)lds));
+    char *const ring = lds + 6 * PLANE;
+    uint32_t *flags = reinterpret_cast<uint32_t *>(ring + 2 * RAW);   // [2][kDenseWaves]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, h = lane >> 4;
+    const int o0 = (blockIdx.y * kDenseWaves + wave) * 32;
+    const bool working = o0 < g.O;
+    const uint32_t per = (g.chunks + gridDim.x - 1) / gridDim.x;
+    uint32_t chunk = blockIdx.x * per;
+    const uint32_t end = min(g.chunks, chunk + per);
+
+    f32x4 acc[2][KT];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) acc[j][kt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    auto place = [&](uint32_t ch, int &n, int &t0) {
+        n = static_cast<int>(ch / static_cast<uint32_t>(g.chunksPerItem));
+        t0 = (static_cast<int>(ch) - n * g.chunksPerItem) * 32;
+    };
+    // x: memory -> ring (group wave + 8 r: rows 8 (wave + 8 r) .. + 7; lane l: row l / 8, samples 4 (l % 8) .. + 3)
+    auto fetch = [&](uint32_t ch, int turn) {
+        const bool live = ch < end;
+        int n, t0;
+        place(live ? ch : 0, n, t0);
+        const int4_ext bx = make_descriptor(g.x + static_cast<int64_t>(n) * g.K * g.T, live ? g.K * g.T * 4 : 0);
+        const uint32_t slot = ldsBase + 6 * PLANE + (turn & 1) * RAW;
+#pragma unroll
+        for (int r = 0; r < RL; ++r) {
+            const int grp = wave + kDenseWaves * r;
+            if (grp >= GROUPS) break;
+            const int k = g.k0 + 8 * grp + (lane >> 3), t = t0 + 4 * (lane & 7);
+            buffer_load4_to_lds(bx, __builtin_amdgcn_readfirstlane(slot + grp * 1024),
+                                masked_offset(k < g.kEnd && t < g.T, (k * g.T + t) * 4));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // ring -> planes (the groups this wavefront fetched itself, two at a time)
+    auto stage = [&](int turn) {
+        const char *slot = ring + (turn & 1) * RAW;
+        char *planes = lds + (turn & 1) * 3 * PLANE;
+        bool beyond = false;
+#pragma unroll
+        for (int r = 0; r < RL; r += 2) {
+            const int ga = wave + kDenseWaves * r, gb = wave + kDenseWaves * (r + 1);
+            if (ga < GROUPS) {
+                const float4 va = *reinterpret_cast<const float4 *>(slot + ga * 1024 + lane * 16);
+                const float4 vb = (r + 1 < RL && gb < GROUPS) ? *reinterpret_cast<const float4 *>(slot + gb * 1024 + lane * 16)
+                                                              : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                const float v[8] = {va.x, va.y, va.z, va.w, vb.x, vb.y, vb.z, vb.w};
+                const SplitPlanes s = split_bf16(v);   // words 0, 1: the four samples of row a; words 2, 3: of row b
+                char *da = planes + (8 * ga + (lane >> 3)) * kWgradPitch + 8 * (lane & 7);
+                *reinterpret_cast<uint2 *>(da) = make_uint2(s.hi[0], s.hi[1]);
+                *reinterpret_cast<uint2 *>(da + PLANE) = make_uint2(s.mid[0], s.mid[1]);
+                *reinterpret_cast<uint2 *>(da + 2 * PLANE) = make_uint2(s.lo[0], s.lo[1]);
+                if (r + 1 < RL && gb < GROUPS) {
+                    char *db = planes + (8 * gb + (lane >> 3)) * kWgradPitch + 8 * (lane & 7);
+                    *reinterpret_cast<uint2 *>(db) = make_uint2(s.hi[2], s.hi[3]);
+                    *reinterpret_cast<uint2 *>(db + PLANE) = make_uint2(s.mid[2], s.mid[3]);
+                    *reinterpret_cast<uint2 *>(db + 2 * PLANE) = make_uint2(s.lo[2], s.lo[3]);
+                }
+                beyond |= ((s.mid[0] | s.mid[1]) | (s.mid[2] | s.mid[3]) | (s.lo[0] | s.lo[1]) | (s.lo[2] | s.lo[3])) != 0u;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const bool any = __builtin_amdgcn_ballot_w64(beyond) != 0;
+        if (lane == 0) flags[(turn & 1) * kDenseWaves + wave] = any ? 1u : 0u;
+    };
+    // gradOut: this lane's samples 8h .. 8h + 7 of rows o0 + 16 j + c of a chunk, straight into registers
+    float4 ga[2][2];
+    auto fetch_grad = [&](uint32_t ch) {
+        const bool live = ch < end;
+        int n, t0;
+        place(live ? ch : 0, n, t0);
+        const BufferRsrc bg = make_buffer(g.gradOut + static_cast<int64_t>(n) * g.O * g.T, live ? g.O * g.T * 4 : 0);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int o = o0 + 16 * j + c, t = t0 + 8 * h;
+            ga[j][0] = buffer_load4<kCached>(bg, masked_offset(o < g.O && t < g.T, (o * g.T + t) * 4), 0);
+            ga[j][1] = buffer_load4<kCached>(bg, masked_offset(o < g.O && t + 4 < g.T, (o * g.T + t + 4) * 4), 0);
+        }
+    };
+
+    if (chunk < end) {
+        fetch_grad(chunk);
+        fetch(chunk, 0);
+        wait_vmem<0>();
+        stage(0);
+        __syncthreads();
+        for (int turn = 0;; ++turn) {
+            // this chunk's rows of gradOut, split (they were fetched a trip ago); then the next chunk's go out, and
+            // the rows of x of the chunk after the next
+            SplitPlanes a[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const float v[8] = {ga[j][0].x, ga[j][0].y, ga[j][0].z, ga[j][0].w, ga[j][1].x, ga[j][1].y, ga[j][1].z, ga[j][1].w};
+                a[j] = split_bf16(v);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            fetch_grad(chunk + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (turn == 0) {
+                fetch(chunk + 1, 1);
+                wait_vmem<0>();      // (the first trip has nothing in flight to hide this behind)
+            } else {
+                // the next chunk's rows of x were fetched a trip ago; behind them: this trip's four loads of gradOut
+                wait_vmem<4>();
+            }
+            stage(turn + 1);
+            fetch(chunk + 2, turn + 2);   // (into the slot whose rows, this chunk's, were split a trip ago)
+            if (working) {
+                const bool allParts = __builtin_amdgcn_ballot_w64(lane < kDenseWaves && flags[(turn & 1) * kDenseWaves + (lane & 7)] != 0u) != 0;
+                const char *base = lds + (turn & 1) * 3 * PLANE + c * kWgradPitch + 16 * h;
+                // (one loop with the test inside: as two loops under the test, the compiler kept the operands of both
+                // in registers at once)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    if (allParts) {
+                        const uint4_ext xm = *reinterpret_cast<const uint4_ext *>(base + PLANE + 16 * kt * kWgradPitch);
+                        const uint4_ext xl = *reinterpret_cast<const uint4_ext *>(base + 2 * PLANE + 16 * kt * kWgradPitch);
+#pragma unroll
+                        for (int j = 0; j < 2; ++j) {
+                            acc[j][kt] = mfma_bf16(a[j].hi, xl, acc[j][kt]);
+                            acc[j][kt] = mfma_bf16(a[j].mid, xm, acc[j][kt]);
+                            acc[j][kt] = mfma_bf16(a[j].hi, xm, acc[j][kt]);
+                        }
+                    }
+                    const uint4_ext xh = *reinterpret_cast<const uint4_ext *>(base + 16 * kt * kWgradPitch);
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        acc[j][kt] = mfma_bf16(a[j].lo, xh, acc[j][kt]);
+                        acc[j][kt] = mfma_bf16(a[j].mid, xh, acc[j][kt]);
+                        acc[j][kt] = mfma_bf16(a[j].hi, xh, acc[j][kt]);
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (++chunk >= end) break;
+            __syncthreads();
+        }
+    }
+    // this work-group's sums: lane (c, h) holds rows 4h .. 4h + 3, column c of every tile
+    if (working) {
+        float *row = g.partial + static_cast<int64_t>(blockIdx.x) * dense_wgrad_pitch(g.O, g.K);
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const int k = g.k0 + 16 * kt + c;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int o = o0 + 16 * j + 4 * h + r;
+                    if (o < g.O && k < g.kEnd) row[o * g.K + k] = acc[j][kt][r];
+                }
+            }
+    }
+}
+
+// out[i] = sum of the rows of partial, in a fixed order: 16 threads share a column of four sums, each adds every
+// sixteenth row, and one of them adds the sixteen results (rows lie `pitch` floats apart, a multiple of 4 that holds
+// n; rows == 0 writes zeros)
+__global__ __launch_bounds__(256) void dense_wgrad_sum_kernel(float *out, const float *partial, int rows, int n, int64_t pitch)
+{
+    __shared__ float4 part[16][17];
+    const int col = threadIdx.x & 15, slice = threadIdx.x >> 4;
+    const int i = (blockIdx.x * 16 + col) * 4;
+    float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (i < n) {
+        const float *p = partial + i;
+        int r = slice;
+        for (; r + 48 < rows; r += 64) {
+            const float4 a = *reinterpret_cast<const float4 *>(p + r * pitch);
+            const float4 b = *reinterpret_cast<const float4 *>(p + (r + 16) * pitch);
+            const float4 c = *reinterpret_cast<const float4 *>(p + (r + 32) * pitch);
+            const float4 d = *reinterpret_cast<const float4 *>(p + (r + 48) * pitch);
+            s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+            s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+            s.x += c.x; s.y += c.y; s.z += c.z; s.w += c.w;
+            s.x += d.x; s.y += d.y; s.z += d.z; s.w += d.w;
+        }
+        for (; r < rows; r += 16) {
+            const float4 a = *reinterpret_cast<const float4 *>(p + r * pitch);
+            s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+        }
+    }
+    part[slice][col] = s;
+    __syncthreads();
+    if (slice == 0 && i < n) {
+        float4 t = part[0][col];
+        for (int q = 1; q < 16; ++q) {
+            const float4 a = part[q][col];
+            t.x += a.x; t.y += a.y; t.z += a.z; t.w += a.w;
+        }
+        if (i + 3 < n) {
+            out[i] = t.x; out[i + 1] = t.y; out[i + 2] = t.z; out[i + 3] = t.w;   // (out need not be 16-byte aligned)
+        } else {
+            out[i] = t.x;
+            if (i + 1 < n) out[i + 1] = t.y;
+            if (i + 2 < n) out[i + 2] = t.z;
+        }
+    }
+}
+
+template <int KT>
+static void launch_dense_wgrad(const DenseWgradArgs &g, dim3 grid, hipStream_t st)
+{
+    const size_t lds = static_cast<size_t>(6) * 16 * KT * kWgradPitch + static_cast<size_t>(2) * 2 * KT * 1024 + 2 * kDenseWaves * 4;
+    hipLaunchKernelGGL((dense_wgrad_split_kernel<KT>), grid, dim3(64 * kDenseWaves), lds, st, g);
+}
+
+static int dense_wgrad_groups(int64_t N, int64_t T)
+{
+    const int64_t chunks = N * ((T + 31) / 32);
+    return static_cast<int>(chunks < compute_units() ? chunks : compute_units());
+}
+
+}  // namespace slayer
+
+extern "C" int slayer_dense_rows_grad_weight_supported(int64_t N, int64_t K, int64_t O, int64_t T)
+{
+    const int64_t lim = (1LL << 31) - 64;
+    return N >= 1 && K >= 1 && K <= 448 && O >= 1 && O <= 256 && T >= 4 && T % 4 == 0 && K * T * 4 < lim && O * T * 4 < lim &&
+           N * ((T + 31) / 32) < (1LL << 31);
+}
+
+extern "C" int64_t slayer_dense_rows_grad_weight_workspace_bytes(int64_t N, int64_t K, int64_t O, int64_t T)
+{
+    if (N < 1 || K < 1 || O < 1 || T < 1) return 0;
+    return static_cast<int64_t>(slayer::dense_wgrad_groups(N, T)) * slayer::dense_wgrad_pitch(O, K) * 4;
+}
+
+extern "C" int slayer_dense_rows_grad_weight_f32(float *gradW, const float *gradOut, const float *x, void *workspace, int64_t N,
+                                                 int64_t K, int64_t O, int64_t T, void *stream)
+{
+    using namespace slayer;
+    if (N < 0 || K < 0 || O < 0 || T < 0) return SLAYER_EINVAL;
+    if (K == 0 || O == 0) return SLAYER_OK;
+    if (!gradW) return SLAYER_EINVAL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (N == 0 || T == 0) {
+        const int n = static_cast<int>(O * K);   // (a sum over no rows: zeros, from a kernel a caller may capture)
+        hipLaunchKernelGGL(dense_wgrad_sum_kernel, dim3((n + 63) / 64), dim3(256), 0, st, gradW, static_cast<const float *>(nullptr), 0, n, dense_wgrad_pitch(O, K));
+        return launch_status();
+    }
+    if (!gradOut || !x || !workspace) return SLAYER_EINVAL;
+    if (!slayer_dense_rows_grad_weight_supported(N, K, O, T) || !aligned16(gradOut) || !aligned16(x) || !aligned16(workspace))
+        return SLAYER_EUNSUPPORTED;
+    const int chunksPerItem = static_cast<int>((T + 31) / 32);
+    const int64_t chunks = N * chunksPerItem;
+    const int groups = dense_wgrad_groups(N, T);
+    // up to 208 inputs a launch; more go in even blocks
+    const int blocks = static_cast<int>((K + kWgradMaxInputs - 1) / kWgradMaxInputs);
+    const int per = static_cast<int>(((K + blocks - 1) / blocks + 15) / 16 * 16);
+    const dim3 grid(static_cast<unsigned>(groups), 1);
+    for (int k0 = 0; k0 < K; k0 += per) {
+        const int kEnd = static_cast<int>(K < k0 + per ? K : k0 + per);
+        DenseWgradArgs g{static_cast<float *>(workspace), gradOut, x, static_cast<int>(N), static_cast<int>(O), static_cast<int>(K),
+                         static_cast<int>(T), k0, kEnd, chunksPerItem, static_cast<uint32_t>(chunks)};
+        switch ((kEnd - k0 + 15) / 16) {
+#define SLAYER_DENSE_WGRAD(KT) case KT: launch_dense_wgrad<KT>(g, grid, st); break
+            SLAYER_DENSE_WGRAD(1); SLAYER_DENSE_WGRAD(2); SLAYER_DENSE_WGRAD(3); SLAYER_DENSE_WGRAD(4); SLAYER_DENSE_WGRAD(5);
+            SLAYER_DENSE_WGRAD(6); SLAYER_DENSE_WGRAD(7); SLAYER_DENSE_WGRAD(8); SLAYER_DENSE_WGRAD(9); SLAYER_DENSE_WGRAD(10);
+            SLAYER_DENSE_WGRAD(11); SLAYER_DENSE_WGRAD(12);
+            default: launch_dense_wgrad<13>(g, grid, st); break;
+#undef SLAYER_DENSE_WGRAD
+        }
+    }
+    const int n = static_cast<int>(O * K);
+    hipLaunchKernelGGL(dense_wgrad_sum_kernel, dim3((n + 63) / 64), dim3(256), 0, st, gradW, static_cast<const float *>(workspace),
+                       groups, n, dense_wgrad_pitch(O, K));
+    return launch_status();
+}

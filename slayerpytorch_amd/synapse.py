@@ -16,7 +16,8 @@ from .slayerCuda import _check_device, _check_input, _on_device_of, _ptr
 
 __all__ = ["conv", "convGradInput", "convGradWeight", "outShape", "supported", "synapseConv", "synapseConvTranspose",
            "denseEvents", "denseEventsGradWeight", "denseEventsSupported", "synapseDenseEvents", "denseRows",
-           "denseRowsSupported", "denseRowsPays", "synapseDenseRows"]
+           "denseRowsSupported", "denseRowsPays", "synapseDenseRows", "denseRowsGradWeight",
+           "denseRowsGradWeightSupported"]
 
 
 def _pair(v, name):
@@ -319,6 +320,34 @@ class _synapseDenseEventsFunction(torch.autograd.Function):
         return gradInput, gradWeight, None, None
 
 
+def denseRowsGradWeightSupported(N, K, O, T):
+    """Whether ``denseRowsGradWeight`` takes these extents (the limits the header states)."""
+    return bool(_lib.load().slayer_dense_rows_grad_weight_supported(N, K, O, T))
+
+
+def denseRowsGradWeight(gradOutput, input):
+    """Weight gradient of the dense layer's product ``out[n] = weight @ input[n]``, ``input`` (N, K, T),
+    ``gradOutput`` (N, O, T): ``sum_n gradOutput[n] @ input[n].T`` as (O, K), on bf16 matrix instructions over split
+    operands (``slayer_dense_rows_grad_weight_f32``), for layers with up to 448 inputs and 256 outputs."""
+    _check_input(gradOutput, "gradOutput")
+    _check_input(input, "input")
+    _check_device(gradOutput, input, "gradOutput", "input")
+    if input.dim() != 3 or gradOutput.dim() != 3 or gradOutput.shape[0] != input.shape[0] \
+            or gradOutput.shape[2] != input.shape[2]:
+        raise RuntimeError("denseRowsGradWeight takes gradOutput (N, O, T) and input (N, K, T); got %r and %r"
+                           % (tuple(gradOutput.shape), tuple(input.shape)))
+    N, K, T = (int(v) for v in input.shape)
+    O = int(gradOutput.shape[1])
+    lib = _lib.load()
+    gradW = torch.empty((O, K), dtype=input.dtype, device=input.device)
+    nbytes = lib.slayer_dense_rows_grad_weight_workspace_bytes(N, K, O, T)
+    workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=input.device)
+    with _on_device_of(input) as stream:
+        _lib.check(lib.slayer_dense_rows_grad_weight_f32(_ptr(gradW), _ptr(gradOutput), _ptr(input), _ptr(workspace),
+                                                         N, K, O, T, stream), "slayer_dense_rows_grad_weight_f32")
+    return gradW
+
+
 DENSE_ROWS_MAX_INPUTS = 448   # two launches of slayer_dense_rows_f32; beyond that the library product
 
 
@@ -347,7 +376,10 @@ class _synapseDenseRowsFunction(torch.autograd.Function):
             else:
                 gradInput = torch.bmm(weight.t().unsqueeze(0).expand(N, K, O), gradOutput)
         if ctx.needs_input_grad[1]:
-            gradWeight = torch.bmm(gradOutput, input.transpose(1, 2)).sum(0)
+            if N * T >= 2048 and denseRowsGradWeightSupported(N, K, O, T):
+                gradWeight = denseRowsGradWeight(gradOutput, input)
+            else:
+                gradWeight = torch.bmm(gradOutput, input.transpose(1, 2)).sum(0)
         return gradInput, gradWeight
 
 

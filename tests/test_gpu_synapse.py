@@ -416,6 +416,60 @@ def test_dense_rows_product(case, transposed):
     assert torch.equal(got, synapse.denseRows(dev(x), dev(w), transposed))            # the same bits every time
 
 
+# (N, K, O, T, spike input)
+DENSE_ROWS_GRAD_WEIGHT_CASES = [
+    (2, 24, 20, 64, False),        # two tiles of inputs, one wavefront at work
+    (3, 200, 256, 300, False),     # the long-sequence network: 13 tiles of inputs, all wavefronts, a chunk of 12 samples at the end
+    (5, 37, 70, 124, True),        # sizes that divide by nothing: a sum row that is not a multiple of four long
+    (2, 208, 256, 96, True),       # the most inputs of one launch
+    (2, 256, 200, 100, True),      # two blocks of 128 inputs; 200 outputs: a wavefront with 8 rows
+    (2, 448, 30, 100, False),      # the most inputs: three blocks
+    (70, 16, 250, 32, True),       # one chunk per item, more items than one per work-group... 70 chunks
+    (1, 16, 16, 4, False),         # a single chunk of four samples
+    (6, 128, 128, 3000, True),     # long rows: more chunks than work-groups, several per group
+]
+
+
+@pytest.mark.parametrize("case", DENSE_ROWS_GRAD_WEIGHT_CASES)
+def test_dense_rows_grad_weight(case):
+    # the dense layer's weight gradient on bf16 matrix instructions over split operands: every element within 1e-6 of
+    # the sum of its terms' magnitudes (the bound the header states), on spikes and on dense inputs of mixed magnitude
+    N, K, O, T, spikes = case
+    rng = np.random.default_rng(N + K + O + T)
+    x = dense_input(rng, (N, K, T), 0.04, True) if spikes else \
+        (rng.standard_normal((N, K, T)) * np.exp2(rng.integers(-8, 8, (N, K, T)))).astype(np.float32)
+    g = (rng.standard_normal((N, O, T)) * np.exp2(rng.integers(-6, 6, (N, O, T)))).astype(np.float32)
+    ref = np.einsum("not,nkt->ok", g.astype(np.float64), x.astype(np.float64))
+    scale = np.einsum("not,nkt->ok", np.abs(g).astype(np.float64), np.abs(x).astype(np.float64))
+    got = synapse.denseRowsGradWeight(dev(g), dev(x))
+    assert got.shape == (O, K)
+    err = np.abs(host(got).astype(np.float64) - ref)
+    assert np.all(err <= 1e-6 * scale + 1e-30), float((err / (scale + 1e-30)).max())
+    assert torch.equal(got, synapse.denseRowsGradWeight(dev(g), dev(x)))                # the same bits every time
+
+
+def test_dense_rows_grad_weight_status_codes_and_limits():
+    lib = _lib.load()
+    t = torch.full((4096,), 7.0, device="cuda")
+    p = t.data_ptr()
+    fn = lib.slayer_dense_rows_grad_weight_f32
+    assert fn(None, None, None, None, 1, 0, 5, 8, None) == 0                              # no weights: nothing to do
+    assert fn(None, p, p, p, 1, 5, 5, 8, None) == 1
+    assert fn(p, p, p, None, 1, 5, 5, 8, None) == 1
+    assert fn(p, p, p, p, 1, 5, 5, 6, None) == 2                                          # T % 4 != 0
+    assert fn(p, p + 4, p, p, 1, 5, 5, 8, None) == 2                                      # gradOut not 16-byte aligned
+    assert fn(p, p, p, p, 1, 449, 5, 8, None) == 2 and fn(p, p, p, p, 1, 5, 257, 8, None) == 2
+    assert fn(p + 4, None, None, None, 0, 3, 5, 8, None) == 0                             # an empty batch: zeros
+    torch.cuda.synchronize()
+    assert host(t[1:16]).tolist() == [0.0] * 15 and host(t[16:18]).tolist() == [7.0, 7.0] and float(t[0]) == 7.0
+    assert not synapse.denseRowsGradWeightSupported(1, 5, 5, 6) and synapse.denseRowsGradWeightSupported(1, 448, 256, 8)
+    assert lib.slayer_dense_rows_grad_weight_workspace_bytes(0, 5, 5, 8) == 0
+    # one row of sums (padded to a multiple of four) for each of the 2 x 3 chunks
+    assert lib.slayer_dense_rows_grad_weight_workspace_bytes(2, 5, 5, 68) == 6 * 28 * 4
+    with pytest.raises(RuntimeError, match="denseRowsGradWeight takes"):
+        synapse.denseRowsGradWeight(torch.zeros((1, 5, 8), device="cuda"), torch.zeros((2, 4, 8), device="cuda"))
+
+
 def test_dense_rows_status_codes_and_limits():
     lib = _lib.load()
     t = torch.full((4096,), 7.0, device="cuda")
@@ -437,7 +491,7 @@ def test_dense_rows_status_codes_and_limits():
 
 
 def test_dense_layer_with_few_inputs_runs_dense_rows(monkeypatch):
-    """_denseLayer with 200 inputs: product and input gradient from synapse.denseRows, against the library products
+    """_denseLayer with 200 inputs: product and both gradients from synapse.denseRows*, against the library products
     (DENSE_ROWS = False): outputs and all gradients to rounding."""
     from slayerpytorch_amd import slayer as slayer_module
     params = {"type": "SRMALPHA", "theta": 10, "tauSr": 10.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
@@ -450,16 +504,19 @@ def test_dense_layer_with_few_inputs_runs_dense_rows(monkeypatch):
     calls = []
     real = synapse.denseRows
     monkeypatch.setattr(synapse, "denseRows", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    realGrad, gradCalls = synapse.denseRowsGradWeight, []
+    monkeypatch.setattr(synapse, "denseRowsGradWeight", lambda *a, **k: (gradCalls.append(1), realGrad(*a, **k))[1])
     for x0 in (dense_input(rng, (4, 200, 1, 1, T), 0.03, True), rng.standard_normal((4, 200, 1, 1, T)).astype(np.float32)):
         results = []
         for mode in (True, False):
             monkeypatch.setattr(slayer_module, "DENSE_ROWS", mode)
             x = dev(x0).requires_grad_(True)
             fc.weight.grad = None
-            n = len(calls)
+            n, m = len(calls), len(gradCalls)
             y = fc(x)
             y.backward(g)
             assert (len(calls) - n) == (2 if mode else 0)        # the product and the input gradient
+            assert (len(gradCalls) - m) == (1 if mode else 0)    # the weight gradient
             results.append((host(y), host(x.grad), host(fc.weight.grad)))
         for a, b in zip(*results):
             assert rel_err(a, b) <= 1e-5
