@@ -18,6 +18,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "fir_core.h"   // split_bf16, mfma_bf16
 
 namespace slayer {
 
@@ -918,6 +919,299 @@ __global__ __launch_bounds__(512) void synapse_gather_mfma_kernel(GatherMfmaArgs
     }
 }
 
+// ---- gather on the matrix cores, bf16 instructions over split operands ---------------------------------------
+// The same work-group, patch and loop as above, with v_mfma_f32_16x16x32_bf16 in place of the fp32 instruction: 32
+// taps per instruction in half the time of the fp32 instruction's four.  Every fp32 number is the sum of three bf16
+// numbers (its upper 16 bits, those of the remainder, and those of what is left), so a product of two is the sum
+// of nine partial products, of which the six largest are kept (the error, below 2^-22 of |x| |w| per term, is that
+// of the fp32 sum itself).  The weights are split once per work-group, in LDS in the register layout of the
+// instruction's second operand ([pass][channel tile][group of 32 taps][part][lane], 16 bytes each).  The patch
+// stays fp32: lane (r, h) reads its sample r of the 8 taps 32 G + 8 h .. + 7 as eight dwords and splits them in
+// registers - or only packs their upper halves when the patch holds nothing else, which the staging wavefronts
+// note per patch (spike tensors: 0 and 1 / Ts with few significant bits): three products instead of six.
+// A pass has room for 5 groups (160 taps >= the 144 of a pass; taps beyond the pass read the zero row and carry zero
+// weights).  With at most two (pass, channel tile) sets of weights the two patches of the kernel above fit beside
+// them; with up to four there is one patch, written between two barriers after the matrix work.  Numbers below
+// 2^-126 in a part are flushed by the instruction; a non-finite input sample gives NaN where the fp32 sum may
+// give an infinity.
+constexpr int kGsGroups = 5;
+constexpr int kGsUnitBytes = kGsGroups * 3 * 1024;      // weights of one (pass, channel tile)
+
+template <int OT, bool BACKWARD, bool DOUBLE>
+__global__ __launch_bounds__(512) void synapse_gather_split_kernel(GatherMfmaArgs g)
+{
+    extern __shared__ __align__(16) float lds[];
+    char *const ldsBytes = reinterpret_cast<char *>(lds);
+    constexpr int NG = kGsGroups;
+    constexpr int STRIDE = DOUBLE ? 2 * kGmRow : kGmRow;     // between patch rows (the rows of two patches alternate)
+    constexpr int PATCH = DOUBLE ? 2 * kGmBuf : kGmBuf;
+    typedef const float __attribute__((address_space(3))) *LdsFloat;
+    typedef const uint4_ext __attribute__((address_space(3))) *LdsUint4;
+    const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char *)ldsBytes));
+    uint32_t rest = xcd_contiguous(blockIdx.x, gridDim.x);
+    uint32_t qq = fastdiv(rest, g.byOGroups);
+    const int og = static_cast<int>(rest - qq * g.byOGroups.d);
+    rest = qq; qq = fastdiv(rest, g.byGroups);
+    const int grp = static_cast<int>(rest - qq * g.byGroups.d);
+    const int slice = static_cast<int>(qq);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, h = lane >> 4;
+    const int KK = g.KH * g.KW;
+    const int64_t srcPlane = static_cast<int64_t>(g.SH) * g.SW * g.T, dstPlane = static_cast<int64_t>(g.DH) * g.DW * g.T;
+    const int rowBytes = g.SW * g.T * 4, pixBytes = g.T * 4, planeBytes = static_cast<int>(srcPlane) * 4;
+    BufferRsrc srcB = make_buffer(g.src), dstB = make_buffer(g.dst);   // (of the batch item at hand: set by place())
+
+    // weights: unit (pass, ot), group G, part, lane (r, h): taps 32 G + 8 h .. + 7 of the pass for channel
+    // 16 (og OT + ot) + r
+    uint4_ext *const wl = reinterpret_cast<uint4_ext *>(ldsBytes + PATCH);
+    uint32_t *const flags = reinterpret_cast<uint32_t *>(ldsBytes + PATCH + g.passes * OT * kGsUnitBytes);   // [2][8]
+    for (int e = tid; e < g.passes * OT * NG * 64; e += 512) {
+        const int l = e & 63, G = (e >> 6) % NG, po = (e >> 6) / NG;
+        const int ot = po % OT, pass = po / OT;
+        const int m = (og * OT + ot) * 16 + (l & 15);
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int k = 32 * G + 8 * (l >> 4) + j;
+            const int cl = static_cast<int>(fastdiv(static_cast<uint32_t>(k), g.byKK)), ij = k - cl * KK, q = pass * g.chansPerPass + cl;
+            v[j] = 0.f;
+            if (cl < g.chansPerPass && q < g.Qg && m < g.Mg) {
+                const int64_t idx = BACKWARD ? (static_cast<int64_t>(grp * g.Og + q) * g.Cg + m) * KK + ij
+                                             : (static_cast<int64_t>(grp * g.Og + m) * g.Cg + q) * KK + ij;
+                v[j] = g.w[idx];
+            }
+        }
+        const SplitPlanes sp = split_bf16(v);
+        uint4_ext *unit = wl + (po * NG + G) * 3 * 64 + l;
+        unit[0] = sp.hi;
+        unit[64] = sp.mid;
+        unit[128] = sp.lo;
+    }
+    if (tid < (DOUBLE ? 2 : 1) * (kGmRow / 4)) lds[kGmMaxRows * STRIDE / 4 + tid] = 0.f;   // the zero row of every patch
+
+    // this lane's sample r (of the first half of a step; the second lies 64 bytes on) of tap 32 G + 8 h + e
+    int aTab[NG][8];
+#pragma unroll
+    for (int G = 0; G < NG; ++G)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int k = 32 * G + 8 * h + e;
+            const uint32_t cl = fastdiv(static_cast<uint32_t>(k), g.byKK);
+            const int ij = k - static_cast<int>(cl * g.byKK.d);
+            const int i = static_cast<int>(fastdiv(static_cast<uint32_t>(ij), g.byKW));
+            const int j = ij - i * g.KW;
+            const int row = static_cast<int>(cl) < g.chansPerPass
+                ? (static_cast<int>(cl) * g.KH + i) * g.WX + wave * g.mulW + j * g.stepW + g.xBias : kGmMaxRows;
+            aTab[G][e] = static_cast<int>(ldsBase) + row * STRIDE + (r << 2);
+        }
+    const uint32_t wAddr = ldsBase + PATCH + lane * 16;
+
+    int oOff[OT];
+#pragma unroll
+    for (int ot = 0; ot < OT; ++ot) {
+        const int m = (og * OT + ot) * 16 + r;
+        oOff[ot] = masked_offset(m < g.Mg, m * static_cast<int>(dstPlane) * 4 + h * 16);
+    }
+
+    // This lane copies unit u (samples 4u..4u+3 of the step) of patch rows tid / 8 + 64 m
+    constexpr int NS = 8;
+    const int u = tid & 7;
+    const int stageAddr = (tid >> 3) * STRIDE + (u << 4);
+
+    const int p0 = slice * g.pairsPerSlice, p1 = min(g.pairs, p0 + g.pairsPerSlice);
+    int sOff[NS];
+    int pixNext = 0;          // byte offset of this wavefront's destination pixel in a channel plane, or -1
+    auto place = [&](int blockOfAll) {
+        const int n = static_cast<int>(fastdiv(static_cast<uint32_t>(blockOfAll), g.byBlocks));
+        const int block = blockOfAll - n * static_cast<int>(g.byBlocks.d);
+        srcB = make_buffer(g.src + (static_cast<int64_t>(n) * g.SC + static_cast<int64_t>(grp) * g.Qg) * srcPlane);
+        const int a = static_cast<int>(fastdiv(static_cast<uint32_t>(block), g.byBlocksPerRow));
+        const int b0 = (block - a * g.blocksPerRow) * kGmPix;
+        const int nv = min(kGmPix, g.DW - b0);
+        const int xLimit = (nv - 1) * g.mulW + (g.KW - 1) * (g.stepW < 0 ? -g.stepW : g.stepW) + 1;
+        const int y0 = a * g.mulH + g.offH, x0 = b0 * g.mulW + g.offW - g.xBias;
+#pragma unroll
+        for (int m = 0; m < NS; ++m) {
+            const int row = (tid >> 3) + 64 * m;
+            const uint32_t cl = fastdiv(static_cast<uint32_t>(row), g.byPatch);
+            const int rem = row - static_cast<int>(cl * g.byPatch.d);
+            const int i = static_cast<int>(fastdiv(static_cast<uint32_t>(rem), g.byWX));
+            const int x = rem - i * g.WX;
+            const int y = y0 + i * g.stepH, xx = x0 + x;
+            const bool ok = row < g.rows && x < xLimit && static_cast<unsigned>(y) < static_cast<unsigned>(g.SH) &&
+                            static_cast<unsigned>(xx) < static_cast<unsigned>(g.SW);
+            sOff[m] = masked_offset(ok, static_cast<int>(cl) * planeBytes + y * rowBytes + xx * pixBytes + u * 16);
+        }
+        const int b = b0 + wave;
+        pixNext = b < g.DW ? (a * g.DW + b) * pixBytes : -1;
+        return n;
+    };
+    auto issue = [&](float4 (&R)[NS], int st, int pass, bool more) {
+        const int uniform = (st << 7) + pass * g.chansPerPass * planeBytes;
+        const bool live = more && (st << 5) + (u << 2) < g.T;
+#pragma unroll
+        for (int m = 0; m < NS; ++m) R[m] = buffer_load4<0>(srcB, live ? sOff[m] : kOutOfRange, uniform);
+    };
+    // registers -> patch; a wavefront notes whether any of its samples has more than the upper 16 bits
+    auto stage = [&](const float4 (&R)[NS], int buf) {
+        uint32_t low = 0;
+#pragma unroll
+        for (int m = 0; m < NS; ++m) {
+            if ((tid >> 3) + 64 * m < kGmMaxRows) *reinterpret_cast<float4 *>(ldsBytes + buf * kGmRow + stageAddr + m * 64 * STRIDE) = R[m];
+            low |= (__builtin_bit_cast(uint32_t, R[m].x) | __builtin_bit_cast(uint32_t, R[m].y)) |
+                   (__builtin_bit_cast(uint32_t, R[m].z) | __builtin_bit_cast(uint32_t, R[m].w));
+        }
+        const bool any = __builtin_amdgcn_ballot_w64((low & 0xffffu) != 0u) != 0;
+        if (lane == 0) flags[buf * 8 + wave] = any ? 1u : 0u;
+    };
+
+    f32x4 acc[2][OT];
+    auto clear = [&]() {
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int ot = 0; ot < OT; ++ot) acc[hf][ot] = f32x4{0.f, 0.f, 0.f, 0.f};
+    };
+    // the matrix work of one pass on the patch in buffer BUF; HALVES = 1 when the second half of the step lies past
+    // the end of the row.  The samples of a group of taps are read while the group before is multiplied.
+    auto multiply = [&](auto bufTag, auto halvesTag, int pass, int buf) {
+        constexpr int BUF = decltype(bufTag)::value, HALVES = decltype(halvesTag)::value;
+        const bool allParts = __builtin_amdgcn_ballot_w64(lane < 8 && flags[buf * 8 + (lane & 7)] != 0u) != 0;
+        const uint32_t wp = wAddr + pass * OT * kGsUnitBytes;
+        uint4_ext wq[OT][3];
+        float av[2][HALVES][8];
+        auto fetch = [&](int set, int G) {
+#pragma unroll
+            for (int hf = 0; hf < HALVES; ++hf)
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    av[set][hf][e] = *reinterpret_cast<LdsFloat>(static_cast<size_t>(static_cast<uint32_t>(aTab[G][e]) + BUF * kGmRow + hf * 64));
+        };
+        fetch(0, 0);
+#pragma unroll
+        for (int G = 0; G < NG; ++G) {
+            const int set = G & 1;
+            // (the weights of this group, then the samples of the next: a second set of weights a group ahead does
+            // not fit the registers)
+#pragma unroll
+            for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+                for (int part = 0; part < 3; ++part)
+                    wq[ot][part] = *reinterpret_cast<LdsUint4>(static_cast<size_t>(wp + ((ot * NG + G) * 3 + part) * 1024));
+            if (G + 1 < NG) fetch(set ^ 1, G + 1);
+            __builtin_amdgcn_sched_barrier(0);   // (issued here, ahead of the matrix instructions of this group)
+            if (allParts) {
+#pragma unroll
+                for (int hf = 0; hf < HALVES; ++hf) {
+                    const SplitPlanes a = split_bf16(av[set][hf]);
+#pragma unroll
+                    for (int ot = 0; ot < OT; ++ot) {
+                        acc[hf][ot] = mfma_bf16(a.hi, wq[ot][2], acc[hf][ot]);
+                        acc[hf][ot] = mfma_bf16(a.lo, wq[ot][0], acc[hf][ot]);
+                        acc[hf][ot] = mfma_bf16(a.mid, wq[ot][1], acc[hf][ot]);
+                        acc[hf][ot] = mfma_bf16(a.hi, wq[ot][1], acc[hf][ot]);
+                        acc[hf][ot] = mfma_bf16(a.mid, wq[ot][0], acc[hf][ot]);
+                        acc[hf][ot] = mfma_bf16(a.hi, wq[ot][0], acc[hf][ot]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int hf = 0; hf < HALVES; ++hf) {
+                    uint4_ext a;
+#pragma unroll
+                    for (int w2 = 0; w2 < 4; ++w2)
+                        a[w2] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, av[set][hf][2 * w2 + 1]),
+                                                      __builtin_bit_cast(uint32_t, av[set][hf][2 * w2]), 0x07060302u);
+#pragma unroll
+                    for (int ot = 0; ot < OT; ++ot) {
+                        acc[hf][ot] = mfma_bf16(a, wq[ot][2], acc[hf][ot]);
+                        acc[hf][ot] = mfma_bf16(a, wq[ot][1], acc[hf][ot]);
+                        acc[hf][ot] = mfma_bf16(a, wq[ot][0], acc[hf][ot]);
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto store = [&](int pix, int st) {
+        if (pix < 0) return;
+        const int uniform = pix + (st << 7);
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            const bool live = (st << 5) + hf * 16 + (h << 2) < g.T;
+#pragma unroll
+            for (int ot = 0; ot < OT; ++ot)
+                buffer_store4<0>(dstB, live ? oOff[ot] : kOutOfRange, uniform + hf * 64,
+                                       make_float4(acc[hf][ot][0], acc[hf][ot][1], acc[hf][ot][2], acc[hf][ot][3]));
+        }
+    };
+
+    {
+        // Trip k loads (pair, pass) number k of the range into registers, multiplies number k - 1 from its patch and
+        // then writes the registers to the other patch (or, with one patch, to the same after a barrier); the first
+        // trip only loads.  Pairs are numbered with the pixel block fastest, then the step, then the batch item.
+        const int perItem = static_cast<int>(g.byBlocks.d);   // pixel blocks of a batch item
+        int image = static_cast<int>(fastdiv(static_cast<uint32_t>(p0), g.byBlocks));
+        int inItem = p0 - image * perItem;
+        int item = static_cast<int>(fastdiv(static_cast<uint32_t>(image), g.bySteps));
+        int st = image - item * g.steps, pass = 0;
+        int stCur = 0, passCur = 0, pixCur = -1, nCur = -1, nNext = -1;
+        float4 R[NS];
+        int buf = DOUBLE ? 1 : 0;
+        bool first = true;
+        const int trips = (p1 - p0) * g.passes;
+        clear();
+#pragma nounroll
+        for (int k = 0;; ++k) {
+            const bool more = k < trips;
+            bool moved = first;
+            if (more && !first) {
+                if (++pass == g.passes) {
+                    pass = 0;
+                    moved = true;
+                    if (++inItem == perItem) {
+                        inItem = 0;
+                        if (++st == g.steps) {
+                            st = 0;
+                            ++item;
+                        }
+                    }
+                }
+            }
+            if (more && moved) nNext = place(item * perItem + inItem);
+            issue(R, st, pass, more);
+            __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the matrix work
+            if (!first) {
+                using I0 = std::integral_constant<int, 0>;
+                using I1 = std::integral_constant<int, 1>;
+                using I2 = std::integral_constant<int, 2>;
+                if ((stCur << 5) + 16 < g.T) {
+                    if (DOUBLE && buf != 0) multiply(I1{}, I2{}, passCur, 1);
+                    else multiply(I0{}, I2{}, passCur, 0);
+                } else {
+                    if (DOUBLE && buf != 0) multiply(I1{}, I1{}, passCur, 1);
+                    else multiply(I0{}, I1{}, passCur, 0);
+                }
+                if (passCur == g.passes - 1) {
+                    if (nCur >= 0) {
+                        dstB = make_buffer(g.dst + (static_cast<int64_t>(nCur) * g.DC + static_cast<int64_t>(grp) * g.Mg) * dstPlane);
+                        store(pixCur, stCur);
+                    }
+                    clear();
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (!more) break;
+            if (DOUBLE) buf ^= 1;
+            else __syncthreads();           // every wavefront has read the one patch
+            stage(R, buf);
+            stCur = st; passCur = pass; pixCur = pixNext; nCur = nNext;
+            __syncthreads();
+            first = false;
+        }
+    }
+}
+
 // ---- weight gradient on the matrix cores, input patch of a block of pixels in LDS -------------------
 // The kernel above fetches every input row once per tap that uses it (the working set of four
 // wavefronts does not stay in the 32 KB L1), 64 bytes at a time: it is bound by the number of cache
@@ -1066,35 +1360,63 @@ __global__ __launch_bounds__(256, 2) void synapse_wgrad_lds_kernel(WgradLdsArgs 
             }
         }
     };
+    // registers -> patch; a wavefront notes whether any of its samples has more than the upper 16 bits
+    uint32_t *const flags = reinterpret_cast<uint32_t *>(ldsBytes + 2 * kWgBuf);   // [2][4]
     auto stage = [&](const float4 (&R)[NS], int buf) {
+        uint32_t low = 0;
 #pragma unroll
-        for (int m = 0; m < NS; ++m) *reinterpret_cast<float4 *>(ldsBytes + buf + stageAddr + m * 32 * kWgRow) = R[m];
-    };
-#define SLAYER_WGRAD_LDS_MFMA(HALF, E)                                                                    \
-    _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)     \
-        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[HALF][mt].E, B[nt].E, acc[mt][nt], 0, 0, 0);
-    // (the second half of a row's last step may lie past the end of the row: nothing to add then)
-    auto multiply = [&](const float4 (&A)[2][MT], int buf, bool second) {
-        {
-            float4 B[NT];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) B[nt] = *reinterpret_cast<const float4 *>(ldsBytes + buf + bAddr[0][nt]);
-            SLAYER_WGRAD_LDS_MFMA(0, x)
-            SLAYER_WGRAD_LDS_MFMA(0, y)
-            SLAYER_WGRAD_LDS_MFMA(0, z)
-            SLAYER_WGRAD_LDS_MFMA(0, w)
+        for (int m = 0; m < NS; ++m) {
+            *reinterpret_cast<float4 *>(ldsBytes + buf + stageAddr + m * 32 * kWgRow) = R[m];
+            low |= (__builtin_bit_cast(uint32_t, R[m].x) | __builtin_bit_cast(uint32_t, R[m].y)) |
+                   (__builtin_bit_cast(uint32_t, R[m].z) | __builtin_bit_cast(uint32_t, R[m].w));
         }
-        if (second) {
-            float4 B[NT];
+        const bool any = __builtin_amdgcn_ballot_w64((low & 0xffffu) != 0u) != 0;
+        if (lane == 0) flags[(buf != 0 ? 4 : 0) + wave] = any ? 1u : 0u;
+    };
+    // One v_mfma_f32_16x16x32_bf16 takes a tile through all 32 samples of the step: slot 8 h + e of the reduction is
+    // sample 4 h + e (e < 4) or 16 + 4 h + e - 4 of the step, which is what a lane holds of a row of gradOut (two
+    // 16-byte loads) and reads of a patch row (two 16-byte reads).  The rows of gradOut are split into three bf16
+    // parts per number (fir_core.h); the patch rows are, too - or, when the patch holds nothing beyond the upper 16
+    // bits of its numbers (spikes), only packed: three products per tile instead of six.  Samples past the end of
+    // a row were loaded as zeros.
+    auto multiply = [&](const float4 (&A)[2][MT], int buf) {
+        const bool allParts = __builtin_amdgcn_ballot_w64(lane < 4 && flags[(buf != 0 ? 4 : 0) + (lane & 3)] != 0u) != 0;
+        SplitPlanes a[MT];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) B[nt] = *reinterpret_cast<const float4 *>(ldsBytes + buf + bAddr[1][nt]);
-            SLAYER_WGRAD_LDS_MFMA(1, x)
-            SLAYER_WGRAD_LDS_MFMA(1, y)
-            SLAYER_WGRAD_LDS_MFMA(1, z)
-            SLAYER_WGRAD_LDS_MFMA(1, w)
+        for (int mt = 0; mt < MT; ++mt) {
+            const float v[8] = {A[0][mt].x, A[0][mt].y, A[0][mt].z, A[0][mt].w, A[1][mt].x, A[1][mt].y, A[1][mt].z, A[1][mt].w};
+            a[mt] = split_bf16(v);
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const float4 b0 = *reinterpret_cast<const float4 *>(ldsBytes + buf + bAddr[0][nt]);
+            const float4 b1 = *reinterpret_cast<const float4 *>(ldsBytes + buf + bAddr[1][nt]);
+            const float v[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+            if (allParts) {
+                const SplitPlanes b = split_bf16(v);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    acc[mt][nt] = mfma_bf16(a[mt].lo, b.hi, acc[mt][nt]);
+                    acc[mt][nt] = mfma_bf16(a[mt].hi, b.lo, acc[mt][nt]);
+                    acc[mt][nt] = mfma_bf16(a[mt].mid, b.mid, acc[mt][nt]);
+                    acc[mt][nt] = mfma_bf16(a[mt].mid, b.hi, acc[mt][nt]);
+                    acc[mt][nt] = mfma_bf16(a[mt].hi, b.mid, acc[mt][nt]);
+                    acc[mt][nt] = mfma_bf16(a[mt].hi, b.hi, acc[mt][nt]);
+                }
+            } else {
+                uint4_ext bh;
+#pragma unroll
+                for (int w2 = 0; w2 < 4; ++w2)
+                    bh[w2] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, v[2 * w2 + 1]), __builtin_bit_cast(uint32_t, v[2 * w2]), 0x07060302u);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    acc[mt][nt] = mfma_bf16(a[mt].lo, bh, acc[mt][nt]);
+                    acc[mt][nt] = mfma_bf16(a[mt].mid, bh, acc[mt][nt]);
+                    acc[mt][nt] = mfma_bf16(a[mt].hi, bh, acc[mt][nt]);
+                }
+            }
         }
     };
-#undef SLAYER_WGRAD_LDS_MFMA
 
     {
         // Trip k of the loop loads pair p0 + k into registers, multiplies pair p0 + k - 1 from its LDS buffer
@@ -1104,7 +1426,7 @@ __global__ __launch_bounds__(256, 2) void synapse_wgrad_lds_kernel(WgradLdsArgs 
         int st = p0 - block * g.steps;
         float4 R[NS], A[2][MT];
         int buf = kWgBuf;
-        bool first = true, second = false;
+        bool first = true;
 #pragma nounroll
         for (int p = p0 - 1;; ++p) {
             const bool more = p + 1 < p1;
@@ -1118,10 +1440,9 @@ __global__ __launch_bounds__(256, 2) void synapse_wgrad_lds_kernel(WgradLdsArgs 
             float4 An[2][MT];
             issue(R, An, st, more);
             __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the pair's matrix work
-            if (!first) multiply(A, buf, second);
+            if (!first) multiply(A, buf);
             __builtin_amdgcn_sched_barrier(0);
             if (!more) break;
-            second = (st << 5) + 16 < s.T;
             buf = kWgBuf - buf;
             stage(R, buf);
 #pragma unroll
@@ -1288,23 +1609,55 @@ static int launch_gather_mfma(const GatherArgs &a, const SynGeom &s, bool stride
     g.byWX = make_fastdiv(static_cast<uint32_t>(g.WX));
     const int64_t blocks = base * g.slices;
     if (blocks >= (1LL << 31)) return SLAYER_EUNSUPPORTED;
-    const int ldsBytes = 2 * kGmBuf + passes * OT * 64 * kGmSteps * 4;
-    // more LDS than a kernel may use without asking; asked once per device (a host-side setting, no allocation)
-    static std::atomic<bool> raised[2][64];
-    int device = 0;
-    hipError_t err = hipGetDevice(&device);
-    if (err == hipSuccess && (device < 0 || device >= 64)) err = hipErrorInvalidDevice;
-    if (err == hipSuccess && !raised[OT - 1][device].load(std::memory_order_acquire)) {
-        const void *fn = OT == 2 ? reinterpret_cast<const void *>(&synapse_gather_mfma_kernel<2, BACKWARD>)
-                                 : reinterpret_cast<const void *>(&synapse_gather_mfma_kernel<1, BACKWARD>);
-        err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kGmBuf + kGmMaxWeightBytes);
-        if (err == hipSuccess) raised[OT - 1][device].store(true, std::memory_order_release);
+    if constexpr (BACKWARD) {
+        // The source is a gradient tensor: numbers with all their bits, which the bf16 kernel would have to split in
+        // registers, tap by tap (137 us against 120 us on the 16 -> 32 channel layer): the fp32 instructions stay.
+        const int ldsBytes = 2 * kGmBuf + passes * OT * 64 * kGmSteps * 4;
+        // more LDS than a kernel may use without asking; asked once per device (a host-side setting, no allocation)
+        static std::atomic<bool> raised[2][64];
+        int device = 0;
+        hipError_t err = hipGetDevice(&device);
+        if (err == hipSuccess && (device < 0 || device >= 64)) err = hipErrorInvalidDevice;
+        if (err == hipSuccess && !raised[OT - 1][device].load(std::memory_order_acquire)) {
+            const void *fn = OT == 2 ? reinterpret_cast<const void *>(&synapse_gather_mfma_kernel<2, BACKWARD>)
+                                     : reinterpret_cast<const void *>(&synapse_gather_mfma_kernel<1, BACKWARD>);
+            err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kGmBuf + kGmMaxWeightBytes);
+            if (err == hipSuccess) raised[OT - 1][device].store(true, std::memory_order_release);
+        }
+        if (err != hipSuccess) return note_hip_error(err);
+        const dim3 grid(static_cast<unsigned>(blocks));
+        if (OT == 2) hipLaunchKernelGGL((synapse_gather_mfma_kernel<2, BACKWARD>), grid, dim3(512), ldsBytes, st, g);
+        else hipLaunchKernelGGL((synapse_gather_mfma_kernel<1, BACKWARD>), grid, dim3(512), ldsBytes, st, g);
+        return launch_status();
+    } else {
+        const int units = passes * OT;
+        const bool twoPatches = units <= 2;      // (beside the weights of two sets; more leave room for one patch)
+        const int ldsBytes = (twoPatches ? 2 * kGmBuf : kGmBuf) + units * kGsUnitBytes + 64;
+        // more LDS than a kernel may use without asking; asked once per device (a host-side setting, no allocation)
+        static std::atomic<bool> raised[2][2][64];
+        int device = 0;
+        hipError_t err = hipGetDevice(&device);
+        if (err == hipSuccess && (device < 0 || device >= 64)) err = hipErrorInvalidDevice;
+        const void *fn = OT == 2 ? (twoPatches ? reinterpret_cast<const void *>(&synapse_gather_split_kernel<2, BACKWARD, true>)
+                                               : reinterpret_cast<const void *>(&synapse_gather_split_kernel<2, BACKWARD, false>))
+                                 : (twoPatches ? reinterpret_cast<const void *>(&synapse_gather_split_kernel<1, BACKWARD, true>)
+                                               : reinterpret_cast<const void *>(&synapse_gather_split_kernel<1, BACKWARD, false>));
+        if (err == hipSuccess && !raised[OT - 1][twoPatches][device].load(std::memory_order_acquire)) {
+            err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (twoPatches ? 2 * kGmBuf + 2 * kGsUnitBytes : kGmBuf + 4 * kGsUnitBytes) + 64);
+            if (err == hipSuccess) raised[OT - 1][twoPatches][device].store(true, std::memory_order_release);
+        }
+        if (err != hipSuccess) return note_hip_error(err);
+        const dim3 grid(static_cast<unsigned>(blocks));
+        if (OT == 2) {
+            if (twoPatches) hipLaunchKernelGGL((synapse_gather_split_kernel<2, BACKWARD, true>), grid, dim3(512), ldsBytes, st, g);
+            else hipLaunchKernelGGL((synapse_gather_split_kernel<2, BACKWARD, false>), grid, dim3(512), ldsBytes, st, g);
+        } else {
+            if (twoPatches) hipLaunchKernelGGL((synapse_gather_split_kernel<1, BACKWARD, true>), grid, dim3(512), ldsBytes, st, g);
+            else hipLaunchKernelGGL((synapse_gather_split_kernel<1, BACKWARD, false>), grid, dim3(512), ldsBytes, st, g);
+        }
+        return launch_status();
     }
-    if (err != hipSuccess) return note_hip_error(err);
-    const dim3 grid(static_cast<unsigned>(blocks));
-    if (OT == 2) hipLaunchKernelGGL((synapse_gather_mfma_kernel<2, BACKWARD>), grid, dim3(512), ldsBytes, st, g);
-    else hipLaunchKernelGGL((synapse_gather_mfma_kernel<1, BACKWARD>), grid, dim3(512), ldsBytes, st, g);
-    return launch_status();
 }
 
 template <bool BACKWARD>
@@ -1578,11 +1931,11 @@ static int launch_wgrad_lds_one(const WgradLdsArgs &g, unsigned blocks, hipStrea
     if (err == hipSuccess && (device < 0 || device >= 64)) err = hipErrorInvalidDevice;
     if (err == hipSuccess && !raised[device].load(std::memory_order_acquire)) {
         err = hipFuncSetAttribute(reinterpret_cast<const void *>(&synapse_wgrad_lds_kernel<MT, NT, NS>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kWgBuf);
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kWgBuf + 32);
         if (err == hipSuccess) raised[device].store(true, std::memory_order_release);
     }
     if (err != hipSuccess) return note_hip_error(err);
-    hipLaunchKernelGGL((synapse_wgrad_lds_kernel<MT, NT, NS>), dim3(blocks), dim3(256), 2 * kWgBuf, st, g);
+    hipLaunchKernelGGL((synapse_wgrad_lds_kernel<MT, NT, NS>), dim3(blocks), dim3(256), 2 * kWgBuf + 32, st, g);
     return launch_status();
 }
 
