@@ -126,6 +126,37 @@ def test_conv_grad_weight_matches_oracle(case, impl):
     close(got, ref, O.synapse_conv_grad_weight(np.abs(go), np.abs(x), w.shape, *a))
 
 
+# the cases whose forward pass and weight gradient run bf16 matrix instructions
+SPLIT_CASES = [c for c in CASES if c[5] >= 16 and (c[1] // c[10]) * c[6][0] * c[6][1] >= 96 and c[4] % 4 == 0 and c[4] >= 16]
+
+
+@pytest.mark.parametrize("case", SPLIT_CASES, ids=["%dx%dx%dx%dx%d-o%d-k%s-s%s-p%s-d%s-g%d" % c for c in SPLIT_CASES])
+@pytest.mark.parametrize("kind", ["spikes", "few bits", "one sample with all bits"])
+def test_conv_and_grad_weight_on_inputs_that_are_bf16_numbers(case, kind):
+    """Input samples with nothing below their upper 16 bits (spikes, small multiples of 1/8) take three of the six
+    partial products; a single sample with more bits anywhere in a patch switches that patch to all six.  Forward
+    pass and weight gradient against the oracle either way."""
+    N, C, H, W, T, Oc, K, s_, p_, d_, g_ = case
+    assert len(SPLIT_CASES) >= 8
+    rng = np.random.default_rng(17)
+    if kind == "spikes":
+        x = (rng.random((N, C, H, W, T)) < 0.1).astype(np.float32)
+    else:
+        x = (rng.integers(-40, 41, (N, C, H, W, T)) / 8.0).astype(np.float32) * (rng.random((N, C, H, W, T)) < 0.5)
+        x = x.astype(np.float32)
+    if kind == "one sample with all bits":
+        x[N - 1, C // 2, H // 2, W // 2, T // 3] = np.float32(np.pi)
+    w = rng.standard_normal((Oc, C // g_, K[0], K[1])).astype(np.float32)
+    a = (s_, p_, d_, g_)
+    close(host(synapse.conv(dev(x), dev(w), *a)), O.synapse_conv(x, w, *a).astype(np.float64),
+          O.synapse_conv(np.abs(x), np.abs(w), *a))
+    shape = O.synapse_geom(x.shape, w.shape, *a)[1]
+    go = rng.standard_normal(shape).astype(np.float32)
+    close(host(synapse.convGradWeight(dev(go), dev(x), w.shape, *a)),
+          O.synapse_conv_grad_weight(go, x, w.shape, *a).astype(np.float64),
+          O.synapse_conv_grad_weight(np.abs(go), np.abs(x), w.shape, *a))
+
+
 def test_unaligned_storage():
     """Tensors that start 4 bytes into an allocation take the one-sample-per-lane kernels."""
     case = (1, 3, 6, 7, 8, 4, (3, 3), 1, 1, 1, 1)
