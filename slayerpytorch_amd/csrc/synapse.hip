@@ -837,11 +837,12 @@ __global__ __launch_bounds__(512) void synapse_gather_mfma_kernel(GatherMfmaArgs
     // instruction writes 64 bytes of each of 16 channel rows, and a pixel's row is 4 T bytes long: cached stores, so
     // that L2 puts the pieces of a line together (streaming stores of these pieces: 137 us instead of 114 us on
     // the 16 -> 32 channel layer)
-    auto store = [&](bool leave, int pix, int st) {
-        const int uniform = leave ? pix + (st << 7) : 0;
+    auto store = [&](int pix, int st) {
+        if (pix < 0) return;
+        const int uniform = pix + (st << 7);
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            const bool live = leave && (st << 5) + hf * 16 + (h << 2) < g.T;
+            const bool live = (st << 5) + hf * 16 + (h << 2) < g.T;
 #pragma unroll
             for (int ot = 0; ot < OT; ++ot)
                 buffer_store4<0>(dstB, live ? oOff[ot] : kOutOfRange, uniform + hf * 64,
@@ -851,7 +852,8 @@ __global__ __launch_bounds__(512) void synapse_gather_mfma_kernel(GatherMfmaArgs
 
     {
         // Trip k of the loop loads (pair, pass) number k of the range into registers, multiplies number k - 1 from
-        // its LDS buffer ((k - 1) % 2) and then writes the registers to the other buffer.
+        // its LDS buffer ((k - 1) % 2) and then writes the registers to the other buffer: the loop's code exists
+        // once, its first trip only loads.
         // Pairs are numbered with the pixel block fastest, then the step, then the batch item: consecutive pairs of
         // a range are neighbouring patches of the same 32 samples, whose shared rows and columns come from L2
         // instead of from memory (with the step fastest every pair fetched all of its patch from beyond L2: 4.7 x
@@ -863,25 +865,15 @@ __global__ __launch_bounds__(512) void synapse_gather_mfma_kernel(GatherMfmaArgs
         int st = image - item * g.steps, pass = 0;        // .. step and pass that are loaded next
         int stCur = 0, passCur = 0, pixCur = -1, nCur = -1, nNext = -1;   // what is multiplied next
         float4 R[NS];
-        int buf = 0;
+        int buf = 1;
+        bool first = true;
         const int trips = (p1 - p0) * g.passes;
         clear();
-        if (trips > 0) {
-            // the first (pair, pass): loaded and written to a patch
-            nNext = place(item * perItem + inItem);
-            issue(R, st, pass, true);
-            stage(R, buf * kGmRow);
-            stCur = st; passCur = pass; pixCur = pixNext; nCur = nNext;
-            __syncthreads();
-        }
-        // Every trip issues the same instructions to memory - the loads of a patch, then the stores of a tile, with
-        // offsets out of range when there is nothing to load or the sums do not leave yet - so the wait for the loads
-        // before they are written to the patch leaves exactly the trip's stores in flight.
 #pragma nounroll
-        for (int k = 1; k <= trips; ++k) {
+        for (int k = 0;; ++k) {
             const bool more = k < trips;
-            bool moved = false;
-            if (more) {
+            bool moved = first;
+            if (more && !first) {
                 if (++pass == g.passes) {
                     pass = 0;
                     moved = true;
@@ -897,26 +889,32 @@ __global__ __launch_bounds__(512) void synapse_gather_mfma_kernel(GatherMfmaArgs
             if (more && moved) nNext = place(item * perItem + inItem);
             issue(R, st, pass, more);
             __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the matrix work
-            using I0 = std::integral_constant<int, 0>;
-            using I1 = std::integral_constant<int, 1>;
-            using I2 = std::integral_constant<int, 2>;
-            if ((stCur << 5) + 16 < g.T) {
-                if (buf == 0) multiply(I0{}, I2{}, passCur);
-                else multiply(I1{}, I2{}, passCur);
-            } else {
-                if (buf == 0) multiply(I0{}, I1{}, passCur);
-                else multiply(I1{}, I1{}, passCur);
+            if (!first) {
+                using I0 = std::integral_constant<int, 0>;
+                using I1 = std::integral_constant<int, 1>;
+                using I2 = std::integral_constant<int, 2>;
+                if ((stCur << 5) + 16 < g.T) {
+                    if (buf == 0) multiply(I0{}, I2{}, passCur);
+                    else multiply(I1{}, I2{}, passCur);
+                } else {
+                    if (buf == 0) multiply(I0{}, I1{}, passCur);
+                    else multiply(I1{}, I1{}, passCur);
+                }
+                if (passCur == g.passes - 1) {
+                    if (nCur >= 0) {
+                        dstB = make_buffer(g.dst + (static_cast<int64_t>(nCur) * g.DC + static_cast<int64_t>(grp) * g.Mg) * dstPlane);
+                        store(pixCur, stCur);
+                    }
+                    clear();
+                }
             }
-            const bool last = passCur == g.passes - 1;
-            dstB = make_buffer(g.dst + (static_cast<int64_t>(nCur) * g.DC + static_cast<int64_t>(grp) * g.Mg) * dstPlane);
-            store(last && pixCur >= 0, pixCur, stCur);
-            if (last) clear();
             __builtin_amdgcn_sched_barrier(0);
             if (!more) break;
             buf ^= 1;
             stage(R, buf * kGmRow);
             stCur = st; passCur = pass; pixCur = pixNext; nCur = nNext;
             __syncthreads();
+            first = false;
         }
     }
 }
@@ -1135,11 +1133,12 @@ __global__ __launch_bounds__(512) void synapse_gather_split_kernel(GatherMfmaArg
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    auto store = [&](bool leave, int pix, int st) {
-        const int uniform = leave ? pix + (st << 7) : 0;
+    auto store = [&](int pix, int st) {
+        if (pix < 0) return;
+        const int uniform = pix + (st << 7);
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            const bool live = leave && (st << 5) + hf * 16 + (h << 2) < g.T;
+            const bool live = (st << 5) + hf * 16 + (h << 2) < g.T;
 #pragma unroll
             for (int ot = 0; ot < OT; ++ot)
                 buffer_store4<0>(dstB, live ? oOff[ot] : kOutOfRange, uniform + hf * 64,
@@ -1149,8 +1148,8 @@ __global__ __launch_bounds__(512) void synapse_gather_split_kernel(GatherMfmaArg
 
     {
         // Trip k loads (pair, pass) number k of the range into registers, multiplies number k - 1 from its patch and
-        // then writes the registers to the other patch (or, with one patch, to the same after a barrier).  Pairs are
-        // numbered with the pixel block fastest, then the step, then the batch item.
+        // then writes the registers to the other patch (or, with one patch, to the same after a barrier); the first
+        // trip only loads.  Pairs are numbered with the pixel block fastest, then the step, then the batch item.
         const int perItem = static_cast<int>(g.byBlocks.d);   // pixel blocks of a batch item
         int image = static_cast<int>(fastdiv(static_cast<uint32_t>(p0), g.byBlocks));
         int inItem = p0 - image * perItem;
@@ -1158,25 +1157,15 @@ __global__ __launch_bounds__(512) void synapse_gather_split_kernel(GatherMfmaArg
         int st = image - item * g.steps, pass = 0;
         int stCur = 0, passCur = 0, pixCur = -1, nCur = -1, nNext = -1;
         float4 R[NS];
-        int buf = 0;
+        int buf = DOUBLE ? 1 : 0;
+        bool first = true;
         const int trips = (p1 - p0) * g.passes;
         clear();
-        if (trips > 0) {
-            // the first (pair, pass): loaded and written to a patch
-            nNext = place(item * perItem + inItem);
-            issue(R, st, pass, true);
-            stage(R, buf);
-            stCur = st; passCur = pass; pixCur = pixNext; nCur = nNext;
-            __syncthreads();
-        }
-        // Every trip issues the same instructions to memory - the loads of a patch, then the stores of a tile, with
-        // offsets out of range when there is nothing to load or the sums do not leave yet - so the wait for the loads
-        // before they are written to the patch leaves exactly the trip's stores in flight.
 #pragma nounroll
-        for (int k = 1; k <= trips; ++k) {
+        for (int k = 0;; ++k) {
             const bool more = k < trips;
-            bool moved = false;
-            if (more) {
+            bool moved = first;
+            if (more && !first) {
                 if (++pass == g.passes) {
                     pass = 0;
                     moved = true;
@@ -1192,20 +1181,25 @@ __global__ __launch_bounds__(512) void synapse_gather_split_kernel(GatherMfmaArg
             if (more && moved) nNext = place(item * perItem + inItem);
             issue(R, st, pass, more);
             __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the matrix work
-            using I0 = std::integral_constant<int, 0>;
-            using I1 = std::integral_constant<int, 1>;
-            using I2 = std::integral_constant<int, 2>;
-            if ((stCur << 5) + 16 < g.T) {
-                if (DOUBLE && buf != 0) multiply(I1{}, I2{}, passCur, 1);
-                else multiply(I0{}, I2{}, passCur, 0);
-            } else {
-                if (DOUBLE && buf != 0) multiply(I1{}, I1{}, passCur, 1);
-                else multiply(I0{}, I1{}, passCur, 0);
+            if (!first) {
+                using I0 = std::integral_constant<int, 0>;
+                using I1 = std::integral_constant<int, 1>;
+                using I2 = std::integral_constant<int, 2>;
+                if ((stCur << 5) + 16 < g.T) {
+                    if (DOUBLE && buf != 0) multiply(I1{}, I2{}, passCur, 1);
+                    else multiply(I0{}, I2{}, passCur, 0);
+                } else {
+                    if (DOUBLE && buf != 0) multiply(I1{}, I1{}, passCur, 1);
+                    else multiply(I0{}, I1{}, passCur, 0);
+                }
+                if (passCur == g.passes - 1) {
+                    if (nCur >= 0) {
+                        dstB = make_buffer(g.dst + (static_cast<int64_t>(nCur) * g.DC + static_cast<int64_t>(grp) * g.Mg) * dstPlane);
+                        store(pixCur, stCur);
+                    }
+                    clear();
+                }
             }
-            const bool last = passCur == g.passes - 1;
-            dstB = make_buffer(g.dst + (static_cast<int64_t>(nCur) * g.DC + static_cast<int64_t>(grp) * g.Mg) * dstPlane);
-            store(last && pixCur >= 0, pixCur, stCur);
-            if (last) clear();
             __builtin_amdgcn_sched_barrier(0);
             if (!more) break;
             if (DOUBLE) buf ^= 1;
@@ -1213,6 +1207,7 @@ __global__ __launch_bounds__(512) void synapse_gather_split_kernel(GatherMfmaArg
             stage(R, buf);
             stCur = st; passCur = pass; pixCur = pixNext; nCur = nNext;
             __syncthreads();
+            first = false;
         }
     }
 }
