@@ -344,6 +344,14 @@ int slayer_loihi_get_spikes_delayed_f32(float *s, float *v, float *u, const floa
  * time extent of 1 dropped), output [N][O][OH][OW][T] with
  * OH = (H + 2*padH - dilH*(KH-1) - 1) / strideH + 1 (0 when the filter does not fit), OW alike.
  * One batch item of the input and of the output must stay below 2 GiB (SLAYER_EUNSUPPORTED).
+ *
+ * Arithmetic: fp32 sums; the order of the additions depends on the geometry, not on the launch (no
+ * atomics).  The forward pass of layers with at least 16 output channels and about 100 or more taps
+ * per output, and the weight gradient of layers large enough for the matrix cores, multiply on bf16
+ * matrix instructions over operands split into three bf16 parts each (six of the nine partial
+ * products; three when the input holds nothing below the upper 16 bits of its numbers, as spike
+ * tensors do): every result within 1e-6 of the sum of its terms' magnitudes.  Parts below 2^-126 are
+ * flushed to zero, and a non-finite input sample gives NaN where an fp32 sum may give an infinity.
  */
 typedef struct slayer_synapse_geom {
     int32_t N, C, H, W, T;

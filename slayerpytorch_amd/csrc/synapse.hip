@@ -12,8 +12,10 @@
 // of a filter row in registers for layers with one or two destination channels).  The weight
 // gradient, a matrix product with time as the reduction axis, runs on the matrix cores from a
 // source patch in LDS (from global memory for patches that do not fit, and a vector kernel for
-// small or unaligned shapes); pooling has a streaming input gradient.  Work-groups that read the
-// same rows are kept on the same die (xcd_contiguous).
+// small or unaligned shapes); pooling has a streaming input gradient.  The forward gather and the
+// weight gradient multiply with bf16 matrix instructions over operands split into three bf16 parts
+// (fir_core.h); the input gradient, whose source is a gradient tensor, with the fp32 instruction.
+// Work-groups that read the same rows are kept on the same die (xcd_contiguous).
 #include <atomic>
 #include <type_traits>
 
