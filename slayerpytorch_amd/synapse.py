@@ -357,6 +357,12 @@ def denseRowsPays(N, K, O, T):
     return K <= DENSE_ROWS_MAX_INPUTS and N * T >= 2048 and O >= 16 and denseRowsSupported(N, K, O, T)
 
 
+def _aligned(t):
+    """``t`` contiguous and on a 16-byte boundary (a view that starts inside an allocation is copied)."""
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 class _synapseDenseRowsFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, weight):
@@ -366,7 +372,7 @@ class _synapseDenseRowsFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gradOutput):
         input, weight = ctx.saved_tensors
-        gradOutput = gradOutput.contiguous()
+        gradOutput = _aligned(gradOutput)
         gradInput = gradWeight = None
         N, K, T = input.shape
         O = weight.shape[0]
@@ -386,8 +392,9 @@ class _synapseDenseRowsFunction(torch.autograd.Function):
 def synapseDenseRows(input, weight):
     """``weight @ input[n]`` for every batch item (``input`` (N, K, T), ``weight`` (O, K)) with its gradients, for
     layers with few inputs: product and input gradient from ``denseRows`` (bf16 matrix instructions over split
-    operands, weights in registers), the weight gradient from the library."""
-    return _synapseDenseRowsFunction.apply(input.contiguous(), weight)
+    operands, weights in registers), the weight gradient from ``denseRowsGradWeight`` (the library's batched product
+    for more than 448 inputs or 256 outputs)."""
+    return _synapseDenseRowsFunction.apply(_aligned(input), weight)
 
 
 def synapseDenseEvents(input, weight, product=True, gradient=True):

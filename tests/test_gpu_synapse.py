@@ -553,6 +553,33 @@ def test_dense_layer_with_few_inputs_runs_dense_rows(monkeypatch):
             assert rel_err(a, b) <= 1e-5
 
 
+def test_dense_rows_layer_on_a_view_that_is_not_16_byte_aligned():
+    """synapseDenseRows copies an input (or an output gradient) that starts 4 bytes into an allocation; same values as
+    on an aligned tensor."""
+    rng = np.random.default_rng(23)
+    N, K, O, T = 2, 40, 32, 1024
+    x = rng.standard_normal((N, K, T)).astype(np.float32)
+    g = rng.standard_normal((N, O, T)).astype(np.float32)
+    w = dev(rng.standard_normal((O, K)).astype(np.float32))
+
+    def off(arr):
+        buf = torch.empty(arr.size + 1, dtype=torch.float32, device="cuda")
+        view = buf[1:].view(arr.shape)
+        view.copy_(torch.from_numpy(arr))
+        return view
+
+    results = []
+    for place in (dev, off):
+        xi = place(x).requires_grad_(True)
+        wi = w.clone().requires_grad_(True)
+        y = synapse.synapseDenseRows(xi, wi)
+        y.backward(place(g))
+        results.append((host(y), host(xi.grad), host(wi.grad)))
+    assert off(x).data_ptr() % 16 != 0
+    for a, b in zip(*results):
+        assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("shape", [((34, 34, 2), 40, 12), (50, 10, 33)])
 def test_dense_layer_sums_over_the_events_of_sparse_input(shape, monkeypatch):
     """_denseLayer with the event-driven product and weight gradient against the library products: same output and
