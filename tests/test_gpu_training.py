@@ -185,19 +185,24 @@ def test_dense_layer_density_follows_the_input_without_waiting(monkeypatch):
 
 
 # ------------------------------------------------------------------------------ HIP graph replay
-def test_training_step_replayed_by_capturedStep():
+@pytest.mark.parametrize("N,T", [(3, 100), (4, 512)], ids=["library dense products", "dense layers on the matrix-core kernels"])
+def test_training_step_replayed_by_capturedStep(N, T):
     """A whole training step - psp, spike, delay, dense, loss, backward - recorded by ``utils.capturedStep``.
-    Every replay, with eager work and synchronisations in between, must reproduce the eager step bit for bit."""
+    Every replay, with eager work and synchronisations in between, must reproduce the eager step bit for bit.  At
+    (4, 512) the first dense layer runs synapse.denseRows and denseRowsGradWeight (workspaces from torch's allocator
+    inside the capture)."""
     params = {"type": "SRMALPHA", "theta": 10, "tauSr": 4.0, "tauRef": 1.0, "scaleRef": 2, "tauRho": 1, "scaleRho": 1}
-    sim = {"Ts": 1.0, "tSample": 100}
+    sim = {"Ts": 1.0, "tSample": T}
     layer = snn.layer(params, sim).cuda()
     error = snn.loss({"neuron": params, "simulation": sim, "training": {"error": {"type": "SpikeTime"}}}).cuda()
     torch.manual_seed(2)
     fc1, fc2 = layer.dense(40, 32, weightScale=30).cuda(), layer.dense(32, 6, weightScale=30).cuda()
     delay = layer.delay(32).cuda()
-    x = (torch.rand((3, 40, 1, 1, 100)) < 0.1).float().cuda()
-    x2 = (torch.rand((3, 40, 1, 1, 100)) < 0.1).float().cuda()
-    target = (torch.rand((3, 6, 1, 1, 100)) < 0.05).float().cuda()
+    x = (torch.rand((N, 40, 1, 1, T)) < 0.1).float().cuda()
+    x2 = (torch.rand((N, 40, 1, 1, T)) < 0.1).float().cuda()
+    target = (torch.rand((N, 6, 1, 1, T)) < 0.05).float().cuda()
+    from slayerpytorch_amd import synapse
+    assert synapse.denseRowsPays(N, 40, 32, T) == (N * T >= 2048)
     batch = x.clone()
     leaves = [fc1.weight, fc2.weight, delay.delay]
     for p in leaves:
