@@ -431,8 +431,8 @@ DENSE_ROWS_CASES = [
 @pytest.mark.parametrize("transposed", [False, True])
 def test_dense_rows_product(case, transposed):
     # the dense layer's product and (transposed) input gradient on bf16 matrix instructions over split operands: every
-    # output within 1e-6 of the sum of its terms' magnitudes (the bound the header states; SUM_TOL for all synapse
-    # kernels is the north star's 1e-5), on spikes and on dense inputs of mixed magnitude
+    # output within 1e-6 of the sum of its terms' magnitudes (the bound the header states; the north star asks for
+    # 1e-5), on spikes and on dense inputs of mixed magnitude
     N, K, O, T, spikes = case
     rng = np.random.default_rng(N + K + O + T)
     x = dense_input(rng, (N, K, T), 0.04, True) if spikes else \
