@@ -157,6 +157,55 @@ def test_conv_and_grad_weight_on_inputs_that_are_bf16_numbers(case, kind):
           O.synapse_conv_grad_weight(np.abs(go), np.abs(x), w.shape, *a))
 
 
+def test_random_geometries_against_conv3d():
+    """60 seeded random layers with at least 16 output channels (the matrix-core kernels and what surrounds them: stride,
+    padding, dilation, groups, ragged extents; spike inputs, dense inputs, inputs with few bits and one sample with all
+    bits): forward pass and both gradients against torch's conv3d with a (KH, KW, 1) kernel and its autograd in
+    double precision on the CPU, within SUM_TOL of the sum of the terms' magnitudes."""
+    import torch.nn.functional as F
+    rng = np.random.default_rng(321)
+    done = 0
+    while done < 60:
+        g = int(rng.choice([1, 1, 1, 2]))
+        Cg, Og = int(rng.choice([4, 8, 11, 12, 16, 16, 24, 32, 48])), int(rng.choice([16, 16, 20, 32, 33, 48, 64]))
+        KH, KW = int(rng.choice([1, 2, 3, 3, 3, 5])), int(rng.choice([2, 3, 3, 3, 4, 5]))
+        C, Oc = Cg * g, Og * g
+        H, W = int(rng.integers(KH, 14)), int(rng.integers(KW, 20))
+        T, N = 4 * int(rng.integers(4, 30)), int(rng.integers(1, 4))
+        st = (int(rng.choice([1, 1, 1, 2])), int(rng.choice([1, 1, 1, 2])))
+        pd = (int(rng.integers(0, 3)), int(rng.integers(0, 3)))
+        dl = (int(rng.choice([1, 1, 1, 2])), int(rng.choice([1, 1, 1, 2])))
+        if H + 2 * pd[0] - dl[0] * (KH - 1) - 1 < 0 or W + 2 * pd[1] - dl[1] * (KW - 1) - 1 < 0:
+            continue
+        kind = done % 3
+        if kind == 0:
+            x = (rng.random((N, C, H, W, T)) < 0.1).astype(np.float32)
+        elif kind == 1:
+            x = rng.standard_normal((N, C, H, W, T)).astype(np.float32)
+        else:
+            x = (rng.integers(-16, 17, (N, C, H, W, T)) / 4.0).astype(np.float32)
+            x[0, 0, 0, 0, 0] = np.float32(0.1)
+        w = rng.standard_normal((Oc, Cg, KH, KW)).astype(np.float32)
+
+        def conv(xx, ww):
+            return F.conv3d(xx, ww.unsqueeze(-1), None, st + (1,), pd + (0,), dl + (1,), g)
+        xt, wt = torch.from_numpy(x).double().requires_grad_(True), torch.from_numpy(w).double().requires_grad_(True)
+        y = conv(xt, wt)
+        go = rng.standard_normal(tuple(y.shape)).astype(np.float32)
+        y.backward(torch.from_numpy(go).double())
+        xa, wa = xt.detach().abs().requires_grad_(True), wt.detach().abs().requires_grad_(True)
+        ya = conv(xa, wa)
+        ya.backward(torch.from_numpy(np.abs(go)).double())
+        a = (st, pd, dl, g)
+        what = "%s -> %d, %dx%d, %s" % ((N, C, H, W, T), Oc, KH, KW, a)
+        for got, ref, scale in ((synapse.conv(dev(x), dev(w), *a), y, ya),
+                                (synapse.convGradInput(dev(go), dev(w), x.shape, *a), xt.grad, xa.grad),
+                                (synapse.convGradWeight(dev(go), dev(x), w.shape, *a), wt.grad, wa.grad)):
+            err = (got.cpu().double() - ref.detach()).abs()
+            assert bool((err <= SUM_TOL * scale.detach() + 1e-30).all()), what
+        done += 1
+
+
 def test_unaligned_storage():
     """Tensors that start 4 bytes into an allocation take the one-sample-per-lane kernels."""
     case = (1, 3, 6, 7, 8, 4, (3, 3), 1, 1, 1, 1)
@@ -499,6 +548,33 @@ def test_dense_rows_grad_weight_status_codes_and_limits():
     assert lib.slayer_dense_rows_grad_weight_workspace_bytes(2, 5, 5, 68) == 6 * 28 * 4
     with pytest.raises(RuntimeError, match="denseRowsGradWeight takes"):
         synapse.denseRowsGradWeight(torch.zeros((1, 5, 8), device="cuda"), torch.zeros((2, 4, 8), device="cuda"))
+
+
+def test_dense_rows_kernels_on_random_shapes():
+    """120 seeded random shapes (1-448 inputs, 1-299 outputs, the limits of a launch and of a block among them; spikes and
+    dense inputs of mixed magnitude): product, input gradient and weight gradient within 1e-6 of the sum of the
+    terms' magnitudes."""
+    rng = np.random.default_rng(123)
+    for it in range(120):
+        N, K, Oc, T = int(rng.integers(1, 6)), int(rng.integers(1, 449)), int(rng.integers(1, 300)), 4 * int(rng.integers(1, 80))
+        if it % 7 == 0:
+            K = int(rng.choice([1, 31, 32, 33, 208, 209, 224, 225, 416, 448]))
+        if it % 11 == 0:
+            Oc = int(rng.choice([1, 15, 16, 17, 255, 256, 257, 290]))
+        x = (rng.random((N, K, T)) < 0.1).astype(np.float32) if it % 2 else \
+            (rng.standard_normal((N, K, T)) * np.exp2(rng.integers(-6, 6, (N, K, T)))).astype(np.float32)
+        w = rng.standard_normal((Oc, K)).astype(np.float32)
+        g = rng.standard_normal((N, Oc, T)).astype(np.float32)
+        x64, w64, g64 = x.astype(np.float64), w.astype(np.float64), g.astype(np.float64)
+        checks = [(synapse.denseRows(dev(x), dev(w)), "ok,nkt->not", (w64, x64)),
+                  (synapse.denseRows(dev(g), dev(w), transposed=True), "ok,not->nkt", (w64, g64))]
+        if synapse.denseRowsGradWeightSupported(N, K, Oc, T):
+            checks.append((synapse.denseRowsGradWeight(dev(g), dev(x)), "not,nkt->ok", (g64, x64)))
+        for got, spec, ops in checks:
+            ref = np.einsum(spec, *ops)
+            scale = np.einsum(spec, *[np.abs(o) for o in ops])
+            err = np.abs(host(got).astype(np.float64) - ref)
+            assert np.all(err <= 1e-6 * scale + 1e-30), (N, K, Oc, T, spec, float((err / (scale + 1e-30)).max()))
 
 
 def test_dense_rows_status_codes_and_limits():
